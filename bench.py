@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the PackKV hot path on one MI355X.
+
+A step = one fused decompress-attention decode (one layer, one query token per sequence) over a
+compressed KV cache resident in HBM.  Workload (BASELINE.json configs[1]): batch 16, 32 query /
+8 KV heads, head_dim 128, 32768 cached tokens per sequence, fp16, K ~ N(0,1) with four outlier
+channels x10, V ~ N(0,1), per-token quantisation at relative step 0.1, 64-token quant blocks.
+
+Prints ONE JSON line: the headline metric (us per layer, lower is better) with `roofline`
+(HBM, algorithmic compressed bytes / measured kernel time) and `cpu_baseline` (the
+decompress-then-attend path restated in PyTorch CPU ops, timed on this host on a bounded
+sample), plus encode / unpack throughput measured in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--ctx", type=int, default=32768)
+    ap.add_argument("--hq", type=int, default=32)
+    ap.add_argument("--hkv", type=int, default=8)
+    ap.add_argument("--rel", type=float, default=0.1)
+    ap.add_argument("--window", type=int, default=0, help="uncompressed fp16 tail tokens")
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip encode / unpack timing")
+    return ap.parse_args()
+
+
+def event_time_ms(torch, fn, iters):
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    e.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def cpu_baseline(torch, args, k1, v1, q1):
+    """Decompress-then-attend for ONE sequence in PyTorch CPU ops (the checker's restatement of
+    utils/compute.py:173-179 + models/llama.py:189-212), median of 5, scaled to the batch."""
+    from oracle import quant as oq
+    ck, zk, sk = oq.quant_ints(k1, 64, args.rel)
+    cv, zv, sv = oq.quant_ints(v1, 64, args.rel)
+    qq = q1.unsqueeze(2)
+
+    def step():
+        kd, vd = oq.dequant(ck, zk, sk), oq.dequant(cv, zv, sv)
+        return oq.eager_attention(qq, kd, vd)
+
+    for _ in range(2):
+        step()
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        step()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    per_seq = ts[len(ts) // 2]
+    return {
+        "value": per_seq * args.batch * 1e6, "unit": "us/layer", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "1 of %d sequences (dequantise + eager attention, %d tokens), median of 5, scaled x%d"
+                  % (args.batch, k1.shape[2], args.batch),
+    }
+
+
+def cpu_encoder(torch, args, k1):
+    """Single-thread scalar encoder on the host: the reference's own k_encode_cpu when its build is
+    present (oracle/_ref), else the restated C codec."""
+    import numpy as np
+    from oracle import codec, quant as oq
+    T = min(k1.shape[2], 4096)
+    c, _, _ = oq.quant_ints(k1[:, :, :T], 64, args.rel)
+    cm = oq.code_matrix(c).numpy()
+    kind = "reference" if codec.have_ref() else "port"
+    enc = codec.ref() if codec.have_ref() else codec.oracle()
+    try:
+        enc.encode(1, cm, 64, 128, 4)
+    except RuntimeError:
+        kind, enc = "port", codec.oracle()
+    t0 = time.perf_counter()
+    _, _, size = enc.encode(1, cm, 64, 128, 4)
+    dt = time.perf_counter() - t0
+    return {"value": cm.size * 2 / dt / 1e9, "unit": "GB/s of fp16 input", "cores": 1, "kind": kind,
+            "sample": "K codes of 1 sequence x %d tokens (%d channels), bit-pack only" % (T, cm.shape[1])}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from packkv_amd import ops, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, Hq, Hkv, T, Tw = args.batch, args.hq, args.hkv, args.ctx, args.window
+    Tc = T - Tw
+    assert Tc % 128 == 0, "compressed tokens must be a multiple of 128"
+
+    k, v = synth.make_kv(B, Hkv, T, seed=0, device=dev)
+    q = synth.make_q(B, Hq, seed=1, device=dev)
+    kc, vc = (k[:, :, :Tc].contiguous(), v[:, :, :Tc].contiguous()) if Tw else (k, v)
+    kw = k[:, :, Tc:].contiguous() if Tw else None
+    vw = v[:, :, Tc:].contiguous() if Tw else None
+
+    bits = ops.bits_for_rel(args.rel)
+    ke = ops.k_quant_encode(kc, args.rel, bits)
+    ve = ops.v_quant_encode(vc, args.rel, bits)
+    hidden = B * Hkv * 128
+    nblk_k, nblk_v = (Tc // 64) * (hidden // 128), (Tc // 128) * (hidden // 64)
+    fp16_bytes = 2 * Tc * hidden * 2
+    algo_bytes = (ke["size"] + ve["size"] + 8 * (nblk_k + nblk_v) + 8 * B * Tc
+                  + 2 * 2 * B * Hkv * Tw * 128 + 2 * 2 * B * Hq * 128)
+
+    out = torch.empty_like(q)
+
+    def step():
+        ops.attn_decode(q, ke, ve, kw, vw, out=out, variant=args.variant)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    s_ev = torch.cuda.Event(enable_timing=True)
+    e_ev = torch.cuda.Event(enable_timing=True)
+    s_ev.record()
+    for _ in range(args.steps):
+        step()
+    e_ev.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / args.steps
+    ms_kernel = s_ev.elapsed_time(e_ev) / args.steps
+
+    result = {
+        "metric": "fused decompress-attn decode us/layer",
+        "value": ms_step * 1e3, "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: GQA decode, batch %d, %d q / %d KV heads, head_dim 128, %d tokens"
+                               " (%d compressed + %d fp16 tail), rel %.3g, %d-bit codes"
+                               % (B, Hq, Hkv, T, Tc, Tw, args.rel, bits),
+                   "variant": args.variant},
+        "tokens_per_s": B / (ms_step * 1e-3),
+        "roofline": {"bound": "hbm", "achieved": algo_bytes / (ms_kernel * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": algo_bytes / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "kernel_ms": ms_kernel, "algorithmic_bytes": algo_bytes},
+        "compression": {"k_bytes": ke["size"], "v_bytes": ve["size"], "fp16_bytes": fp16_bytes,
+                        "ratio_k": fp16_bytes / 2 / ke["size"], "ratio_v": fp16_bytes / 2 / ve["size"]},
+    }
+
+    if not args.no_extras:
+        # encode: fused quantize + bit-pack, fp16 in -> stream out (GB/s of fp16 input consumed)
+        x_bytes = Tc * hidden * 2
+        k_ms = event_time_ms(torch, lambda: ops.k_quant_encode(kc, args.rel, bits, ke["stream"], ke["info"],
+                                                               want_size=False), 5)
+        v_ms = event_time_ms(torch, lambda: ops.v_quant_encode(vc, args.rel, bits, ve["stream"], ve["info"],
+                                                               want_size=False), 5)
+        codes = torch.empty(Tc, hidden, dtype=torch.uint8, device=dev)
+        uk_ms = event_time_ms(torch, lambda: ops.k_decode(ke["stream"], ke["info"], codes, 64, 128, bits), 5)
+        uv_ms = event_time_ms(torch, lambda: ops.v_decode(ve["stream"], ve["info"], codes, 128, 64, bits), 5)
+        del codes
+        enc_algo_k = x_bytes + ke["size"] + 8 * nblk_k + 4 * B * Tc
+        enc_algo_v = x_bytes + ve["size"] + 8 * nblk_v + 4 * B * Tc
+        result["encode"] = {
+            "k_ms": k_ms, "v_ms": v_ms,
+            "k_gbs_fp16_in": x_bytes / (k_ms * 1e-3) / 1e9, "v_gbs_fp16_in": x_bytes / (v_ms * 1e-3) / 1e9,
+            "k_roofline_frac": enc_algo_k / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "v_roofline_frac": enc_algo_v / (v_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        }
+        result["unpack"] = {
+            "k_ms": uk_ms, "v_ms": uv_ms,
+            "k_gbs": (ke["size"] + 8 * nblk_k + Tc * hidden) / (uk_ms * 1e-3) / 1e9,
+            "v_gbs": (ve["size"] + 8 * nblk_v + Tc * hidden) / (uv_ms * 1e-3) / 1e9,
+        }
+
+    if not args.no_cpu:
+        k1, v1, q1 = kc[:1].cpu(), vc[:1].cpu(), q[:1].cpu()
+        result["cpu_baseline"] = cpu_baseline(torch, args, k1, v1, q1)
+        result["cpu_encode"] = cpu_encoder(torch, args, k1)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

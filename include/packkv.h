@@ -1,0 +1,165 @@
+/*
+ * packkv.h -- C ABI of libpackkv_hip.so: the PackKV compressed-KV-cache hot path on one
+ * AMD gfx950 GPU (quantize -> bit-pack encode, bit-unpack decode, fused
+ * decompress-attention decode).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the parameter is documented as host;
+ *     buffers are caller-allocated and written in place, nothing is returned but a status;
+ *   - `s` is a hipStream_t (NULL = the default stream); work is enqueued on it;
+ *   - `ms_out` (host, may be NULL): when non-NULL the call brackets its kernels with HIP
+ *     events, waits for them and stores the elapsed milliseconds -- the reference's
+ *     launchers are synchronous and return milliseconds the same way
+ *     (packkv_cuda_ext/src/kernels.cu:560-608, src/fused_kernels.cu:118-168);
+ *   - return value 0 = success, otherwise a PKV_ERR_* code with text in pkv_last_error();
+ *     the library never aborts the process (the reference's CPU codec aborts on a failed
+ *     precondition, include/utils.h:8-16, and throws "not supported" for shapes outside
+ *     its dispatch table, src/k_encode_cpu.cpp:328-330 -- both map to error codes here);
+ *   - `dtype`: PKV_F16 or PKV_BF16, the 16-bit storage type of q / scale / zero / outputs
+ *     (the reference dispatches on at::Half / at::BFloat16, src/kernels.cu:622-629);
+ *   - code matrices are uint8 [ctx_len, hidden_dim] row-major with channel index
+ *     (b * H + h) * 128 + d (evaluation/evaluation.py:406); streams and block_info are laid
+ *     out exactly as the reference encoders write them (block_info[i] = (byte offset, byte
+ *     size) as uint32, i = ctx_blk * n_hid_blk + hid_blk).
+ */
+#ifndef PACKKV_H
+#define PACKKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PKV_ABI_VERSION 1
+
+#define PKV_F16 0
+#define PKV_BF16 1
+
+#define PKV_OK 0
+#define PKV_ERR_UNSUPPORTED 1 /* shape / width outside what the kernels implement */
+#define PKV_ERR_INVALID 2     /* bad argument */
+#define PKV_ERR_HIP 3         /* a HIP runtime call failed */
+#define PKV_ERR_CAPACITY 4    /* output buffer too small for the produced stream */
+#define PKV_ERR_INTERNAL 5    /* device-side protocol failure */
+
+typedef void *pkv_stream_t;
+
+int pkv_abi_version(void);
+/* Text of the last error raised on the calling thread. */
+const char *pkv_last_error(void);
+/* Worst-case bytes of one block (every pack at full width). */
+uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits);
+
+/* ---- bit-pack / bit-unpack of uint8 code matrices ---------------------------------
+ * Device counterparts of k_encode_cpu / v_encode_cpu / k_decode_cpu / v_decode_cpu
+ * (packkv_cuda_ext/packkv_cuda.pyi:4-24, :38-58; src/k_encode_cpu.cpp:286-331,
+ * src/v_encode_cpu.cpp:301-346, src/k_decode_cpu.cpp:281-326, src/v_decode_cpu.cpp:258-303).
+ * Generalised from the reference's dispatch table to any hidden_dim that is a multiple of
+ * the block width, bits in {2,3,4}; K blocks are ctx_blk x 128 (ctx_blk a multiple of 16,
+ * at most 256), V blocks are 128 x hid_blk (hid_blk a multiple of 32, at most 256).
+ * `capacity` = bytes available at `stream`; `size_out` (host, may be NULL) receives the
+ * stream size and makes the call synchronous. */
+int pkv_k_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
+                 int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
+                 float *ms_out, pkv_stream_t s);
+int pkv_v_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
+                 int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
+                 float *ms_out, pkv_stream_t s);
+int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                 int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
+int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                 int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
+
+/* ---- per-token affine quantizer ------------------------------------------------------
+ * Device counterpart of quant_ints(..., QuantMode.TokenQuant) and of the dequantisation
+ * (code + zero) * scale (utils/compute.py:84-112, :173-179): x is [B, H, T, 128] in
+ * `dtype`; scale and zero are [B, T] in `dtype` (one pair per batch and token, shared by
+ * all heads and channels); every intermediate is rounded to `dtype` exactly where the
+ * PyTorch op chain rounds it.  `codes` is the uint8 code matrix [T, B*H*128].
+ * `max_code_out` (device uint32, may be NULL) receives the largest code produced. */
+int pkv_quant_params(const void *x, int dtype, int B, int H, int T, float rel, void *scale, void *zero,
+                     float *ms_out, pkv_stream_t s);
+int pkv_quantize(const void *x, int dtype, int B, int H, int T, const void *scale, const void *zero,
+                 uint8_t *codes, uint32_t *max_code_out, float *ms_out, pkv_stream_t s);
+int pkv_dequantize(const uint8_t *codes, int dtype, int B, int H, int T, const void *scale,
+                   const void *zero, void *x_out, float *ms_out, pkv_stream_t s);
+
+/* ---- fused quantize + encode (the encode hot path) -----------------------------------
+ * x [B, H, T, 128] `dtype` -> stream + block_info + scale/zero [B, T], never materialising
+ * the code matrix.  Same stream as pkv_quant_params + pkv_quantize + pkv_{k,v}_encode.
+ * K uses blocks of 64 x 128, V blocks of 128 x 64 (the shapes the reference's kernels
+ * consume, src/kernels.cu:564-589, :795-818).  `bits` is the raw code width W; a code
+ * that does not fit W bits raises PKV_ERR_UNSUPPORTED when size_out is requested. */
+int pkv_k_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *stream,
+                       uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
+                       uint64_t *size_out, float *ms_out, pkv_stream_t s);
+int pkv_v_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *stream,
+                       uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
+                       uint64_t *size_out, float *ms_out, pkv_stream_t s);
+
+/* ---- the reference's GEMV surface -----------------------------------------------------
+ * kq_mat_vec_mul (packkv_cuda.pyi:26-36, src/kernels.cu:611-630):
+ *     kq_out[h, tok] = sum_d q[h, d] * code[tok, h*128 + d]        (dtype, [H, ctx_len])
+ *   q_interleaved != 0: q is in the lane order the reference kernel expects
+ *   (evaluation/evaluation.py:465-468); 0: plain [H, 128].
+ * wv_mat_vec_mul (packkv_cuda.pyi:60-70, src/kernels.cu:840-859):
+ *     wv_out[c] += sum_tok w[c / 128, tok] * code[tok, c]          (fp32 [hidden_dim], caller
+ *   zeroes it; accumulated with atomics like the reference, src/kernels.cu:756-763)
+ * fused_kq (packkv_cuda.pyi:72-78, src/fused_kernels.cu:13-76):
+ *     our_kq[m, n] = (sum_d q[m, d] * zero[n] + t[m, n]) * scale[n]
+ * fused_wv (packkv_cuda.pyi:80-86, src/fused_kernels.cu:187-261):
+ *     our_wv[m, d] = sum_n w[m, n] * zero[n] * scale[n] + term1[m, d]
+ * Any head count M and any hidden_dim multiple of 128 are accepted (the reference
+ * instantiates hidden_dim in {5120, 1024}, M in {40, 8} only). */
+int pkv_kq_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *q, void *kq_out,
+                       int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
+                       int q_interleaved, float *ms_out, pkv_stream_t s);
+int pkv_wv_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *w, float *wv_out,
+                       int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
+                       float *ms_out, pkv_stream_t s);
+int pkv_fused_kq(void *our_kq, const void *q, const void *k_zero, const void *k_scale, const void *t, int M,
+                 int K, int N, int dtype, float *ms_out, pkv_stream_t s);
+int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_scale, const void *term1,
+                 int M, int N, int D, int dtype, float *ms_out, pkv_stream_t s);
+
+/* ---- fused decompress-attention decode ------------------------------------------------
+ * One decode step over a compressed cache, without materialising K or V:
+ *   out[b, hq, :] = softmax_t( sm_scale * q[b, hq, :] . K[b, hq / G, t, :] ) @ V[b, hq / G, t, :]
+ * with K = (k_code + k_zero) * k_scale, V likewise, G = Hq / Hkv, fp32 accumulation.
+ * It fuses what the reference runs as kq_mat_vec_mul -> fused_kq -> softmax
+ * (models/llama.py:202-209) -> w * v_scale (evaluation/evaluation.py:661) ->
+ * wv_mat_vec_mul -> fused_wv, and adds the batch and GQA-group dimensions.
+ *
+ *   k_stream/k_info   K stream of the code matrix [T_c, B*Hkv*128], blocks 64 x 128
+ *   v_stream/v_info   V stream of the same shape, blocks 128 x 64
+ *   k_scale..v_zero   [B, T_c] `dtype`
+ *   q, out            [B, Hq, 128] `dtype`
+ *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype` (the residual
+ *                     window the cache keeps in 16-bit, utils/compute.py:54-67); T_w may be 0
+ *   T_c               compressed tokens, a multiple of 128 (may be 0 when T_w > 0)
+ *   variant           0 = default kernel; other values select alternative implementations
+ *                     of the same contract (used by tests to cross-check)
+ */
+typedef struct pkv_attn_args {
+    const uint8_t *k_stream;
+    const uint32_t *k_info;
+    const uint8_t *v_stream;
+    const uint32_t *v_info;
+    const void *k_scale, *k_zero, *v_scale, *v_zero;
+    const void *q;
+    void *out;
+    const void *k_win, *v_win;
+    int B, Hq, Hkv, T_c, T_w;
+    int k_bits, v_bits;
+    int dtype;
+    float sm_scale;
+    int variant;
+} pkv_attn_args;
+
+int pkv_attn_decode(const pkv_attn_args *args, float *ms_out, pkv_stream_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PACKKV_H */

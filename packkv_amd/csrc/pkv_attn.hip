@@ -1,0 +1,389 @@
+// Fused decompress-attention decode: one query token per sequence attends over a compressed
+// K/V cache (plus an optional 16-bit tail window) without materialising K or V.
+//
+// Fuses the reference's chain  kq_mat_vec_mul -> fused_kq -> softmax -> w * v_scale ->
+// wv_mat_vec_mul -> fused_wv  (packkv_cuda_ext/src/kernels.cu:426-535, :632-765,
+// src/fused_kernels.cu:13-76, :187-261, models/llama.py:202-209,
+// evaluation/evaluation.py:661) and adds batch and GQA-group dimensions.
+//
+// Work decomposition (flash-decoding): grid (split, kv_head, batch).  A workgroup walks
+// 128-token super-tiles = 2 K blocks (64 x 128) + 2 V blocks (128 x 64) of its head and keeps
+// an online-softmax state; each split writes (m, l, acc[128]) per query head, a small merge
+// kernel combines the splits and the tail window.
+#include "pkv_block.hpp"
+#include "pkv_runtime.hpp"
+
+namespace pkv {
+
+constexpr int kTile = 128;              // tokens per super-tile
+constexpr int kPartStride = 2 + kHeadDim;  // floats per partial: m, l, acc[128]
+
+__device__ __forceinline__ float a_ld16(const uint16_t *p, size_t i, int dtype) {
+    const uint32_t u = p[i];
+    return dtype == PKV_F16 ? __half2float(__ushort_as_half((unsigned short)u)) : __uint_as_float(u << 16);
+}
+
+__device__ __forceinline__ uint16_t a_st16(float x, int dtype) {
+    if (dtype == PKV_F16) return __half_as_ushort(__float2half_rn(x));
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+struct AttnParams {
+    const uint8_t *k_stream;
+    const uint32_t *k_info;
+    const uint8_t *v_stream;
+    const uint32_t *v_info;
+    const uint16_t *k_scale, *k_zero, *v_scale, *v_zero;
+    const uint16_t *q;
+    const uint16_t *k_win, *v_win;
+    float *part;          // [B, Hq, nparts, kPartStride]
+    int B, Hq, Hkv, T_c, T_w;
+    int k_bits, v_bits, dtype;
+    float sm_scale;
+    int tiles_per_split, nsplit, nparts;
+    uint32_t k_cap, v_cap, blk_stride;
+};
+
+// ---- variant 1: decode tiles into LDS, then plain VALU attention --------------------------
+// Straightforward and easy to audit; kept as the cross-check for the tuned kernel.
+template <int G>
+__global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t *ktile = lds;                                   // [128 tok][128 ch]
+    uint8_t *vtile = ktile + kTile * kHeadDim;              // [128 tok][128 ch]
+    uint8_t *blkbuf = vtile + kTile * kHeadDim;             // 4 x blk_stride
+    float *fl = reinterpret_cast<float *>(blkbuf + 4 * p.blk_stride);
+    float *qf = fl;                       // [G][128]
+    float *S = qf + G * kHeadDim;         // [G][128]
+    float *P = S + G * kTile;             // [G][128]
+    float *ks = P + G * kTile;            // [128] x4
+    float *kz = ks + kTile, *vs = kz + kTile, *vz = vs + kTile;
+    float *st_m = vz + kTile;             // [G] each
+    float *st_l = st_m + G, *st_a = st_l + G, *st_z = st_a + G, *qsum = st_z + G;
+    __shared__ uint32_t s_phase[4], s_off[4];
+
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int lane32 = tid & 31, hw = tid >> 5;
+    const int bh = b * p.Hkv + h;
+    const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
+    const UnitGeom gk = unit_geom(p.k_bits), gv = unit_geom(p.v_bits);
+
+    for (int i = tid; i < G * kHeadDim; i += 256)
+        qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
+    if (tid < G) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; }
+    __syncthreads();
+    if (tid < G) {
+        float s = 0.f;
+        for (int d = 0; d < kHeadDim; d++) s += qf[tid * kHeadDim + d];
+        qsum[tid] = s;
+    }
+    float acc[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) acc[g] = 0.f;
+
+    const int n_tiles = p.T_c / kTile;
+    const int tile0 = split * p.tiles_per_split;
+    const int tile1 = min(n_tiles, tile0 + p.tiles_per_split);
+    for (int tau = tile0; tau < tile1; tau++) {
+        // 1. stage the four blocks and the per-token quantizer parameters
+        for (int j = 0; j < 4; j++) {
+            const bool is_k = j < 2;
+            const uint32_t bidx = is_k ? (uint32_t)((2 * tau + j) * n_hid_k + bh)
+                                       : (uint32_t)(tau * n_hid_v + 2 * bh + (j - 2));
+            const uint32_t *info = is_k ? p.k_info : p.v_info;
+            const uint8_t *stream = is_k ? p.k_stream : p.v_stream;
+            const uint32_t off = info[2 * bidx];
+            uint32_t size = info[2 * bidx + 1];
+            const uint32_t cap = is_k ? p.k_cap : p.v_cap;
+            if (size > cap) size = cap;
+            const uint32_t ph = stage_to_lds(stream + off, size, blkbuf + j * p.blk_stride, tid, 256);
+            if (tid == 0) s_phase[j] = ph;
+        }
+        if (tid < kTile) {
+            const size_t ti = (size_t)b * p.T_c + (size_t)tau * kTile + tid;
+            ks[tid] = a_ld16(p.k_scale, ti, p.dtype);
+            kz[tid] = a_ld16(p.k_zero, ti, p.dtype);
+            vs[tid] = a_ld16(p.v_scale, ti, p.dtype);
+            vz[tid] = a_ld16(p.v_zero, ti, p.dtype);
+        }
+        __syncthreads();
+        // 2. unpack: half-wave hw handles K unit (block hw/4, round hw%4) and V unit
+        //    (block hw/4 = channel half, segment hw%4)
+        {
+            const int j = hw >> 2, unit = hw & 3;
+            const uint8_t *kb = blkbuf + j * p.blk_stride;
+            const uint32_t kph = s_phase[j];
+            const uint16_t *kcum = reinterpret_cast<const uint16_t *>(kb + kph);
+            const uint32_t kstart = kph + 8u + (unit ? (uint32_t)kcum[unit - 1] : 0u);
+            unit_decode<true>(kb, kstart, unit, lane32, gk, ktile + j * 64 * kHeadDim, kHeadDim);
+            const uint8_t *vb = blkbuf + (2 + j) * p.blk_stride;
+            const uint32_t vph = s_phase[2 + j];
+            const uint16_t *vcum = reinterpret_cast<const uint16_t *>(vb + vph);
+            const uint32_t vstart = vph + 8u + (unit ? (uint32_t)vcum[unit - 1] : 0u);
+            unit_decode<false>(vb, vstart, unit, lane32, gv, vtile + j * 64, kHeadDim);
+        }
+        __syncthreads();
+        // 3. scores: two threads per token, 64 channels each
+        {
+            const int tok = tid >> 1, half = tid & 1;
+            const uint32_t *row = reinterpret_cast<const uint32_t *>(ktile + tok * kHeadDim + half * 64);
+            float dot[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) dot[g] = 0.f;
+#pragma unroll 4
+            for (int i = 0; i < 16; i++) {
+                const uint32_t w = row[i];
+                const float c0 = (float)(w & 0xFFu), c1 = (float)((w >> 8) & 0xFFu),
+                            c2 = (float)((w >> 16) & 0xFFu), c3 = (float)(w >> 24);
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    const float *qq = qf + g * kHeadDim + half * 64 + 4 * i;
+                    dot[g] += qq[0] * c0 + qq[1] * c1 + qq[2] * c2 + qq[3] * c3;
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float d = dot[g] + __shfl_xor(dot[g], 1, 64);
+                if (half == 0) S[g * kTile + tok] = p.sm_scale * ks[tok] * (d + kz[tok] * qsum[g]);
+            }
+        }
+        __syncthreads();
+        // 4. online softmax: wavefront w owns query heads w, w+4, ...
+        for (int g = tid >> 6; g < G; g += 4) {
+            const int lane = tid & 63;
+            const float s0 = S[g * kTile + lane], s1 = S[g * kTile + 64 + lane];
+            float mx = fmaxf(s0, s1);
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+            const float m_old = st_m[g];
+            const float m_new = fmaxf(m_old, mx);
+            const float p0 = __expf(s0 - m_new), p1 = __expf(s1 - m_new);
+            const float w0 = p0 * vs[lane], w1 = p1 * vs[64 + lane];
+            P[g * kTile + lane] = w0;
+            P[g * kTile + 64 + lane] = w1;
+            float sum = p0 + p1;
+            float zs = w0 * vz[lane] + w1 * vz[64 + lane];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                sum += __shfl_xor(sum, d, 64);
+                zs += __shfl_xor(zs, d, 64);
+            }
+            if (lane == 0) {
+                const float alpha = __expf(m_old - m_new);   // exp(-inf) = 0 on the first tile
+                st_a[g] = alpha;
+                st_m[g] = m_new;
+                st_l[g] = st_l[g] * alpha + sum;
+                st_z[g] = st_z[g] * alpha + zs;
+            }
+        }
+        __syncthreads();
+        // 5. PV: thread = (channel, token half)
+        {
+            const int ch = tid & 127, half = tid >> 7;
+            float part[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) part[g] = 0.f;
+#pragma unroll 8
+            for (int t = 0; t < 64; t++) {
+                const float c = (float)vtile[(half * 64 + t) * kHeadDim + ch];
+#pragma unroll
+                for (int g = 0; g < G; g++) part[g] += P[g * kTile + half * 64 + t] * c;
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) acc[g] = acc[g] * st_a[g] + part[g];
+        }
+        __syncthreads();
+    }
+    // combine the two token halves and write the partial
+    {
+        const int ch = tid & 127, half = tid >> 7;
+        float *red = S;   // reuse: [G][128]
+        if (half == 1)
+            for (int g = 0; g < G; g++) red[g * kTile + ch] = acc[g];
+        __syncthreads();
+        if (half == 0) {
+            for (int g = 0; g < G; g++) {
+                const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+                float *dst = p.part + (hq * p.nparts + split) * kPartStride;
+                dst[2 + ch] = acc[g] + red[g * kTile + ch] + st_z[g];
+                if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+            }
+        }
+    }
+}
+
+// ---- 16-bit tail window: dense attention over T_w tokens, one workgroup per (kv head, batch)
+template <int G>
+__global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    float *qf = reinterpret_cast<float *>(lds);   // [G][128]
+    float *S = qf + G * kHeadDim;                 // [G][T_w]
+    __shared__ float st_m[G], st_l[G];
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int Tw = p.T_w;
+    for (int i = tid; i < G * kHeadDim; i += 256)
+        qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
+    __syncthreads();
+    const uint16_t *kbase = p.k_win + ((size_t)b * p.Hkv + h) * Tw * kHeadDim;
+    const uint16_t *vbase = p.v_win + ((size_t)b * p.Hkv + h) * Tw * kHeadDim;
+    for (int t = tid; t < Tw; t += 256) {
+        float dot[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) dot[g] = 0.f;
+        for (int d = 0; d < kHeadDim; d++) {
+            const float kv = a_ld16(kbase, (size_t)t * kHeadDim + d, p.dtype);
+#pragma unroll
+            for (int g = 0; g < G; g++) dot[g] += qf[g * kHeadDim + d] * kv;
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) S[g * Tw + t] = dot[g] * p.sm_scale;
+    }
+    __syncthreads();
+    for (int g = tid >> 6; g < G; g += 4) {
+        const int lane = tid & 63;
+        float mx = -INFINITY;
+        for (int t = lane; t < Tw; t += 64) mx = fmaxf(mx, S[g * Tw + t]);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+        float sum = 0.f;
+        for (int t = lane; t < Tw; t += 64) {
+            const float e = __expf(S[g * Tw + t] - mx);
+            S[g * Tw + t] = e;
+            sum += e;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+        if (lane == 0) { st_m[g] = mx; st_l[g] = sum; }
+    }
+    __syncthreads();
+    if (tid < kHeadDim) {
+        float acc[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) acc[g] = 0.f;
+        for (int t = 0; t < Tw; t++) {
+            const float v = a_ld16(vbase, (size_t)t * kHeadDim + tid, p.dtype);
+#pragma unroll
+            for (int g = 0; g < G; g++) acc[g] += S[g * Tw + t] * v;
+        }
+        for (int g = 0; g < G; g++) {
+            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            float *dst = p.part + (hq * p.nparts + (p.nparts - 1)) * kPartStride;
+            dst[2 + tid] = acc[g];
+            if (tid == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+        }
+    }
+}
+
+// ---- merge of the per-split partials: grid (Hq, B), 128 threads ---------------------------
+__global__ void attn_merge_kernel(const float *__restrict__ part, uint16_t *__restrict__ out, int Hq,
+                                  int nparts, int dtype) {
+    const size_t hq = (size_t)blockIdx.y * Hq + blockIdx.x;
+    const float *base = part + hq * nparts * kPartStride;
+    float M = -INFINITY;
+    for (int s = 0; s < nparts; s++) M = fmaxf(M, base[s * kPartStride]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < nparts; s++) {
+        const float w = __expf(base[s * kPartStride] - M);
+        den += w * base[s * kPartStride + 1];
+        num += w * base[s * kPartStride + 2 + threadIdx.x];
+    }
+    out[hq * kHeadDim + threadIdx.x] = a_st16(num / den, dtype);
+}
+
+template <int G>
+static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
+    (void)variant;
+    if (p.T_c > 0) {
+        const uint32_t lds_bytes = 2u * kTile * kHeadDim + 4u * p.blk_stride +
+                                   (uint32_t)sizeof(float) * (G * kHeadDim + 2 * G * kTile + 4 * kTile + 5 * G);
+        const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_tiles_kernel<G>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attn_tiles_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
+        PKV_HIP_CHECK(hipGetLastError());
+    }
+    if (p.T_w > 0) {
+        const uint32_t lds_bytes = (uint32_t)sizeof(float) * (G * kHeadDim + G * p.T_w);
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_window_kernel<G>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attn_window_kernel<G><<<dim3((unsigned)p.Hkv, (unsigned)p.B), 256, lds_bytes, s>>>(p);
+        PKV_HIP_CHECK(hipGetLastError());
+    }
+    attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), kHeadDim, 0, s>>>(p.part, out, p.Hq, p.nparts,
+                                                                              p.dtype);
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
+}  // namespace pkv
+
+extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream_t s_) {
+    using namespace pkv;
+    hipStream_t s = (hipStream_t)s_;
+    PKV_REQUIRE(a != nullptr, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(a->dtype == PKV_F16 || a->dtype == PKV_BF16, PKV_ERR_UNSUPPORTED, "Unsupported data type");
+    PKV_REQUIRE(a->B > 0 && a->Hq > 0 && a->Hkv > 0 && a->Hq % a->Hkv == 0, PKV_ERR_INVALID,
+                "need B, Hq, Hkv > 0 and Hq divisible by Hkv");
+    PKV_REQUIRE(a->B <= 65535 && a->Hkv <= 65535, PKV_ERR_UNSUPPORTED, "batch / head count above 65535");
+    PKV_REQUIRE(a->T_c >= 0 && a->T_w >= 0 && a->T_c + a->T_w > 0, PKV_ERR_INVALID, "empty cache");
+    PKV_REQUIRE(a->T_c % kTile == 0, PKV_ERR_INVALID, "compressed length must be a multiple of 128 tokens");
+    PKV_REQUIRE(a->T_w <= 2048, PKV_ERR_UNSUPPORTED, "tail window longer than 2048 tokens");
+    PKV_REQUIRE(a->q && a->out, PKV_ERR_INVALID, "null pointer argument");
+    if (a->T_c > 0) {
+        PKV_REQUIRE(a->k_stream && a->k_info && a->v_stream && a->v_info && a->k_scale && a->k_zero &&
+                        a->v_scale && a->v_zero,
+                    PKV_ERR_INVALID, "null pointer argument");
+        PKV_REQUIRE(a->k_bits >= 2 && a->k_bits <= 4 && a->v_bits >= 2 && a->v_bits <= 4, PKV_ERR_UNSUPPORTED,
+                    "not supported: bits_len outside 2..4");
+    }
+    if (a->T_w > 0) PKV_REQUIRE(a->k_win && a->v_win, PKV_ERR_INVALID, "null pointer argument");
+    const int G = a->Hq / a->Hkv;
+    PKV_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, PKV_ERR_UNSUPPORTED,
+                "not supported: query heads per KV head must be 1, 2, 4 or 8");
+
+    AttnParams p;
+    p.k_stream = a->k_stream; p.k_info = a->k_info; p.v_stream = a->v_stream; p.v_info = a->v_info;
+    p.k_scale = (const uint16_t *)a->k_scale; p.k_zero = (const uint16_t *)a->k_zero;
+    p.v_scale = (const uint16_t *)a->v_scale; p.v_zero = (const uint16_t *)a->v_zero;
+    p.q = (const uint16_t *)a->q;
+    p.k_win = (const uint16_t *)a->k_win; p.v_win = (const uint16_t *)a->v_win;
+    p.B = a->B; p.Hq = a->Hq; p.Hkv = a->Hkv; p.T_c = a->T_c; p.T_w = a->T_w;
+    p.k_bits = a->k_bits; p.v_bits = a->v_bits; p.dtype = a->dtype; p.sm_scale = a->sm_scale;
+    const int n_tiles = a->T_c / kTile;
+    int nsplit = 0, tps = 0;
+    if (n_tiles > 0) {
+        const int pairs = a->B * a->Hkv;
+        int want = (2048 + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
+        if (want < 1) want = 1;
+        if (want > n_tiles) want = n_tiles;
+        tps = (n_tiles + want - 1) / want;
+        nsplit = (n_tiles + tps - 1) / tps;
+    }
+    p.tiles_per_split = tps; p.nsplit = nsplit;
+    p.nparts = nsplit + (a->T_w > 0 ? 1 : 0);
+    p.k_cap = a->T_c > 0 ? (uint32_t)k_block_bound(64, a->k_bits) : 0;
+    p.v_cap = a->T_c > 0 ? (uint32_t)v_block_bound(64, a->v_bits) : 0;
+    const uint32_t cap = p.k_cap > p.v_cap ? p.k_cap : p.v_cap;
+    p.blk_stride = ((cap + 15u) & ~15u) + 32u;
+    void *scratch = nullptr;
+    const size_t part_bytes = (size_t)a->B * a->Hq * p.nparts * kPartStride * sizeof(float);
+    int rc = scratch_get(part_bytes, &scratch);
+    if (rc) return rc;
+    p.part = (float *)scratch;
+
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    switch (G) {
+        case 1: rc = launch_attn<1>(p, a->variant, (uint16_t *)a->out, s); break;
+        case 2: rc = launch_attn<2>(p, a->variant, (uint16_t *)a->out, s); break;
+        case 4: rc = launch_attn<4>(p, a->variant, (uint16_t *)a->out, s); break;
+        default: rc = launch_attn<8>(p, a->variant, (uint16_t *)a->out, s); break;
+    }
+    if (rc) return rc;
+    return tm.end(ms_out);
+}

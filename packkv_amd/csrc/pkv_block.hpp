@@ -1,0 +1,288 @@
+// Block-level codec building blocks shared by the unpack, encode and fused
+// quantize+encode kernels.  A "unit" is what one 32-lane half-wavefront handles:
+//   K: one round  (16 tokens x 128 channels), lane t <-> channels 4t..4t+3, slot i = channel 4t+i
+//   V: one segment (64 tokens x 32 channels), lane t <-> channel 32*warp+t, slot i = round 4*seg+i
+// In both cases the unit's bytes are  mins | lens | payload  with payload ordered slot-major,
+// lane-minor, so parsing and emitting are the same code; only the tile scatter differs.
+#pragma once
+#include "pkv_common.hpp"
+
+namespace pkv {
+
+struct UnitGeom {
+    int mins_bytes;   // W * 128 / 8
+    int lens_bytes;   // LB * 128 / 8
+    int W, LB;
+};
+
+__host__ __device__ inline UnitGeom unit_geom(int W) {
+    UnitGeom g;
+    g.W = W;
+    g.LB = len_field_bits(W);
+    g.mins_bytes = W * 16;
+    g.lens_bytes = g.LB * 16;
+    return g;
+}
+
+#ifdef __HIPCC__
+
+// Tile addressing: the uint8 code tile in LDS is row-major [tokens][hid_blk].
+template <bool IS_K>
+__device__ __forceinline__ int tile_index(int unit, int slot, int k, int t, int hid_blk) {
+    if (IS_K) return (unit * kPackTok + k) * hid_blk + 4 * t + slot;
+    const int warp = unit >> 1, seg = unit & 1;
+    return ((seg * 4 + slot) * kPackTok + k) * hid_blk + warp * kLanes + t;
+}
+
+// Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
+template <bool IS_K>
+__device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,
+                                            const UnitGeom g, uint8_t *tile, int hid_blk) {
+    const uint32_t minsw = lds_meta_word(blk + unit_off, t, g.W);
+    const uint32_t lensw = lds_meta_word(blk + unit_off + g.mins_bytes, t, g.LB);
+    uint32_t run = unit_off + g.mins_bytes + g.lens_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t len = (lensw >> (i * g.LB)) & ((1u << g.LB) - 1u);
+        const uint32_t mn = (minsw >> (i * g.W)) & ((1u << g.W) - 1u);
+        uint32_t tot;
+        const uint32_t off = run + half_excl_scan(2u * len, tot);
+        run += tot;
+        uint64_t word = lds_load64(blk, off);
+        const uint64_t mask = (1ull << len) - 1ull;
+        if (IS_K) {
+#pragma unroll
+            for (int k = 0; k < kPackTok; k++) {
+                const uint32_t c = (uint32_t)((word >> ((15 - k) * len)) & mask) + mn;
+                tile[tile_index<true>(unit, i, k, t, hid_blk)] = (uint8_t)c;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < kPackTok; k++) {
+                const uint32_t c = (uint32_t)((word >> ((15 - k) * len)) & mask) + mn;
+                tile[tile_index<false>(unit, i, k, t, hid_blk)] = (uint8_t)c;
+            }
+        }
+    }
+}
+
+struct UnitPacks {
+    uint64_t word[4];
+    uint32_t len[4];
+    uint32_t mn[4];
+    uint32_t off[4];     // byte offset of each pack inside the unit's payload
+    uint32_t payload;    // payload bytes of the whole unit
+};
+
+// Gather lane t's four packs of `unit` from the LDS code tile and compute min / len / word
+// and the payload offsets (one 32-lane exclusive scan per slot).
+template <bool IS_K>
+__device__ __forceinline__ void unit_analyse(const uint8_t *tile, int hid_blk, int unit, int t,
+                                             UnitPacks &u) {
+    uint32_t run = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t c[kPackTok];
+        uint32_t mn = 255u, mx = 0u;
+#pragma unroll
+        for (int k = 0; k < kPackTok; k++) {
+            c[k] = tile[tile_index<IS_K>(unit, i, k, t, hid_blk)];
+            mn = min(mn, c[k]);
+            mx = max(mx, c[k]);
+        }
+        const uint32_t len = (uint32_t)bit_length_u32(mx - mn);
+        uint64_t w = 0;
+#pragma unroll
+        for (int k = 0; k < kPackTok; k++) w = (w << len) | (uint64_t)(c[k] - mn);
+        u.word[i] = w;
+        u.len[i] = len;
+        u.mn[i] = mn;
+        uint32_t tot;
+        u.off[i] = run + half_excl_scan(2u * len, tot);
+        run += tot;
+    }
+    u.payload = run;
+}
+
+// Write lane t's 4*nbits-bit metadata word into an LSB-first bit array (nbits in {2,3,4}).
+__device__ __forceinline__ void lds_put_meta(uint8_t *arr, int t, int nbits, uint32_t w) {
+    if (nbits == 4) {
+        reinterpret_cast<uint16_t *>(arr)[t] = (uint16_t)w;
+    } else if (nbits == 2) {
+        arr[t] = (uint8_t)w;
+    } else {  // 12 bits per lane: an even/odd lane pair shares three bytes
+        const uint32_t hi = __shfl_down(w, 1, 32);
+        if ((t & 1) == 0) {
+            const uint32_t v = w | (hi << 12);
+            uint8_t *p = arr + (t >> 1) * 3;
+            p[0] = (uint8_t)v;
+            p[1] = (uint8_t)(v >> 8);
+            p[2] = (uint8_t)(v >> 16);
+        }
+    }
+}
+
+// Emit one analysed unit at blk[unit_off] (unit_off even, blk 4-byte aligned).
+__device__ __forceinline__ void unit_emit(uint8_t *blk, uint32_t unit_off, int t, const UnitGeom g,
+                                          const UnitPacks &u) {
+    uint32_t minsw = 0, lensw = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        minsw |= u.mn[i] << (i * g.W);
+        lensw |= u.len[i] << (i * g.LB);
+    }
+    lds_put_meta(blk + unit_off, t, g.W, minsw);
+    lds_put_meta(blk + unit_off + g.mins_bytes, t, g.LB, lensw);
+    uint8_t *pay = blk + unit_off + g.mins_bytes + g.lens_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(pay + u.off[i]);
+        uint64_t w = u.word[i];
+        for (uint32_t b = 0; b < u.len[i]; b++) {
+            dst[b] = (uint16_t)w;
+            w >>= 16;
+        }
+    }
+}
+
+// Encode the LDS code tile of one block into the LDS buffer `blk`; every thread of the
+// workgroup must call it, and the workgroup must hold at least one half-wavefront per unit
+// (blockDim.x >= 32 * nunits).  `unit_bytes` is an LDS array of >= nunits uint32.  Returns
+// the block size in bytes (uniform).  Contains __syncthreads().
+template <bool IS_K>
+__device__ __forceinline__ uint32_t block_encode(const uint8_t *tile, int hid_blk, int nunits, int W,
+                                                 uint8_t *blk, uint32_t *unit_bytes) {
+    const UnitGeom g = unit_geom(W);
+    const int t = threadIdx.x & 31;
+    const int unit = threadIdx.x >> 5;
+    const bool active = unit < nunits;
+    const uint32_t hdr = 2u * (uint32_t)nunits;
+    UnitPacks u;
+    if (active) {
+        unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
+        if (t == 0) unit_bytes[unit] = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+    }
+    __syncthreads();
+    uint32_t total = hdr;
+    for (int q = 0; q < nunits; q++) total += unit_bytes[q];
+    if (active) {
+        uint32_t base = hdr;
+        for (int q = 0; q < unit; q++) base += unit_bytes[q];
+        if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - hdr + unit_bytes[unit]);
+        unit_emit(blk, base, t, g, u);
+    }
+    __syncthreads();
+    return total;
+}
+
+// Decode a staged block (bytes at blk[phase..]) into the LDS code tile; needs one
+// half-wavefront per unit like block_encode.
+template <bool IS_K>
+__device__ __forceinline__ void block_decode(const uint8_t *blk, uint32_t phase, int nunits, int W,
+                                             uint8_t *tile, int hid_blk) {
+    const UnitGeom g = unit_geom(W);
+    const int t = threadIdx.x & 31;
+    const int unit = threadIdx.x >> 5;
+    const uint32_t hdr = 2u * (uint32_t)nunits;
+    const uint16_t *cum = reinterpret_cast<const uint16_t *>(blk + phase);  // phase is even
+    if (unit < nunits) {
+        const uint32_t start = phase + hdr + (unit ? (uint32_t)cum[unit - 1] : 0u);
+        unit_decode<IS_K>(blk, start, unit, t, g, tile, hid_blk);
+    }
+}
+
+// ---- single-pass global offsets: decoupled look-back over block order -------------------
+// status word: bits 63..62 = flag (0 empty, 1 aggregate, 2 inclusive), bits 61..0 = bytes.
+constexpr uint64_t kFlagAgg = 1ull << 62;
+constexpr uint64_t kFlagIncl = 2ull << 62;
+constexpr uint64_t kValueMask = (1ull << 62) - 1ull;
+constexpr int kSpinLimit = 1 << 20;
+
+struct ScanState {
+    uint32_t ticket;      // next block index to hand out
+    uint32_t error;       // non-zero: PKV_ERR_* raised on the device
+    uint64_t total;       // stream bytes (written by the last block)
+    uint32_t max_code;    // largest code seen by a fused quantize+encode launch
+    uint32_t pad_;
+    uint64_t status[1];   // one per block
+};
+
+// Called by every lane of the FIRST wavefront of the workgroup that owns block `idx`.
+// Returns the byte offset of the block in the stream.
+__device__ __forceinline__ uint64_t lookback_offset(ScanState *st, uint32_t idx, uint32_t my_bytes) {
+    const int lane = threadIdx.x & 63;
+    uint64_t *status = st->status;
+    if (idx == 0) {
+        if (lane == 0)
+            __hip_atomic_store(&status[0], kFlagIncl | (uint64_t)my_bytes, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        return 0;
+    }
+    if (lane == 0)
+        __hip_atomic_store(&status[idx], kFlagAgg | (uint64_t)my_bytes, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t prefix = 0;
+    int64_t base = (int64_t)idx - 1;
+    bool failed = false;
+    while (true) {
+        const int64_t j = base - lane;
+        uint64_t s = kFlagIncl;  // the virtual block before block 0: inclusive sum 0
+        int spins = 0;
+        if (j >= 0) {
+            s = __hip_atomic_load(&status[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            while ((s >> 62) == 0 && spins < kSpinLimit) {
+                __builtin_amdgcn_s_sleep(1);
+                s = __hip_atomic_load(&status[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                spins++;
+            }
+        }
+        if (__any((s >> 62) == 0)) { failed = true; break; }
+        const uint64_t incl_mask = __ballot((s >> 62) == 2);
+        const int first_incl = incl_mask ? (__ffsll((unsigned long long)incl_mask) - 1) : 64;
+        uint64_t v = (lane <= first_incl) ? (s & kValueMask) : 0ull;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+        prefix += v;
+        if (incl_mask) break;
+        base -= 64;
+    }
+    if (failed) {
+        if (lane == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);
+        prefix = 0;
+    }
+    if (lane == 0)
+        __hip_atomic_store(&status[idx], kFlagIncl | (prefix + (uint64_t)my_bytes), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    return prefix;
+}
+
+// Everything after the code tile is in LDS: encode the block, obtain its stream offset by
+// look-back, record block_info and copy the bytes out.  Every thread of the workgroup calls
+// it; `s_off` is an LDS uint64, `unit_bytes` an LDS array of 16 uint32.
+template <bool IS_K>
+__device__ __forceinline__ void block_finish(const uint8_t *tile, uint8_t *blk, uint32_t *unit_bytes,
+                                             uint64_t *s_off, ScanState *st, uint32_t b, uint32_t nblocks,
+                                             uint8_t *__restrict__ stream, uint64_t capacity,
+                                             uint32_t *__restrict__ info, int hid_blk, int nunits, int W) {
+    const uint32_t bytes = block_encode<IS_K>(tile, hid_blk, nunits, W, blk, unit_bytes);
+    if (threadIdx.x < 64) {
+        const uint64_t off = lookback_offset(st, b, bytes);
+        if (threadIdx.x == 0) {
+            *s_off = off;
+            info[2 * b] = (uint32_t)off;
+            info[2 * b + 1] = bytes;
+            if (b == nblocks - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = *s_off;
+    if (off + bytes > capacity) return;
+    uint16_t *dst = reinterpret_cast<uint16_t *>(stream + off);   // block offsets are even
+    const uint16_t *src = reinterpret_cast<const uint16_t *>(blk);
+    for (uint32_t i = threadIdx.x; i < (bytes >> 1); i += blockDim.x) dst[i] = src[i];
+}
+
+#endif  // __HIPCC__
+
+}  // namespace pkv

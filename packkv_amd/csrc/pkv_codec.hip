@@ -1,0 +1,223 @@
+// Bit-unpack (stream -> uint8 codes) and bit-pack (uint8 codes -> stream) kernels, one
+// workgroup per block, one 32-lane half-wavefront per round (K) or segment (V).
+//
+// Replaces the reference's scalar CPU codec on the device:
+//   packkv_cuda_ext/src/k_encode_cpu.cpp:203-231, v_encode_cpu.cpp:230-259  (encode drivers)
+//   packkv_cuda_ext/src/k_decode_cpu.cpp:201-225, v_decode_cpu.cpp:184-216  (decode drivers)
+#include "pkv_block.hpp"
+#include "pkv_runtime.hpp"
+
+namespace pkv {
+
+// LDS layout of both kernels: [code tile: ctx_blk*hid_blk][block buffer: bound + 32][unit_bytes]
+__host__ __device__ inline uint32_t round_up16(uint32_t v) { return (v + 15u) & ~15u; }
+
+template <bool IS_K>
+__global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+                              uint8_t *__restrict__ codes, int hidden_dim, int ctx_blk, int hid_blk,
+                              int nunits, int W, uint32_t blk_cap) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t *tile = lds;
+    uint8_t *blk = lds + round_up16((uint32_t)(ctx_blk * hid_blk));
+    const int n_hid = hidden_dim / hid_blk;
+    const uint32_t b = blockIdx.x;
+    const uint32_t cb = b / n_hid, hb = b % n_hid;
+    const uint32_t off = info[2 * b];
+    uint32_t size = info[2 * b + 1];
+    if (size > blk_cap) size = blk_cap;   // corrupt block_info must not overrun LDS
+    const uint32_t phase = stage_to_lds(stream + off, size, blk, threadIdx.x, blockDim.x);
+    __syncthreads();
+    block_decode<IS_K>(blk, phase, nunits, W, tile, hid_blk);
+    __syncthreads();
+    // coalesced write-back: rows of hid_blk bytes, as dwords
+    const int row_dw = hid_blk >> 2;
+    const uint32_t *t4 = reinterpret_cast<const uint32_t *>(tile);
+    for (int i = threadIdx.x; i < ctx_blk * row_dw; i += blockDim.x) {
+        const int row = i / row_dw, c = i % row_dw;
+        uint32_t *dst = reinterpret_cast<uint32_t *>(
+            codes + ((size_t)cb * ctx_blk + row) * hidden_dim + (size_t)hb * hid_blk);
+        dst[c] = t4[i];
+    }
+}
+
+template <bool IS_K>
+__global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                            uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                            int hidden_dim, int ctx_blk, int hid_blk, int nunits, int W,
+                            uint32_t nblocks) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t unit_bytes[16];
+    uint8_t *tile = lds;
+    uint8_t *blk = lds + round_up16((uint32_t)(ctx_blk * hid_blk));
+    if (threadIdx.x == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t b = s_idx;
+    if (b >= nblocks) return;
+    const int n_hid = hidden_dim / hid_blk;
+    const uint32_t cb = b / n_hid, hb = b % n_hid;
+    const int row_dw = hid_blk >> 2;
+    uint32_t *t4 = reinterpret_cast<uint32_t *>(tile);
+    for (int i = threadIdx.x; i < ctx_blk * row_dw; i += blockDim.x) {
+        const int row = i / row_dw, c = i % row_dw;
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(
+            codes + ((size_t)cb * ctx_blk + row) * hidden_dim + (size_t)hb * hid_blk);
+        t4[i] = src[c];
+    }
+    __syncthreads();
+    block_finish<IS_K>(tile, blk, unit_bytes, &s_off, st, b, nblocks, stream, capacity, info, hid_blk,
+                       nunits, W);
+}
+
+__global__ void zero_state_kernel(uint64_t *p, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+struct CodecShape {
+    int nunits, threads, nblocks;
+    uint32_t blk_cap, lds_bytes;
+};
+
+static int codec_shape(bool is_k, int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits,
+                       CodecShape *o) {
+    PKV_REQUIRE(bits >= 2 && bits <= 4, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (need 2..4)", bits);
+    PKV_REQUIRE(ctx_len > 0 && hidden_dim > 0 && ctx_blk > 0 && hid_blk > 0, PKV_ERR_INVALID,
+                "sizes must be positive");
+    PKV_REQUIRE(ctx_len % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
+    PKV_REQUIRE(hidden_dim % hid_blk == 0, PKV_ERR_INVALID,
+                "hidden_dim must be divisible by hidden_dim_block_size");
+    PKV_REQUIRE(ctx_blk % kPackTok == 0, PKV_ERR_INVALID, "ctx_len_block_size must be divisible by 16");
+    if (is_k) {
+        PKV_REQUIRE(hid_blk == kHeadDim, PKV_ERR_UNSUPPORTED,
+                    "not supported: K hidden_dim_block_size must be 128");
+        PKV_REQUIRE(ctx_blk <= 256, PKV_ERR_UNSUPPORTED, "not supported: K ctx_len_block_size > 256");
+        o->nunits = ctx_blk / kPackTok;
+        o->blk_cap = (uint32_t)k_block_bound(ctx_blk, bits);
+    } else {
+        PKV_REQUIRE(ctx_blk == 128, PKV_ERR_UNSUPPORTED, "not supported: V ctx_len_block_size must be 128");
+        PKV_REQUIRE(hid_blk % kLanes == 0 && hid_blk <= 256, PKV_ERR_UNSUPPORTED,
+                    "not supported: V hidden_dim_block_size must be a multiple of 32, at most 256");
+        o->nunits = 2 * (hid_blk / kLanes);
+        o->blk_cap = (uint32_t)v_block_bound(hid_blk, bits);
+    }
+    o->threads = ((32 * o->nunits + 63) / 64) * 64;
+    o->nblocks = (ctx_len / ctx_blk) * (hidden_dim / hid_blk);
+    o->lds_bytes = round_up16((uint32_t)(ctx_blk * hid_blk)) + round_up16(o->blk_cap) + 32u;
+    return PKV_OK;
+}
+
+static int run_unpack(bool is_k, const uint8_t *stream, const uint32_t *info, uint8_t *codes,
+                      int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out,
+                      hipStream_t s) {
+    PKV_REQUIRE(stream && info && codes, PKV_ERR_INVALID, "null pointer argument");
+    CodecShape cs;
+    int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
+    if (rc) return rc;
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    if (is_k)
+        unpack_kernel<true><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
+            stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
+    else
+        unpack_kernel<false><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
+            stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
+    PKV_HIP_CHECK(hipGetLastError());
+    return tm.end(ms_out);
+}
+
+// Shared tail of every encoder: read back {error, total} when the caller wants the size.
+int finish_encode(ScanState *st, uint64_t *size_out, int bits, hipStream_t s) {
+    if (!size_out) return PKV_OK;
+    struct { uint32_t ticket, error; uint64_t total; uint32_t max_code, pad; } h;
+    PKV_HIP_CHECK(hipMemcpyAsync(&h, st, sizeof(h), hipMemcpyDeviceToHost, s));
+    PKV_HIP_CHECK(hipStreamSynchronize(s));
+    if (h.error == (uint32_t)PKV_ERR_CAPACITY) {
+        set_error("compressed stream does not fit the output buffer");
+        return PKV_ERR_CAPACITY;
+    }
+    if (h.error) {
+        set_error("device-side encode failure (code %u)", h.error);
+        return (int)h.error;
+    }
+    if (bits > 0 && h.max_code >= (1u << bits)) {
+        set_error("not supported: code %u does not fit bits_len %d", h.max_code, bits);
+        return PKV_ERR_UNSUPPORTED;
+    }
+    *size_out = h.total;
+    return PKV_OK;
+}
+
+int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s) {
+    void *p = nullptr;
+    const size_t bytes = sizeof(ScanState) + (size_t)nblocks * sizeof(uint64_t);
+    int rc = scratch_get(bytes, &p);
+    if (rc) return rc;
+    const size_t n64 = (bytes + 7) / 8;
+    zero_state_kernel<<<(unsigned)((n64 + 255) / 256), 256, 0, s>>>((uint64_t *)p, n64);
+    PKV_HIP_CHECK(hipGetLastError());
+    *out = (ScanState *)p;
+    return PKV_OK;
+}
+
+static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *info,
+                    int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
+                    float *ms_out, hipStream_t s) {
+    PKV_REQUIRE(stream && info && codes, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
+    CodecShape cs;
+    int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
+    if (rc) return rc;
+    ScanState *st = nullptr;
+    if ((rc = prepare_scan_state((uint32_t)cs.nblocks, &st, s))) return rc;
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    if (is_k)
+        pack_kernel<true><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
+            codes, stream, capacity, info, st, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits,
+            (uint32_t)cs.nblocks);
+    else
+        pack_kernel<false><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
+            codes, stream, capacity, info, st, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits,
+            (uint32_t)cs.nblocks);
+    PKV_HIP_CHECK(hipGetLastError());
+    if ((rc = tm.end(ms_out))) return rc;
+    return finish_encode(st, size_out, 0, s);
+}
+
+}  // namespace pkv
+
+extern "C" {
+
+int pkv_k_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
+                 int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
+                 float *ms_out, pkv_stream_t s) {
+    return pkv::run_pack(true, codes, stream, capacity, block_info, ctx_len, hidden_dim, ctx_blk, hid_blk,
+                         bits, size_out, ms_out, (hipStream_t)s);
+}
+
+int pkv_v_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
+                 int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
+                 float *ms_out, pkv_stream_t s) {
+    return pkv::run_pack(false, codes, stream, capacity, block_info, ctx_len, hidden_dim, ctx_blk, hid_blk,
+                         bits, size_out, ms_out, (hipStream_t)s);
+}
+
+int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                 int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s) {
+    return pkv::run_unpack(true, stream, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+                           ms_out, (hipStream_t)s);
+}
+
+int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                 int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s) {
+    return pkv::run_unpack(false, stream, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+                           ms_out, (hipStream_t)s);
+}
+
+uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits) {
+    return is_k ? (uint64_t)pkv::k_block_bound(ctx_blk, bits) : (uint64_t)pkv::v_block_bound(hid_blk, bits);
+}
+
+}  // extern "C"

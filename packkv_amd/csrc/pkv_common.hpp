@@ -1,0 +1,111 @@
+// Shared definitions for the PackKV gfx950 kernels: stream-format constants, error
+// plumbing, and the small wavefront-level helpers every kernel uses.
+//
+// Stream format (restated from packkv_cuda_ext/src/{k,v}_encode_cpu.cpp of the reference):
+//   pack    16 consecutive tokens of one channel; min, len = bit_length(max - min),
+//           word = sum_k (code_k - min) << ((15 - k) * len), stored as 2*len bytes LE
+//   K block ctx_blk tokens x 128 channels: u16 cumulative round sizes, then per round
+//           (16 tokens): mins (W bits/pack) | lens (LB bits/pack) | payload in the order
+//           slot-major, lane-minor, lane t owning channels 4t..4t+3 (slot i = channel 4t+i)
+//   V block 128 tokens x 32*warps channels: u16 cumulative segment sizes in (warp, seg)
+//           order, then per segment (64 tokens x 32 channels): mins | lens | payload,
+//           lane t owning channel 32*warp + t, slot i = round 4*seg + i
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/packkv.h"   // PKV_* status codes and the exported prototypes
+
+namespace pkv {
+
+constexpr int kPackTok = 16;    // tokens per pack        (static_def.h:6)
+constexpr int kLanes = 32;      // format lanes per round (static_def.h:4)
+constexpr int kHeadDim = 128;   // K block width          (static_def.h:5)
+
+__host__ __device__ constexpr int len_field_bits(int W) {  // include/utils.h:24-36
+    return W >= 4 ? 3 : (W >= 2 ? 2 : 1);
+}
+__host__ __device__ constexpr int k_block_bound(int ctx_blk, int W) {
+    return 2 * (ctx_blk / kPackTok) +
+           (ctx_blk / kPackTok) * kHeadDim * (W + len_field_bits(W)) / 8 +
+           (ctx_blk / kPackTok) * kHeadDim * 2 * W;
+}
+__host__ __device__ constexpr int v_block_bound(int hid_blk, int W) {
+    return 4 * (hid_blk / kLanes) + 8 * hid_blk * (W + len_field_bits(W)) / 8 + 8 * hid_blk * 2 * W;
+}
+
+void set_error(const char *fmt, ...);
+
+#define PKV_HIP_CHECK(expr)                                                              \
+    do {                                                                                 \
+        hipError_t e__ = (expr);                                                         \
+        if (e__ != hipSuccess) {                                                         \
+            ::pkv::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__),     \
+                             __FILE__, __LINE__);                                        \
+            return PKV_ERR_HIP;                                                   \
+        }                                                                                \
+    } while (0)
+
+#define PKV_REQUIRE(cond, code, ...)                                                     \
+    do {                                                                                 \
+        if (!(cond)) {                                                                   \
+            ::pkv::set_error(__VA_ARGS__);                                               \
+            return (code);                                                               \
+        }                                                                                \
+    } while (0)
+
+// ---- device helpers ---------------------------------------------------------
+#ifdef __HIPCC__
+
+__device__ __forceinline__ int bit_length_u32(uint32_t v) { return 32 - __clz((int)v); }
+
+// Exclusive prefix sum over the 32 lanes of a half-wavefront; `total` receives the sum.
+__device__ __forceinline__ uint32_t half_excl_scan(uint32_t v, uint32_t &total) {
+    const int t = threadIdx.x & 31;
+    uint32_t incl = v;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) {
+        uint32_t up = __shfl_up(incl, d, 32);
+        if (t >= d) incl += up;
+    }
+    total = __shfl(incl, 31, 32);
+    return incl - v;
+}
+
+// 64 bits starting at byte offset `off` (2-byte aligned) of an LDS byte array whose base
+// is 4-byte aligned.  Reads three aligned dwords; never issues an unaligned LDS access.
+__device__ __forceinline__ uint64_t lds_load64(const uint8_t *lds, uint32_t off) {
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(lds + (off & ~3u));
+    uint32_t d0 = p[0], d1 = p[1], d2 = p[2];
+    uint32_t sh = (off & 2u) * 8u;
+    uint32_t lo = __builtin_amdgcn_alignbit(d1, d0, sh);
+    uint32_t hi = __builtin_amdgcn_alignbit(d2, d1, sh);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// The 4*nbits-bit metadata word of format lane t from an LSB-first bit array (4 fields
+// of nbits each; nbits in {2,3,4}).
+__device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int nbits) {
+    const uint32_t bit = (uint32_t)t * 4u * (uint32_t)nbits;
+    const uint32_t byte = bit >> 3;
+    uint32_t v = (uint32_t)arr[byte] | ((uint32_t)arr[byte + 1] << 8);
+    return (v >> (bit & 7u)) & ((1u << (4 * nbits)) - 1u);
+}
+
+// Copy `nbytes` from global `src` (any alignment) into LDS `dst` (4-byte aligned) so that
+// dst[(src & 3) + i] == src[i]; touches only the aligned dwords that overlap the range.
+// Returns the phase (src & 3).
+__device__ __forceinline__ uint32_t stage_to_lds(const uint8_t *src, uint32_t nbytes, uint8_t *dst,
+                                                 int tid, int nthreads) {
+    const uint32_t phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 3u);
+    const uint32_t *s4 = reinterpret_cast<const uint32_t *>(src - phase);
+    uint32_t *d4 = reinterpret_cast<uint32_t *>(dst);
+    const uint32_t ndw = (phase + nbytes + 3u) >> 2;
+    for (uint32_t i = tid; i < ndw; i += nthreads) d4[i] = s4[i];
+    return phase;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace pkv

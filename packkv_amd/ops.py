@@ -1,0 +1,435 @@
+"""Python op surface over the C ABI: the reference's eight ``packkv_cuda`` functions with the
+same positional signatures (packkv_cuda_ext/packkv_cuda.pyi:4-86, bound in
+packkv_cuda_ext/export_packkv.cpp:9-18), plus the device-native ops the reference does not
+have (GPU encode / unpack, fused quantize+encode, fused decompress-attention).
+
+All tensors are caller-allocated and written in place, as in the reference.  PyTorch is used
+for device memory and the current stream only; every computation happens in
+libpackkv_hip.so.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import AttnArgs, PackKVError  # noqa: F401  (re-exported)
+
+__all__ = [
+    "k_encode_cpu", "k_decode_cpu", "v_encode_cpu", "v_decode_cpu",
+    "kq_mat_vec_mul", "wv_mat_vec_mul", "fused_kq", "fused_wv",
+    "k_encode", "v_encode", "k_decode", "v_decode",
+    "quant_params", "quantize", "dequantize", "k_quant_encode", "v_quant_encode",
+    "attn_decode", "block_bound", "bits_for_rel",
+]
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float16:
+        return _lib.F16
+    if t.dtype == torch.bfloat16:
+        return _lib.BF16
+    raise RuntimeError("Unsupported data type")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _require(cond, msg):
+    if not cond:
+        raise RuntimeError("PackKV Assertion failed: " + msg)
+
+
+def _device_of(*tensors):
+    dev = None
+    for t in tensors:
+        if t.is_cuda:
+            dev = t.device
+    if dev is None:
+        if not torch.cuda.is_available():
+            raise RuntimeError("packkv needs a GPU: the ops run in libpackkv_hip.so, there is no CPU path")
+        dev = torch.device("cuda", torch.cuda.current_device())
+    return dev
+
+
+def block_bound(is_k, ctx_blk, hid_blk, bits):
+    return int(_lib.load().pkv_block_bound(int(is_k), ctx_blk, hid_blk, bits))
+
+
+def bits_for_rel(rel):
+    """Raw code width W for a relative quant step: codes span 0..ceil(1/rel), plus at most one
+    more level from rounding the quotient to the storage type."""
+    import math
+    top = math.ceil(1.0 / rel - 1e-9) + 1
+    return max(2, top.bit_length())
+
+
+# ------------------------------------------------------------------ codec ------------
+
+def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k):
+    # mirrors k_encode_cpu_assert / v_encode_cpu_assert (src/k_encode_cpu.cpp:247-284,
+    # src/v_encode_cpu.cpp:262-299); raises instead of aborting the process
+    _require(codes.dim() == 2 and codes.size(0) == ctx_len, "ctx_len mismatch")
+    _require(codes.size(1) == hidden_dim, "hidden_dim mismatch")
+    _require(ctx_blk > 0, "ctx_len_block_size must be greater than 0")
+    _require(hid_blk > 0, "hidden_dim_block_size must be greater than 0")
+    _require(ctx_len % ctx_blk == 0, "ctx_len must be divisible by ctx_len_block_size")
+    _require(hidden_dim % hid_blk == 0, "hidden_dim must be divisible by hidden_dim_block_size")
+    nblk = (ctx_len // ctx_blk) * (hidden_dim // hid_blk)
+    _require(info.dim() == 2 and info.size(0) == nblk, "block_info_buffer block num mismatch")
+    _require(info.size(1) == 2, "block_info_buffer.size(1) must be 2")
+    _require(bits <= 4, "bits_len must be less than or equal to 4")
+    _require(ctx_blk % 16 == 0, "ctx_len_block_size must be divisible by PACK_ELE_NUM")
+    if is_k:
+        _require(hid_blk == 128, "hidden_dim_block_size must be 128, because this is most common head dim")
+    _require(codes.dtype == torch.uint8, "quant_ints_tensor must be a UInt8 tensor")
+    _require(stream.dtype == torch.uint8, "compressed_buffer must be a UInt8 tensor")
+    _require(stream.numel() > 0, "compressed_buffer must be a non-empty tensor")
+    _require(info.dtype == torch.uint32, "block_info_buffer must be a UInt32 tensor")
+    _require(codes.is_contiguous() and stream.is_contiguous() and info.is_contiguous(),
+             "tensors must be contiguous")
+
+
+def _encode(is_k, codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, want_size=True,
+            timed=False):
+    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k)
+    lib = _lib.load()
+    dev = _device_of(codes, stream, info)
+    on_host = not codes.is_cuda
+    _require(stream.is_cuda != on_host and info.is_cuda != on_host, "all tensors must be on one device")
+    d_codes = codes.to(dev) if on_host else codes
+    d_stream = torch.empty(stream.numel(), dtype=torch.uint8, device=dev) if on_host else stream
+    d_info = torch.empty_like(info, device=dev) if on_host else info
+    size = ctypes.c_uint64(0)
+    ms = ctypes.c_float(0.0)
+    fn = lib.pkv_k_encode if is_k else lib.pkv_v_encode
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(d_codes), _ptr(d_stream), d_stream.numel(), _ptr(d_info), ctx_len, hidden_dim,
+                ctx_blk, hid_blk, bits, ctypes.byref(size) if (want_size or on_host) else None,
+                ctypes.byref(ms) if timed else None, _stream(dev))
+    _lib.check(rc)
+    if on_host:
+        n = int(size.value)
+        stream.view(-1)[:n].copy_(d_stream[:n].cpu())
+        info.copy_(d_info.cpu())
+    return (int(size.value), float(ms.value)) if timed else int(size.value)
+
+
+def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, timed=False):
+    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k)
+    lib = _lib.load()
+    dev = _device_of(codes, stream, info)
+    on_host = not codes.is_cuda
+    _require(stream.is_cuda != on_host and info.is_cuda != on_host, "all tensors must be on one device")
+    d_stream = stream.to(dev) if on_host else stream
+    d_info = info.to(dev) if on_host else info
+    d_codes = torch.empty_like(codes, device=dev) if on_host else codes
+    ms = ctypes.c_float(0.0)
+    fn = lib.pkv_k_decode if is_k else lib.pkv_v_decode
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(d_stream), _ptr(d_info), _ptr(d_codes), ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+                ctypes.byref(ms) if timed else None, _stream(dev))
+    _lib.check(rc)
+    if on_host:
+        codes.copy_(d_codes.cpu())
+    return float(ms.value) if timed else None
+
+
+def k_encode_cpu(quant_ints_tensor, compressed_buffer, block_info_buffer, ctx_len, hidden_dim,
+                 ctx_len_block_size, hidden_dim_block_size, bits_len):
+    """Drop-in for packkv_cuda.k_encode_cpu (packkv_cuda.pyi:4-13): host tensors in, host tensors
+    written in place, stream size returned -- but encoded on the GPU (staged through device
+    memory).  Device tensors are accepted too and then nothing is copied."""
+    return _encode(True, quant_ints_tensor, compressed_buffer, block_info_buffer, ctx_len, hidden_dim,
+                   ctx_len_block_size, hidden_dim_block_size, bits_len)
+
+
+def v_encode_cpu(quant_ints_tensor, compressed_buffer, block_info_buffer, ctx_len, hidden_dim,
+                 ctx_len_block_size, hidden_dim_block_size, bits_len):
+    """Drop-in for packkv_cuda.v_encode_cpu (packkv_cuda.pyi:38-47)."""
+    return _encode(False, quant_ints_tensor, compressed_buffer, block_info_buffer, ctx_len, hidden_dim,
+                   ctx_len_block_size, hidden_dim_block_size, bits_len)
+
+
+def k_decode_cpu(compressed_buffer, block_info_buffer, quant_ints_tensor, ctx_len, hidden_dim,
+                 ctx_len_block_size, hidden_dim_block_size, bits_len):
+    """Drop-in for packkv_cuda.k_decode_cpu (packkv_cuda.pyi:15-24)."""
+    _decode(True, compressed_buffer, block_info_buffer, quant_ints_tensor, ctx_len, hidden_dim,
+            ctx_len_block_size, hidden_dim_block_size, bits_len)
+
+
+def v_decode_cpu(compressed_buffer, block_info_buffer, quant_ints_tensor, ctx_len, hidden_dim,
+                 ctx_len_block_size, hidden_dim_block_size, bits_len):
+    """Drop-in for packkv_cuda.v_decode_cpu (packkv_cuda.pyi:49-58)."""
+    _decode(False, compressed_buffer, block_info_buffer, quant_ints_tensor, ctx_len, hidden_dim,
+            ctx_len_block_size, hidden_dim_block_size, bits_len)
+
+
+def k_encode(codes, stream, info, ctx_blk=64, hid_blk=128, bits=4, want_size=True, timed=False):
+    """Device encode of a uint8 code matrix [ctx_len, hidden]; returns the stream size (and ms)."""
+    return _encode(True, codes, stream, info, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits,
+                   want_size, timed)
+
+
+def v_encode(codes, stream, info, ctx_blk=128, hid_blk=64, bits=4, want_size=True, timed=False):
+    return _encode(False, codes, stream, info, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits,
+                   want_size, timed)
+
+
+def k_decode(stream, info, codes, ctx_blk=64, hid_blk=128, bits=4, timed=False):
+    return _decode(True, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed)
+
+
+def v_decode(stream, info, codes, ctx_blk=128, hid_blk=64, bits=4, timed=False):
+    return _decode(False, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed)
+
+
+# --------------------------------------------------------------- quantizer -----------
+
+def _check_x(x):
+    _require(x.is_cuda and x.dim() == 4 and x.size(3) == 128 and x.is_contiguous(),
+             "x must be a contiguous device tensor [B, H, T, 128]")
+    return x.size(0), x.size(1), x.size(2)
+
+
+def quant_params(x, rel, timed=False):
+    """Per-(batch, token) scale and zero of quant_ints(TokenQuant) (utils/compute.py:84-112);
+    returns (scale, zero) as [B, T] tensors of x.dtype."""
+    B, H, T = _check_x(x)
+    scale = torch.empty(B, T, dtype=x.dtype, device=x.device)
+    zero = torch.empty(B, T, dtype=x.dtype, device=x.device)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().pkv_quant_params(_ptr(x), _dtype_code(x), B, H, T, float(rel), _ptr(scale),
+                                          _ptr(zero), ctypes.byref(ms) if timed else None, _stream(x.device))
+    _lib.check(rc)
+    return (scale, zero, float(ms.value)) if timed else (scale, zero)
+
+
+def quantize(x, scale, zero):
+    """uint8 code matrix [T, B*H*128] (layout of evaluation/evaluation.py:406) and the largest code."""
+    B, H, T = _check_x(x)
+    codes = torch.empty(T, B * H * 128, dtype=torch.uint8, device=x.device)
+    mx = torch.zeros(1, dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().pkv_quantize(_ptr(x), _dtype_code(x), B, H, T, _ptr(scale), _ptr(zero), _ptr(codes),
+                                      _ptr(mx), None, _stream(x.device))
+    _lib.check(rc)
+    return codes, int(mx.item())
+
+
+def dequantize(codes, scale, zero, B, H):
+    """(code + zero) * scale in the storage dtype -> [B, H, T, 128] (utils/compute.py:173-179)."""
+    T = codes.size(0)
+    x = torch.empty(B, H, T, 128, dtype=scale.dtype, device=codes.device)
+    with torch.cuda.device(codes.device):
+        rc = _lib.load().pkv_dequantize(_ptr(codes), _dtype_code(scale), B, H, T, _ptr(scale), _ptr(zero),
+                                        _ptr(x), None, _stream(codes.device))
+    _lib.check(rc)
+    return x
+
+
+def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed):
+    B, H, T = _check_x(x)
+    hidden = B * H * 128
+    ctx_blk, hid_blk = (64, 128) if is_k else (128, 64)
+    nblk = (T // ctx_blk) * (hidden // hid_blk)
+    if stream is None:
+        stream = torch.empty(T * hidden, dtype=torch.uint8, device=x.device)
+    if info is None:
+        info = torch.empty(nblk, 2, dtype=torch.uint32, device=x.device)
+    _require(info.numel() == 2 * nblk and info.dtype == torch.uint32, "block_info_buffer block num mismatch")
+    scale = torch.empty(B, T, dtype=x.dtype, device=x.device)
+    zero = torch.empty(B, T, dtype=x.dtype, device=x.device)
+    size = ctypes.c_uint64(0)
+    ms = ctypes.c_float(0.0)
+    fn = _lib.load().pkv_k_quant_encode if is_k else _lib.load().pkv_v_quant_encode
+    with torch.cuda.device(x.device):
+        rc = fn(_ptr(x), _dtype_code(x), B, H, T, float(rel), bits, _ptr(stream), stream.numel(), _ptr(info),
+                _ptr(scale), _ptr(zero), ctypes.byref(size) if want_size else None,
+                ctypes.byref(ms) if timed else None, _stream(x.device))
+    _lib.check(rc)
+    return {"stream": stream, "info": info, "scale": scale, "zero": zero, "size": int(size.value),
+            "ms": float(ms.value), "bits": bits}
+
+
+def k_quant_encode(x, rel, bits=None, stream=None, info=None, want_size=True, timed=False):
+    """Fused quantize + K encode of x [B, H, T, 128]; returns a dict with stream, info (block_info),
+    scale, zero [B, T], size (bytes), ms and bits."""
+    return _quant_encode(True, x, rel, bits or bits_for_rel(rel), stream, info, want_size, timed)
+
+
+def v_quant_encode(x, rel, bits=None, stream=None, info=None, want_size=True, timed=False):
+    return _quant_encode(False, x, rel, bits or bits_for_rel(rel), stream, info, want_size, timed)
+
+
+# ------------------------------------------------------- reference GEMV surface ------
+
+def _require_cuda(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError("tensor must be a CUDA tensor")
+
+
+def kq_mat_vec_mul(compressed_buffer, block_info_buffer, q, kq_out, ctx_len, hidden_dim,
+                   ctx_len_block_size, hidden_dim_block_size, bits_len, q_interleaved=True):
+    """Drop-in for packkv_cuda.kq_mat_vec_mul (packkv_cuda.pyi:26-36): kq_out[h, tok] =
+    sum_d q[h, d] * code[tok, h*128 + d]; returns kernel milliseconds.  `q` is expected in the
+    reference's lane-interleaved layout (evaluation/evaluation.py:465-468) unless
+    q_interleaved=False.  Like the reference, an unsupported shape or dtype prints a message
+    and returns 0.0 (src/kernels.cu:586-589, :626-629)."""
+    _require_cuda(compressed_buffer, block_info_buffer, q, kq_out)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        print("Unsupported data type")
+        return 0.0
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().pkv_kq_mat_vec_mul(_ptr(compressed_buffer), _ptr(block_info_buffer), _ptr(q),
+                                            _ptr(kq_out), ctx_len, hidden_dim, ctx_len_block_size,
+                                            hidden_dim_block_size, bits_len, _dtype_code(q),
+                                            int(bool(q_interleaved)), ctypes.byref(ms), _stream(q.device))
+    if rc == _lib.ERR_UNSUPPORTED:
+        print("no such case")
+        return 0.0
+    _lib.check(rc)
+    return float(ms.value)
+
+
+def wv_mat_vec_mul(compressed_buffer, block_info_buffer, w, wv_out, ctx_len, hidden_dim,
+                   ctx_len_block_size, hidden_dim_block_size, bits_len):
+    """Drop-in for packkv_cuda.wv_mat_vec_mul (packkv_cuda.pyi:60-70): wv_out (fp32, caller-zeroed,
+    [hidden_dim] or [H, 128]) += sum_tok w[c // 128, tok] * code[tok, c]; returns milliseconds."""
+    _require_cuda(compressed_buffer, block_info_buffer, w, wv_out)
+    if w.dtype not in (torch.float16, torch.bfloat16):
+        print("Unsupported data type")
+        return 0.0
+    if wv_out.dtype != torch.float32:
+        raise RuntimeError("wv_out must be a float32 tensor")
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(w.device):
+        rc = _lib.load().pkv_wv_mat_vec_mul(_ptr(compressed_buffer), _ptr(block_info_buffer), _ptr(w),
+                                            _ptr(wv_out), ctx_len, hidden_dim, ctx_len_block_size,
+                                            hidden_dim_block_size, bits_len, _dtype_code(w),
+                                            ctypes.byref(ms), _stream(w.device))
+    if rc == _lib.ERR_UNSUPPORTED:
+        print("no such case")
+        return 0.0
+    _lib.check(rc)
+    return float(ms.value)
+
+
+def fused_kq(our_kq, q, k_quant_zero, k_quant_scale, t):
+    """Drop-in for packkv_cuda.fused_kq (packkv_cuda.pyi:72-78; checks of
+    src/fused_kernels.cu:90-108): our_kq[m, n] = (sum(q[m]) * zero[n] + t[m, n]) * scale[n]."""
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("Unsupported data type for fused_kq_launcher")
+    if q.dim() != 2: raise RuntimeError("q must be a 2D tensor")
+    if t.dim() != 2: raise RuntimeError("t must be a 2D tensor")
+    if k_quant_zero.dim() != 1: raise RuntimeError("k_quant_zero must be a 1D tensor")
+    if k_quant_scale.dim() != 1: raise RuntimeError("k_quant_scale must be a 1D tensor")
+    if our_kq.dim() != 2: raise RuntimeError("our_kq must be a 2D tensor")
+    M, K = q.shape
+    N = t.size(1)
+    if t.size(0) != M: raise RuntimeError("t.size(0) must be equal to q.size(0)")
+    if k_quant_zero.size(0) != N: raise RuntimeError("k_quant_zero.size(0) must be equal to t.size(1)")
+    if k_quant_scale.size(0) != N: raise RuntimeError("k_quant_scale.size(0) must be equal to t.size(1)")
+    if our_kq.size(0) != M: raise RuntimeError("our_kq.size(0) must be equal to q.size(0)")
+    if our_kq.size(1) != N: raise RuntimeError("our_kq.size(1) must be equal to t.size(1)")
+    for name, x in (("q", q), ("t", t), ("k_quant_zero", k_quant_zero), ("k_quant_scale", k_quant_scale),
+                    ("our_kq", our_kq)):
+        if not x.is_cuda:
+            raise RuntimeError("%s must be a CUDA tensor" % name)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().pkv_fused_kq(_ptr(our_kq), _ptr(q.contiguous()), _ptr(k_quant_zero.contiguous()),
+                                      _ptr(k_quant_scale.contiguous()), _ptr(t.contiguous()), M, K, N,
+                                      _dtype_code(q), ctypes.byref(ms), _stream(q.device))
+    _lib.check(rc)
+    return float(ms.value)
+
+
+def fused_wv(our_wv, w, v_quant_zero, v_quant_scale, term1):
+    """Drop-in for packkv_cuda.fused_wv (packkv_cuda.pyi:80-86; checks of
+    src/fused_kernels.cu:275-293): our_wv[m, d] = sum_n w[m, n] * zero[n] * scale[n] + term1[m, d]."""
+    if w.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("Unsupported data type for fused_wv_launcher")
+    if w.dim() != 2: raise RuntimeError("w must be a 2D tensor")
+    if term1.dim() != 2: raise RuntimeError("term1 must be a 2D tensor")
+    if v_quant_zero.dim() != 1: raise RuntimeError("v_quant_zero must be a 1D tensor")
+    if v_quant_scale.dim() != 1: raise RuntimeError("v_quant_scale must be a 1D tensor")
+    if our_wv.dim() != 2: raise RuntimeError("our_wv must be a 2D tensor")
+    M, N = w.shape
+    D = term1.size(1)
+    if term1.size(0) != M: raise RuntimeError("term1.size(0) must be equal to w.size(0)")
+    if v_quant_zero.size(0) != N: raise RuntimeError("v_quant_zero.size(0) must be equal to w.size(1)")
+    if v_quant_scale.size(0) != N: raise RuntimeError("v_quant_scale.size(0) must be equal to w.size(1)")
+    if tuple(our_wv.shape) != (M, D): raise RuntimeError("our_wv shape must match term1")
+    if term1.dtype != w.dtype: raise RuntimeError("term1 must have the dtype of w")
+    for name, x in (("w", w), ("term1", term1), ("v_quant_zero", v_quant_zero),
+                    ("v_quant_scale", v_quant_scale), ("our_wv", our_wv)):
+        if not x.is_cuda:
+            raise RuntimeError("%s must be a CUDA tensor" % name)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(w.device):
+        rc = _lib.load().pkv_fused_wv(_ptr(our_wv), _ptr(w.contiguous()), _ptr(v_quant_zero.contiguous()),
+                                      _ptr(v_quant_scale.contiguous()), _ptr(term1.contiguous()), M, N, D,
+                                      _dtype_code(w), ctypes.byref(ms), _stream(w.device))
+    _lib.check(rc)
+    return float(ms.value)
+
+
+# ------------------------------------------------- fused decompress-attention --------
+
+def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False):
+    """One decode step over a compressed cache.
+
+    q [B, Hq, 128]; k and v are the dicts returned by k_quant_encode / v_quant_encode (stream,
+    info, scale, zero, bits) or None when only the 16-bit window exists; k_win / v_win are
+    optional [B, Hkv, T_w, 128] tails.  Returns out [B, Hq, 128] (and ms when timed)."""
+    _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
+             "q must be a contiguous device tensor [B, Hq, 128]")
+    B, Hq, _ = q.shape
+    a = AttnArgs()
+    T_c = 0
+    Hkv = None
+    keep = [q]
+    if k is not None:
+        T_c = k["scale"].size(1)
+        for name, d in (("k", k), ("v", v)):
+            for f in ("stream", "info", "scale", "zero"):
+                _require(d[f].is_cuda and d[f].is_contiguous(), "%s.%s must be a contiguous device tensor" % (name, f))
+        nblk_k = k["info"].numel() // 2
+        Hkv = nblk_k // (T_c // 64) // B
+        a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
+        a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
+        a.k_scale, a.k_zero = _ptr(k["scale"]), _ptr(k["zero"])
+        a.v_scale, a.v_zero = _ptr(v["scale"]), _ptr(v["zero"])
+        a.k_bits, a.v_bits = int(k["bits"]), int(v["bits"])
+    T_w = 0
+    if k_win is not None:
+        _require(k_win.is_cuda and v_win.is_cuda and k_win.is_contiguous() and v_win.is_contiguous()
+                 and k_win.shape == v_win.shape and k_win.dim() == 4 and k_win.size(3) == 128
+                 and k_win.dtype == q.dtype and v_win.dtype == q.dtype,
+                 "window tensors must be contiguous [B, Hkv, T_w, 128] of q's dtype")
+        T_w = k_win.size(2)
+        _require(Hkv is None or Hkv == k_win.size(1), "window head count mismatch")
+        Hkv = k_win.size(1)
+        a.k_win, a.v_win = _ptr(k_win), _ptr(v_win)
+    _require(Hkv is not None, "empty cache")
+    if out is None:
+        out = torch.empty_like(q)
+    a.q, a.out = _ptr(q), _ptr(out)
+    a.B, a.Hq, a.Hkv, a.T_c, a.T_w = B, Hq, Hkv, T_c, T_w
+    a.dtype = _dtype_code(q)
+    a.sm_scale = float(sm_scale if sm_scale is not None else 128 ** -0.5)
+    a.variant = int(variant)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().pkv_attn_decode(ctypes.byref(a), ctypes.byref(ms) if timed else None,
+                                         _stream(q.device))
+    _lib.check(rc)
+    return (out, float(ms.value)) if timed else out

@@ -1,0 +1,144 @@
+"""GPU parity of the bit-pack / bit-unpack kernels against the CPU oracle: bit-exact stream,
+block_info, size and decoded codes, through the C ABI (packkv_amd.ops -> libpackkv_hip.so)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import codec
+from packkv_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _rand_codes(rng, T, H, W, kind):
+    if kind == "uniform":
+        c = rng.integers(0, 1 << W, (T, H))
+    elif kind == "const":
+        c = np.full((T, H), (1 << W) - 1)
+    elif kind == "narrow":
+        c = rng.integers(0, 2, (T, H)) + rng.integers(0, (1 << W) - 1, (1, H))
+    else:
+        c = np.clip(np.rint(rng.normal(1 << (W - 1), 1.0, (T, H))), 0, (1 << W) - 1)
+    return c.astype(np.uint8)
+
+
+def _gpu_encode(cuda, is_k, c, cb, hb, W):
+    T, H = c.shape
+    d_codes = torch.from_numpy(c).to(cuda)
+    d_stream = torch.zeros(T * H, dtype=torch.uint8, device=cuda)
+    d_info = torch.zeros((T // cb) * (H // hb), 2, dtype=torch.uint32, device=cuda)
+    fn = ops.k_encode if is_k else ops.v_encode
+    size = fn(d_codes, d_stream, d_info, cb, hb, W)
+    return d_stream, d_info, size
+
+
+SHAPES = {1: [(64, 128, 64, 128), (256, 512, 64, 128), (128, 4096, 64, 128), (64, 256, 32, 128),
+              (256, 128, 128, 128), (32, 128, 16, 128)],
+          0: [(128, 64, 128, 64), (512, 512, 128, 64), (128, 4096, 128, 64), (256, 128, 128, 32),
+              (128, 256, 128, 128)]}
+
+
+@pytest.mark.parametrize("is_k", [1, 0])
+@pytest.mark.parametrize("W", [2, 3, 4])
+def test_encode_decode_bit_exact_vs_oracle(cuda, oracle_codec, is_k, W):
+    rng = np.random.default_rng(100 + 10 * is_k + W)
+    for (T, H, cb, hb) in SHAPES[is_k]:
+        for kind in ("uniform", "const", "narrow", "gauss"):
+            _say("codec case", "K" if is_k else "V", T, H, cb, hb, W, kind)
+            c = _rand_codes(rng, T, H, W, kind)
+            so, io, zo = oracle_codec.encode(is_k, c, cb, hb, W)
+            d_stream, d_info, size = _gpu_encode(cuda, is_k, c, cb, hb, W)
+            assert size == zo
+            assert np.array_equal(d_info.cpu().numpy(), io)
+            assert np.array_equal(d_stream[:size].cpu().numpy(), so[:zo])
+            # unpack both the GPU stream and (independently) the oracle stream
+            d_out = torch.zeros(T, H, dtype=torch.uint8, device=cuda)
+            (ops.k_decode if is_k else ops.v_decode)(d_stream, d_info, d_out, cb, hb, W)
+            assert np.array_equal(d_out.cpu().numpy(), c)
+            d_out.zero_()
+            s2 = torch.from_numpy(so[:zo].copy()).to(cuda)      # exactly-sized stream buffer
+            (ops.k_decode if is_k else ops.v_decode)(s2, torch.from_numpy(io).to(cuda), d_out, cb, hb, W)
+            assert np.array_equal(d_out.cpu().numpy(), c)
+
+
+def test_golden_vectors_from_reference_codec(cuda, golden):
+    for name in [str(n) for n in golden["cases"]]:
+        is_k, T, H, cb, hb, W, size = [int(x) for x in golden[name + "_meta"]]
+        _say("golden", name)
+        c = golden[name + "_codes"]
+        d_stream, d_info, got = _gpu_encode(cuda, is_k, c, cb, hb, W)
+        assert got == size
+        assert np.array_equal(d_info.cpu().numpy(), golden[name + "_info"])
+        assert np.array_equal(d_stream[:size].cpu().numpy(), golden[name + "_stream"])
+        d_out = torch.zeros(T, H, dtype=torch.uint8, device=cuda)
+        (ops.k_decode if is_k else ops.v_decode)(torch.from_numpy(golden[name + "_stream"]).to(cuda),
+                                                 torch.from_numpy(golden[name + "_info"]).to(cuda),
+                                                 d_out, cb, hb, W)
+        assert np.array_equal(d_out.cpu().numpy(), c)
+
+
+def test_drop_in_cpu_signatures_round_trip(cuda, oracle_codec):
+    """The reference call sequence (evaluation/evaluation.py:419-456) with host tensors."""
+    import packkv_cuda
+    rng = np.random.default_rng(7)
+    for is_k, (cb, hb, W) in ((1, (64, 128, 4)), (0, (128, 64, 3))):
+        T, H = 256, 1024
+        block = torch.from_numpy(_rand_codes(rng, T, H, W, "gauss"))
+        info = torch.zeros((T // cb) * (H // hb), 2, dtype=torch.uint32)
+        comp = torch.zeros_like(block)
+        enc = packkv_cuda.k_encode_cpu if is_k else packkv_cuda.v_encode_cpu
+        dec = packkv_cuda.k_decode_cpu if is_k else packkv_cuda.v_decode_cpu
+        size = enc(block, comp, info, T, H, cb, hb, W)
+        so, io, zo = oracle_codec.encode(is_k, block.numpy(), cb, hb, W)
+        assert size == zo and np.array_equal(info.numpy(), io)
+        assert np.array_equal(comp.flatten()[:size].numpy(), so[:zo])
+        back = torch.zeros_like(block)
+        dec(comp, info, back, T, H, cb, hb, W)
+        assert (block == back).all()
+
+
+def test_error_conventions(cuda):
+    c = torch.zeros(64, 128, dtype=torch.uint8, device=cuda)
+    s = torch.zeros(64 * 128, dtype=torch.uint8, device=cuda)
+    i = torch.zeros(1, 2, dtype=torch.uint32, device=cuda)
+    with pytest.raises(RuntimeError, match="not supported"):
+        ops.k_encode(c, s, i, 64, 128, 1)
+    with pytest.raises(RuntimeError, match="bits_len"):
+        ops.k_encode(c, s, i, 64, 128, 5)
+    with pytest.raises(RuntimeError, match="block num mismatch"):
+        ops.k_encode(c, s, torch.zeros(2, 2, dtype=torch.uint32, device=cuda), 64, 128, 4)
+    with pytest.raises(RuntimeError, match="UInt8"):
+        ops.k_encode(c.to(torch.int32), s, i, 64, 128, 4)
+    # output buffer too small for the stream: reported, nothing written out of bounds
+    rnd = torch.randint(0, 16, (64, 128), dtype=torch.uint8, device=cuda)
+    small = torch.zeros(1000, dtype=torch.uint8, device=cuda)
+    with pytest.raises(ops.PackKVError) as e:
+        ops.k_encode(rnd, small, i, 64, 128, 4)
+    assert e.value.code == 4
+
+
+def test_round_trip_at_bench_scale(cuda):
+    """Size-independent property at a full-size shape (8 KV heads x 128 x 32768 tokens x batch 4):
+    decode(encode(x)) == x, offsets are the prefix sum of sizes, sizes are within the block bounds."""
+    T, H = 32768, 4 * 8 * 128
+    g = torch.Generator(device=cuda)
+    g.manual_seed(11)
+    x = torch.randn(T, H, device=cuda, generator=g)
+    codes = ((x - x.amin(1, keepdim=True)) / (x.amax(1, keepdim=True) - x.amin(1, keepdim=True)) * 10).round().to(torch.uint8)
+    del x
+    for is_k, (cb, hb) in ((1, (64, 128)), (0, (128, 64))):
+        stream = torch.empty(T * H, dtype=torch.uint8, device=cuda)
+        info = torch.empty((T // cb) * (H // hb), 2, dtype=torch.uint32, device=cuda)
+        size = (ops.k_encode if is_k else ops.v_encode)(codes, stream, info, cb, hb, 4)
+        inf = info.cpu().numpy().astype(np.int64)
+        assert int(inf[:, 1].sum()) == size
+        assert np.array_equal(inf[:, 0], np.concatenate([[0], np.cumsum(inf[:, 1])[:-1]]))
+        assert inf[:, 1].min() >= (456 if is_k else 8 + 4 * 112) and inf[:, 1].max() <= 4552
+        out = torch.zeros_like(codes)
+        (ops.k_decode if is_k else ops.v_decode)(stream, info, out, cb, hb, 4)
+        assert torch.equal(out, codes)
+        _say("bench-scale", "K" if is_k else "V", "ratio uint8/stream = %.3f" % (T * H / size))

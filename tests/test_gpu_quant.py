@@ -1,0 +1,62 @@
+"""GPU parity of the quantizer and the fused quantize+encode kernels: integer codes, scale, zero,
+dequantised values and the packed stream are bit-exact against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from packkv_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rel", [0.1, 0.2, 0.14])
+def test_quantizer_bit_exact(cuda, dtype, rel):
+    B, H, T = 2, 8, 256
+    k, v = synth.make_kv(B, H, T, seed=21, dtype=dtype)
+    for name, x in (("k", k), ("v", v)):
+        _say("quant case", name, dtype, rel)
+        c, z, s = oq.quant_ints(x, 64, rel)
+        want_codes = oq.code_matrix(c)
+        xd = x.to(cuda)
+        scale, zero = ops.quant_params(xd, rel)
+        assert torch.equal(scale.cpu().view(torch.int16), s.reshape(B, T).view(torch.int16))
+        assert torch.equal(zero.cpu().view(torch.int16), z.reshape(B, T).view(torch.int16))
+        codes, mx = ops.quantize(xd, scale, zero)
+        assert torch.equal(codes.cpu(), want_codes)
+        assert mx == int(want_codes.max())
+        y = ops.dequantize(codes, scale, zero, B, H)
+        want_y = oq.dequant(c, z, s)
+        assert torch.equal(y.cpu().view(torch.int16), want_y.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
+    for (B, H, T, rel) in ((1, 2, 128, 0.1), (2, 8, 256, 0.1), (1, 32, 128, 0.1), (2, 4, 256, 0.2), (1, 8, 128, 0.34)):
+        k, v = synth.make_kv(B, H, T, seed=31 + H, dtype=dtype)
+        for is_k, x in ((1, k), (0, v)):
+            _say("fused quant+encode", "K" if is_k else "V", dtype, B, H, T, rel)
+            c, z, s = oq.quant_ints(x, 64, rel)
+            cm = oq.code_matrix(c).numpy()
+            W = ops.bits_for_rel(rel)
+            assert oq.bits_for_codes(torch.from_numpy(cm)) <= W
+            cb, hb = (64, 128) if is_k else (128, 64)
+            so, io, zo = oracle_codec.encode(is_k, cm, cb, hb, W)
+            r = (ops.k_quant_encode if is_k else ops.v_quant_encode)(x.to(cuda), rel, W)
+            assert r["size"] == zo
+            assert np.array_equal(r["info"].cpu().numpy(), io)
+            assert np.array_equal(r["stream"][:zo].cpu().numpy(), so[:zo])
+            assert torch.equal(r["scale"].cpu().view(torch.int16), s.reshape(B, T).view(torch.int16))
+            assert torch.equal(r["zero"].cpu().view(torch.int16), z.reshape(B, T).view(torch.int16))
+
+
+def test_code_wider_than_bits_is_reported(cuda):
+    k, _ = synth.make_kv(1, 2, 128, seed=5)
+    with pytest.raises(ops.PackKVError) as e:
+        ops.k_quant_encode(k.to(cuda), 0.1, 3)     # codes reach 10..11: needs 4 bits
+    assert e.value.code == 1 and "does not fit" in str(e.value)

@@ -1,0 +1,87 @@
+"""Pins the restated quantizer / attention (oracle/quant.py) against an independent NumPy
+emulation with explicit rounding, closed forms, and fp64 attention."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from packkv_amd import synth
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.float16, "fp16"), (torch.bfloat16, "bf16")])
+@pytest.mark.parametrize("rel", [0.05, 0.1, 0.14, 0.2])
+def test_quant_chain_matches_explicit_rounding(dtype, name, rel):
+    k, v = synth.make_kv(2, 4, 128, seed=3, dtype=dtype)
+    for x in (k, v):
+        c, z, s = oq.quant_ints(x, 64, rel)
+        cn, zn, sn = oq.quant_ints_np(x.float().numpy(), name, 64, rel)
+        assert np.array_equal(c.reshape(x.shape).float().numpy(), cn)
+        assert np.array_equal(z.flatten().float().numpy(), zn.flatten())
+        assert np.array_equal(s.flatten().float().numpy(), sn.flatten())
+        assert cn.min() == 0
+        assert cn.max() in (int(np.ceil(1 / rel - 1e-9)), int(np.ceil(1 / rel - 1e-9)) + 1)
+
+
+def test_quant_is_per_batch_and_token():
+    k, _ = synth.make_kv(2, 4, 64, seed=4)
+    c, z, s = oq.quant_ints(k, 64, 0.1)
+    assert tuple(z.shape) == (2, 1, 1, 64, 1) and tuple(s.shape) == (2, 1, 1, 64, 1)
+    mn = k.float().amin(dim=(1, 3))
+    mx = k.float().amax(dim=(1, 3))
+    want = ((mx - mn).half().float() * np.float32(0.1)).half()
+    assert torch.equal(s.flatten(), want.flatten())
+
+
+def test_dequant_error_bound_and_layout():
+    k, _ = synth.make_kv(1, 2, 64, seed=5)
+    c, z, s = oq.quant_ints(k, 64, 0.1)
+    y = oq.dequant(c, z, s)
+    err = (y.float() - k.float()).abs()
+    bound = 0.5 * s.flatten().float().view(1, 1, 64, 1) * 1.02 + 1e-2
+    assert (err <= bound).all()
+    m = oq.code_matrix(c)
+    assert tuple(m.shape) == (64, 256)
+    assert int(m[7, 1 * 128 + 5]) == int(c.reshape(1, 2, 64, 128)[0, 1, 7, 5])
+
+
+def test_q_interleave_is_lane_order():
+    q = torch.arange(128, dtype=torch.float32).view(1, 128)
+    qi = oq.q_interleave(q)[0]
+    for lane in range(32):
+        assert qi[2 * lane].item() == 4 * lane and qi[2 * lane + 1].item() == 4 * lane + 1
+        assert qi[64 + 2 * lane].item() == 4 * lane + 2 and qi[64 + 2 * lane + 1].item() == 4 * lane + 3
+
+
+def test_cut_counts_residual_window():
+    # block 64, buffer 192: a prompt below 192 tokens is never compressed; 8192 -> 8064 + 128; the
+    # window then cycles 128..191
+    assert oq.cut_counts(0, 191, 64, 192) == (0, 191)
+    assert oq.cut_counts(0, 192, 64, 192) == (64, 128)
+    assert oq.cut_counts(0, 8192, 64, 192) == (8064, 128)
+    n = 128
+    for _ in range(200):
+        cut, n = oq.cut_counts(n, 1, 64, 192)
+        assert cut in (0, 64) and 128 <= n <= 191
+
+
+def test_bit_pack_closed_form():
+    # 2 channels x 32 tokens: packs with ranges 0, 1, 3, 15 -> lens 0, 1, 2, 4
+    c = np.zeros((32, 2), dtype=np.int64)
+    c[16:, 0] = np.arange(16) % 2
+    c[:16, 1] = np.arange(16) % 4
+    c[16:, 1] = np.arange(16)
+    bits = 16 * (0 + 1 + 2 + 4) + 4 * (4 + 3)
+    assert oq.bit_pack_bytes(c, 16, W=4) == bits // 8
+
+
+def test_attention_versions_agree_with_fp64():
+    k, v = synth.make_kv(2, 2, 256, seed=6)
+    q = synth.make_q(2, 8, seed=7).unsqueeze(2)
+    ck, zk, sk = oq.quant_ints(k, 64, 0.1)
+    cv, zv, sv = oq.quant_ints(v, 64, 0.1)
+    kd, vd = oq.dequant(ck, zk, sk), oq.dequant(cv, zv, sv)
+    want = oq.attention_f64_np(q, kd, vd)
+    got32 = oq.attention_f32(q, kd, vd).double().numpy()
+    got16 = oq.eager_attention(q, kd, vd).double().numpy()
+    assert np.abs(got32 - want).max() < 1e-5
+    assert np.abs(got16 - want).max() < 5e-3
