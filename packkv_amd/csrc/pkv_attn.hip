@@ -216,6 +216,391 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
     }
 }
 
+// ---- variant 0: matrix-core kernel ---------------------------------------------------------
+// K side: every half-wavefront unpacks one round (16 tokens x 128 channels, lane t = channels
+// 4t..4t+3) into an int8 tile in LDS laid out [token][channel]; the tile is read back in the
+// operand layout of v_mfma_i32_16x16x32_i8 (lane = token, 8 consecutive channels) and
+// contracted against q, which is split per query head into three signed 7-bit digits
+// (q = qs * (d0 * 2^14 + d1 * 2^7 + d2)), one MFMA row per (digit, head).  Integer arithmetic
+// is exact, so the scores carry only the 2^-21 relative rounding of that split.
+// V side: lane = channel as in the stream; each pack yields four v_mfma_f32_4x4x4_16B_f16
+// (4 tokens each) whose A operand holds the softmax weights (times v_scale) of the 4 query
+// heads, so the per-lane accumulators are out[g][channel] and need no cross-lane reduction.
+// Codes enter as fp16 16 + delta (exponent bits OR-ed over the field); the 16 * sum(p) and the
+// per-pack minimum are corrected with sums kept beside the softmax state.
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
+
+constexpr int kKtStride = 136;         // bytes per token row of the int8 K tile (128 + 8 pad)
+constexpr int kKtDw = kKtStride / 4;
+constexpr float kPScale = 256.f;       // softmax weights are stored as fp16(p * v_scale * 256)
+
+__device__ __forceinline__ uint32_t pk_shr16(uint32_t v, uint32_t sh) {
+    ushort2v a = __builtin_bit_cast(ushort2v, v), b = __builtin_bit_cast(ushort2v, sh);
+    return __builtin_bit_cast(uint32_t, (ushort2v)(a >> b));
+}
+
+template <int G>
+__global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
+    constexpr int ROWS = 3 * G;                  // MFMA rows: (digit, head)
+    constexpr int NSETS = (ROWS + 15) / 16;
+    constexpr int NG4 = (G + 3) / 4;             // groups of 4 heads on the V side
+    constexpr int GP = NG4 * 4;                  // heads padded to a multiple of 4
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t *stage = lds;
+    uint8_t *kt = stage + 4 * p.blk_stride;                               // [8*16][136] int8
+    int32_t *sraw = reinterpret_cast<int32_t *>(kt + 8 * 16 * kKtStride); // [8*16][16*NSETS]
+    _Float16 *pbuf = reinterpret_cast<_Float16 *>(sraw + 8 * 16 * 16 * NSETS);   // [GP][128]
+    _Float16 *p16hi = pbuf + GP * kTile;                                  // [GP][8]
+    _Float16 *p16lo = p16hi + GP * 8;                                     // [GP][8]
+    float *ks = reinterpret_cast<float *>(p16lo + GP * 8);                // 4 x [128]
+    float *kz = ks + kTile, *vs = kz + kTile, *vz = vs + kTile;
+    float *st_m = vz + kTile;                                             // 8 floats each
+    float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8, *st_ps = st_z + 8;
+    float *qsum = st_ps + 8, *qs = qsum + 8;
+    uint8_t *aq = reinterpret_cast<uint8_t *>(qs + 8);                    // [NSETS][4][16][32]
+    __shared__ uint32_t s_phase[4];
+
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int t = tid & 31, hw = tid >> 5;
+    const int bh = b * p.Hkv + h;
+    const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
+    const UnitGeom gk = unit_geom(p.k_bits), gv = unit_geom(p.v_bits);
+
+    // ---- prologue: split q into digits, zero the padded rows ----
+    for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
+    for (int i = tid; i < GP * kTile / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
+    for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
+    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_ps[tid] = 0.f; st_a[tid] = 0.f; }
+    __syncthreads();
+    for (int g = wave; g < G; g += 4) {
+        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
+        const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
+        float mx = fmaxf(fabsf(q0), fabsf(q1)), sm = q0 + q1;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+            sm += __shfl_xor(sm, d, 64);
+        }
+        const float inv = mx > 0.f ? 1048576.f / mx : 0.f;
+        if (lane == 0) { qsum[g] = sm; qs[g] = mx * (1.f / 1048576.f); }
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int d = lane + 64 * e;
+            int Q = (int)rintf((e ? q1 : q0) * inv);
+            const int d2 = ((Q + 64) & 127) - 64;
+            Q = (Q - d2) >> 7;
+            const int d1 = ((Q + 64) & 127) - 64;
+            const int d0 = (Q - d1) >> 7;
+            const int dig[3] = {d0, d1, d2};
+#pragma unroll
+            for (int pp = 0; pp < 3; pp++) {
+                const int m = pp * G + g;
+                aq[(((m >> 4) * 4 + (d >> 5)) * 16 + (m & 15)) * 32 + (d & 31)] = (uint8_t)(int8_t)dig[pp];
+            }
+        }
+    }
+    __syncthreads();
+    long aop[NSETS][4];
+#pragma unroll
+    for (int s = 0; s < NSETS; s++)
+#pragma unroll
+        for (int sl = 0; sl < 4; sl++)
+            aop[s][sl] = *reinterpret_cast<const long *>(aq + ((s * 4 + sl) * 16 + (lane & 15)) * 32 + 8 * (lane >> 4));
+
+    float4v acc[NG4];
+#pragma unroll
+    for (int i = 0; i < NG4; i++) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+
+    const int n_tiles = p.T_c / kTile;
+    const int tile0 = split * p.tiles_per_split;
+    const int tile1 = min(n_tiles, tile0 + p.tiles_per_split);
+
+    // Software pipeline over tiles: while tile tau is processed from LDS, the stream bytes and
+    // quantizer parameters of tile tau+1 are in flight into registers, and the block_info of
+    // tile tau+2 into one more; they are written to LDS at the bottom of the iteration.
+    __shared__ uint32_t s_info[3][4][2];     // ring over tiles: (byte offset, byte size) of 2 K + 2 V blocks
+    constexpr int kPre = 5;                  // dwords per thread per block: 5 * 256 * 4 >= 4552 + 6
+    uint32_t pre[4][kPre];
+    uint32_t pre_q[2];
+
+    auto block_index = [&](int tau, int j) -> uint32_t {
+        return j < 2 ? (uint32_t)((2 * tau + j) * n_hid_k + bh) : (uint32_t)(tau * n_hid_v + 2 * bh + (j - 2));
+    };
+    auto fetch_info = [&](int tau) -> uint2 {     // by threads 0..3
+        uint2 r = make_uint2(0u, 0u);
+        if (tid < 4 && tau < tile1) {
+            const uint32_t *info = tid < 2 ? p.k_info : p.v_info;
+            r = *reinterpret_cast<const uint2 *>(info + 2 * (size_t)block_index(tau, tid));
+            const uint32_t cap = tid < 2 ? p.k_cap : p.v_cap;
+            if (r.y > cap) r.y = cap;             // corrupt block_info must not overrun LDS
+        }
+        return r;
+    };
+    auto issue_loads = [&](int tau, int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint8_t *src = (j < 2 ? p.k_stream : p.v_stream) + s_info[slot][j][0];
+            const uint32_t phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 3u);
+            const uint32_t ndw = (phase + s_info[slot][j][1] + 3u) >> 2;
+            const uint32_t *s4 = reinterpret_cast<const uint32_t *>(src - phase);
+#pragma unroll
+            for (int k = 0; k < kPre; k++) {
+                const uint32_t i = (uint32_t)tid + 256u * k;
+                pre[j][k] = i < ndw ? s4[i] : 0u;
+            }
+        }
+        if (tid < kTile) {
+            const size_t ti = (size_t)b * p.T_c + (size_t)tau * kTile + tid;
+            pre_q[0] = (uint32_t)p.k_scale[ti] | ((uint32_t)p.k_zero[ti] << 16);
+            pre_q[1] = (uint32_t)p.v_scale[ti] | ((uint32_t)p.v_zero[ti] << 16);
+        }
+    };
+    auto commit_loads = [&](int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint8_t *src = (j < 2 ? p.k_stream : p.v_stream) + s_info[slot][j][0];
+            const uint32_t phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 3u);
+            const uint32_t ndw = (phase + s_info[slot][j][1] + 3u) >> 2;
+            uint32_t *d4 = reinterpret_cast<uint32_t *>(stage + j * p.blk_stride);
+#pragma unroll
+            for (int k = 0; k < kPre; k++) {
+                const uint32_t i = (uint32_t)tid + 256u * k;
+                if (i < ndw) d4[i] = pre[j][k];
+            }
+            if (tid == 0) s_phase[j] = phase;
+        }
+        if (tid < kTile) {
+            const uint32_t lo_sh = p.dtype == PKV_F16 ? 0u : 16u;
+            auto cvt = [&](uint32_t u16) -> float {
+                return p.dtype == PKV_F16 ? __half2float(__ushort_as_half((unsigned short)u16))
+                                          : __uint_as_float(u16 << 16);
+            };
+            (void)lo_sh;
+            ks[tid] = cvt(pre_q[0] & 0xFFFFu);
+            kz[tid] = cvt(pre_q[0] >> 16);
+            vs[tid] = cvt(pre_q[1] & 0xFFFFu);
+            vz[tid] = cvt(pre_q[1] >> 16);
+        }
+    };
+
+    if (tile0 < tile1) {
+        const uint2 i0 = fetch_info(tile0), i1 = fetch_info(tile0 + 1);
+        if (tid < 4) {
+            s_info[0][tid][0] = i0.x; s_info[0][tid][1] = i0.y;
+            s_info[1][tid][0] = i1.x; s_info[1][tid][1] = i1.y;
+        }
+        __syncthreads();
+        issue_loads(tile0, 0);
+        commit_loads(0);
+        __syncthreads();
+    }
+    for (int tau = tile0; tau < tile1; tau++) {
+        const int rel = tau - tile0;
+        const bool more = tau + 1 < tile1;
+        // 1. prefetch the next tile (registers) and the block_info of the one after
+        const uint2 inext = fetch_info(tau + 2);
+        if (more) issue_loads(tau + 1, (rel + 1) % 3);
+
+        // 2. K round hw -> int8 tile rows [hw*16, hw*16+16)
+        {
+            const int j = hw >> 2, unit = hw & 3;
+            const uint8_t *kb = stage + j * p.blk_stride;
+            const uint32_t kph = s_phase[j];
+            const uint16_t *kcum = reinterpret_cast<const uint16_t *>(kb + kph);
+            const uint32_t kstart = kph + 8u + (unit ? (uint32_t)kcum[unit - 1] : 0u);
+            UnitPacks u;
+            unit_parse(kb, kstart, t, gk, u);
+            uint32_t hlf[4][2];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                hlf[i][0] = (uint32_t)(u.word[i] >> (8u * u.len[i]));   // tokens 0..7
+                hlf[i][1] = (uint32_t)u.word[i];                        // tokens 8..15 (+ junk above)
+            }
+            const uint32_t len01 = u.len[0] | (u.len[1] << 16), len23 = u.len[2] | (u.len[3] << 16);
+            const uint32_t mq = ((1u << u.len[0]) - 1u) | (((1u << u.len[1]) - 1u) << 8) |
+                                (((1u << u.len[2]) - 1u) << 16) | (((1u << u.len[3]) - 1u) << 24);
+            const uint32_t minq = u.mn[0] | (u.mn[1] << 8) | (u.mn[2] << 16) | (u.mn[3] << 24);
+            uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
+#pragma unroll
+            for (int qtr = 0; qtr < 4; qtr++) {
+                uint32_t qd[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t src = hlf[i][qtr >> 1];
+                    qd[i] = (qtr & 1) ? src : (src >> (4u * u.len[i]));
+                }
+                const uint32_t u01 = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);
+                const uint32_t u23 = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
+#pragma unroll
+                for (int pp = 0; pp < 4; pp++) {
+                    const uint32_t x01 = pp == 3 ? u01 : pk_shr16(u01, len01 * (uint32_t)(3 - pp));
+                    const uint32_t x23 = pp == 3 ? u23 : pk_shr16(u23, len23 * (uint32_t)(3 - pp));
+                    const uint32_t quad = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + minq;
+                    dst[(qtr * 4 + pp) * kKtDw] = quad;
+                }
+            }
+        }
+        __syncthreads();
+
+        // 3. scores on the matrix cores: wave handles rounds 2*wave, 2*wave+1
+#pragma unroll
+        for (int rr = 0; rr < 2; rr++) {
+            const int R = 2 * wave + rr;
+            const uint8_t *row = kt + (R * 16 + (lane & 15)) * kKtStride + 8 * (lane >> 4);
+            long bop[4];
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++) bop[sl] = *reinterpret_cast<const long *>(row + 32 * sl);
+#pragma unroll
+            for (int s = 0; s < NSETS; s++) {
+                int4v d = {0, 0, 0, 0};
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) d = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[s][sl], bop[sl], d, 0, 0, 0);
+                *reinterpret_cast<int4v *>(sraw + ((R * 16 + (lane & 15)) * NSETS + s) * 16 + 4 * (lane >> 4)) = d;
+            }
+        }
+        __syncthreads();
+
+        // 4. online softmax: wave <-> query head
+        for (int g = wave; g < G; g += 4) {
+            float sv[2], pv[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int tok = lane + 64 * e;
+                const int32_t *r = sraw + tok * NSETS * 16;
+                const int m0 = g, m1 = G + g, m2 = 2 * G + g;
+                const float d0 = (float)r[(m0 >> 4) * 16 + (m0 & 15)];
+                const float d1 = (float)r[(m1 >> 4) * 16 + (m1 & 15)];
+                const float d2 = (float)r[(m2 >> 4) * 16 + (m2 & 15)];
+                const float dot = qs[g] * (d0 * 16384.f + d1 * 128.f + d2);
+                sv[e] = p.sm_scale * ks[tok] * (dot + kz[tok] * qsum[g]);
+            }
+            float mx = fmaxf(sv[0], sv[1]);
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+            const float m_old = st_m[g];
+            const float m_new = fmaxf(m_old, mx);
+            float sum = 0.f, psum = 0.f, zs = 0.f;
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int tok = lane + 64 * e;
+                pv[e] = __expf(sv[e] - m_new);
+                const _Float16 ph = (_Float16)(pv[e] * vs[tok] * kPScale);
+                pbuf[g * kTile + (tok ^ 1)] = ph;       // pairs swapped: matches the unpack order
+                const float pf = (float)ph;
+                sum += pv[e];
+                zs += pf * vz[tok];
+                // per-round (16 token) sums of the rounded weights, for the pack-minimum term
+                float r16 = pf;
+#pragma unroll
+                for (int d = 8; d >= 1; d >>= 1) r16 += __shfl_xor(r16, d, 64);
+                if ((lane & 15) == 0) {
+                    const int R = tok >> 4;
+                    const _Float16 hi = (_Float16)r16;
+                    p16hi[g * 8 + R] = hi;
+                    p16lo[g * 8 + R] = (_Float16)(r16 - (float)hi);
+                }
+                psum += pf;
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                sum += __shfl_xor(sum, d, 64);
+                psum += __shfl_xor(psum, d, 64);
+                zs += __shfl_xor(zs, d, 64);
+            }
+            if (lane == 0) {
+                const float alpha = __expf(m_old - m_new);
+                st_a[g] = alpha;
+                st_m[g] = m_new;
+                st_l[g] = st_l[g] * alpha + sum;
+                st_z[g] = st_z[g] * alpha + zs;
+                st_ps[g] = st_ps[g] * alpha + psum;
+            }
+        }
+        __syncthreads();
+
+        // 5. V segment hw: lane = channel, 4 packs x 4 MFMAs (4 tokens each) per head group
+        {
+            const int j = hw >> 2, unit = hw & 3, seg = unit & 1;
+            const uint8_t *vb = stage + (2 + j) * p.blk_stride;
+            const uint32_t vph = s_phase[2 + j];
+            const uint16_t *vcum = reinterpret_cast<const uint16_t *>(vb + vph);
+            const uint32_t vstart = vph + 8u + (unit ? (uint32_t)vcum[unit - 1] : 0u);
+            UnitPacks u;
+            unit_parse(vb, vstart, t, gv, u);
+#pragma unroll
+            for (int i4 = 0; i4 < NG4; i4++) {
+                const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
+                acc[i4] *= al;
+            }
+            const int gl = lane & 3;
+            half4v mins;
+#pragma unroll
+            for (int i = 0; i < 4; i++) mins[i] = (_Float16)(float)u.mn[i];
+#pragma unroll
+            for (int i4 = 0; i4 < NG4; i4++) {
+                const half4v ahi = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
+                const half4v alo = *reinterpret_cast<const half4v *>(p16lo + (4 * i4 + gl) * 8 + 4 * seg);
+                acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(ahi, mins, acc[i4], 0, 0, 0);
+                acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(alo, mins, acc[i4], 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t len = u.len[i];
+                const uint32_t len2 = 2u * len;
+                const uint32_t hi8 = (uint32_t)(u.word[i] >> (8u * len));
+                const uint32_t lo8 = (uint32_t)u.word[i];
+                const uint32_t mult = 64u + (0x400000u >> len);
+                const uint32_t msk = ((1u << len) - 1u) * 0x00400040u;
+                const int tokbase = (seg * 4 + i) * 16;
+#pragma unroll
+                for (int uu = 0; uu < 4; uu++) {
+                    const uint32_t src = uu < 2 ? hi8 : lo8;
+                    // pairs inside the 8-token half: pair 0 is the most significant
+                    const uint32_t pa = 2 * (uu & 1), pb = pa + 1;
+                    const uint32_t xa = __builtin_amdgcn_ubfe(src, (3u - pa) * len2, len2);
+                    const uint32_t xb = __builtin_amdgcn_ubfe(src, (3u - pb) * len2, len2);
+                    const uint32_t ra = (__umul24(xa, mult) & msk) | 0x4C004C00u;
+                    const uint32_t rb = (__umul24(xb, mult) & msk) | 0x4C004C00u;
+                    const half4v bop = __builtin_bit_cast(half4v, make_uint2(ra, rb));
+#pragma unroll
+                    for (int i4 = 0; i4 < NG4; i4++) {
+                        const half4v aopv = *reinterpret_cast<const half4v *>(
+                            pbuf + (4 * i4 + gl) * kTile + tokbase + 4 * uu);
+                        acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(aopv, bop, acc[i4], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // 6. land the prefetched tile in LDS
+        if (tid < 4) { s_info[(rel + 2) % 3][tid][0] = inext.x; s_info[(rel + 2) % 3][tid][1] = inext.y; }
+        if (more) commit_loads((rel + 1) % 3);
+        __syncthreads();
+    }
+
+    // epilogue: the two half-waves of a wave hold the two 64-token halves of the same channels
+#pragma unroll
+    for (int i4 = 0; i4 < NG4; i4++)
+#pragma unroll
+        for (int m = 0; m < 4; m++) acc[i4][m] += __shfl_xor(acc[i4][m], 32, 64);
+    if ((lane >> 5) == 0) {
+        const int j = hw >> 2, w = (hw & 3) >> 1;
+        const int ch = 64 * j + 32 * w + t;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            float *dst = p.part + (hq * p.nparts + split) * kPartStride;
+            dst[2 + ch] = (acc[g >> 2][g & 3] - 16.f * st_ps[g] + st_z[g]) * (1.f / kPScale);
+            if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+        }
+    }
+}
+
 // ---- 16-bit tail window: dense attention over T_w tokens, one workgroup per (kv head, batch)
 template <int G>
 __global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
@@ -297,14 +682,23 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint16_t *__re
 
 template <int G>
 static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
-    (void)variant;
-    if (p.T_c > 0) {
+    if (p.T_c > 0 && variant == 1) {
         const uint32_t lds_bytes = 2u * kTile * kHeadDim + 4u * p.blk_stride +
                                    (uint32_t)sizeof(float) * (G * kHeadDim + 2 * G * kTile + 4 * kTile + 5 * G);
         const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
         PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_tiles_kernel<G>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         attn_tiles_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
+        PKV_HIP_CHECK(hipGetLastError());
+    } else if (p.T_c > 0) {
+        constexpr int NSETS = (3 * G + 15) / 16, GP = ((G + 3) / 4) * 4;
+        const uint32_t lds_bytes = 4u * p.blk_stride + 8u * 16u * kKtStride + 8u * 16u * 16u * NSETS * 4u +
+                                   GP * kTile * 2u + 2u * GP * 8u * 2u + 4u * kTile * 4u + 7u * 8u * 4u +
+                                   NSETS * 4u * 16u * 32u;
+        const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel<G>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attn_mfma_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
     if (p.T_w > 0) {

@@ -34,38 +34,6 @@ __device__ __forceinline__ int tile_index(int unit, int slot, int k, int t, int 
     return ((seg * 4 + slot) * kPackTok + k) * hid_blk + warp * kLanes + t;
 }
 
-// Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
-template <bool IS_K>
-__device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,
-                                            const UnitGeom g, uint8_t *tile, int hid_blk) {
-    const uint32_t minsw = lds_meta_word(blk + unit_off, t, g.W);
-    const uint32_t lensw = lds_meta_word(blk + unit_off + g.mins_bytes, t, g.LB);
-    uint32_t run = unit_off + g.mins_bytes + g.lens_bytes;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t len = (lensw >> (i * g.LB)) & ((1u << g.LB) - 1u);
-        const uint32_t mn = (minsw >> (i * g.W)) & ((1u << g.W) - 1u);
-        uint32_t tot;
-        const uint32_t off = run + half_excl_scan(2u * len, tot);
-        run += tot;
-        uint64_t word = lds_load64(blk, off);
-        const uint64_t mask = (1ull << len) - 1ull;
-        if (IS_K) {
-#pragma unroll
-            for (int k = 0; k < kPackTok; k++) {
-                const uint32_t c = (uint32_t)((word >> ((15 - k) * len)) & mask) + mn;
-                tile[tile_index<true>(unit, i, k, t, hid_blk)] = (uint8_t)c;
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < kPackTok; k++) {
-                const uint32_t c = (uint32_t)((word >> ((15 - k) * len)) & mask) + mn;
-                tile[tile_index<false>(unit, i, k, t, hid_blk)] = (uint8_t)c;
-            }
-        }
-    }
-}
-
 struct UnitPacks {
     uint64_t word[4];
     uint32_t len[4];
@@ -74,12 +42,47 @@ struct UnitPacks {
     uint32_t payload;    // payload bytes of the whole unit
 };
 
+// Read lane t's four packs (min, len, word) of the unit whose bytes start at blk[unit_off].
+__device__ __forceinline__ void unit_parse(const uint8_t *blk, uint32_t unit_off, int t, const UnitGeom g,
+                                           UnitPacks &u) {
+    const uint32_t minsw = lds_meta_word(blk + unit_off, t, g.W);
+    const uint32_t lensw = lds_meta_word(blk + unit_off + g.mins_bytes, t, g.LB);
+    const uint32_t pay0 = unit_off + g.mins_bytes + g.lens_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        u.len[i] = (lensw >> (i * g.LB)) & ((1u << g.LB) - 1u);
+        u.mn[i] = (minsw >> (i * g.W)) & ((1u << g.W) - 1u);
+    }
+    pack_offsets(u.len, u.off, u.payload);
+    // bits above 16*len belong to the next pack; every consumer masks per field
+#pragma unroll
+    for (int i = 0; i < 4; i++) u.word[i] = lds_load64(blk, pay0 + u.off[i]);
+}
+
+// Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
+template <bool IS_K>
+__device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,
+                                            const UnitGeom g, uint8_t *tile, int hid_blk) {
+    UnitPacks u;
+    unit_parse(blk, unit_off, t, g, u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t len = u.len[i];
+        const uint64_t mask = (1ull << len) - 1ull;
+#pragma unroll
+        for (int k = 0; k < kPackTok; k++) {
+            const uint32_t c = (uint32_t)((u.word[i] >> ((15 - k) * len)) & mask) + u.mn[i];
+            tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] = (uint8_t)c;
+        }
+    }
+}
+
+
 // Gather lane t's four packs of `unit` from the LDS code tile and compute min / len / word
 // and the payload offsets (one 32-lane exclusive scan per slot).
 template <bool IS_K>
 __device__ __forceinline__ void unit_analyse(const uint8_t *tile, int hid_blk, int unit, int t,
                                              UnitPacks &u) {
-    uint32_t run = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         uint32_t c[kPackTok];
@@ -97,11 +100,8 @@ __device__ __forceinline__ void unit_analyse(const uint8_t *tile, int hid_blk, i
         u.word[i] = w;
         u.len[i] = len;
         u.mn[i] = mn;
-        uint32_t tot;
-        u.off[i] = run + half_excl_scan(2u * len, tot);
-        run += tot;
     }
-    u.payload = run;
+    pack_offsets(u.len, u.off, u.payload);
 }
 
 // Write lane t's 4*nbits-bit metadata word into an LSB-first bit array (nbits in {2,3,4}).

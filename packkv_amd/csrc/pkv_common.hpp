@@ -60,17 +60,45 @@ void set_error(const char *fmt, ...);
 
 __device__ __forceinline__ int bit_length_u32(uint32_t v) { return 32 - __clz((int)v); }
 
+// Inclusive prefix sum inside each 32-lane half of the wavefront, on the DPP data path
+// (row_shr 1/2/4/8 inside 16-lane rows, then row_bcast:15 into rows 1 and 3).
+__device__ __forceinline__ uint32_t half_incl_scan(uint32_t v) {
+    uint32_t x = v;
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x111, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x112, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x114, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x118, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x142, 0xA, 0xF, true);
+    return x;
+}
+
+// Value held by the last lane of the caller's 32-lane half.
+__device__ __forceinline__ uint32_t half_last(uint32_t x) {
+    const uint32_t a = __builtin_amdgcn_readlane(x, 31), b = __builtin_amdgcn_readlane(x, 63);
+    return (threadIdx.x & 32) ? b : a;
+}
+
 // Exclusive prefix sum over the 32 lanes of a half-wavefront; `total` receives the sum.
 __device__ __forceinline__ uint32_t half_excl_scan(uint32_t v, uint32_t &total) {
-    const int t = threadIdx.x & 31;
-    uint32_t incl = v;
-#pragma unroll
-    for (int d = 1; d < 32; d <<= 1) {
-        uint32_t up = __shfl_up(incl, d, 32);
-        if (t >= d) incl += up;
-    }
-    total = __shfl(incl, 31, 32);
+    const uint32_t incl = half_incl_scan(v);
+    total = half_last(incl);
     return incl - v;
+}
+
+// Payload byte offsets of a lane's four packs (stream order: slot-major, lane-minor) from
+// their bit widths: two packed 16-bit scans instead of four.
+__device__ __forceinline__ void pack_offsets(const uint32_t len[4], uint32_t off[4], uint32_t &payload) {
+    const uint32_t a = (2u * len[0]) | ((2u * len[1]) << 16);
+    const uint32_t b = (2u * len[2]) | ((2u * len[3]) << 16);
+    const uint32_t ia = half_incl_scan(a), ib = half_incl_scan(b);
+    const uint32_t ta = half_last(ia), tb = half_last(ib);
+    const uint32_t ea = ia - a, eb = ib - b;
+    const uint32_t t0 = ta & 0xFFFFu, t01 = t0 + (ta >> 16), t012 = t01 + (tb & 0xFFFFu);
+    off[0] = ea & 0xFFFFu;
+    off[1] = t0 + (ea >> 16);
+    off[2] = t01 + (eb & 0xFFFFu);
+    off[3] = t012 + (eb >> 16);
+    payload = t012 + (tb >> 16);
 }
 
 // 64 bits starting at byte offset `off` (2-byte aligned) of an LDS byte array whose base
