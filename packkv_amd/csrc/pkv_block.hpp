@@ -59,6 +59,32 @@ __device__ __forceinline__ void unit_parse(const uint8_t *blk, uint32_t unit_off
     for (int i = 0; i < 4; i++) u.word[i] = lds_load64(blk, pay0 + u.off[i]);
 }
 
+// Parse two independent units at once (same lane t in both), batching the LDS round trips:
+// all metadata reads first, then both offset scans, then all eight pack words.
+__device__ __forceinline__ void unit_parse2(const uint8_t *blk_a, uint32_t off_a, const UnitGeom ga, UnitPacks &ua,
+                                            const uint8_t *blk_b, uint32_t off_b, const UnitGeom gb, UnitPacks &ub,
+                                            int t) {
+    const uint32_t mins_a = lds_meta_word(blk_a + off_a, t, ga.W);
+    const uint32_t lens_a = lds_meta_word(blk_a + off_a + ga.mins_bytes, t, ga.LB);
+    const uint32_t mins_b = lds_meta_word(blk_b + off_b, t, gb.W);
+    const uint32_t lens_b = lds_meta_word(blk_b + off_b + gb.mins_bytes, t, gb.LB);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ua.len[i] = (lens_a >> (i * ga.LB)) & ((1u << ga.LB) - 1u);
+        ua.mn[i] = (mins_a >> (i * ga.W)) & ((1u << ga.W) - 1u);
+        ub.len[i] = (lens_b >> (i * gb.LB)) & ((1u << gb.LB) - 1u);
+        ub.mn[i] = (mins_b >> (i * gb.W)) & ((1u << gb.W) - 1u);
+    }
+    pack_offsets(ua.len, ua.off, ua.payload);
+    pack_offsets(ub.len, ub.off, ub.payload);
+    const uint32_t pay_a = off_a + ga.mins_bytes + ga.lens_bytes, pay_b = off_b + gb.mins_bytes + gb.lens_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ua.word[i] = lds_load64(blk_a, pay_a + ua.off[i]);
+        ub.word[i] = lds_load64(blk_b, pay_b + ub.off[i]);
+    }
+}
+
 // Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
 template <bool IS_K>
 __device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,

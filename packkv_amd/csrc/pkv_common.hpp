@@ -101,24 +101,29 @@ __device__ __forceinline__ void pack_offsets(const uint32_t len[4], uint32_t off
     payload = t012 + (tb >> 16);
 }
 
-// 64 bits starting at byte offset `off` (2-byte aligned) of an LDS byte array whose base
-// is 4-byte aligned.  Reads three aligned dwords; never issues an unaligned LDS access.
+// 64 bits starting at byte offset `off` (2-byte aligned) of an LDS byte array whose base is
+// 4-byte aligned.  gfx950 does execute DS reads at any alignment, but a misaligned 64-bit read
+// stalls the LDS pipeline (SQ_LDS_UNALIGNED_STALL), so this reads the three aligned dwords that
+// cover the range and funnel-shifts them.
 __device__ __forceinline__ uint64_t lds_load64(const uint8_t *lds, uint32_t off) {
     const uint32_t *p = reinterpret_cast<const uint32_t *>(lds + (off & ~3u));
-    uint32_t d0 = p[0], d1 = p[1], d2 = p[2];
-    uint32_t sh = (off & 2u) * 8u;
-    uint32_t lo = __builtin_amdgcn_alignbit(d1, d0, sh);
-    uint32_t hi = __builtin_amdgcn_alignbit(d2, d1, sh);
+    const uint32_t d0 = p[0], d1 = p[1], d2 = p[2];
+    const uint32_t sh = (off & 2u) * 8u;
+    const uint32_t lo = __builtin_amdgcn_alignbit(d1, d0, sh);
+    const uint32_t hi = __builtin_amdgcn_alignbit(d2, d1, sh);
     return ((uint64_t)hi << 32) | lo;
 }
 
-// The 4*nbits-bit metadata word of format lane t from an LSB-first bit array (4 fields
-// of nbits each; nbits in {2,3,4}).
+// The 4*nbits-bit metadata word of format lane t from an LSB-first bit array in LDS (4 fields
+// of nbits each; nbits in {2,3,4}; `arr` 2-byte aligned).  Reads the two aligned dwords around
+// the field and funnel-shifts: adjacent byte reads would be merged into misaligned 16-bit DS
+// reads, which stall the LDS pipeline.
 __device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int nbits) {
-    const uint32_t bit = (uint32_t)t * 4u * (uint32_t)nbits;
-    const uint32_t byte = bit >> 3;
-    uint32_t v = (uint32_t)arr[byte] | ((uint32_t)arr[byte + 1] << 8);
-    return (v >> (bit & 7u)) & ((1u << (4 * nbits)) - 1u);
+    const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>(arr);      // LDS byte address
+    const uint32_t bit = (addr & 3u) * 8u + (uint32_t)t * 4u * (uint32_t)nbits;
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(arr - (addr & 3u)) + (bit >> 5);
+    const uint32_t v = __builtin_amdgcn_alignbit(p[1], p[0], bit & 31u);
+    return v & ((1u << (4 * nbits)) - 1u);
 }
 
 // Copy `nbytes` from global `src` (any alignment) into LDS `dst` (4-byte aligned) so that
