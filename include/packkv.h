@@ -133,6 +133,10 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *
  *   k_stream/k_info   K stream of the code matrix [T_c, B*Hkv*128], blocks 64 x 128
  *   v_stream/v_info   V stream of the same shape, blocks 128 x 64
+ *   k_bytes, v_bytes  readable bytes of each stream BUFFER (below 4 GiB).  The kernels never read
+ *                     past this, whatever block_info says; they fetch pack words as whole
+ *                     8-byte words, so the buffer must extend at least 7 bytes past the encoded
+ *                     size (size_out of the encoder) or the last block decodes wrongly
  *   k_scale..v_zero   [B, T_c] `dtype`
  *   q, out            [B, Hq, 128] `dtype`
  *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype` (the residual
@@ -146,6 +150,7 @@ typedef struct pkv_attn_args {
     const uint32_t *k_info;
     const uint8_t *v_stream;
     const uint32_t *v_info;
+    uint64_t k_bytes, v_bytes;
     const void *k_scale, *k_zero, *v_scale, *v_zero;
     const void *q;
     void *out;

@@ -24,6 +24,7 @@ _u64p = ctypes.POINTER(ctypes.c_uint64)
 class AttnArgs(ctypes.Structure):
     _fields_ = [
         ("k_stream", _vp), ("k_info", _vp), ("v_stream", _vp), ("v_info", _vp),
+        ("k_bytes", _u64), ("v_bytes", _u64),
         ("k_scale", _vp), ("k_zero", _vp), ("v_scale", _vp), ("v_zero", _vp),
         ("q", _vp), ("out", _vp), ("k_win", _vp), ("v_win", _vp),
         ("B", _i), ("Hq", _i), ("Hkv", _i), ("T_c", _i), ("T_w", _i),

@@ -47,6 +47,7 @@ struct AttnParams {
     int dbg;
     int tiles_per_split, nsplit, nparts;
     uint32_t k_cap, v_cap, blk_stride;
+    uint32_t k_bytes, v_bytes;   // valid bytes of the streams
 };
 
 // ---- variant 1: decode tiles into LDS, then plain VALU attention --------------------------
@@ -745,9 +746,44 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint16_t *__re
     out[hq * kHeadDim + threadIdx.x] = a_st16(num / den, dtype);
 }
 
+}  // namespace pkv
+#include "pkv_attn_direct.hpp"
+namespace pkv {
+
+template <int G, int KW, int VW>
+static int launch_direct(const AttnParams &p, hipStream_t s) {
+    constexpr int GP = ((G + 3) / 4) * 4;
+    const uint32_t lds_bytes = 8u * 16u * kKtStride + kRing * 16u * 4u + GP * kTile * 2u + 2u * GP * 8u * 2u + 6u * 8u * 4u;
+    const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
+    if (p.dtype == PKV_BF16)
+        attn_direct_kernel<G, KW, VW, true><<<grid, 256, lds_bytes, s>>>(p);
+    else
+        attn_direct_kernel<G, KW, VW, false><<<grid, 256, lds_bytes, s>>>(p);
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
+template <int G>
+static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
+    switch (p.k_bits * 8 + p.v_bits) {
+        case 2 * 8 + 2: return launch_direct<G, 2, 2>(p, s);
+        case 2 * 8 + 3: return launch_direct<G, 2, 3>(p, s);
+        case 2 * 8 + 4: return launch_direct<G, 2, 4>(p, s);
+        case 3 * 8 + 2: return launch_direct<G, 3, 2>(p, s);
+        case 3 * 8 + 3: return launch_direct<G, 3, 3>(p, s);
+        case 3 * 8 + 4: return launch_direct<G, 3, 4>(p, s);
+        case 4 * 8 + 2: return launch_direct<G, 4, 2>(p, s);
+        case 4 * 8 + 3: return launch_direct<G, 4, 3>(p, s);
+        default: return launch_direct<G, 4, 4>(p, s);
+    }
+}
+
 template <int G>
 static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
-    if (p.T_c > 0 && (variant & 0xFF) == 1) {
+    if (p.T_c > 0 && (variant & 0xFF) == 0) {
+        const int rc = launch_direct_bits<G>(p, s);
+        if (rc) return rc;
+    } else if (p.T_c > 0 && (variant & 0xFF) == 1) {
         const uint32_t lds_bytes = 2u * kTile * kHeadDim + 4u * p.blk_stride +
                                    (uint32_t)sizeof(float) * (G * kHeadDim + 2 * G * kTile + 4 * kTile + 5 * G);
         const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
@@ -800,6 +836,8 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
                     PKV_ERR_INVALID, "null pointer argument");
         PKV_REQUIRE(a->k_bits >= 2 && a->k_bits <= 4 && a->v_bits >= 2 && a->v_bits <= 4, PKV_ERR_UNSUPPORTED,
                     "not supported: bits_len outside 2..4");
+        PKV_REQUIRE(a->k_bytes > 0 && a->v_bytes > 0 && a->k_bytes < (1ull << 32) && a->v_bytes < (1ull << 32),
+                    PKV_ERR_INVALID, "stream sizes must be in 1 .. 4 GiB - 1");
     }
     if (a->T_w > 0) PKV_REQUIRE(a->k_win && a->v_win, PKV_ERR_INVALID, "null pointer argument");
     const int G = a->Hq / a->Hkv;
@@ -830,7 +868,8 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     p.k_cap = a->T_c > 0 ? (uint32_t)k_block_bound(64, a->k_bits) : 0;
     p.v_cap = a->T_c > 0 ? (uint32_t)v_block_bound(64, a->v_bits) : 0;
     const uint32_t cap = p.k_cap > p.v_cap ? p.k_cap : p.v_cap;
-    p.blk_stride = ((cap + 14u + 15u) & ~15u) + 32u;   // up to 14 bytes of phase in front, slack behind
+    p.blk_stride = ((cap + 14u + 15u) & ~15u) + 32u;
+    p.k_bytes = (uint32_t)a->k_bytes; p.v_bytes = (uint32_t)a->v_bytes;   // up to 14 bytes of phase in front, slack behind
     void *scratch = nullptr;
     const size_t part_bytes = (size_t)a->B * a->Hq * p.nparts * kPartStride * sizeof(float);
     int rc = scratch_get(part_bytes, &scratch);

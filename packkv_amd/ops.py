@@ -406,6 +406,12 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
         Hkv = nblk_k // (T_c // 64) // B
         a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
         a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
+        # readable bytes of each buffer: pack words are fetched as whole 8-byte words, so the last
+        # block needs 7 bytes of readable slack behind the encoded size
+        for d in (k, v):
+            _require(not d.get("size") or d["stream"].numel() >= int(d["size"]) + 7,
+                     "stream buffers need 7 readable bytes behind the encoded size")
+        a.k_bytes, a.v_bytes = k["stream"].numel(), v["stream"].numel()
         a.k_scale, a.k_zero = _ptr(k["scale"]), _ptr(k["zero"])
         a.v_scale, a.v_zero = _ptr(v["scale"]), _ptr(v["zero"])
         a.k_bits, a.v_bits = int(k["bits"]), int(v["bits"])
