@@ -763,6 +763,36 @@ static int launch_direct(const AttnParams &p, hipStream_t s) {
     return PKV_OK;
 }
 
+}  // namespace pkv
+#include "pkv_attn_dma.hpp"
+namespace pkv {
+
+template <int G, int KW, int VW>
+static int launch_dma(const AttnParams &p, hipStream_t s) {
+    const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
+    if (p.dtype == PKV_BF16)
+        attn_dma_kernel<G, KW, VW, true><<<grid, 256, 0, s>>>(p);
+    else
+        attn_dma_kernel<G, KW, VW, false><<<grid, 256, 0, s>>>(p);
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
+template <int G>
+static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
+    switch (p.k_bits * 8 + p.v_bits) {
+        case 2 * 8 + 2: return launch_dma<G, 2, 2>(p, s);
+        case 2 * 8 + 3: return launch_dma<G, 2, 3>(p, s);
+        case 2 * 8 + 4: return launch_dma<G, 2, 4>(p, s);
+        case 3 * 8 + 2: return launch_dma<G, 3, 2>(p, s);
+        case 3 * 8 + 3: return launch_dma<G, 3, 3>(p, s);
+        case 3 * 8 + 4: return launch_dma<G, 3, 4>(p, s);
+        case 4 * 8 + 2: return launch_dma<G, 4, 2>(p, s);
+        case 4 * 8 + 3: return launch_dma<G, 4, 3>(p, s);
+        default: return launch_dma<G, 4, 4>(p, s);
+    }
+}
+
 template <int G>
 static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
     switch (p.k_bits * 8 + p.v_bits) {
@@ -780,7 +810,11 @@ static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
 
 template <int G>
 static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
-    if (p.T_c > 0 && (variant & 0xFF) == 0) {
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(p.k_stream) | reinterpret_cast<uintptr_t>(p.v_stream)) & 15u) == 0;
+    if (p.T_c > 0 && (variant & 0xFF) == 0 && aligned16) {
+        const int rc = launch_dma_bits<G>(p, s);
+        if (rc) return rc;
+    } else if (p.T_c > 0 && ((variant & 0xFF) == 0 || (variant & 0xFF) == 3)) {
         const int rc = launch_direct_bits<G>(p, s);
         if (rc) return rc;
     } else if (p.T_c > 0 && (variant & 0xFF) == 1) {
@@ -839,6 +873,10 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
         PKV_REQUIRE(a->k_bytes > 0 && a->v_bytes > 0 && a->k_bytes < (1ull << 32) && a->v_bytes < (1ull << 32),
                     PKV_ERR_INVALID, "stream sizes must be in 1 .. 4 GiB - 1");
     }
+    PKV_REQUIRE((uint64_t)a->B * (uint64_t)a->T_c < (1ull << 28), PKV_ERR_UNSUPPORTED,
+                "batch x compressed tokens above 2^28");
+    PKV_REQUIRE((uint64_t)(a->T_c / 64) * (uint64_t)a->B * (uint64_t)a->Hkv < (1ull << 27), PKV_ERR_UNSUPPORTED,
+                "more than 2^27 blocks per stream");
     if (a->T_w > 0) PKV_REQUIRE(a->k_win && a->v_win, PKV_ERR_INVALID, "null pointer argument");
     const int G = a->Hq / a->Hkv;
     PKV_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, PKV_ERR_UNSUPPORTED,
@@ -857,7 +895,8 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     int nsplit = 0, tps = 0;
     if (n_tiles > 0) {
         const int pairs = a->B * a->Hkv;
-        int want = (2048 + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
+        const int target = 1024;
+        int want = (target + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
         if (want < 1) want = 1;
         if (want > n_tiles) want = n_tiles;
         tps = (n_tiles + want - 1) / want;

@@ -64,6 +64,47 @@ __device__ __forceinline__ void unit_windows(const UnitRegs &u, uint32_t win01[4
 
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
+// Cross-lane float reductions with the lane permutation fused into the arithmetic instruction
+// (one VALU instruction per step).  Lanes whose row is masked off keep their value.  The leading
+// s_nop covers the two wait states a DPP read needs after the VALU write of its source.
+#define PKV_DPP_STEP(op, x, ctrl) asm("s_nop 1\n\t" op " %0, %0, %0 " ctrl : "+v"(x))
+
+__device__ __forceinline__ float wave_max_fused(float x) {
+    PKV_DPP_STEP("v_max_f32_dpp", x, "quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_max_f32_dpp", x, "quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_max_f32_dpp", x, "row_half_mirror row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_max_f32_dpp", x, "row_mirror row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_max_f32_dpp", x, "row_bcast:15 row_mask:0xa bank_mask:0xf");
+    PKV_DPP_STEP("v_max_f32_dpp", x, "row_bcast:31 row_mask:0xc bank_mask:0xf");
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
+__device__ __forceinline__ float oct_sum_fused(float x) {   // every lane gets the sum over its 8-lane group
+    PKV_DPP_STEP("v_add_f32_dpp", x, "quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_add_f32_dpp", x, "quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf");
+    PKV_DPP_STEP("v_add_f32_dpp", x, "row_half_mirror row_mask:0xf bank_mask:0xf");
+    return x;
+}
+
+// Payload offsets (in 2-byte units) of a lane's four packs from their widths `lens_b` (one per
+// byte): a single packed scan over the 32 lanes of the half-wavefront.  A slot's widths sum to at
+// most 32 * 4 = 128, so the four running sums never carry into each other.
+__device__ __forceinline__ void pack_offsets8(uint32_t lens_b, uint32_t off2[4]) {
+    const uint32_t incl = half_incl_scan(lens_b);
+    const uint32_t excl = incl - lens_b;
+    const uint32_t ta = __builtin_amdgcn_readlane(incl, 31), tb = __builtin_amdgcn_readlane(incl, 63);
+    // slot bases = running sums of the slot totals; uniform per half, so this is scalar work
+    const uint32_t a0 = ta & 0xFFu, a01 = a0 + ((ta >> 8) & 0xFFu), a012 = a01 + ((ta >> 16) & 0xFFu);
+    const uint32_t b0 = tb & 0xFFu, b01 = b0 + ((tb >> 8) & 0xFFu), b012 = b01 + ((tb >> 16) & 0xFFu);
+    const bool upper = (threadIdx.x & 32) != 0;
+    const uint32_t base12 = upper ? (b0 | (b01 << 16)) : (a0 | (a01 << 16));
+    const uint32_t base3 = upper ? b012 : a012;
+    off2[0] = excl & 0xFFu;
+    off2[1] = ((excl >> 8) & 0xFFu) + (base12 & 0xFFFFu);
+    off2[2] = ((excl >> 16) & 0xFFu) + (base12 >> 16);
+    off2[3] = (excl >> 24) + base3;
+}
+
 template <int G, int KW, int VW, bool BF>
 __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     constexpr int ROWS = 3 * G;
@@ -97,6 +138,14 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.k_stream), 0, (int)p.k_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.v_stream), 0, (int)p.v_bytes, 0x00020000);
+
+    const int par_bytes = p.B * p.T_c * 2, info_bytes = (p.T_c / 64) * p.B * p.Hkv * 8;
+    const __amdgpu_buffer_rsrc_t ks_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.k_scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t kz_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.k_zero), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.v_scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vz_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.v_zero), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ki_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.k_info), 0, info_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vi_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.v_info), 0, info_bytes, 0x00020000);
 
     // ---- prologue: split q into digits (through LDS, aliased onto the K tile) ----
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
@@ -158,7 +207,9 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     const int f_j = tid & 3;
     auto fill_info = [&](int rel) -> uint32_t {              // byte offset of block f_j of tile rel (clamped)
         const uint32_t bi = block_index(tile0 + min(rel, ntl - 1), f_j);
-        const uint32_t ko = p.k_info[2 * (size_t)bi], vo = p.v_info[2 * (size_t)bi];   // both in range: K has the larger table
+        // the two tables have the same number of entries, so either index is in range for both
+        const uint32_t ko = __builtin_amdgcn_raw_buffer_load_b32(ki_rsrc, 8u * bi, 0, 0);
+        const uint32_t vo = __builtin_amdgcn_raw_buffer_load_b32(vi_rsrc, 8u * bi, 0, 0);
         return f_j < 2 ? ko : vo;
     };
     auto fill_header = [&](uint32_t off) -> uint2v {         // the block's four cumulative u16 sizes
@@ -211,17 +262,18 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
         m.v_lens = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, m.v_start + v_lens_off, 0, 0);
     };
     auto words_issue = [&](const Meta &m, UnitRegs &ku_r, UnitRegs &vu_r) {
-        uint32_t klen[4], vlen[4], koff[4], voff[4], kpay, vpay;
+        uint32_t klen[4], vlen[4], koff[4], voff[4];
         meta_fields<KW>((m.k_mins >> k_mins_sh) & ((1u << (4 * KW)) - 1u), (m.k_lens >> k_lens_sh) & ((1u << (4 * KLB)) - 1u),
                         klen, ku_r.lens, ku_r.mins);
         meta_fields<VW>((m.v_mins >> v_mins_sh) & ((1u << (4 * VW)) - 1u), (m.v_lens >> v_lens_sh) & ((1u << (4 * VLB)) - 1u),
                         vlen, vu_r.lens, vu_r.mins);
-        pack_offsets(klen, koff, kpay);
-        pack_offsets(vlen, voff, vpay);
+        pack_offsets8(ku_r.lens, koff);
+        pack_offsets8(vu_r.lens, voff);
+        const uint32_t kpay0 = m.k_start + K_META, vpay0 = m.v_start + V_META;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint2v kwd = __builtin_amdgcn_raw_buffer_load_b64(k_rsrc, m.k_start + K_META + koff[i], 0, 0);
-            const uint2v vwd = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, m.v_start + V_META + voff[i], 0, 0);
+            const uint2v kwd = __builtin_amdgcn_raw_buffer_load_b64(k_rsrc, kpay0 + 2u * koff[i], 0, 0);
+            const uint2v vwd = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, vpay0 + 2u * voff[i], 0, 0);
             ku_r.word[i] = ((uint64_t)kwd[1] << 32) | kwd[0];
             vu_r.word[i] = ((uint64_t)vwd[1] << 32) | vwd[0];
         }
@@ -229,11 +281,11 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     // quantizer parameters of the two tokens (2*lane, 2*lane+1) this lane handles in the softmax stage
     struct QPar { uint32_t ks, kz, vs, vz; };
     auto qpar_issue = [&](int rel, QPar &q) {
-        const size_t ti = ((size_t)b * p.T_c + (size_t)(tile0 + min(rel, ntl - 1)) * kTile) / 2 + lane;
-        q.ks = reinterpret_cast<const uint32_t *>(p.k_scale)[ti];
-        q.kz = reinterpret_cast<const uint32_t *>(p.k_zero)[ti];
-        q.vs = reinterpret_cast<const uint32_t *>(p.v_scale)[ti];
-        q.vz = reinterpret_cast<const uint32_t *>(p.v_zero)[ti];
+        const int tile_off = (b * p.T_c + (tile0 + min(rel, ntl - 1)) * kTile) * 2;     // bytes, wave-uniform
+        q.ks = __builtin_amdgcn_raw_buffer_load_b32(ks_rsrc, 4 * lane, tile_off, 0);
+        q.kz = __builtin_amdgcn_raw_buffer_load_b32(kz_rsrc, 4 * lane, tile_off, 0);
+        q.vs = __builtin_amdgcn_raw_buffer_load_b32(vs_rsrc, 4 * lane, tile_off, 0);
+        q.vz = __builtin_amdgcn_raw_buffer_load_b32(vz_rsrc, 4 * lane, tile_off, 0);
     };
     auto cvt2 = [&](uint32_t w, float &lo, float &hi) {
         if (!BF) {
@@ -317,7 +369,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
                     const float dot = qs_r[gi] * (d0 * 16384.f + d1 * 128.f + d2);
                     sv[e] = p.sm_scale * (e ? ks1 : ks0) * (dot + (e ? kz1 : kz0) * qsum_r[gi]);
                 }
-                const float mx = wave_max(fmaxf(sv[0], sv[1]));
+                const float mx = wave_max_fused(fmaxf(sv[0], sv[1]));
                 const float m_new = fmaxf(m_run[gi], mx);
                 const float alpha = __expf(m_run[gi] - m_new);    // exp(-inf) = 0 on the first tile
                 m_run[gi] = m_new;
@@ -332,10 +384,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
                 l_part[gi] = l_part[gi] * alpha + (p0 + p1);
                 z_part[gi] = z_part[gi] * alpha + (f0 * vz0 + f1 * vz1);
                 // per-round sums (16 tokens = 8 lanes) of the rounded weights, for the pack-minimum term
-                float r16 = f0 + f1;
-                r16 += dpp_keep<0xB1, 0xF>(r16);
-                r16 += dpp_keep<0x4E, 0xF>(r16);
-                r16 += dpp_keep<0x141, 0xF>(r16);     // row_half_mirror: lanes 8k..8k+7 all hold the sum
+                const float r16 = oct_sum_fused(f0 + f1);
                 if ((lane & 7) == 0) {
                     const _Float16 hi = (_Float16)r16;
                     p16hi[g * 8 + (lane >> 3)] = hi;

@@ -1,0 +1,436 @@
+// Fused decompress-attention decode, asynchronous-copy kernel.  The compressed blocks of a tile
+// travel global memory -> LDS with LDS-direct buffer loads (no registers, 16 bytes per lane,
+// fully coalesced) into one of two tile slots, one tile ahead of their use; lanes then parse their
+// packs out of LDS.  Included by pkv_attn.hip after pkv_attn_direct.hpp (shares UnitRegs,
+// meta_fields, unit_windows, pack_offsets8 and the fused DPP reductions).
+//
+// Tile = 128 tokens of one (sequence, KV head) = 2 K blocks (64 x 128) + 2 V blocks (128 x 64);
+// wave w copies block w (0, 1: K; 2, 3: V) and quantizer-parameter array w of the tile.
+// Per tile and half-wavefront hw (0..7): K unit = round hw%4 of K block hw/4, V unit = segment
+// hw%4 of V block hw/4 -- both blocks are wave-uniform (hw/4 == wave/2).
+//
+// Step s of the pipeline (slot = s & 1 holds tile s, already parsed into registers):
+//   K stage      packs -> int8 K tile, written OVER the block bytes of slot s (dead once parsed),
+//                scores on the matrix cores                                        | barrier 1
+//   softmax      reads scores and the slot's parameters; then wait for the copy of tile s+1
+//                                                                                  | barrier 2
+//   issue the copy of tile s+2 into slot s;  V stage of tile s  together with the parse of
+//   tile s+1 out of the other slot                                                 | barrier 3
+// so a copy has a whole step to land and a tile's LDS round trips hide behind the V arithmetic.
+// LDS per workgroup is 2 slots + 2 KiB: four workgroups fit a CU.
+//
+// Ordering.  The copies are issued from inline assembly, so the compiler neither sees them nor
+// waits for them; every wait on a copy is written out here (s_waitcnt vmcnt(0): the loop has no
+// other vector memory instruction, block_info comes through scalar loads).  The barriers are bare
+// s_barrier with an LDS-only wait: a workgroup fence would also drain the copies in flight.
+// The slots sit at the bottom of LDS, below 64 KiB.
+#pragma once
+#include <type_traits>
+
+namespace pkv {
+
+#define PKV_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor (base, stride 0, num_records = bytes, 32-bit raw format): reads past
+// `bytes` return zero instead of touching memory.
+__device__ __forceinline__ u32x4 dma_rsrc(const void *base, uint32_t bytes) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(base);
+    return (u32x4){(uint32_t)a, (uint32_t)(a >> 32) & 0xFFFFu, bytes, 0x00020000u};
+}
+
+// One LDS-direct load: lane l's 16 (4) bytes at buffer offset voff (+ soff) land at LDS byte
+// lds_addr + 16 l (4 l).  lds_addr, rsrc and soff are wave-uniform.
+__device__ __forceinline__ void dma_b128(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+__device__ __forceinline__ void dma_b32(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+template <int KW, int VW>
+struct DmaGeom {
+    static constexpr int kMaxBlock = k_block_bound(64, KW) > v_block_bound(64, VW) ? k_block_bound(64, KW) : v_block_bound(64, VW);
+    // a block is copied from the 16-byte boundary below its start: up to 14 bytes of phase in front
+    static constexpr int kRegion = (kMaxBlock + 14 + 511) / 512 * 512;      // LDS bytes per block
+    static constexpr int kMaxInstr = (kRegion + 1023) / 1024;              // 64-lane copy instructions per block
+    static constexpr int kKTile = 8 * 16 * 136;                            // the int8 K tile shares the block regions
+    static constexpr int kParOff = 4 * kRegion > kKTile ? 4 * kRegion : kKTile;   // then 4 arrays x 128 tokens x 2 bytes
+    static constexpr int kSlot = kParOff + 4 * kTile * 2;
+    static_assert(2 * kSlot <= 65536, "the slots must stay below 64 KiB of LDS");
+    static_assert(kKTile == 8 * 16 * kKtStride, "K tile geometry");
+};
+
+template <int G, int KW, int VW, bool BF>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) attn_dma_kernel(const AttnParams p) {
+    using Geo = DmaGeom<KW, VW>;
+    constexpr int ROWS = 3 * G;
+    constexpr int NSETS = (ROWS + 15) / 16;
+    constexpr int NG4 = (G + 3) / 4;
+    constexpr int GP = NG4 * 4;
+    constexpr int GW = (G + 3) / 4;
+    constexpr int KLB = len_field_bits(KW), VLB = len_field_bits(VW);
+    constexpr uint32_t K_META = KW * 16 + KLB * 16, V_META = VW * 16 + VLB * 16;
+    constexpr int kRoundBytes = 16 * kKtStride;
+    static_assert(16 * NSETS * 16 * 4 + 64 <= kRoundBytes, "score rows must fit the K-tile rows they reuse");
+    static_assert(NSETS * 4 * 16 * 32 <= 8 * kRoundBytes, "q digits borrow a slot");
+
+    constexpr int kLdsBytes = 2 * Geo::kSlot + GP * kTile * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t smem[kLdsBytes];
+    uint8_t *ring = smem;                                                    // [2 slots][4 block regions | parameters]
+    _Float16 *pbuf = reinterpret_cast<_Float16 *>(smem + 2 * Geo::kSlot);    // [GP][128]
+    _Float16 *p16hi = pbuf + GP * kTile;                                     // [GP][8]
+    _Float16 *p16lo = p16hi + GP * 8;
+    float *st_m = reinterpret_cast<float *>(p16lo + GP * 8);                 // 8 floats each
+    float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8, *qsum = st_z + 8, *qs = qsum + 8;
+    const uint32_t ring_lds = (uint32_t)reinterpret_cast<uintptr_t>(ring);   // LDS byte address of the slots
+    uint8_t *aq = ring;                                                      // q digits, prologue only
+
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t = tid & 31, hw = tid >> 5;
+    const int bh = b * p.Hkv + h;
+    const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
+
+    // the stream this wave copies from, range-checked: block_info is never trusted with an address
+    const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, wave < 2 ? p.k_bytes : p.v_bytes);
+    const uint16_t *par_arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
+    const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.T_c * 2));
+
+    // ---- prologue: split q into digits (through LDS, aliased onto the K tile) ----
+    for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
+    for (int i = tid; i < GP * kTile / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
+    for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
+    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 0.f; }
+    __syncthreads();
+    for (int g = wave; g < G; g += 4) {
+        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
+        const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
+        const float mx = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
+        const float sm = wave_sum(q0 + q1);
+        const float inv = mx > 0.f ? 1048576.f / mx : 0.f;
+        if (lane == 0) { qsum[g] = sm; qs[g] = mx * (1.f / 1048576.f); }
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int d = lane + 64 * e;
+            int Q = (int)rintf((e ? q1 : q0) * inv);
+            const int d2 = ((Q + 64) & 127) - 64;
+            Q = (Q - d2) >> 7;
+            const int d1 = ((Q + 64) & 127) - 64;
+            const int d0 = (Q - d1) >> 7;
+            const int dig[3] = {d0, d1, d2};
+#pragma unroll
+            for (int pp = 0; pp < 3; pp++) {
+                const int m = pp * G + g;
+                aq[(((m >> 4) * 4 + (d >> 5)) * 16 + (m & 15)) * 32 + (d & 31)] = (uint8_t)(int8_t)dig[pp];
+            }
+        }
+    }
+    __syncthreads();
+    long aop[NSETS][4];
+#pragma unroll
+    for (int s = 0; s < NSETS; s++)
+#pragma unroll
+        for (int sl = 0; sl < 4; sl++)
+            aop[s][sl] = *reinterpret_cast<const long *>(aq + ((s * 4 + sl) * 16 + (lane & 15)) * 32 + 8 * (lane >> 4));
+    float qs_r[GW], qsum_r[GW];
+#pragma unroll
+    for (int gi = 0; gi < GW; gi++) {
+        const int g = min(wave + 4 * gi, G - 1);
+        qs_r[gi] = qs[g];
+        qsum_r[gi] = qsum[g];
+    }
+    __syncthreads();      // slot 0 is free from here on; the last workgroup fence of the kernel
+
+    const int n_tiles = p.T_c / kTile;
+    const int tile0 = split * p.tiles_per_split;
+    const int tile1 = min(n_tiles, tile0 + p.tiles_per_split);
+    const int ntl = tile1 - tile0;                 // tiles of this split (>= 1)
+
+    // ---- block_info: wave-uniform scalar loads, fetched well before use ----
+    // this wave copies block `wave` of a tile and parses K block wave/2 and V block 2 + wave/2
+    // (read through the constant address space: block_info is read-only for the whole launch, and
+    // only loads known to be unclobbered are issued as scalar loads; a vector load here would make
+    // every later vmcnt wait drain the copies in flight)
+    typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
+    const int kj = wave >> 1;
+    const const_u32_ptr k_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.k_info));
+    const const_u32_ptr v_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.v_info));
+    const const_u32_ptr dma_info = wave < 2 ? k_info_c : v_info_c;
+    struct TileInfo { uint32_t dma_off, dma_size, k_off, v_off; };
+    auto load_info = [&](int rel) -> TileInfo {
+        const int tau = tile0 + min(rel, ntl - 1);
+        const uint32_t ik0 = (uint32_t)((2 * tau) * n_hid_k + bh), iv0 = (uint32_t)(tau * n_hid_v + 2 * bh);
+        const uint32_t id = wave < 2 ? ik0 + (uint32_t)wave * (uint32_t)n_hid_k : iv0 + (uint32_t)(wave - 2);
+        TileInfo ti;
+        ti.dma_off = dma_info[2 * (size_t)id];
+        ti.dma_size = dma_info[2 * (size_t)id + 1];
+        ti.k_off = k_info_c[2 * (size_t)(ik0 + (uint32_t)kj * (uint32_t)n_hid_k)];
+        ti.v_off = v_info_c[2 * (size_t)(iv0 + (uint32_t)kj)];
+        return ti;
+    };
+
+    // ---- copy of one tile into slot `slot` ----
+    auto dma_issue = [&](int slot, int rel, const TileInfo &ti) {
+        const uint32_t phase = ti.dma_off & 15u;                  // the streams themselves are 16-byte aligned
+        const uint32_t src = ti.dma_off - phase;
+        uint32_t nq = (phase + ti.dma_size + 15u) >> 4;           // 16-byte quads to copy
+        nq = min(max(nq, 1u), (uint32_t)(Geo::kRegion / 16));     // corrupt block_info must not overrun the region
+        const uint32_t last = nq - 1u;
+        const uint32_t dst = ring_lds + (uint32_t)(slot * Geo::kSlot + wave * Geo::kRegion);
+#pragma unroll
+        for (int i = 0; i < Geo::kMaxInstr; i++) {
+            if ((uint32_t)(i * 64) < nq) {                        // wave-uniform
+                if (i * 1024 + 1024 <= Geo::kRegion || lane < (Geo::kRegion - i * 1024) / 16)
+                    dma_b128(blk_rsrc, dst + i * 1024, src + 16u * min((uint32_t)(i * 64 + lane), last));
+            }
+        }
+        // parameter array `wave` of the tile: 128 tokens x 2 bytes = 64 lanes x 4 bytes
+        const int tile_off = (b * p.T_c + (tile0 + min(rel, ntl - 1)) * kTile) * 2;
+        dma_b32(par_rsrc, ring_lds + (uint32_t)(slot * Geo::kSlot + Geo::kParOff + wave * 256), 4 * lane, (uint32_t)tile_off);
+    };
+
+    // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
+    const int ku = hw & 3;
+    auto parse = [&](int slot, const TileInfo &ti, UnitRegs &kr, UnitRegs &vr) {
+        const uint8_t *kb = ring + slot * Geo::kSlot + kj * Geo::kRegion;
+        const uint8_t *vb = ring + slot * Geo::kSlot + (2 + kj) * Geo::kRegion;
+        const uint32_t kph = ti.k_off & 15u, vph = ti.v_off & 15u;
+        // header: four cumulative u16 unit sizes; unit u starts at 8 + cum[u - 1] (read unconditionally, then selected)
+        const uint32_t hsel = 2u * (uint32_t)max(ku - 1, 0);
+        uint32_t kc = *reinterpret_cast<const uint16_t *>(kb + kph + hsel);
+        uint32_t vc = *reinterpret_cast<const uint16_t *>(vb + vph + hsel);
+        kc = ku ? kc : 0u;
+        vc = ku ? vc : 0u;
+        // a corrupt header must not send the reads below out of the block's region
+        const uint32_t k_unit = min(kph + 8u + kc, (uint32_t)(Geo::kRegion - K_META - 16));
+        const uint32_t v_unit = min(vph + 8u + vc, (uint32_t)(Geo::kRegion - V_META - 16));
+        const uint32_t k_mins = lds_meta_word(kb + k_unit, t, KW), k_lens = lds_meta_word(kb + k_unit + KW * 16, t, KLB);
+        const uint32_t v_mins = lds_meta_word(vb + v_unit, t, VW), v_lens = lds_meta_word(vb + v_unit + VW * 16, t, VLB);
+        uint32_t klen[4], vlen[4], koff[4], voff[4];
+        meta_fields<KW>(k_mins, k_lens, klen, kr.lens, kr.mins);
+        meta_fields<VW>(v_mins, v_lens, vlen, vr.lens, vr.mins);
+        pack_offsets8(kr.lens, koff);
+        pack_offsets8(vr.lens, voff);
+        const uint32_t kpay0 = k_unit + K_META, vpay0 = v_unit + V_META;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            kr.word[i] = lds_load64(kb, min(kpay0 + 2u * koff[i], (uint32_t)(Geo::kRegion - 12)));
+            vr.word[i] = lds_load64(vb, min(vpay0 + 2u * voff[i], (uint32_t)(Geo::kRegion - 12)));
+        }
+    };
+
+    auto cvt2 = [&](uint32_t w, float &lo, float &hi) {
+        if (!BF) {
+            lo = __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu)));
+            hi = __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+        } else {
+            lo = __uint_as_float(w << 16);
+            hi = __uint_as_float(w & 0xFFFF0000u);
+        }
+    };
+
+    float4v acc[NG4];
+#pragma unroll
+    for (int i = 0; i < NG4; i++) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+    float m_run[GW], l_part[GW], z_part[GW];
+#pragma unroll
+    for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
+
+    // ---- stage 1: K round hw -> int8 tile rows [hw*16, hw*16+16), then scores on the matrix cores ----
+    auto k_stage = [&](const UnitRegs &kr, uint8_t *kt) {
+        {
+            uint32_t w01[4], w23[4];
+            unit_windows(kr, w01, w23);
+            const uint32_t len01 = (kr.lens & 0xFFu) | ((kr.lens & 0xFF00u) << 8);
+            const uint32_t len23 = ((kr.lens >> 16) & 0xFFu) | ((kr.lens >> 8) & 0xFF0000u);
+            const uint32_t l0 = kr.lens & 0xFFu, l1 = (kr.lens >> 8) & 0xFFu, l2 = (kr.lens >> 16) & 0xFFu, l3 = kr.lens >> 24;
+            const uint32_t mq = ((1u << l0) - 1u) | (((1u << l1) - 1u) << 8) | (((1u << l2) - 1u) << 16) |
+                                (((1u << l3) - 1u) << 24);
+            uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+#pragma unroll
+                for (int pp = 0; pp < 4; pp++) {
+                    const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
+                    const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
+                    dst[(q * 4 + pp) * kKtDw] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + kr.mins;
+                }
+            }
+        }
+        // the rounds a wavefront multiplies are the two its own halves just wrote: LDS executes a
+        // wavefront's accesses in order, so only the compiler must be kept from reordering
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int rr = 0; rr < 2; rr++) {
+            const int R = 2 * wave + rr;
+            const uint8_t *row = kt + (R * 16 + (lane & 15)) * kKtStride + 8 * (lane >> 4);
+            long bop[4];
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++) bop[sl] = *reinterpret_cast<const long *>(row + 32 * sl);
+#pragma unroll
+            for (int s = 0; s < NSETS; s++) {
+                int4v d = {0, 0, 0, 0};
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) d = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[s][sl], bop[sl], d, 0, 0, 0);
+                // row-major [m][token]; odd rounds sit 16 banks further so the softmax reads spread over all banks
+                int32_t *o = reinterpret_cast<int32_t *>(kt + R * kRoundBytes + (R & 1) * 64) +
+                             (s * 16 + 4 * (lane >> 4)) * 16 + (lane & 15);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) o[jj * 16] = d[jj];
+            }
+        }
+    };
+
+    // ---- stage 2: online softmax; wave <-> query head, lane <-> tokens 2*lane, 2*lane+1 ----
+    auto softmax_stage = [&](int slot, const uint8_t *kt) {
+        const uint32_t *par = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff) + lane;
+        float ks0, ks1, kz0, kz1, vs0, vs1, vz0, vz1;
+        cvt2(par[0], ks0, ks1); cvt2(par[64], kz0, kz1); cvt2(par[128], vs0, vs1); cvt2(par[192], vz0, vz1);
+#pragma unroll
+        for (int gi = 0; gi < GW; gi++) {
+            const int g = wave + 4 * gi;
+            if (g < G) {
+                const int32_t *r =
+                    reinterpret_cast<const int32_t *>(kt + (lane >> 3) * kRoundBytes + ((lane >> 3) & 1) * 64) + 2 * (lane & 7);
+                float sv[2];
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const float d0 = (float)r[g * 16 + e], d1 = (float)r[(G + g) * 16 + e], d2 = (float)r[(2 * G + g) * 16 + e];
+                    const float dot = qs_r[gi] * (d0 * 16384.f + d1 * 128.f + d2);
+                    sv[e] = p.sm_scale * (e ? ks1 : ks0) * (dot + (e ? kz1 : kz0) * qsum_r[gi]);
+                }
+                const float mx = wave_max_fused(fmaxf(sv[0], sv[1]));
+                const float m_new = fmaxf(m_run[gi], mx);
+                const float alpha = __expf(m_run[gi] - m_new);    // exp(-inf) = 0 on the first tile
+                m_run[gi] = m_new;
+                const float p0 = __expf(sv[0] - m_new), p1 = __expf(sv[1] - m_new);
+                const _Float16 h0 = (_Float16)(p0 * vs0 * kPScale), h1 = (_Float16)(p1 * vs1 * kPScale);
+                const float f0 = (float)h0, f1 = (float)h1;
+                // V-side order: MFMA k of a segment contracts token k of its four rounds
+                const int tok0 = 2 * lane;
+                _Float16 *pb = pbuf + g * kTile + (tok0 & 64) + ((tok0 & 15) << 2) + ((tok0 >> 4) & 3);
+                pb[0] = h0;
+                pb[4] = h1;      // token 2*lane+1: same round, next k
+                l_part[gi] = l_part[gi] * alpha + (p0 + p1);
+                z_part[gi] = z_part[gi] * alpha + (f0 * vz0 + f1 * vz1);
+                // per-round sums (16 tokens = 8 lanes) of the rounded weights, for the pack-minimum term
+                const float r16 = oct_sum_fused(f0 + f1);
+                if ((lane & 7) == 0) {
+                    const _Float16 hi = (_Float16)r16;
+                    p16hi[g * 8 + (lane >> 3)] = hi;
+                    p16lo[g * 8 + (lane >> 3)] = (_Float16)(r16 - (float)hi);
+                }
+                if (lane == 0) st_a[g] = alpha;
+            }
+        }
+    };
+
+    // ---- stage 3: V segment hw; lane = channel, MFMA k contracts token k of the lane's four packs ----
+    auto v_stage = [&](const UnitRegs &vr) {
+        const int seg = hw & 1;
+        uint32_t w01[4], w23[4];
+        unit_windows(vr, w01, w23);
+        const uint32_t len01 = (vr.lens & 0xFFu) | ((vr.lens & 0xFF00u) << 8);
+        const uint32_t len23 = ((vr.lens >> 16) & 0xFFu) | ((vr.lens >> 8) & 0xFF0000u);
+        const uint32_t m01 = ((1u << (vr.lens & 7u)) - 1u) | (((1u << ((vr.lens >> 8) & 7u)) - 1u) << 16);
+        const uint32_t m23 = ((1u << ((vr.lens >> 16) & 7u)) - 1u) | (((1u << ((vr.lens >> 24) & 7u)) - 1u) << 16);
+#pragma unroll
+        for (int i4 = 0; i4 < NG4; i4++) {
+            const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
+            acc[i4] *= al;
+        }
+        const int gl = lane & 3;
+        // pack minima: raw bits are the same fp16-subnormal encoding as the fields
+        const half4v mins = __builtin_bit_cast(half4v, make_uint2((vr.mins & 0xFFu) | ((vr.mins & 0xFF00u) << 8),
+                                                                  ((vr.mins >> 16) & 0xFFu) | ((vr.mins >> 8) & 0xFF0000u)));
+#pragma unroll
+        for (int i4 = 0; i4 < NG4; i4++) {
+            const half4v ahi = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
+            const half4v alo = *reinterpret_cast<const half4v *>(p16lo + (4 * i4 + gl) * 8 + 4 * seg);
+            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(ahi, mins, acc[i4], 0, 0, 0);
+            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(alo, mins, acc[i4], 0, 0, 0);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#pragma unroll
+            for (int pp = 0; pp < 4; pp++) {
+                const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
+                const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
+                const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
+#pragma unroll
+                for (int i4 = 0; i4 < NG4; i4++) {
+                    const half4v aopv = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kTile + 64 * seg + 4 * (4 * q + pp));
+                    acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(aopv, bop, acc[i4], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    // ---- pipeline ----
+    TileInfo i0 = load_info(0), i1 = load_info(1), i2 = load_info(2);
+    UnitRegs kcur, vcur;
+    dma_issue(0, 0, i0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PKV_LDS_BARRIER();
+    dma_issue(1, 1, i1);
+    parse(0, i0, kcur, vcur);
+    PKV_LDS_BARRIER();
+
+    // at step s: i1, i2 = block_info of tiles s+1, s+2
+    for (int s = 0; s < ntl; s++) {
+        const int slot = s & 1;
+        uint8_t *kt = ring + slot * Geo::kSlot;
+        const TileInfo i3 = load_info(s + 3);
+        if (!(p.dbg & 2)) k_stage(kcur, kt);
+        PKV_LDS_BARRIER();
+        if (!(p.dbg & 4)) softmax_stage(slot, kt);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
+        PKV_LDS_BARRIER();
+        if (!(p.dbg & 1)) dma_issue(slot, s + 2, i2);
+        UnitRegs knext, vnext;
+        parse(slot ^ 1, i1, knext, vnext);
+        if (!(p.dbg & 8)) v_stage(vcur);
+        kcur = knext;
+        vcur = vnext;
+        i1 = i2; i2 = i3;
+        PKV_LDS_BARRIER();
+    }
+    // drain: the copy issued in the last step must land before the workgroup's LDS is released
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int gi = 0; gi < GW; gi++) {
+        const int g = wave + 4 * gi;
+        if (g < G) {
+            const float l = wave_sum(l_part[gi]), z = wave_sum(z_part[gi]);
+            if (lane == 0) { st_m[g] = m_run[gi]; st_l[g] = l; st_z[g] = z; }
+        }
+    }
+    PKV_LDS_BARRIER();
+#pragma unroll
+    for (int i4 = 0; i4 < NG4; i4++)
+#pragma unroll
+        for (int m = 0; m < 4; m++) acc[i4][m] += __shfl_xor(acc[i4][m], 32, 64);
+    if ((lane >> 5) == 0) {
+        const int j = hw >> 2, w = (hw & 3) >> 1;
+        const int ch = 64 * j + 32 * w + t;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            float *dst = p.part + (hq * p.nparts + split) * kPartStride;
+            // fields were consumed as fp16 subnormals (delta * 2^-24)
+            dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
+            if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+        }
+    }
+}
+
+}  // namespace pkv
