@@ -64,6 +64,75 @@ struct DmaGeom {
     static_assert(kKTile == 8 * 16 * kKtStride, "K tile geometry");
 };
 
+// One unit's packs in registers: pack words, the four widths as two 16-bit pairs, minima as bytes.
+struct UnitPairs {
+    uint64_t word[4];
+    uint32_t len01, len23;   // widths of packs (0, 1) and (2, 3), one per 16-bit half
+    uint32_t mins;           // the four minima, one per byte
+};
+
+__device__ __forceinline__ uint32_t pk_mask16(uint32_t len_pair) {   // (1 << len) - 1 in both halves
+    const ushort2v one = {1, 1};
+    return __builtin_bit_cast(uint32_t, (ushort2v)((ushort2v)(one << __builtin_bit_cast(ushort2v, len_pair)) - one));
+}
+
+// 64 bits at byte offset `off` (even) of an LDS array whose base is 4-byte aligned: the three
+// aligned dwords that cover it, funnel-shifted by bytes (a misaligned DS read stalls the LDS pipe).
+__device__ __forceinline__ uint64_t lds_word64(const uint8_t *base, uint32_t off) {
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (off & ~3u));
+    const uint32_t d0 = q[0], d1 = q[1], d2 = q[2];
+    const uint32_t lo = __builtin_amdgcn_alignbyte(d1, d0, off), hi = __builtin_amdgcn_alignbyte(d2, d1, off);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Lane t's 4*NB-bit metadata word of the LSB-first bit array at byte offset `off` (even) of `base`.
+template <int NB>
+__device__ __forceinline__ uint32_t lds_meta(const uint8_t *base, uint32_t off, int t) {
+    if (NB == 4) return *reinterpret_cast<const uint16_t *>(base + off + 2 * t);
+    if (NB == 2) return base[off + t];
+    const uint32_t a = off + ((uint32_t)(t * 12) >> 3);          // NB == 3: 12 bits at bit 12 t
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (a & ~3u));
+    const uint32_t v = __builtin_amdgcn_alignbyte(q[1], q[0], a);
+    return (v >> ((t & 1) * 4)) & 0xFFFu;
+}
+
+template <int W>
+__device__ __forceinline__ void meta_pairs(uint32_t minsw, uint32_t lensw, UnitPairs &u) {
+    constexpr int LB = len_field_bits(W);
+    u.len01 = __builtin_amdgcn_ubfe(lensw, 0, LB) | (__builtin_amdgcn_ubfe(lensw, LB, LB) << 16);
+    u.len23 = __builtin_amdgcn_ubfe(lensw, 2 * LB, LB) | (__builtin_amdgcn_ubfe(lensw, 3 * LB, LB) << 16);
+    if (W == 4) {   // four nibbles -> four bytes
+        const uint32_t y = (minsw | (minsw << 8)) & 0x00FF00FFu;
+        u.mins = (y | (y << 4)) & 0x0F0F0F0Fu;
+    } else {
+        u.mins = __builtin_amdgcn_ubfe(minsw, 0, W) | (__builtin_amdgcn_ubfe(minsw, W, W) << 8) |
+                 (__builtin_amdgcn_ubfe(minsw, 2 * W, W) << 16) | (__builtin_amdgcn_ubfe(minsw, 3 * W, W) << 24);
+    }
+}
+
+// win01[q] = tokens 4q..4q+3 of packs 0 and 1 in the low / high 16 bits (token 4q on top), win23
+// likewise; bits above 4*len in a half are other tokens' fields, every consumer masks.
+__device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[4], uint32_t win23[4]) {
+    const uint32_t len[4] = {u.len01 & 0xFFFFu, u.len01 >> 16, u.len23 & 0xFFFFu, u.len23 >> 16};
+    uint32_t hlf[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        hlf[i][0] = (uint32_t)(u.word[i] >> (8u * len[i]));   // tokens 0..7
+        hlf[i][1] = (uint32_t)u.word[i];                      // tokens 8..15
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        uint32_t qd[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t src = hlf[i][q >> 1];
+            qd[i] = (q & 1) ? src : (src >> (4u * len[i]));
+        }
+        win01[q] = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);
+        win23[q] = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
+    }
+}
+
 template <int G, int KW, int VW, bool BF>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) attn_dma_kernel(const AttnParams p) {
     using Geo = DmaGeom<KW, VW>;
@@ -105,7 +174,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
     for (int i = tid; i < GP * kTile / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
     for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
-    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 0.f; }
+    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 1.f; }
     __syncthreads();
     for (int g = wave; g < G; g += 4) {
         const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
@@ -196,7 +265,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 
     // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
     const int ku = hw & 3;
-    auto parse = [&](int slot, const TileInfo &ti, UnitRegs &kr, UnitRegs &vr) {
+    auto parse = [&](int slot, const TileInfo &ti, UnitPairs &kr, UnitPairs &vr) {
         const uint8_t *kb = ring + slot * Geo::kSlot + kj * Geo::kRegion;
         const uint8_t *vb = ring + slot * Geo::kSlot + (2 + kj) * Geo::kRegion;
         const uint32_t kph = ti.k_off & 15u, vph = ti.v_off & 15u;
@@ -206,21 +275,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         uint32_t vc = *reinterpret_cast<const uint16_t *>(vb + vph + hsel);
         kc = ku ? kc : 0u;
         vc = ku ? vc : 0u;
-        // a corrupt header must not send the reads below out of the block's region
+        // A corrupt header must not send the metadata reads out of the block's region.  The pack
+        // reads below start less than 1.1 KiB behind the unit, which keeps them inside this
+        // workgroup's LDS (2.3 KiB follow the last region); garbage in, garbage out, no fault.
         const uint32_t k_unit = min(kph + 8u + kc, (uint32_t)(Geo::kRegion - K_META - 16));
         const uint32_t v_unit = min(vph + 8u + vc, (uint32_t)(Geo::kRegion - V_META - 16));
-        const uint32_t k_mins = lds_meta_word(kb + k_unit, t, KW), k_lens = lds_meta_word(kb + k_unit + KW * 16, t, KLB);
-        const uint32_t v_mins = lds_meta_word(vb + v_unit, t, VW), v_lens = lds_meta_word(vb + v_unit + VW * 16, t, VLB);
-        uint32_t klen[4], vlen[4], koff[4], voff[4];
-        meta_fields<KW>(k_mins, k_lens, klen, kr.lens, kr.mins);
-        meta_fields<VW>(v_mins, v_lens, vlen, vr.lens, vr.mins);
-        pack_offsets8(kr.lens, koff);
-        pack_offsets8(vr.lens, voff);
+        const uint32_t k_mins = lds_meta<KW>(kb, k_unit, t), k_lens = lds_meta<KLB>(kb, k_unit + KW * 16, t);
+        const uint32_t v_mins = lds_meta<VW>(vb, v_unit, t), v_lens = lds_meta<VLB>(vb, v_unit + VW * 16, t);
+        uint32_t koff[4], voff[4];
+        meta_pairs<KW>(k_mins, k_lens, kr);
+        meta_pairs<VW>(v_mins, v_lens, vr);
+        pack_offsets8(__builtin_amdgcn_perm(kr.len23, kr.len01, 0x06040200u), koff);
+        pack_offsets8(__builtin_amdgcn_perm(vr.len23, vr.len01, 0x06040200u), voff);
         const uint32_t kpay0 = k_unit + K_META, vpay0 = v_unit + V_META;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            kr.word[i] = lds_load64(kb, min(kpay0 + 2u * koff[i], (uint32_t)(Geo::kRegion - 12)));
-            vr.word[i] = lds_load64(vb, min(vpay0 + 2u * voff[i], (uint32_t)(Geo::kRegion - 12)));
+            kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
+            vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
         }
     };
 
@@ -242,15 +313,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
 
     // ---- stage 1: K round hw -> int8 tile rows [hw*16, hw*16+16), then scores on the matrix cores ----
-    auto k_stage = [&](const UnitRegs &kr, uint8_t *kt) {
+    auto k_stage = [&](const UnitPairs &kr, uint8_t *kt) {
         {
             uint32_t w01[4], w23[4];
-            unit_windows(kr, w01, w23);
-            const uint32_t len01 = (kr.lens & 0xFFu) | ((kr.lens & 0xFF00u) << 8);
-            const uint32_t len23 = ((kr.lens >> 16) & 0xFFu) | ((kr.lens >> 8) & 0xFF0000u);
-            const uint32_t l0 = kr.lens & 0xFFu, l1 = (kr.lens >> 8) & 0xFFu, l2 = (kr.lens >> 16) & 0xFFu, l3 = kr.lens >> 24;
-            const uint32_t mq = ((1u << l0) - 1u) | (((1u << l1) - 1u) << 8) | (((1u << l2) - 1u) << 16) |
-                                (((1u << l3) - 1u) << 24);
+            pair_windows(kr, w01, w23);
+            const uint32_t len01 = kr.len01, len23 = kr.len23;
+            const uint32_t mq = __builtin_amdgcn_perm(pk_mask16(len23), pk_mask16(len01), 0x06040200u);   // byte masks
             uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
@@ -333,23 +401,30 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     };
 
     // ---- stage 3: V segment hw; lane = channel, MFMA k contracts token k of the lane's four packs ----
-    auto v_stage = [&](const UnitRegs &vr) {
+    auto v_stage = [&](const UnitPairs &vr) {
         const int seg = hw & 1;
         uint32_t w01[4], w23[4];
-        unit_windows(vr, w01, w23);
-        const uint32_t len01 = (vr.lens & 0xFFu) | ((vr.lens & 0xFF00u) << 8);
-        const uint32_t len23 = ((vr.lens >> 16) & 0xFFu) | ((vr.lens >> 8) & 0xFF0000u);
-        const uint32_t m01 = ((1u << (vr.lens & 7u)) - 1u) | (((1u << ((vr.lens >> 8) & 7u)) - 1u) << 16);
-        const uint32_t m23 = ((1u << ((vr.lens >> 16) & 7u)) - 1u) | (((1u << ((vr.lens >> 24) & 7u)) - 1u) << 16);
+        pair_windows(vr, w01, w23);
+        const uint32_t len01 = vr.len01, len23 = vr.len23;
+        const uint32_t m01 = pk_mask16(len01), m23 = pk_mask16(len23);
+        // rescale the accumulators only when some head's running maximum moved (alpha <= 1, so the
+        // product is 1 exactly when every alpha is)
+        {
+            float prod = 1.f;
 #pragma unroll
-        for (int i4 = 0; i4 < NG4; i4++) {
-            const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
-            acc[i4] *= al;
+            for (int g = 0; g < GP; g++) prod *= st_a[g];
+            if (__builtin_amdgcn_readfirstlane(__float_as_uint(prod)) != 0x3F800000u) {
+#pragma unroll
+                for (int i4 = 0; i4 < NG4; i4++) {
+                    const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
+                    acc[i4] *= al;
+                }
+            }
         }
         const int gl = lane & 3;
         // pack minima: raw bits are the same fp16-subnormal encoding as the fields
-        const half4v mins = __builtin_bit_cast(half4v, make_uint2((vr.mins & 0xFFu) | ((vr.mins & 0xFF00u) << 8),
-                                                                  ((vr.mins >> 16) & 0xFFu) | ((vr.mins >> 8) & 0xFF0000u)));
+        const half4v mins = __builtin_bit_cast(half4v, make_uint2(__builtin_amdgcn_perm(0u, vr.mins, 0x0C010C00u),
+                                                                  __builtin_amdgcn_perm(0u, vr.mins, 0x0C030C02u)));
 #pragma unroll
         for (int i4 = 0; i4 < NG4; i4++) {
             const half4v ahi = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
@@ -375,7 +450,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 
     // ---- pipeline ----
     TileInfo i0 = load_info(0), i1 = load_info(1), i2 = load_info(2);
-    UnitRegs kcur, vcur;
+    UnitPairs kcur, vcur;
     dma_issue(0, 0, i0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     PKV_LDS_BARRIER();
@@ -394,7 +469,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
         PKV_LDS_BARRIER();
         if (!(p.dbg & 1)) dma_issue(slot, s + 2, i2);
-        UnitRegs knext, vnext;
+        UnitPairs knext, vnext;
         parse(slot ^ 1, i1, knext, vnext);
         if (!(p.dbg & 8)) v_stage(vcur);
         kcur = knext;
