@@ -142,8 +142,10 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype` (the residual
  *                     window the cache keeps in 16-bit, utils/compute.py:54-67); T_w may be 0
  *   T_c               compressed tokens, a multiple of 128 (may be 0 when T_w > 0)
- *   variant           0 = default kernel; other values select alternative implementations
- *                     of the same contract (used by tests to cross-check)
+ *   variant           0 = default (asynchronous-copy matrix-core kernel; streams must be 16-byte
+ *                     aligned, otherwise variant 2 runs); 1 = plain VALU kernel; 2 = matrix-core
+ *                     kernel that gathers straight from global memory.  All three implement the
+ *                     same contract; tests cross-check them.
  */
 typedef struct pkv_attn_args {
     const uint8_t *k_stream;

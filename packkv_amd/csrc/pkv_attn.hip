@@ -12,7 +12,6 @@
 // kernel combines the splits and the tail window.
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
-#include <cstdlib>
 
 namespace pkv {
 
@@ -44,7 +43,6 @@ struct AttnParams {
     int B, Hq, Hkv, T_c, T_w;
     int k_bits, v_bits, dtype;
     float sm_scale;
-    int dbg;
     int tiles_per_split, nsplit, nparts;
     uint32_t k_cap, v_cap, blk_stride;
     uint32_t k_bytes, v_bytes;   // valid bytes of the streams
@@ -219,7 +217,7 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
     }
 }
 
-// ---- variant 0: matrix-core kernel ---------------------------------------------------------
+// ---- matrix-core kernels (variants 0 and 2): shared arithmetic ----------------------------
 // K side: every half-wavefront unpacks one round (16 tokens x 128 channels, lane t = channels
 // 4t..4t+3) into an int8 tile in LDS laid out [token][channel]; the tile is read back in the
 // operand layout of v_mfma_i32_16x16x32_i8 (lane = token, 8 consecutive channels) and
@@ -278,393 +276,6 @@ __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
     for (int r = 0; r < 4; r++) s += __builtin_bit_cast(float, __builtin_amdgcn_readlane(v, 16 * r));
     return s;
-}
-
-// The four packs of a lane as 16-bit windows: win01[q] holds tokens 4q..4q+3 of packs 0 and 1 in
-// its low and high half (token 4q at bits [3*len, 4*len) of the half), win23[q] packs 2 and 3.
-// Bits above 4*len in a half are other tokens' fields; every consumer masks.
-__device__ __forceinline__ void pack_windows(const UnitPacks &u, uint32_t win01[4], uint32_t win23[4]) {
-    uint32_t hlf[4][2];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        hlf[i][0] = (uint32_t)(u.word[i] >> (8u * u.len[i]));   // tokens 0..7
-        hlf[i][1] = (uint32_t)u.word[i];                        // tokens 8..15
-    }
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        uint32_t qd[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t src = hlf[i][q >> 1];
-            qd[i] = (q & 1) ? src : (src >> (4u * u.len[i]));
-        }
-        win01[q] = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);
-        win23[q] = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
-    }
-}
-
-template <int G>
-__global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
-    constexpr int ROWS = 3 * G;                  // MFMA rows: (digit, head)
-    constexpr int NSETS = (ROWS + 15) / 16;
-    constexpr int NG4 = (G + 3) / 4;             // groups of 4 heads on the V side
-    constexpr int GP = NG4 * 4;                  // heads padded to a multiple of 4
-    constexpr int GW = (G + 3) / 4;              // query heads per wavefront in the softmax stage
-    extern __shared__ __align__(16) uint8_t lds[];
-    uint8_t *stage = lds;
-    uint8_t *aq = lds;       // [NSETS][4][16][32] q digits; only alive in the prologue, before the first tile lands
-    _Float16 *pbuf = reinterpret_cast<_Float16 *>(stage + 4 * p.blk_stride);      // [GP][128]
-    _Float16 *p16hi = pbuf + GP * kTile;                                  // [GP][8]
-    _Float16 *p16lo = p16hi + GP * 8;                                     // [GP][8]
-    float *qpar = reinterpret_cast<float *>(p16lo + GP * 8);              // [4][128]: ks, kz, vs, vz
-    float *st_m = qpar + 4 * kTile;                                       // 8 floats each
-    float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8;
-    float *qsum = st_z + 8, *qs = qsum + 8;
-    uint8_t *kt = reinterpret_cast<uint8_t *>(qs + 8);                    // [8 rounds][16 tok][136] int8
-    // scores of round R ([16*NSETS rows][16 tok] int32) overwrite the K-tile rows of round R once the
-    // wavefront that owns the round has loaded its B operands
-    constexpr int kRoundBytes = 16 * kKtStride;
-    static_assert(16 * NSETS * 16 * 4 <= kRoundBytes, "score rows must fit the K-tile rows they reuse");
-    __shared__ uint32_t s_info[3][4][2];   // ring over tiles: (byte offset, byte size) of 2 K + 2 V blocks
-
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index in an SGPR
-    const int t = tid & 31, hw = tid >> 5;
-    const int bh = b * p.Hkv + h;
-    const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
-    const UnitGeom gk = unit_geom(p.k_bits), gv = unit_geom(p.v_bits);
-
-    // ---- prologue: split q into digits, zero the padded rows ----
-    for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
-    for (int i = tid; i < GP * kTile / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
-    for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
-    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 0.f; }
-    __syncthreads();
-    for (int g = wave; g < G; g += 4) {
-        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
-        const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
-        const float mx = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
-        const float sm = wave_sum(q0 + q1);
-        const float inv = mx > 0.f ? 1048576.f / mx : 0.f;
-        if (lane == 0) { qsum[g] = sm; qs[g] = mx * (1.f / 1048576.f); }
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const int d = lane + 64 * e;
-            int Q = (int)rintf((e ? q1 : q0) * inv);
-            const int d2 = ((Q + 64) & 127) - 64;
-            Q = (Q - d2) >> 7;
-            const int d1 = ((Q + 64) & 127) - 64;
-            const int d0 = (Q - d1) >> 7;
-            const int dig[3] = {d0, d1, d2};
-#pragma unroll
-            for (int pp = 0; pp < 3; pp++) {
-                const int m = pp * G + g;
-                aq[(((m >> 4) * 4 + (d >> 5)) * 16 + (m & 15)) * 32 + (d & 31)] = (uint8_t)(int8_t)dig[pp];
-            }
-        }
-    }
-    __syncthreads();
-    long aop[NSETS][4];
-#pragma unroll
-    for (int s = 0; s < NSETS; s++)
-#pragma unroll
-        for (int sl = 0; sl < 4; sl++)
-            aop[s][sl] = *reinterpret_cast<const long *>(aq + ((s * 4 + sl) * 16 + (lane & 15)) * 32 + 8 * (lane >> 4));
-
-    float4v acc[NG4];
-#pragma unroll
-    for (int i = 0; i < NG4; i++) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
-    // softmax state of the query heads this wavefront owns: running max (uniform) and per-lane
-    // partial sums, reduced across lanes once at the end
-    float m_run[GW], l_part[GW], z_part[GW];
-#pragma unroll
-    for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
-
-    const int n_tiles = p.T_c / kTile;
-    const int tile0 = split * p.tiles_per_split;
-    const int tile1 = min(n_tiles, tile0 + p.tiles_per_split);
-
-    // Software pipeline over tiles: while tile tau is processed from LDS, the stream bytes and
-    // quantizer parameters of tile tau+1 are in flight into registers, and the block_info of
-    // tile tau+2 into one more; they are written to LDS at the bottom of the iteration.
-    // Blocks are fetched as 16-byte quads from the 16-byte-aligned address below their start;
-    // the distance to the start (phase, even, < 16) is added to every in-block offset.
-    uint4 pa0, pb0, pa1, pb1, pa2, pb2, pa3, pb3;   // two 16-byte quads per block (scalars: an array here lands in scratch)
-    uint2 pre_q;
-
-    auto block_index = [&](int tau, int j) -> uint32_t {
-        return j < 2 ? (uint32_t)((2 * tau + j) * n_hid_k + bh) : (uint32_t)(tau * n_hid_v + 2 * bh + (j - 2));
-    };
-    // All loads below are unconditional (clamped indices instead of predicates): a load inside a
-    // divergent branch makes the compiler wait for it right there, which serialises the prefetch.
-    // Pointer choices are kept wave-uniform (a per-lane choice between kernel-argument pointers
-    // turns into a vector load of the pointer itself, one more memory round trip).
-    auto fetch_info = [&](int tau) -> uint2 {     // even waves read the K entries, odd waves the V entries
-        const int tc = min(tau, tile1 - 1);
-        const int j = 2 * (wave & 1) + (lane & 1);
-        const uint32_t *info = (wave & 1) ? p.v_info : p.k_info;
-        return *reinterpret_cast<const uint2 *>(info + 2 * (size_t)block_index(tc, j));
-    };
-    auto store_info = [&](int slot, uint2 r) {
-        if (wave < 2 && lane < 2) {
-            const uint32_t cap = wave ? p.v_cap : p.k_cap;
-            s_info[slot][2 * wave + lane][0] = r.x;
-            s_info[slot][2 * wave + lane][1] = r.y > cap ? cap : r.y;   // corrupt block_info must not overrun LDS
-        }
-    };
-    auto block_src = [&](int slot, int j, uint32_t &phase, uint32_t &nquad) -> const uint4 * {
-        const uint32_t off = __builtin_amdgcn_readfirstlane(s_info[slot][j][0]);
-        const uint32_t size = __builtin_amdgcn_readfirstlane(s_info[slot][j][1]);
-        const uint8_t *a = (j < 2 ? p.k_stream : p.v_stream) + off;     // stays a global pointer
-        phase = (uint32_t)(reinterpret_cast<uintptr_t>(a) & 15u);
-        nquad = (phase + size + 15u) >> 4;
-        return reinterpret_cast<const uint4 *>(a - phase);
-    };
-    auto load_block = [&](int slot, int j, uint4 &qa, uint4 &qb) {
-        uint32_t phase, nquad;
-        const uint4 *src = block_src(slot, j, phase, nquad);
-        const uint32_t last = nquad - 1u;                      // nquad >= 1: blocks are never empty
-        qa = src[min((uint32_t)tid, last)];
-        qb = src[min((uint32_t)tid + 256u, last)];             // only blocks above 4 KiB use it
-    };
-    auto store_block = [&](int slot, int j, const uint4 &qa, const uint4 &qb) {
-        uint32_t phase, nquad;
-        (void)block_src(slot, j, phase, nquad);
-        uint4 *dst = reinterpret_cast<uint4 *>(stage + j * p.blk_stride);
-        if ((uint32_t)tid < nquad) dst[tid] = qa;
-        if ((uint32_t)tid + 256u < nquad) dst[tid + 256] = qb;
-    };
-    auto issue_loads = [&](int tau, int slot) {
-        load_block(slot, 0, pa0, pb0);
-        load_block(slot, 1, pa1, pb1);
-        load_block(slot, 2, pa2, pb2);
-        load_block(slot, 3, pa3, pb3);
-        // wave w fetches parameter array w: 32 lanes x 4 tokens (8 bytes); the upper half-wave repeats
-        const uint16_t *arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
-        pre_q = *reinterpret_cast<const uint2 *>(arr + (size_t)b * p.T_c + (size_t)tau * kTile + 4 * t);
-    };
-    auto commit_loads = [&](int slot) {
-        store_block(slot, 0, pa0, pb0);
-        store_block(slot, 1, pa1, pb1);
-        store_block(slot, 2, pa2, pb2);
-        store_block(slot, 3, pa3, pb3);
-        if (lane < 32) {
-            const uint32_t w0 = pre_q.x, w1 = pre_q.y;
-            float4v f;
-            if (p.dtype == PKV_F16) {
-                f[0] = __half2float(__ushort_as_half((unsigned short)(w0 & 0xFFFFu)));
-                f[1] = __half2float(__ushort_as_half((unsigned short)(w0 >> 16)));
-                f[2] = __half2float(__ushort_as_half((unsigned short)(w1 & 0xFFFFu)));
-                f[3] = __half2float(__ushort_as_half((unsigned short)(w1 >> 16)));
-            } else {
-                f[0] = __uint_as_float(w0 << 16);
-                f[1] = __uint_as_float(w0 & 0xFFFF0000u);
-                f[2] = __uint_as_float(w1 << 16);
-                f[3] = __uint_as_float(w1 & 0xFFFF0000u);
-            }
-            *reinterpret_cast<float4v *>(qpar + wave * kTile + 4 * t) = f;
-        }
-    };
-    const float *ks = qpar, *kz = qpar + kTile, *vs = qpar + 2 * kTile, *vz = qpar + 3 * kTile;
-
-    if (tile0 < tile1) {
-        store_info(0, fetch_info(tile0));
-        store_info(1, fetch_info(tile0 + 1));
-        __syncthreads();
-        issue_loads(tile0, 0);
-        commit_loads(0);
-        __syncthreads();
-    }
-    for (int tau = tile0; tau < tile1; tau++) {
-        const int rel = tau - tile0;
-        const int slot = rel % 3;
-        const bool more = tau + 1 < tile1;
-        // 1. prefetch the next tile (registers) and the block_info of the one after
-        const uint2 inext = fetch_info(tau + 2);
-        if (!(p.dbg & 16)) issue_loads(more ? tau + 1 : tau, more ? (rel + 1) % 3 : slot);
-
-        // 2. parse this half-wave's K round and V segment together (one batch of LDS round trips),
-        //    then K round hw -> int8 tile rows [hw*16, hw*16+16)
-        UnitPacks u, uv;
-        {
-            const int j = hw >> 2, unit = hw & 3;
-            const uint8_t *kb = stage + j * p.blk_stride;
-            const uint8_t *vb = stage + (2 + j) * p.blk_stride;
-            const uint32_t kph = s_info[slot][j][0] + (uint32_t)(reinterpret_cast<uintptr_t>(p.k_stream)) & 15u;
-            const uint32_t vph = s_info[slot][2 + j][0] + (uint32_t)(reinterpret_cast<uintptr_t>(p.v_stream)) & 15u;
-            const uint16_t *kcum = reinterpret_cast<const uint16_t *>(kb + kph);
-            const uint16_t *vcum = reinterpret_cast<const uint16_t *>(vb + vph);
-            const uint32_t kc = unit ? (uint32_t)kcum[unit - 1] : 0u, vc = unit ? (uint32_t)vcum[unit - 1] : 0u;
-            unit_parse2(kb, kph + 8u + kc, gk, u, vb, vph + 8u + vc, gv, uv, t);
-        }
-        if (!(p.dbg & 1)) {
-            uint32_t w01[4], w23[4];
-            pack_windows(u, w01, w23);
-            const uint32_t len01 = u.len[0] | (u.len[1] << 16), len23 = u.len[2] | (u.len[3] << 16);
-            const uint32_t mq = ((1u << u.len[0]) - 1u) | (((1u << u.len[1]) - 1u) << 8) |
-                                (((1u << u.len[2]) - 1u) << 16) | (((1u << u.len[3]) - 1u) << 24);
-            const uint32_t minq = u.mn[0] | (u.mn[1] << 8) | (u.mn[2] << 16) | (u.mn[3] << 24);
-            uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-#pragma unroll
-                for (int pp = 0; pp < 4; pp++) {
-                    const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
-                    const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
-                    dst[(q * 4 + pp) * kKtDw] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + minq;
-                }
-            }
-        }
-        // the rounds a wavefront multiplies are the two its own halves just wrote: LDS executes a
-        // wavefront's accesses in order, so only the compiler must be kept from reordering
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        // 3. scores on the matrix cores: wave handles rounds 2*wave, 2*wave+1
-        if (!(p.dbg & 2))
-#pragma unroll
-        for (int rr = 0; rr < 2; rr++) {
-            const int R = 2 * wave + rr;
-            const uint8_t *row = kt + (R * 16 + (lane & 15)) * kKtStride + 8 * (lane >> 4);
-            long bop[4];
-#pragma unroll
-            for (int sl = 0; sl < 4; sl++) bop[sl] = *reinterpret_cast<const long *>(row + 32 * sl);
-#pragma unroll
-            for (int s = 0; s < NSETS; s++) {
-                int4v d = {0, 0, 0, 0};
-#pragma unroll
-                for (int sl = 0; sl < 4; sl++) d = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[s][sl], bop[sl], d, 0, 0, 0);
-                // row-major [R][m][token]: conflict-free here and in the softmax stage
-                int32_t *o = reinterpret_cast<int32_t *>(kt + R * kRoundBytes) + (s * 16 + 4 * (lane >> 4)) * 16 + (lane & 15);
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) o[jj * 16] = d[jj];
-            }
-        }
-        __syncthreads();
-
-        // 4. online softmax: wave <-> query head
-        if (!(p.dbg & 4))
-#pragma unroll
-        for (int gi = 0; gi < GW; gi++) {
-            const int g = wave + 4 * gi;
-            if (g < G) {
-                float sv[2], pf[2];
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int tok = lane + 64 * e;
-                    const int32_t *r = reinterpret_cast<const int32_t *>(kt + (tok >> 4) * kRoundBytes) + (tok & 15);
-                    const int m0 = g, m1 = G + g, m2 = 2 * G + g;
-                    const float d0 = (float)r[m0 * 16], d1 = (float)r[m1 * 16], d2 = (float)r[m2 * 16];
-                    const float dot = qs[g] * (d0 * 16384.f + d1 * 128.f + d2);
-                    sv[e] = p.sm_scale * ks[tok] * (dot + kz[tok] * qsum[g]);
-                }
-                const float mx = wave_max(fmaxf(sv[0], sv[1]));
-                const float m_new = fmaxf(m_run[gi], mx);
-                const float alpha = __expf(m_run[gi] - m_new);    // exp(-inf) = 0 on the first tile
-                m_run[gi] = m_new;
-                float lsum = 0.f, zs = 0.f;
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int tok = lane + 64 * e;
-                    const float pe = __expf(sv[e] - m_new);
-                    const _Float16 ph = (_Float16)(pe * vs[tok] * kPScale);
-                    // V-side order: MFMA k of a segment contracts token k of its four rounds
-                    pbuf[g * kTile + (tok & 64) + ((tok & 15) << 2) + ((tok >> 4) & 3)] = ph;
-                    pf[e] = (float)ph;
-                    lsum += pe;
-                    zs += pf[e] * vz[tok];
-                    // per-round (16 token) sums of the rounded weights, for the pack-minimum term
-                    const float r16 = row16_sum(pf[e]);
-                    if ((lane & 15) == 0) {
-                        const _Float16 hi = (_Float16)r16;
-                        p16hi[g * 8 + (tok >> 4)] = hi;
-                        p16lo[g * 8 + (tok >> 4)] = (_Float16)(r16 - (float)hi);
-                    }
-                }
-                l_part[gi] = l_part[gi] * alpha + lsum;
-                z_part[gi] = z_part[gi] * alpha + zs;
-                if (lane == 0) st_a[g] = alpha;
-            }
-        }
-        __syncthreads();
-
-        // 5. V segment hw: lane = channel; MFMA k contracts token k of the lane's four packs
-        if (!(p.dbg & 8)) {
-            const int seg = hw & 1;
-            const UnitPacks &u = uv;
-            uint32_t w01[4], w23[4];
-            pack_windows(u, w01, w23);
-            const uint32_t len01 = u.len[0] | (u.len[1] << 16), len23 = u.len[2] | (u.len[3] << 16);
-            const uint32_t m01 = ((1u << u.len[0]) - 1u) | (((1u << u.len[1]) - 1u) << 16);
-            const uint32_t m23 = ((1u << u.len[2]) - 1u) | (((1u << u.len[3]) - 1u) << 16);
-#pragma unroll
-            for (int i4 = 0; i4 < NG4; i4++) {
-                const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
-                acc[i4] *= al;
-            }
-            const int gl = lane & 3;
-            // pack minima: raw bits are the same subnormal encoding as the fields
-            const half4v mins = __builtin_bit_cast(half4v, make_uint2(u.mn[0] | (u.mn[1] << 16), u.mn[2] | (u.mn[3] << 16)));
-#pragma unroll
-            for (int i4 = 0; i4 < NG4; i4++) {
-                const half4v ahi = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
-                const half4v alo = *reinterpret_cast<const half4v *>(p16lo + (4 * i4 + gl) * 8 + 4 * seg);
-                acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(ahi, mins, acc[i4], 0, 0, 0);
-                acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(alo, mins, acc[i4], 0, 0, 0);
-            }
-            if (!(p.dbg & 64))
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-#pragma unroll
-                for (int pp = 0; pp < 4; pp++) {
-                    const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
-                    const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
-                    const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
-#pragma unroll
-                    for (int i4 = 0; i4 < NG4; i4++) {
-                        const half4v aopv = *reinterpret_cast<const half4v *>(
-                            pbuf + (4 * i4 + gl) * kTile + 64 * seg + 4 * (4 * q + pp));
-                        acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(aopv, bop, acc[i4], 0, 0, 0);
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        // 6. land the prefetched tile in LDS
-        store_info((rel + 2) % 3, inext);
-        if (more && !(p.dbg & 16)) commit_loads((rel + 1) % 3);
-        __syncthreads();
-    }
-
-    // epilogue: reduce the softmax sums, then the two half-waves of a wave hold the two 64-token
-    // halves of the same channels
-#pragma unroll
-    for (int gi = 0; gi < GW; gi++) {
-        const int g = wave + 4 * gi;
-        if (g < G) {
-            const float l = wave_sum(l_part[gi]), z = wave_sum(z_part[gi]);
-            if (lane == 0) { st_m[g] = m_run[gi]; st_l[g] = l; st_z[g] = z; }
-        }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i4 = 0; i4 < NG4; i4++)
-#pragma unroll
-        for (int m = 0; m < 4; m++) acc[i4][m] += __shfl_xor(acc[i4][m], 32, 64);
-    if ((lane >> 5) == 0) {
-        const int j = hw >> 2, w = (hw & 3) >> 1;
-        const int ch = 64 * j + 32 * w + t;
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
-            float *dst = p.part + (hq * p.nparts + split) * kPartStride;
-            // fields were consumed as fp16 subnormals (delta * 2^-24)
-            dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
-            if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
-        }
-    }
 }
 
 // ---- 16-bit tail window: dense attention over T_w tokens, one workgroup per (kv head, batch)
@@ -811,30 +422,22 @@ static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
 template <int G>
 static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(p.k_stream) | reinterpret_cast<uintptr_t>(p.v_stream)) & 15u) == 0;
-    if (p.T_c > 0 && (variant & 0xFF) == 0 && aligned16) {
+    PKV_REQUIRE(variant >= 0 && variant <= 2, PKV_ERR_INVALID, "variant must be 0, 1 or 2");
+    // variant 0: asynchronous-copy kernel (needs 16-byte aligned streams; otherwise, and as
+    // variant 2, the kernel that gathers straight from global memory); variant 1: plain VALU kernel
+    if (p.T_c > 0 && variant == 0 && aligned16) {
         const int rc = launch_dma_bits<G>(p, s);
         if (rc) return rc;
-    } else if (p.T_c > 0 && ((variant & 0xFF) == 0 || (variant & 0xFF) == 3)) {
+    } else if (p.T_c > 0 && (variant == 0 || variant == 2)) {
         const int rc = launch_direct_bits<G>(p, s);
         if (rc) return rc;
-    } else if (p.T_c > 0 && (variant & 0xFF) == 1) {
+    } else if (p.T_c > 0) {
         const uint32_t lds_bytes = 2u * kTile * kHeadDim + 4u * p.blk_stride +
                                    (uint32_t)sizeof(float) * (G * kHeadDim + 2 * G * kTile + 4 * kTile + 5 * G);
         const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
         PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_tiles_kernel<G>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         attn_tiles_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
-        PKV_HIP_CHECK(hipGetLastError());
-    } else if (p.T_c > 0) {
-        constexpr int NSETS = (3 * G + 15) / 16, GP = ((G + 3) / 4) * 4;
-        static_assert(NSETS * 4 * 16 * 32 <= 4 * 4096, "q digits must fit the stage area they borrow");
-        uint32_t lds_bytes = 4u * p.blk_stride + 8u * 16u * kKtStride + GP * kTile * 2u + 2u * GP * 8u * 2u +
-                             4u * kTile * 4u + 6u * 8u * 4u;
-        if (getenv("PKV_DBG_LDS_BYTES")) lds_bytes = (uint32_t)atoi(getenv("PKV_DBG_LDS_BYTES"));
-        const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
-        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel<G>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attn_mfma_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
     if (p.T_w > 0) {
@@ -890,12 +493,11 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     p.k_win = (const uint16_t *)a->k_win; p.v_win = (const uint16_t *)a->v_win;
     p.B = a->B; p.Hq = a->Hq; p.Hkv = a->Hkv; p.T_c = a->T_c; p.T_w = a->T_w;
     p.k_bits = a->k_bits; p.v_bits = a->v_bits; p.dtype = a->dtype; p.sm_scale = a->sm_scale;
-    p.dbg = (a->variant >> 8) & 0xFF;
     const int n_tiles = a->T_c / kTile;
     int nsplit = 0, tps = 0;
     if (n_tiles > 0) {
         const int pairs = a->B * a->Hkv;
-        const int target = 1024;
+        const int target = 1024;                   // four resident workgroups on each of 256 CUs
         int want = (target + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
         if (want < 1) want = 1;
         if (want > n_tiles) want = n_tiles;

@@ -463,15 +463,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         const int slot = s & 1;
         uint8_t *kt = ring + slot * Geo::kSlot;
         const TileInfo i3 = load_info(s + 3);
-        if (!(p.dbg & 2)) k_stage(kcur, kt);
+        k_stage(kcur, kt);
         PKV_LDS_BARRIER();
-        if (!(p.dbg & 4)) softmax_stage(slot, kt);
+        softmax_stage(slot, kt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
         PKV_LDS_BARRIER();
-        if (!(p.dbg & 1)) dma_issue(slot, s + 2, i2);
+        dma_issue(slot, s + 2, i2);
         UnitPairs knext, vnext;
         parse(slot ^ 1, i1, knext, vnext);
-        if (!(p.dbg & 8)) v_stage(vcur);
+        v_stage(vcur);
         kcur = knext;
         vcur = vnext;
         i1 = i2; i2 = i3;
