@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip encode / unpack timing")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     return ap.parse_args()
 
 
@@ -135,6 +138,13 @@ def main():
                   + 2 * 2 * B * Hkv * Tw * 128 + 2 * 2 * B * Hq * 128)
 
     out = torch.empty_like(q)
+
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)           # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         ops.attn_decode(q, ke, ve, kw, vw, out=out, variant=args.variant)

@@ -134,7 +134,7 @@ __device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[
 }
 
 template <int G, int KW, int VW, bool BF>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) attn_dma_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 3, 4))) attn_dma_kernel(const AttnParams p) {
     using Geo = DmaGeom<KW, VW>;
     constexpr int ROWS = 3 * G;
     constexpr int NSETS = (ROWS + 15) / 16;

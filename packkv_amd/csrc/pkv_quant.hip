@@ -154,60 +154,356 @@ __global__ void dequantize_kernel(const uint8_t *__restrict__ codes, int H, int 
         make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-// ---- fused quantize + encode -------------------------------------------------------------
-// One workgroup per block, in ticket order.  The workgroup quantizes its tile of x straight
-// into the LDS code tile and then runs the same block encoder as the codes->stream kernel.
-template <bool IS_K, int DT>
-__global__ void quant_pack_kernel(const uint16_t *__restrict__ x, int H, int T,
-                                  const uint16_t *__restrict__ scale, const uint16_t *__restrict__ zero,
-                                  uint8_t *__restrict__ stream, uint64_t capacity,
-                                  uint32_t *__restrict__ info, ScanState *st, int hidden_dim, int ctx_blk,
-                                  int hid_blk, int nunits, int W, uint32_t nblocks) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    __shared__ uint32_t s_idx;
-    __shared__ uint64_t s_off;
-    __shared__ uint32_t unit_bytes[16];
-    uint8_t *tile = lds;
-    uint8_t *blk = lds + ((uint32_t)(ctx_blk * hid_blk + 15) & ~15u);
-    if (threadIdx.x == 0) s_idx = atomicAdd(&st->ticket, 1u);
-    __syncthreads();
-    const uint32_t bidx = s_idx;
-    if (bidx >= nblocks) return;
-    const int n_hid = hidden_dim / hid_blk;
-    const uint32_t cb = bidx / n_hid, hb = bidx % n_hid;
-    const uint32_t ch0 = hb * hid_blk;              // first channel of the block in [0, B*H*128)
-    const uint32_t bh = ch0 / kHeadDim;             // b * H + h
-    const uint32_t b = bh / H;
-    const uint32_t d0 = ch0 % kHeadDim;
-    const int lanes_per_row = hid_blk / 8;          // 8 channels per thread
-    const int rows_per_pass = blockDim.x / lanes_per_row;
-    const int lr = threadIdx.x % lanes_per_row;
-    uint32_t cmax = 0;
-    for (int r = threadIdx.x / lanes_per_row; r < ctx_blk; r += rows_per_pass) {
-        const size_t tok = (size_t)cb * ctx_blk + r;
-        const float sc = T16<DT>::from_bits(scale[(size_t)b * T + tok]);
-        const float z = T16<DT>::from_bits(zero[(size_t)b * T + tok]);
-        const uint4 v = *reinterpret_cast<const uint4 *>(
-            x + ((size_t)bh * T + tok) * kHeadDim + d0 + lr * 8);
+// ---- fused quantize + encode: the cell ---------------------------------------------------
+// 128 threads work on one block.  Thread = "cell": 16 tokens (one round) x 4 adjacent channels,
+// i.e. four packs.  The cell is loaded straight from x (8 bytes per token row, rows of a
+// half-wavefront contiguous), quantized and analysed in registers with packed 16-bit arithmetic;
+// no code tile is ever formed.
+//   K block (64 x 128):  cell (round r = tid / 32, channels 4t..4t+3, t = tid % 32) IS lane t of
+//                        unit r, so the packs are emitted where they were computed.
+//   V block (128 x 64):  cell (round r = tid / 16, channels 4g..4g+3, g = tid % 16); V units want
+//                        lane = channel with the packs of four consecutive rounds, so the pack
+//                        records change hands once through LDS.
+//
+// Exact division without the division sequence.  code = rint(T(x / scale)) - zero needs
+// h = RN16(RN32(x / scale)), which equals RN16(x / scale) (24 >= 2 * 11 + 2 bits: double rounding
+// is innocuous).  With r = 1 / scale refined to half an ulp once per token,
+//   q0 = x * r;  e = fma(-scale, q0, x);  q1 = fma(e, r, q0)
+// is within 2^-24 (1 + 2^-20) of the quotient, while a quotient of two 11-bit significands is
+// either exactly an fp16 rounding midpoint (then e is exact and q1 hits it exactly, so the tie is
+// broken as in the reference) or at least 2^-23 away from every midpoint; so RN16(q1) is the
+// reference's value.  bf16 inputs take the plain path (quant_code).
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+struct TokPar { float s, r; uint32_t neg_zero2, pad; };   // scale, 1 / scale, (-zero, -zero) as two fp16 (or zero as fp32 bits for bf16)
+
+__device__ __forceinline__ uint32_t pk_u16(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
+
+// codes of four adjacent channels of one token as two pairs of 16-bit integers
+template <int DT>
+__device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01, uint32_t &c23) {
+    if (DT == PKV_F16) {
+        const f16x2 x01 = __builtin_bit_cast(f16x2, xw.x), x23 = __builtin_bit_cast(f16x2, xw.y);
+        auto quot = [&](_Float16 xh) -> _Float16 {
+            const float f = (float)xh;
+            const float q0 = __fmul_rn(f, tp.r);
+            const float e = __fmaf_rn(-tp.s, q0, f);
+            return (_Float16)__fmaf_rn(e, tp.r, q0);
+        };
+        const f16x2 h01 = {quot(x01[0]), quot(x01[1])}, h23 = {quot(x23[0]), quot(x23[1])};
+        const f16x2 nz = __builtin_bit_cast(f16x2, tp.neg_zero2);
+        const f16x2 magic = {(_Float16)1024.f, (_Float16)1024.f};    // 1024 + c has c in its low mantissa bits
+        const f16x2 d01 = __builtin_elementwise_roundeven(h01) + nz, d23 = __builtin_elementwise_roundeven(h23) + nz;
+        c01 = __builtin_bit_cast(uint32_t, (f16x2)(d01 + magic)) & 0x00FF00FFu;
+        c23 = __builtin_bit_cast(uint32_t, (f16x2)(d23 + magic)) & 0x00FF00FFu;
+    } else {
+        const float z = __uint_as_float(tp.neg_zero2);
+        const uint32_t a = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.x & 0xFFFFu), tp.s, z) & 0xFFu;
+        const uint32_t b = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.x >> 16), tp.s, z) & 0xFFu;
+        const uint32_t c = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.y & 0xFFFFu), tp.s, z) & 0xFFu;
+        const uint32_t d = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.y >> 16), tp.s, z) & 0xFFu;
+        c01 = a | (b << 16);
+        c23 = c | (d << 16);
+    }
+}
+
+// bit_length of both 16-bit halves, clamped to 4 (values above 15 mean the codes overflow the
+// format; the launch reports that through max_code)
+__device__ __forceinline__ uint32_t pk_bitlen4(uint32_t d) {
+    const u16x2 v = as_u16x2(d), one = {1, 1};
+    const u16x2 l = __builtin_elementwise_min(v, one) + __builtin_elementwise_min((u16x2)(v >> 1), one) +
+                    __builtin_elementwise_min((u16x2)(v >> 2), one) + __builtin_elementwise_min((u16x2)(v >> 3), one);
+    return pk_u16(l);
+}
+
+// The two packs held in one register pair column: codes c[k] (k = token, two channels per word)
+// -> minima, widths and the two 64-bit pack words  sum (c_k - min) << ((15 - k) * len).
+__device__ __forceinline__ void build_pair(const uint32_t c[16], uint32_t &mn2, uint32_t &len2, uint32_t &mx2,
+                                           uint64_t &w_lo, uint64_t &w_hi) {
+    u16x2 mn = as_u16x2(c[0]), mx = as_u16x2(c[0]);
+#pragma unroll
+    for (int k = 1; k < 16; k++) {
+        mn = __builtin_elementwise_min(mn, as_u16x2(c[k]));
+        mx = __builtin_elementwise_max(mx, as_u16x2(c[k]));
+    }
+    mn2 = pk_u16(mn);
+    mx2 = pk_u16(mx);
+    len2 = pk_bitlen4(pk_u16((u16x2)(mx - mn)));
+    const u16x2 one = {1, 1};
+    const u16x2 p = one << as_u16x2(len2);                       // 2^len per half
+    // quarter windows (4 tokens, 4 * len <= 16 bits), all arithmetic modulo 2^16 per half:
+    //   sum c_k p^(3-k) - min (1 + p + p^2 + p^3)
+    const u16x2 rep = ((p + one) * p + one) * p + one;
+    const u16x2 mnrep = mn * rep;
+    uint32_t qw[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        u16x2 w = as_u16x2(c[4 * j]);
+        w = w * p + as_u16x2(c[4 * j + 1]);
+        w = w * p + as_u16x2(c[4 * j + 2]);
+        w = w * p + as_u16x2(c[4 * j + 3]);
+        qw[j] = pk_u16((u16x2)(w - mnrep));
+    }
+    // 64-bit words: tokens 0..7 above tokens 8..15
+    const uint32_t l0 = len2 & 0xFFFFu, l1 = len2 >> 16;
+    const uint32_t a0 = ((qw[0] & 0xFFFFu) << (4u * l0)) | (qw[1] & 0xFFFFu), b0 = ((qw[2] & 0xFFFFu) << (4u * l0)) | (qw[3] & 0xFFFFu);
+    const uint32_t a1 = ((qw[0] >> 16) << (4u * l1)) | (qw[1] >> 16), b1 = ((qw[2] >> 16) << (4u * l1)) | (qw[3] >> 16);
+    w_lo = ((uint64_t)a0 << (8u * l0)) | b0;
+    w_hi = ((uint64_t)a1 << (8u * l1)) | b1;
+}
+
+// running (min, max) of the 8 values of one 16-byte row chunk
+template <int DT>
+__device__ __forceinline__ void minmax8(const uint4 v, float &mn, float &mx) {
+    if (DT == PKV_F16) {   // packed fp16 comparisons, converted once
+        const f16x2 a = __builtin_bit_cast(f16x2, v.x), b = __builtin_bit_cast(f16x2, v.y), c = __builtin_bit_cast(f16x2, v.z),
+                    d = __builtin_bit_cast(f16x2, v.w);
+        const f16x2 lo = __builtin_elementwise_min(__builtin_elementwise_min(a, b), __builtin_elementwise_min(c, d));
+        const f16x2 hi = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        mn = fminf(mn, fminf((float)lo[0], (float)lo[1]));
+        mx = fmaxf(mx, fmaxf((float)hi[0], (float)hi[1]));
+    } else {
         float f[8];
         unpack8<DT>(v, f);
-        uint32_t lo = 0, hi = 0;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t c0 = (uint32_t)(int)quant_code<DT>(f[i], sc, z) & 0xFFu;
-            const uint32_t c1 = (uint32_t)(int)quant_code<DT>(f[4 + i], sc, z) & 0xFFu;
-            lo |= c0 << (8 * i);
-            hi |= c1 << (8 * i);
-            cmax = max(cmax, max(c0, c1));
+        for (int i = 0; i < 8; i++) {
+            mn = fminf(mn, f[i]);
+            mx = fmaxf(mx, f[i]);
         }
-        *reinterpret_cast<uint2 *>(tile + r * hid_blk + lr * 8) = make_uint2(lo, hi);
+    }
+}
+
+__device__ __forceinline__ void cell_load(const uint16_t *xc, uint2 xr[16]) {
+#pragma unroll
+    for (int k = 0; k < 16; k++) xr[k] = *reinterpret_cast<const uint2 *>(xc + (size_t)k * kHeadDim);
+}
+
+template <int DT>
+__device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
+    float r = __builtin_amdgcn_rcpf(sc);
+    r = __fmaf_rn(__fmaf_rn(-sc, r, 1.f), r, r);
+    TokPar tp;
+    tp.s = sc;
+    tp.r = r;
+    tp.neg_zero2 = DT == PKV_F16 ? ((zero_bits ^ 0x8000u) * 0x00010001u) : __float_as_uint(T16<DT>::from_bits(zero_bits));
+    tp.pad = 0;
+    return tp;
+}
+
+// The four packs of a loaded cell (rows xr, the 16 tokens' constants at par): words, minima, widths.
+template <int DT>
+__device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par, UnitPacks &u, uint32_t &cmax) {
+    uint32_t c01[16], c23[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+    uint32_t mn01, mn23, len01, len23, mx01, mx23;
+    build_pair(c01, mn01, len01, mx01, u.word[0], u.word[1]);
+    build_pair(c23, mn23, len23, mx23, u.word[2], u.word[3]);
+    const u16x2 m = __builtin_elementwise_max(as_u16x2(mx01), as_u16x2(mx23));
+    cmax = max((uint32_t)m[0], (uint32_t)m[1]);
+    u.mn[0] = mn01 & 0xFFFFu; u.mn[1] = mn01 >> 16; u.mn[2] = mn23 & 0xFFFFu; u.mn[3] = mn23 >> 16;
+    u.len[0] = len01 & 0xFFFFu; u.len[1] = len01 >> 16; u.len[2] = len23 & 0xFFFFu; u.len[3] = len23 >> 16;
+}
+
+// V blocks: a wavefront's 64 cells (round 4 sg + i, channels 4 g .. 4 g + 3; lane = 16 i + g) cover
+// one segment sg of the block; V units want lane c = channel c holding the packs of rounds
+// 4 sg .. 4 sg + 3.  The packs change lanes inside the wavefront through a 1 KiB LDS area
+// ([channel][round] dwords), one 32-bit field at a time.  LDS serves a wavefront's accesses in
+// order, so only the compiler needs fencing.
+__device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane) {
+    uint32_t *a = reinterpret_cast<uint32_t *>(area);
+    const int i = lane >> 4, g = lane & 15;
+    uint32_t f[3][4];
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) {
+        f[0][sl] = (uint32_t)u.word[sl];
+        f[1][sl] = (uint32_t)(u.word[sl] >> 32);
+        f[2][sl] = u.mn[sl] | (u.len[sl] << 8);
     }
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) cmax = max(cmax, __shfl_xor(cmax, d, 64));
-    if ((threadIdx.x & 63) == 0 && cmax >= (1u << W)) atomicMax(&st->max_code, cmax);
+    for (int kind = 0; kind < 3; kind++) {
+#pragma unroll
+        for (int sl = 0; sl < 4; sl++) a[(4 * g + sl) * 4 + i] = f[kind][sl];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint4 r = *reinterpret_cast<const uint4 *>(a + lane * 4);
+        f[kind][0] = r.x; f[kind][1] = r.y; f[kind][2] = r.z; f[kind][3] = r.w;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) {
+        u.word[sl] = ((uint64_t)f[1][sl] << 32) | f[0][sl];
+        u.mn[sl] = f[2][sl] & 0xFFu;
+        u.len[sl] = f[2][sl] >> 8;
+    }
+}
+
+// ---- fused parameters + quantize + encode, one workgroup per sub-group ---------------------
+// A group is the run of blocks that share one (context block, sequence): H blocks for K, 2 H for
+// V, consecutive in stream order; a sub-group is up to eight consecutive blocks of a group.  One
+// workgroup of 256 threads (two blocks at a time)
+//   1. reads the group's x for the per-token min / max over ALL heads (sub-groups of one group
+//      repeat this read; they run at the same time, so the repeats are served by the caches);
+//      the first sub-group writes scale / zero;
+//   2. re-reads its own blocks (cache-hot) cell by cell, quantizes and encodes them into LDS;
+//   3. obtains the sub-group's stream offset with ONE look-back (one ticket and one status word
+//      per sub-group) and writes its bytes, contiguous in the stream, in one sweep of aligned
+//      16-byte stores.
+// So x crosses HBM once, and the ordered-ticket / look-back traffic shrinks eightfold.
+constexpr int kSubBlocks = 8;
+
+template <bool IS_K, int DT>
+__global__ void __launch_bounds__(256) quant_encode_group_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t nsub, uint32_t bound) {
+    constexpr int CTX = IS_K ? 64 : 128;
+    extern __shared__ __align__(16) uint8_t gbuf[];        // the sub-group's encoded bytes (8 x block bound)
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t unit_bytes[2][4];
+    __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the sub-group
+    __shared__ __attribute__((aligned(16))) TokPar s_par[CTX];
+    const int tid = threadIdx.x;
+    const int HB = IS_K ? H : 2 * H;                      // blocks per group
+    const int SG = (HB + kSubBlocks - 1) / kSubBlocks;    // sub-groups per group
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    block_finish<IS_K>(tile, blk, unit_bytes, &s_off, st, bidx, nblocks, stream, capacity, info, hid_blk,
-                       nunits, W);
+    const uint32_t sidx = s_idx;
+    if (sidx >= nsub) return;
+    const uint32_t gidx = sidx / (uint32_t)SG, sg = sidx % (uint32_t)SG;
+    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * CTX;
+    const int jbase = (int)sg * kSubBlocks;               // first block of the sub-group inside the group
+    const int nb = min(kSubBlocks, HB - jbase);
+
+    // ---- 1. per-token parameters: 16 lanes x 8 channels per token, all heads ----
+    for (int tt = tid >> 4; tt < CTX; tt += 16) {
+        const int l16 = tid & 15;
+        float mn = INFINITY, mx = -INFINITY;
+        // eight rows in flight at a time (head indices clamped: a repeated row changes no min / max)
+        for (int h0 = 0; h0 < H; h0 += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                v[i] = *reinterpret_cast<const uint4 *>(
+                    x + (((size_t)b * H + min(h0 + i, H - 1)) * T + tok0 + tt) * kHeadDim + l16 * 8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+        }
+#pragma unroll
+        for (int d = 8; d >= 1; d >>= 1) {
+            mn = fminf(mn, __shfl_xor(mn, d, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, d, 16));
+        }
+        if (l16 == 0) {
+            const float range = round_t<DT>(mx - mn);
+            const float sc = round_t<DT>(range * rel);
+            const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+            if (sg == 0) {
+                scale[(size_t)b * T + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[(size_t)b * T + tok0 + tt] = (uint16_t)zb;
+            }
+            s_par[tt] = token_par<DT>(sc, zb);
+        }
+    }
+    if (tid == 0) blk_off[0] = 0;
+    __syncthreads();
+
+    // ---- 2. encode, two blocks at a time ----
+    const UnitGeom g = unit_geom(W);
+    const int jl = tid >> 7, ct = tid & 127;             // local block, cell
+    const int round = IS_K ? ct >> 5 : ct >> 4;
+    const int cgrp = IS_K ? ct & 31 : ct & 15;
+    const int unit = IS_K ? ct >> 5 : 2 * ((ct >> 5) & 1) + (ct >> 6);
+    const int t = tid & 31;
+    uint32_t cmax_all = 0;
+    for (int j0 = 0; j0 < nb; j0 += 2) {
+        const int jj = j0 + jl;                           // block inside the sub-group
+        const bool active = jj < nb;
+        const int j = jbase + min(jj, nb - 1);            // block inside the group (clamped: loads are unconditional)
+        const int h = IS_K ? j : j >> 1, d0 = IS_K ? 0 : (j & 1) * 64;
+        uint2 xr[16];
+        cell_load(x + (((size_t)b * H + h) * T + tok0 + 16 * round) * kHeadDim + d0 + 4 * cgrp, xr);
+        UnitPacks u;
+        uint32_t cmax;
+        cell_packs<DT>(xr, s_par + 16 * round, u, cmax);
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            // V: the exchange area (1 KiB per wavefront) sits in the block's own worst-case slot,
+            // which lies behind everything encoded so far
+            if (!IS_K) v_exchange(u, gbuf + (((size_t)jj * bound + 15) & ~(size_t)15) + ((tid >> 6) & 1) * 1024, tid & 63);
+            pack_offsets(u.len, u.off, u.payload);
+            if (t == 0) unit_bytes[jl][unit] = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        }
+        __syncthreads();
+        if (tid == 0) {                                   // block sizes of this pair -> offsets inside the sub-group
+            uint32_t off = blk_off[j0];
+            off += 8u + unit_bytes[0][0] + unit_bytes[0][1] + unit_bytes[0][2] + unit_bytes[0][3];
+            blk_off[j0 + 1] = off;
+            if (j0 + 1 < nb) blk_off[j0 + 2] = off + 8u + unit_bytes[1][0] + unit_bytes[1][1] + unit_bytes[1][2] + unit_bytes[1][3];
+        }
+        __syncthreads();
+        if (active) {
+            uint8_t *blk = gbuf + blk_off[jj];
+            uint32_t base = 8u;
+#pragma unroll
+            for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
+            if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
+            unit_emit(blk, base, t, g, u);
+        }
+        __syncthreads();
+    }
+    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+
+    // ---- 3. one look-back for the whole sub-group, then one contiguous copy ----
+    const uint32_t bytes = blk_off[nb];
+    if (tid < 64) {
+        const uint64_t off = lookback_offset(st, sidx, bytes);
+        if (tid == 0) {
+            s_off = off;
+            if (sidx == nsub - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < nb) {
+        const uint32_t first = cb * (uint32_t)(B * HB) + b * (uint32_t)HB + (uint32_t)jbase;   // stream index of the first block
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    // head (to the first 16-byte boundary of the stream) and tail in 2-byte pieces, the body as
+    // aligned 16-byte stores fed by aligned LDS reads and byte funnel shifts
+    uint8_t *dst = stream + off;
+    const uint32_t head = min(bytes, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
+    const uint32_t nq = (bytes - head) >> 4;
+    for (uint32_t i = tid; i < (head >> 1); i += 256)
+        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(gbuf)[i];
+    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(gbuf + (head & ~3u));
+    for (uint32_t i = tid; i < nq; i += 256) {
+        const uint32_t *q = src32 + 4 * i;
+        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+        uint4 v;
+        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
+        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
+        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
+        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+        *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
+    }
+    const uint32_t done = head + 16u * nq;
+    for (uint32_t i = tid; i < ((bytes - done) >> 1); i += 256)
+        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(gbuf + done)[i];
 }
 
 static int check_xshape(const void *x, int dtype, int B, int H, int T) {
@@ -230,32 +526,28 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
-    const int hidden = B * H * kHeadDim;
-    const int nunits = 4;
-    const uint32_t nblocks = (uint32_t)(T / ctx_blk) * (uint32_t)(hidden / hid_blk);
-    const uint32_t cap = IS_K ? (uint32_t)k_block_bound(ctx_blk, bits) : (uint32_t)v_block_bound(hid_blk, bits);
-    const uint32_t lds_bytes = (uint32_t)(ctx_blk * hid_blk) + ((cap + 15u) & ~15u) + 32u;
     ScanState *st = nullptr;
-    if ((rc = prepare_scan_state(nblocks, &st, s))) return rc;
-    LaunchTimer tm(s, ms_out != nullptr);
-    if ((rc = tm.begin())) return rc;
-    const dim3 pgrid((unsigned)((T + 15) / 16), (unsigned)B);
-    if (dtype == PKV_F16) {
-        quant_params_kernel<PKV_F16><<<pgrid, 256, 0, s>>>((const uint16_t *)x, H, T, rel, (uint16_t *)scale,
-                                                           (uint16_t *)zero);
-        quant_pack_kernel<IS_K, PKV_F16><<<nblocks, 128, lds_bytes, s>>>(
-            (const uint16_t *)x, H, T, (const uint16_t *)scale, (const uint16_t *)zero, stream, capacity, info,
-            st, hidden, ctx_blk, hid_blk, nunits, bits, nblocks);
-    } else {
-        quant_params_kernel<PKV_BF16><<<pgrid, 256, 0, s>>>((const uint16_t *)x, H, T, rel, (uint16_t *)scale,
-                                                            (uint16_t *)zero);
-        quant_pack_kernel<IS_K, PKV_BF16><<<nblocks, 128, lds_bytes, s>>>(
-            (const uint16_t *)x, H, T, (const uint16_t *)scale, (const uint16_t *)zero, stream, capacity, info,
-            st, hidden, ctx_blk, hid_blk, nunits, bits, nblocks);
+    // One workgroup per sub-group of up to eight consecutive blocks that share (context block, sequence).
+    {
+        const int HB = IS_K ? H : 2 * H;
+        const uint32_t bound = IS_K ? (uint32_t)k_block_bound(ctx_blk, bits) : (uint32_t)v_block_bound(hid_blk, bits);
+        const uint32_t gbytes = (uint32_t)kSubBlocks * bound + 32u;
+        const uint32_t nsub = (uint32_t)(T / ctx_blk) * (uint32_t)B * (uint32_t)((HB + kSubBlocks - 1) / kSubBlocks);
+        if ((rc = prepare_scan_state(nsub, &st, s))) return rc;
+        LaunchTimer tm(s, ms_out != nullptr);
+        if ((rc = tm.begin())) return rc;
+        if (dtype == PKV_F16)
+            quant_encode_group_kernel<IS_K, PKV_F16><<<nsub, 256, gbytes, s>>>(
+                (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
+                bits, nsub, bound);
+        else
+            quant_encode_group_kernel<IS_K, PKV_BF16><<<nsub, 256, gbytes, s>>>(
+                (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
+                bits, nsub, bound);
+        PKV_HIP_CHECK(hipGetLastError());
+        if ((rc = tm.end(ms_out))) return rc;
+        return finish_encode(st, size_out, bits, s);
     }
-    PKV_HIP_CHECK(hipGetLastError());
-    if ((rc = tm.end(ms_out))) return rc;
-    return finish_encode(st, size_out, bits, s);
 }
 
 }  // namespace pkv

@@ -37,7 +37,8 @@ def test_quantizer_bit_exact(cuda, dtype, rel):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
-    for (B, H, T, rel) in ((1, 2, 128, 0.1), (2, 8, 256, 0.1), (1, 32, 128, 0.1), (2, 4, 256, 0.2), (1, 8, 128, 0.34)):
+    for (B, H, T, rel) in ((1, 2, 128, 0.1), (2, 8, 256, 0.1), (1, 32, 128, 0.1), (2, 4, 256, 0.2), (1, 8, 128, 0.34),
+                           (1, 3, 128, 0.1), (2, 5, 256, 0.14), (3, 1, 128, 0.1)):
         k, v = synth.make_kv(B, H, T, seed=31 + H, dtype=dtype)
         for is_k, x in ((1, k), (0, v)):
             _say("fused quant+encode", "K" if is_k else "V", dtype, B, H, T, rel)
@@ -60,3 +61,23 @@ def test_code_wider_than_bits_is_reported(cuda):
     with pytest.raises(ops.PackKVError) as e:
         ops.k_quant_encode(k.to(cuda), 0.1, 3)     # codes reach 10..11: needs 4 bits
     assert e.value.code == 1 and "does not fit" in str(e.value)
+
+
+@pytest.mark.gpu
+def test_fused_quant_encode_round_trip_medium(cuda):
+    """Size-independent property at a size the CPU oracle would take minutes for: unpacking the fused
+    encoder's stream gives back exactly the codes of the stand-alone quantizer."""
+    B, H, T, rel = 4, 8, 4096, 0.1
+    k, v = synth.make_kv(B, H, T, seed=77)
+    for is_k, x in ((True, k), (False, v)):
+        x = x.to(cuda)
+        r = (ops.k_quant_encode if is_k else ops.v_quant_encode)(x, rel, 4)
+        scale, zero = ops.quant_params(x, rel)
+        assert torch.equal(scale, r["scale"]) and torch.equal(zero, r["zero"])
+        codes, _ = ops.quantize(x, scale, zero)
+        back = torch.empty_like(codes)
+        if is_k:
+            ops.k_decode(r["stream"], r["info"], back, 64, 128, 4)
+        else:
+            ops.v_decode(r["stream"], r["info"], back, 128, 64, 4)
+        assert torch.equal(back, codes)
