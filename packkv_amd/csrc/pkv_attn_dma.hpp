@@ -147,11 +147,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
     static_assert(16 * NSETS * 16 * 4 + 64 <= kRoundBytes, "score rows must fit the K-tile rows they reuse");
     static_assert(NSETS * 4 * 16 * 32 <= 8 * kRoundBytes, "q digits borrow a slot");
 
-    constexpr int kLdsBytes = 2 * Geo::kSlot + GP * kTile * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
+    constexpr int kPStride = kTile + 4;          // halves per head row of the weights: rows 8 bytes apart in bank space
+    constexpr int kLdsBytes = 2 * Geo::kSlot + GP * kPStride * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLdsBytes];
     uint8_t *ring = smem;                                                    // [2 slots][4 block regions | parameters]
-    _Float16 *pbuf = reinterpret_cast<_Float16 *>(smem + 2 * Geo::kSlot);    // [GP][128]
-    _Float16 *p16hi = pbuf + GP * kTile;                                     // [GP][8]
+    _Float16 *pbuf = reinterpret_cast<_Float16 *>(smem + 2 * Geo::kSlot);    // [GP][128 + 4]
+    _Float16 *p16hi = pbuf + GP * kPStride;                                     // [GP][8]
     _Float16 *p16lo = p16hi + GP * 8;
     float *st_m = reinterpret_cast<float *>(p16lo + GP * 8);                 // 8 floats each
     float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8, *qsum = st_z + 8, *qs = qsum + 8;
@@ -172,7 +173,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 
     // ---- prologue: split q into digits (through LDS, aliased onto the K tile) ----
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
-    for (int i = tid; i < GP * kTile / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
+    for (int i = tid; i < GP * kPStride / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
     for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
     if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 1.f; }
     __syncthreads();
@@ -348,15 +349,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 #pragma unroll
                 for (int sl = 0; sl < 4; sl++) d = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[s][sl], bop[sl], d, 0, 0, 0);
                 // row-major [m][token]; odd rounds sit 16 banks further so the softmax reads spread over all banks
+                // (the four rows one instruction writes, m = 4 (lane / 16) + jj, are stored as 4 jj + lane / 16:
+                // adjacent, so they alternate between the two halves of the banks)
                 int32_t *o = reinterpret_cast<int32_t *>(kt + R * kRoundBytes + (R & 1) * 64) +
-                             (s * 16 + 4 * (lane >> 4)) * 16 + (lane & 15);
+                             (s * 16 + (lane >> 4)) * 16 + (lane & 15);
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) o[jj * 16] = d[jj];
+                for (int jj = 0; jj < 4; jj++) o[jj * 64] = d[jj];
             }
         }
     };
 
     // ---- stage 2: online softmax; wave <-> query head, lane <-> tokens 2*lane, 2*lane+1 ----
+    auto score_row = [](int m) -> int { return (m & ~15) | ((m & 3) << 2) | ((m >> 2) & 3); };   // where row m of the scores is stored
     auto softmax_stage = [&](int slot, const uint8_t *kt) {
         const uint32_t *par = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff) + lane;
         float ks0, ks1, kz0, kz1, vs0, vs1, vz0, vz1;
@@ -370,7 +374,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
                 float sv[2];
 #pragma unroll
                 for (int e = 0; e < 2; e++) {
-                    const float d0 = (float)r[g * 16 + e], d1 = (float)r[(G + g) * 16 + e], d2 = (float)r[(2 * G + g) * 16 + e];
+                    const float d0 = (float)r[score_row(g) * 16 + e], d1 = (float)r[score_row(G + g) * 16 + e],
+                                d2 = (float)r[score_row(2 * G + g) * 16 + e];
                     const float dot = qs_r[gi] * (d0 * 16384.f + d1 * 128.f + d2);
                     sv[e] = p.sm_scale * (e ? ks1 : ks0) * (dot + (e ? kz1 : kz0) * qsum_r[gi]);
                 }
@@ -383,7 +388,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
                 const float f0 = (float)h0, f1 = (float)h1;
                 // V-side order: MFMA k of a segment contracts token k of its four rounds
                 const int tok0 = 2 * lane;
-                _Float16 *pb = pbuf + g * kTile + (tok0 & 64) + ((tok0 & 15) << 2) + ((tok0 >> 4) & 3);
+                _Float16 *pb = pbuf + g * kPStride + (tok0 & 64) + ((tok0 & 15) << 2) + ((tok0 >> 4) & 3);
                 pb[0] = h0;
                 pb[4] = h1;      // token 2*lane+1: same round, next k
                 l_part[gi] = l_part[gi] * alpha + (p0 + p1);
@@ -441,7 +446,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
                 const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
 #pragma unroll
                 for (int i4 = 0; i4 < NG4; i4++) {
-                    const half4v aopv = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kTile + 64 * seg + 4 * (4 * q + pp));
+                    const half4v aopv = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kPStride + 64 * seg + 4 * (4 * q + pp));
                     acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(aopv, bop, acc[i4], 0, 0, 0);
                 }
             }
@@ -464,18 +469,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
         uint8_t *kt = ring + slot * Geo::kSlot;
         const TileInfo i3 = load_info(s + 3);
         k_stage(kcur, kt);
-        PKV_LDS_BARRIER();
-        softmax_stage(slot, kt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
-        PKV_LDS_BARRIER();
-        dma_issue(slot, s + 2, i2);
+        PKV_LDS_BARRIER();                                    // publishes the scores and tile s+1
         UnitPairs knext, vnext;
         parse(slot ^ 1, i1, knext, vnext);
+        softmax_stage(slot, kt);
+        PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile s+1 is parsed
+        dma_issue(slot, s + 2, i2);
         v_stage(vcur);
         kcur = knext;
         vcur = vnext;
         i1 = i2; i2 = i3;
-        PKV_LDS_BARRIER();
     }
     // drain: the copy issued in the last step must land before the workgroup's LDS is released
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
