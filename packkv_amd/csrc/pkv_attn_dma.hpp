@@ -406,6 +406,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
     };
 
     // ---- stage 3: V segment hw; lane = channel, MFMA k contracts token k of the lane's four packs ----
+    // A operands of the V-side MFMAs (4 heads x 4 tokens of weights): every block of 4 lanes wants
+    // the same values, so only lanes 0..3 of each half-wavefront read them from LDS and the MFMA
+    // broadcasts block 0 of each group of 8 blocks (cbsz = 3, abid = 0).  The other lanes' copies
+    // are never read; they stay at their initial zero.
+    half4v a_w[4][NG4], a_hi[NG4], a_lo[NG4];
+#pragma unroll
+    for (int i4 = 0; i4 < NG4; i4++) {
+        a_hi[i4] = a_lo[i4] = (half4v){0, 0, 0, 0};
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) a_w[pp][i4] = (half4v){0, 0, 0, 0};
+    }
+    const bool a_loader = (lane & 31) < 4;
     auto v_stage = [&](const UnitPairs &vr) {
         const int seg = hw & 1;
         uint32_t w01[4], w23[4];
@@ -430,25 +442,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
         // pack minima: raw bits are the same fp16-subnormal encoding as the fields
         const half4v mins = __builtin_bit_cast(half4v, make_uint2(__builtin_amdgcn_perm(0u, vr.mins, 0x0C010C00u),
                                                                   __builtin_amdgcn_perm(0u, vr.mins, 0x0C030C02u)));
+        if (a_loader) {
+#pragma unroll
+            for (int i4 = 0; i4 < NG4; i4++) {
+                a_hi[i4] = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
+                a_lo[i4] = *reinterpret_cast<const half4v *>(p16lo + (4 * i4 + gl) * 8 + 4 * seg);
+            }
+        }
 #pragma unroll
         for (int i4 = 0; i4 < NG4; i4++) {
-            const half4v ahi = *reinterpret_cast<const half4v *>(p16hi + (4 * i4 + gl) * 8 + 4 * seg);
-            const half4v alo = *reinterpret_cast<const half4v *>(p16lo + (4 * i4 + gl) * 8 + 4 * seg);
-            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(ahi, mins, acc[i4], 0, 0, 0);
-            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(alo, mins, acc[i4], 0, 0, 0);
+            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(a_hi[i4], mins, acc[i4], 3, 0, 0);
+            acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(a_lo[i4], mins, acc[i4], 3, 0, 0);
         }
 #pragma unroll
         for (int q = 0; q < 4; q++) {
+            if (a_loader) {
+#pragma unroll
+                for (int pp = 0; pp < 4; pp++)
+#pragma unroll
+                    for (int i4 = 0; i4 < NG4; i4++)
+                        a_w[pp][i4] = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kPStride + 64 * seg + 4 * (4 * q + pp));
+            }
 #pragma unroll
             for (int pp = 0; pp < 4; pp++) {
                 const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
                 const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
                 const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
 #pragma unroll
-                for (int i4 = 0; i4 < NG4; i4++) {
-                    const half4v aopv = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kPStride + 64 * seg + 4 * (4 * q + pp));
-                    acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(aopv, bop, acc[i4], 0, 0, 0);
-                }
+                for (int i4 = 0; i4 < NG4; i4++)
+                    acc[i4] = __builtin_amdgcn_mfma_f32_4x4x4f16(a_w[pp][i4], bop, acc[i4], 3, 0, 0);
             }
         }
     };
