@@ -506,6 +506,135 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
         reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(gbuf + done)[i];
 }
 
+// ---- K, all heads in one workgroup: round-major single trip over x --------------------------
+// For H <= 8 the eight blocks of a (context block, sequence) group are the eight heads, so one
+// workgroup of 256 threads (head j = tid / 32, lane t = tid % 32) can go through the group ROUND BY
+// ROUND (16 tokens): read the round's rows of all heads for the token parameters (32 KiB per
+// workgroup), then at once re-read them as cells -- the lines are still in L2 -- quantize, and emit
+// unit `round` of every block behind the units already there.  x therefore crosses HBM once.
+// Blocks sit in worst-case slots in LDS and are compacted by the final copy.
+template <int DT>
+__global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound) {
+    extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the group's bytes
+    __shared__ __attribute__((aligned(16))) TokPar s_par[16];
+    const int tid = threadIdx.x;
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = s_idx;
+    if (gidx >= ngroups) return;
+    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * 64;
+    const UnitGeom g = unit_geom(W);
+    const int j = tid >> 5, t = tid & 31;                 // block (= head) and lane of the unit
+    const bool active = j < H;
+    const int jc = min(j, H - 1);
+    uint8_t *blk = gbuf + (size_t)j * bound;
+    uint32_t my_off = 8u;                                 // bytes of this block so far (uniform per half-wavefront)
+    uint32_t cmax_all = 0;
+    for (int r = 0; r < 4; r++) {
+        // token parameters of the round: 16 lanes x 8 channels per token, all heads
+        {
+            const int tt = tid >> 4, l16 = tid & 15;
+            float mn = INFINITY, mx = -INFINITY;
+            uint4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                v[i] = *reinterpret_cast<const uint4 *>(
+                    x + (((size_t)b * H + min(i, H - 1)) * T + tok0 + 16 * r + tt) * kHeadDim + l16 * 8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+#pragma unroll
+            for (int d = 8; d >= 1; d >>= 1) {
+                mn = fminf(mn, __shfl_xor(mn, d, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, d, 16));
+            }
+            if (l16 == 0) {
+                const float range = round_t<DT>(mx - mn);
+                const float sc = round_t<DT>(range * rel);
+                const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+                scale[(size_t)b * T + tok0 + 16 * r + tt] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[(size_t)b * T + tok0 + 16 * r + tt] = (uint16_t)zb;
+                s_par[tt] = token_par<DT>(sc, zb);
+            }
+        }
+        // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
+        uint2 xr[16];
+        cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
+        __syncthreads();
+        UnitPacks u;
+        uint32_t cmax;
+        cell_packs<DT>(xr, s_par, u, cmax);
+        __syncthreads();                                  // s_par is rewritten by the next round
+        pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+            if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
+            unit_emit(blk, my_off, t, g, u);
+            my_off += usz;
+        }
+    }
+    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+    if (active && t == 0) blk_off[j + 1] = my_off;          // sizes first ...
+    if (tid == 0) blk_off[0] = 0;
+    __syncthreads();
+    if (tid == 0)                                           // ... then their running sum
+        for (int q = 1; q <= H; q++) blk_off[q] += blk_off[q - 1];
+    __syncthreads();
+    const uint32_t bytes = blk_off[H];
+    if (tid < 64) {
+        const uint64_t off = lookback_offset(st, gidx, bytes);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < H) {
+        const uint32_t first = cb * (uint32_t)(B * H) + b * (uint32_t)H;
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    // each half-wavefront copies its own block: head to the first 16-byte boundary of the stream
+    // and tail in 2-byte pieces, the body as aligned 16-byte stores fed by aligned LDS reads and
+    // byte funnel shifts
+    if (active) {
+        uint8_t *dst = stream + off + blk_off[j];
+        const uint32_t nbytes = my_off;
+        const uint32_t head = min(nbytes, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
+        const uint32_t nq = (nbytes - head) >> 4;
+        for (uint32_t i = t; i < (head >> 1); i += 32)
+            reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(blk)[i];
+        const uint32_t *src32 = reinterpret_cast<const uint32_t *>(blk + (head & ~3u));
+        for (uint32_t i = t; i < nq; i += 32) {
+            const uint32_t *q = src32 + 4 * i;
+            const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+            uint4 v;
+            v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
+            v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
+            v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
+            v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+            *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
+        }
+        const uint32_t done = head + 16u * nq;
+        for (uint32_t i = t; i < ((nbytes - done) >> 1); i += 32)
+            reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(blk + done)[i];
+    }
+}
+
 static int check_xshape(const void *x, int dtype, int B, int H, int T) {
     PKV_REQUIRE(x != nullptr, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(dtype == PKV_F16 || dtype == PKV_BF16, PKV_ERR_UNSUPPORTED, "Unsupported data type");
@@ -536,7 +665,18 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
         if ((rc = prepare_scan_state(nsub, &st, s))) return rc;
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
-        if (dtype == PKV_F16)
+        if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
+            const uint32_t slot = (bound + 15u) & ~15u;
+            const uint32_t lds = (uint32_t)H * slot + 32u;
+            if (dtype == PKV_F16)
+                k_quant_encode_rounds_kernel<PKV_F16><<<nsub, 256, lds, s>>>(
+                    (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
+                    bits, nsub, slot);
+            else
+                k_quant_encode_rounds_kernel<PKV_BF16><<<nsub, 256, lds, s>>>(
+                    (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
+                    bits, nsub, slot);
+        } else if (dtype == PKV_F16)
             quant_encode_group_kernel<IS_K, PKV_F16><<<nsub, 256, gbytes, s>>>(
                 (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
                 bits, nsub, bound);
