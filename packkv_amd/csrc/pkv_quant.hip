@@ -382,7 +382,32 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     const int jbase = (int)sg * kSubBlocks;               // first block of the sub-group inside the group
     const int nb = min(kSubBlocks, HB - jbase);
 
-    // ---- 1. per-token parameters: 16 lanes x 8 channels per token, all heads ----
+    // ---- 1. per-token parameters ----
+    // Sub-group 0 of a group computes them (16 lanes x 8 channels per token, all heads) and
+    // publishes each token's (scale, zero) as ONE 64-bit word (valid bit | scale | zero) behind the
+    // status words -- single relaxed agent-scope atomics like the look-back, no fence, so no cache
+    // write-back.  Later sub-groups of the group, whose tickets are younger (so sub-group 0 is
+    // already running and never waits for them), poll those words instead of reading all heads
+    // again.  A wait that expires falls back to computing.
+    uint64_t *tokw = st->status + nsub + ((size_t)b * T + tok0);
+    __shared__ int s_miss;
+    if (tid == 0) s_miss = 0;
+    __syncthreads();
+    if (sg != 0) {
+        if (tid < CTX) {
+            uint64_t w = __hip_atomic_load(tokw + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int spins = 0;
+            while ((w >> 63) == 0 && spins < kSpinLimit) {
+                __builtin_amdgcn_s_sleep(16);
+                w = __hip_atomic_load(tokw + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                spins++;
+            }
+            if ((w >> 63) == 0) s_miss = 1;
+            else s_par[tid] = token_par<DT>(T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu), (uint32_t)w & 0xFFFFu);
+        }
+        __syncthreads();
+    }
+    if (sg == 0 || s_miss)
     for (int tt = tid >> 4; tt < CTX; tt += 16) {
         const int l16 = tid & 15;
         float mn = INFINITY, mx = -INFINITY;
@@ -408,6 +433,9 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
             if (sg == 0) {
                 scale[(size_t)b * T + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
                 zero[(size_t)b * T + tok0 + tt] = (uint16_t)zb;
+                if (SG > 1)
+                    __hip_atomic_store(tokw + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(sc) << 16) | (uint64_t)zb,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             s_par[tt] = token_par<DT>(sc, zb);
         }
@@ -662,7 +690,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
         const uint32_t bound = IS_K ? (uint32_t)k_block_bound(ctx_blk, bits) : (uint32_t)v_block_bound(hid_blk, bits);
         const uint32_t gbytes = (uint32_t)kSubBlocks * bound + 32u;
         const uint32_t nsub = (uint32_t)(T / ctx_blk) * (uint32_t)B * (uint32_t)((HB + kSubBlocks - 1) / kSubBlocks);
-        if ((rc = prepare_scan_state(nsub, &st, s))) return rc;
+        const bool shared_params = (HB > kSubBlocks);            // sub-groups of a group hand the token parameters on
+        PKV_REQUIRE((uint64_t)nsub + (uint64_t)B * (uint64_t)T < (1ull << 31), PKV_ERR_UNSUPPORTED, "batch x tokens too large");
+        if ((rc = prepare_scan_state(nsub + (shared_params ? (uint32_t)B * (uint32_t)T : 0u), &st, s))) return rc;   // status words, then one word per token
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
         if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
