@@ -11,12 +11,11 @@
 //
 // Step s of the pipeline (slot = s & 1 holds tile s, already parsed into registers):
 //   K stage      packs -> int8 K tile, written OVER the block bytes of slot s (dead once parsed),
-//                scores on the matrix cores                                        | barrier 1
-//   softmax      reads scores and the slot's parameters; then wait for the copy of tile s+1
-//                                                                                  | barrier 2
-//   issue the copy of tile s+2 into slot s;  V stage of tile s  together with the parse of
-//   tile s+1 out of the other slot                                                 | barrier 3
-// so a copy has a whole step to land and a tile's LDS round trips hide behind the V arithmetic.
+//                scores on the matrix cores; then wait for this wave's share of the copy of
+//                tile s+1                                                           | barrier 1
+//   softmax      reads scores and the slot's parameters, together with the parse of tile s+1
+//                out of the other slot                                              | barrier 2
+//   issue the copy of tile s+2 into slot s (its scores and parameters are consumed); V stage.
 // LDS per workgroup is 2 slots + 2 KiB: four workgroups fit a CU.
 //
 // Ordering.  The copies are issued from inline assembly, so the compiler neither sees them nor
@@ -25,7 +24,6 @@
 // s_barrier with an LDS-only wait: a workgroup fence would also drain the copies in flight.
 // The slots sit at the bottom of LDS, below 64 KiB.
 #pragma once
-#include <type_traits>
 
 namespace pkv {
 
