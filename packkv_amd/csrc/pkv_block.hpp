@@ -86,23 +86,52 @@ __device__ __forceinline__ void unit_parse2(const uint8_t *blk_a, uint32_t off_a
 }
 
 // Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
+// The four pack words are cut into 16-bit windows of four tokens (packs 0|1 and 2|3 share a
+// register), so one packed 16-bit shift moves two packs at a time and a byte permute gathers the
+// four codes of a token: 5 instructions per four codes instead of a 64-bit shift per code.
 template <bool IS_K>
 __device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,
                                             const UnitGeom g, uint8_t *tile, int hid_blk) {
+    typedef unsigned short u16pair __attribute__((ext_vector_type(2)));
     UnitPacks u;
     unit_parse(blk, unit_off, t, g, u);
+    uint32_t hlf[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t len = u.len[i];
-        const uint64_t mask = (1ull << len) - 1ull;
+        hlf[i][0] = (uint32_t)(u.word[i] >> (8u * u.len[i]));   // tokens 0..7
+        hlf[i][1] = (uint32_t)u.word[i];                        // tokens 8..15
+    }
+    const uint32_t len01 = u.len[0] | (u.len[1] << 16), len23 = u.len[2] | (u.len[3] << 16);
+    const uint32_t mq = ((1u << u.len[0]) - 1u) | (((1u << u.len[1]) - 1u) << 8) | (((1u << u.len[2]) - 1u) << 16) |
+                        (((1u << u.len[3]) - 1u) << 24);
+    const uint32_t minq = u.mn[0] | (u.mn[1] << 8) | (u.mn[2] << 16) | (u.mn[3] << 24);
 #pragma unroll
-        for (int k = 0; k < kPackTok; k++) {
-            const uint32_t c = (uint32_t)((u.word[i] >> ((15 - k) * len)) & mask) + u.mn[i];
-            tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] = (uint8_t)c;
+    for (int q = 0; q < 4; q++) {
+        uint32_t qd[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t src = hlf[i][q >> 1];
+            qd[i] = (q & 1) ? src : (src >> (4u * u.len[i]));
+        }
+        const uint32_t w01 = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);   // tokens 4q..4q+3 of packs 0 | 1
+        const uint32_t w23 = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) {
+            const int k = 4 * q + pp;
+            const u16pair s01 = __builtin_bit_cast(u16pair, len01 * (uint32_t)(3 - pp));
+            const u16pair s23 = __builtin_bit_cast(u16pair, len23 * (uint32_t)(3 - pp));
+            const uint32_t x01 = __builtin_bit_cast(uint32_t, (u16pair)(__builtin_bit_cast(u16pair, w01) >> s01));
+            const uint32_t x23 = __builtin_bit_cast(uint32_t, (u16pair)(__builtin_bit_cast(u16pair, w23) >> s23));
+            const uint32_t c4 = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + minq;   // codes of slots 0..3
+            if (IS_K) {   // slots are the four adjacent channels 4t..4t+3 of token k
+                *reinterpret_cast<uint32_t *>(tile + tile_index<true>(unit, 0, k, t, hid_blk)) = c4;
+            } else {      // slots are four rounds of channel t
+#pragma unroll
+                for (int i = 0; i < 4; i++) tile[tile_index<false>(unit, i, k, t, hid_blk)] = (uint8_t)(c4 >> (8 * i));
+            }
         }
     }
 }
-
 
 // Gather lane t's four packs of `unit` from the LDS code tile and compute min / len / word
 // and the payload offsets (one 32-lane exclusive scan per slot).
