@@ -309,12 +309,13 @@ __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par
 
 // V blocks: a wavefront's 64 cells (round 4 sg + i, channels 4 g .. 4 g + 3; lane = 16 i + g) cover
 // one segment sg of the block; V units want lane c = channel c holding the packs of rounds
-// 4 sg .. 4 sg + 3.  The packs change lanes inside the wavefront through a 1 KiB LDS area
-// ([channel][round] dwords), one 32-bit field at a time.  LDS serves a wavefront's accesses in
-// order, so only the compiler needs fencing.
+// 4 sg .. 4 sg + 3.  The packs change lanes inside the wavefront through a 1 KiB LDS area, one
+// 32-bit field at a time: every lane stores its four channels as one 16-byte word (area[lane][slot]
+// = area[round i][channel 4 g + slot]), then lane c reads area[i][c] for i = 0..3 -- both sides
+// touch consecutive dwords, no bank conflicts.  LDS serves a wavefront's accesses in order, so
+// only the compiler needs fencing.
 __device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane) {
     uint32_t *a = reinterpret_cast<uint32_t *>(area);
-    const int i = lane >> 4, g = lane & 15;
     uint32_t f[3][4];
 #pragma unroll
     for (int sl = 0; sl < 4; sl++) {
@@ -324,13 +325,12 @@ __device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane
     }
 #pragma unroll
     for (int kind = 0; kind < 3; kind++) {
-#pragma unroll
-        for (int sl = 0; sl < 4; sl++) a[(4 * g + sl) * 4 + i] = f[kind][sl];
+        *reinterpret_cast<uint4 *>(a + 4 * lane) = make_uint4(f[kind][0], f[kind][1], f[kind][2], f[kind][3]);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const uint4 r = *reinterpret_cast<const uint4 *>(a + lane * 4);
-        f[kind][0] = r.x; f[kind][1] = r.y; f[kind][2] = r.z; f[kind][3] = r.w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[kind][i] = a[64 * i + lane];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
