@@ -39,7 +39,8 @@ __device__ __forceinline__ u32x4 dma_rsrc(const void *base, uint32_t bytes) {
 }
 
 // One LDS-direct load: lane l's 16 (4) bytes at buffer offset voff (+ soff) land at LDS byte
-// lds_addr + 16 l (4 l).  lds_addr, rsrc and soff are wave-uniform.
+// lds_addr + 16 l (4 l).  lds_addr, rsrc and soff are wave-uniform.  M0 (the LDS base of the copy)
+// is written and consumed inside the one asm statement; nothing else in these kernels depends on M0.
 __device__ __forceinline__ void dma_b128(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
