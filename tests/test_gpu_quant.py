@@ -81,3 +81,27 @@ def test_fused_quant_encode_round_trip_medium(cuda):
         else:
             ops.v_decode(r["stream"], r["info"], back, 128, 64, 4)
         assert torch.equal(back, codes)
+
+
+@pytest.mark.gpu
+def test_fused_quant_encode_round_trip_full_size(cuda):
+    """The benchmark workload itself (16 x 8 heads x 32768 tokens, 1 GiB of fp16 per tensor): block_info tiles the
+    stream without gaps, and unpacking the stream reproduces the stand-alone quantizer's codes."""
+    B, H, T, rel = 16, 8, 32768, 0.1
+    k, v = synth.make_kv(B, H, T, seed=0, device=cuda)
+    for is_k, x in ((True, k), (False, v)):
+        r = (ops.k_quant_encode if is_k else ops.v_quant_encode)(x, rel, 4)
+        info = r["info"].view(-1, 2).to(torch.int64)
+        assert int(info[0, 0]) == 0
+        assert torch.equal(info[1:, 0], torch.cumsum(info[:-1, 1], 0))          # back to back, in block order
+        assert int(info[-1, 0] + info[-1, 1]) == r["size"]
+        scale, zero = ops.quant_params(x, rel)
+        assert torch.equal(scale, r["scale"]) and torch.equal(zero, r["zero"])
+        codes, _ = ops.quantize(x, scale, zero)
+        back = torch.empty_like(codes)
+        if is_k:
+            ops.k_decode(r["stream"], r["info"], back, 64, 128, 4)
+        else:
+            ops.v_decode(r["stream"], r["info"], back, 128, 64, 4)
+        assert torch.equal(back, codes)
+        del r, codes, back
