@@ -139,7 +139,7 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *                     size (size_out of the encoder) or the last block decodes wrongly
  *   k_scale..v_zero   [B, T_c] `dtype`
  *   q, out            [B, Hq, 128] `dtype`
- *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype` (the residual
+ *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype`, k_win 16-byte aligned (the residual
  *                     window the cache keeps in 16-bit, utils/compute.py:54-67); T_w may be 0
  *   T_c               compressed tokens, a multiple of 128 (may be 0 when T_w > 0)
  *   variant           0 = default (asynchronous-copy matrix-core kernel; streams must be 16-byte

@@ -44,6 +44,8 @@ struct AttnParams {
     int k_bits, v_bits, dtype;
     float sm_scale;
     int tiles_per_split, nsplit, nparts;
+    int win_piece;        // > 0: split i of the compressed part also takes window tokens [i * win_piece, ...) and
+                          // writes partial nsplit + i; 0: the window has a kernel of its own (partial nparts - 1)
     uint32_t k_cap, v_cap, blk_stride;
     uint32_t k_bytes, v_bytes;   // valid bytes of the streams
 };
@@ -279,31 +281,55 @@ __device__ __forceinline__ float wave_sum(float x) {
 }
 
 // ---- 16-bit tail window: dense attention over T_w tokens, one workgroup per (kv head, batch)
+// Attention of the G query heads of KV head (h, b) over tokens [t0, t1) of the uncompressed tail window, written
+// as partial `part_idx` (an empty range writes a partial of weight zero).  `lds` provides G * (128 + t1 - t0)
+// floats.  Called by all 256 threads of a workgroup.
+constexpr int kWinPieceLds = 36864;   // LDS every instance of the async-copy kernel has in its two slots
+
 template <int G>
-__global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
-    extern __shared__ __align__(16) uint8_t lds[];
+__device__ __forceinline__ void window_body(const AttnParams &p, uint8_t *lds, int h, int b, int t0, int t1,
+                                            int part_idx) {
     float *qf = reinterpret_cast<float *>(lds);   // [G][128]
-    float *S = qf + G * kHeadDim;                 // [G][T_w]
+    float *S = qf + G * kHeadDim;                 // [G][Tw]
     __shared__ float st_m[G], st_l[G];
-    const int h = blockIdx.x, b = blockIdx.y;
     const int tid = threadIdx.x;
-    const int Tw = p.T_w;
+    const int Tw = t1 > t0 ? t1 - t0 : 0;
     for (int i = tid; i < G * kHeadDim; i += 256)
         qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
     __syncthreads();
-    const uint16_t *kbase = p.k_win + ((size_t)b * p.Hkv + h) * Tw * kHeadDim;
-    const uint16_t *vbase = p.v_win + ((size_t)b * p.Hkv + h) * Tw * kHeadDim;
-    for (int t = tid; t < Tw; t += 256) {
-        float dot[G];
+    const uint16_t *kbase = p.k_win + (((size_t)b * p.Hkv + h) * p.T_w + t0) * kHeadDim;
+    const uint16_t *vbase = p.v_win + (((size_t)b * p.Hkv + h) * p.T_w + t0) * kHeadDim;
+    {   // scores: 16 tokens per pass, 16 threads per token, each with 8 channels of the row
+        const int c = tid & 15;
+        float qr[G][8];
 #pragma unroll
-        for (int g = 0; g < G; g++) dot[g] = 0.f;
-        for (int d = 0; d < kHeadDim; d++) {
-            const float kv = a_ld16(kbase, (size_t)t * kHeadDim + d, p.dtype);
+        for (int g = 0; g < G; g++)
 #pragma unroll
-            for (int g = 0; g < G; g++) dot[g] += qf[g * kHeadDim + d] * kv;
+            for (int j = 0; j < 8; j++) qr[g][j] = qf[g * kHeadDim + 8 * c + j];
+        for (int base = 0; base < Tw; base += 16) {
+            const int t = base + (tid >> 4);
+            float dot[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) dot[g] = 0.f;
+            if (t < Tw) {
+                const uint4 v = reinterpret_cast<const uint4 *>(kbase + (size_t)t * kHeadDim)[c];
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float k0 = p.dtype == PKV_F16 ? __half2float(__ushort_as_half((unsigned short)(w[i] & 0xFFFFu)))
+                                                        : __uint_as_float(w[i] << 16);
+                    const float k1 = p.dtype == PKV_F16 ? __half2float(__ushort_as_half((unsigned short)(w[i] >> 16)))
+                                                        : __uint_as_float(w[i] & 0xFFFF0000u);
+#pragma unroll
+                    for (int g = 0; g < G; g++) dot[g] += qr[g][2 * i] * k0 + qr[g][2 * i + 1] * k1;
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float d = row16_sum(dot[g]);
+                if (c == 0 && t < Tw) S[g * Tw + t] = d * p.sm_scale;
+            }
         }
-#pragma unroll
-        for (int g = 0; g < G; g++) S[g * Tw + t] = dot[g] * p.sm_scale;
     }
     __syncthreads();
     for (int g = tid >> 6; g < G; g += 4) {
@@ -323,22 +349,47 @@ __global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
         if (lane == 0) { st_m[g] = mx; st_l[g] = sum; }
     }
     __syncthreads();
-    if (tid < kHeadDim) {
+    {   // weighted V sum: thread = (token parity, channel); the odd half hands its sums over through qf
+        const int half = tid >> 7, ch = tid & (kHeadDim - 1);
         float acc[G];
 #pragma unroll
         for (int g = 0; g < G; g++) acc[g] = 0.f;
-        for (int t = 0; t < Tw; t++) {
-            const float v = a_ld16(vbase, (size_t)t * kHeadDim + tid, p.dtype);
+        int t = half;
+        for (; t + 6 < Tw; t += 8) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = a_ld16(vbase, (size_t)(t + 2 * u) * kHeadDim + ch, p.dtype);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int g = 0; g < G; g++) acc[g] += S[g * Tw + t + 2 * u] * v[u];
+        }
+        for (; t < Tw; t += 2) {
+            const float v = a_ld16(vbase, (size_t)t * kHeadDim + ch, p.dtype);
 #pragma unroll
             for (int g = 0; g < G; g++) acc[g] += S[g * Tw + t] * v;
         }
-        for (int g = 0; g < G; g++) {
-            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
-            float *dst = p.part + (hq * p.nparts + (p.nparts - 1)) * kPartStride;
-            dst[2 + tid] = acc[g];
-            if (tid == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+        if (half) {
+#pragma unroll
+            for (int g = 0; g < G; g++) qf[g * kHeadDim + ch] = acc[g];
+        }
+        __syncthreads();
+        if (!half) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+                float *dst = p.part + (hq * p.nparts + part_idx) * kPartStride;
+                dst[2 + ch] = acc[g] + qf[g * kHeadDim + ch];
+                if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
+            }
         }
     }
+}
+
+template <int G>
+__global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    window_body<G>(p, lds, blockIdx.x, blockIdx.y, 0, p.T_w, p.nparts - 1);
 }
 
 // ---- merge of the per-split partials: grid (Hq, B), 128 threads ---------------------------
@@ -380,6 +431,7 @@ namespace pkv {
 
 template <int G, int KW, int VW>
 static int launch_dma(const AttnParams &p, hipStream_t s) {
+    static_assert(dma_lds_bytes<G, KW, VW>() >= kWinPieceLds, "window pieces borrow the slots");
     const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
     if (p.dtype == PKV_BF16)
         attn_dma_kernel<G, KW, VW, true><<<grid, 256, 0, s>>>(p);
@@ -420,8 +472,7 @@ static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
 }
 
 template <int G>
-static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStream_t s) {
-    const bool aligned16 = ((reinterpret_cast<uintptr_t>(p.k_stream) | reinterpret_cast<uintptr_t>(p.v_stream)) & 15u) == 0;
+static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_t *out, hipStream_t s) {
     PKV_REQUIRE(variant >= 0 && variant <= 2, PKV_ERR_INVALID, "variant must be 0, 1 or 2");
     // variant 0: asynchronous-copy kernel (needs 16-byte aligned streams; otherwise, and as
     // variant 2, the kernel that gathers straight from global memory); variant 1: plain VALU kernel
@@ -440,7 +491,7 @@ static int launch_attn(const AttnParams &p, int variant, uint16_t *out, hipStrea
         attn_tiles_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
-    if (p.T_w > 0) {
+    if (p.T_w > 0 && p.win_piece == 0) {
         const uint32_t lds_bytes = (uint32_t)sizeof(float) * (G * kHeadDim + G * p.T_w);
         PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_window_kernel<G>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
@@ -480,7 +531,11 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
                 "batch x compressed tokens above 2^28");
     PKV_REQUIRE((uint64_t)(a->T_c / 64) * (uint64_t)a->B * (uint64_t)a->Hkv < (1ull << 27), PKV_ERR_UNSUPPORTED,
                 "more than 2^27 blocks per stream");
-    if (a->T_w > 0) PKV_REQUIRE(a->k_win && a->v_win, PKV_ERR_INVALID, "null pointer argument");
+    if (a->T_w > 0) {
+        PKV_REQUIRE(a->k_win && a->v_win, PKV_ERR_INVALID, "null pointer argument");
+        PKV_REQUIRE((reinterpret_cast<uintptr_t>(a->k_win) & 15u) == 0, PKV_ERR_INVALID,
+                    "k_win must be 16-byte aligned");
+    }
     const int G = a->Hq / a->Hkv;
     PKV_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, PKV_ERR_UNSUPPORTED,
                 "not supported: query heads per KV head must be 1, 2, 4 or 8");
@@ -505,7 +560,16 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
         nsplit = (n_tiles + tps - 1) / tps;
     }
     p.tiles_per_split = tps; p.nsplit = nsplit;
-    p.nparts = nsplit + (a->T_w > 0 ? 1 : 0);
+    // The async-copy kernel spreads the tail window over its splits (each takes win_piece tokens after its
+    // tiles and writes one more partial), so the window costs no launch and no idle tail; other paths
+    // give the window a kernel of its own.
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
+    p.win_piece = 0;
+    if (a->T_w > 0 && nsplit > 0 && a->variant == 0 && aligned16) {
+        const int piece = (a->T_w + nsplit - 1) / nsplit;
+        if ((size_t)G * (kHeadDim + piece) * sizeof(float) <= (size_t)kWinPieceLds) p.win_piece = piece;
+    }
+    p.nparts = nsplit + (a->T_w > 0 ? (p.win_piece ? nsplit : 1) : 0);
     p.k_cap = a->T_c > 0 ? (uint32_t)k_block_bound(64, a->k_bits) : 0;
     p.v_cap = a->T_c > 0 ? (uint32_t)v_block_bound(64, a->v_bits) : 0;
     const uint32_t cap = p.k_cap > p.v_cap ? p.k_cap : p.v_cap;
@@ -520,10 +584,10 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     switch (G) {
-        case 1: rc = launch_attn<1>(p, a->variant, (uint16_t *)a->out, s); break;
-        case 2: rc = launch_attn<2>(p, a->variant, (uint16_t *)a->out, s); break;
-        case 4: rc = launch_attn<4>(p, a->variant, (uint16_t *)a->out, s); break;
-        default: rc = launch_attn<8>(p, a->variant, (uint16_t *)a->out, s); break;
+        case 1: rc = launch_attn<1>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
+        case 2: rc = launch_attn<2>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
+        case 4: rc = launch_attn<4>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
+        default: rc = launch_attn<8>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
     }
     if (rc) return rc;
     return tm.end(ms_out);

@@ -132,6 +132,12 @@ __device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[
     }
 }
 
+template <int G, int KW, int VW>
+constexpr int dma_lds_bytes() {          // static LDS of attn_dma_kernel: two slots, weights, round sums, state
+    constexpr int GP = (G + 3) / 4 * 4;
+    return 2 * DmaGeom<KW, VW>::kSlot + GP * (kTile + 4) * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
+}
+
 template <int G, int KW, int VW, bool BF>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 3, 4))) attn_dma_kernel(const AttnParams p) {
     using Geo = DmaGeom<KW, VW>;
@@ -147,7 +153,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
     static_assert(NSETS * 4 * 16 * 32 <= 8 * kRoundBytes, "q digits borrow a slot");
 
     constexpr int kPStride = kTile + 4;          // halves per head row of the weights: rows 8 bytes apart in bank space
-    constexpr int kLdsBytes = 2 * Geo::kSlot + GP * kPStride * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
+    constexpr int kLdsBytes = dma_lds_bytes<G, KW, VW>();
+    static_assert(kLdsBytes == 2 * Geo::kSlot + GP * kPStride * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4, "LDS layout");
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLdsBytes];
     uint8_t *ring = smem;                                                    // [2 slots][4 block regions | parameters]
     _Float16 *pbuf = reinterpret_cast<_Float16 *>(smem + 2 * Geo::kSlot);    // [GP][128 + 4]
@@ -530,6 +537,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
             dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
             if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
         }
+    }
+    // this split's share of the 16-bit tail window, as a partial of its own (the slots are free: every
+    // wave drained its copies before the barrier above)
+    if (p.win_piece > 0) {
+        const int t0 = split * p.win_piece, t1 = min(t0 + p.win_piece, p.T_w);
+        window_body<G>(p, smem, h, b, t0, t1, p.nsplit + split);
     }
 }
 

@@ -126,7 +126,10 @@ def test_attn_decode_baseline_shapes_contract_tolerance(cuda, dtype, variant):
 @pytest.mark.parametrize("variant", [0, 1, 2])
 def test_attn_decode_with_tail_window(cuda, variant):
     dtype = torch.float16
-    for (B, Hq, Hkv, T, Tw) in ((2, 32, 8, 512, 150), (1, 8, 8, 0, 191), (1, 16, 4, 128, 1)):
+    # the default kernel spreads the window over its splits: cover pieces of unequal size, more splits than
+    # window tokens (empty pieces), the largest piece that fits and one that does not (window kernel of its own)
+    for (B, Hq, Hkv, T, Tw) in ((2, 32, 8, 512, 150), (1, 8, 8, 0, 191), (1, 16, 4, 128, 1), (1, 8, 2, 1024, 3),
+                                (1, 8, 1, 256, 2048), (1, 8, 1, 128, 2048)):
         _say("attn window case", B, Hq, Hkv, T, Tw)
         k, v = synth.make_kv(B, Hkv, T + Tw, seed=60 + Tw, dtype=dtype)
         q = synth.make_q(B, Hq, seed=61, dtype=dtype)
