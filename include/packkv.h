@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PKV_ABI_VERSION 1
+#define PKV_ABI_VERSION 2
 
 #define PKV_F16 0
 #define PKV_BF16 1
@@ -98,6 +98,25 @@ int pkv_v_quant_encode(const void *x, int dtype, int B, int H, int T, float rel,
                        uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
                        uint64_t *size_out, float *ms_out, pkv_stream_t s);
 
+/* ---- incremental encode: append T_new more tokens to an existing stream ----------------
+ * For a cache that grows (models/cache/packkv_quant.py:45-85 re-quantizes each cut of the
+ * buffer, utils/compute.py:54-67; per-token parameters make a chunked encode produce the
+ * codes of a one-shot encode).  x [B, H, T_new, 128] are the new tokens (T_new a multiple
+ * of 64 for K, 128 for V).  Their blocks are written back-to-back from byte `stream_used`
+ * of `stream`; `block_info_tail` points at the entry after the last existing block (entries
+ * hold offsets from the start of `stream`), `scale_tail` / `zero_tail` at the first new
+ * token of row 0 of arrays [B, par_stride].  Appending chunk after chunk gives the stream,
+ * block_info and parameters of one pkv_{k,v}_quant_encode call over all tokens.  size_out
+ * receives the bytes in use after the append. */
+int pkv_k_quant_encode_append(const void *x, int dtype, int B, int H, int T_new, float rel, int bits,
+                               uint8_t *stream, uint64_t capacity, uint64_t stream_used, uint32_t *block_info_tail,
+                               void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
+                               float *ms_out, pkv_stream_t s);
+int pkv_v_quant_encode_append(const void *x, int dtype, int B, int H, int T_new, float rel, int bits,
+                               uint8_t *stream, uint64_t capacity, uint64_t stream_used, uint32_t *block_info_tail,
+                               void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
+                               float *ms_out, pkv_stream_t s);
+
 /* ---- the reference's GEMV surface -----------------------------------------------------
  * kq_mat_vec_mul (packkv_cuda.pyi:26-36, src/kernels.cu:611-630):
  *     kq_out[h, tok] = sum_d q[h, d] * code[tok, h*128 + d]        (dtype, [H, ctx_len])
@@ -142,6 +161,9 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype`, k_win 16-byte aligned (the residual
  *                     window the cache keeps in 16-bit, utils/compute.py:54-67); T_w may be 0
  *   T_c               compressed tokens, a multiple of 128 (may be 0 when T_w > 0)
+ *   par_stride        tokens per row of the scale / zero arrays when they are allocated longer than
+ *                     T_c (a cache that grows); 0 = T_c
+ *   win_stride        tokens per (sequence, KV head) row of k_win / v_win; 0 = T_w
  *   variant           0 = default (asynchronous-copy matrix-core kernel; streams must be 16-byte
  *                     aligned, otherwise variant 2 runs); 1 = plain VALU kernel; 2 = matrix-core
  *                     kernel that gathers straight from global memory.  All three implement the
@@ -162,6 +184,7 @@ typedef struct pkv_attn_args {
     int dtype;
     float sm_scale;
     int variant;
+    int par_stride, win_stride;
 } pkv_attn_args;
 
 int pkv_attn_decode(const pkv_attn_args *args, float *ms_out, pkv_stream_t s);

@@ -29,6 +29,7 @@ class AttnArgs(ctypes.Structure):
         ("q", _vp), ("out", _vp), ("k_win", _vp), ("v_win", _vp),
         ("B", _i), ("Hq", _i), ("Hkv", _i), ("T_c", _i), ("T_w", _i),
         ("k_bits", _i), ("v_bits", _i), ("dtype", _i), ("sm_scale", _f), ("variant", _i),
+        ("par_stride", _i), ("win_stride", _i),
     ]
 
 
@@ -46,6 +47,8 @@ SIGNATURES = {
     "pkv_dequantize": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _fp, _vp]),
     "pkv_k_quant_encode": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
     "pkv_v_quant_encode": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
+    "pkv_k_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),
+    "pkv_v_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),
     "pkv_kq_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_wv_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_fused_kq": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),

@@ -41,6 +41,8 @@ struct AttnParams {
     const uint16_t *k_win, *v_win;
     float *part;          // [B, Hq, nparts, kPartStride]
     int B, Hq, Hkv, T_c, T_w;
+    int par_stride;       // tokens per sequence row of the scale / zero arrays (>= T_c)
+    int win_stride;       // tokens per (sequence, KV head) row of k_win / v_win (>= T_w)
     int k_bits, v_bits, dtype;
     float sm_scale;
     int tiles_per_split, nsplit, nparts;
@@ -107,7 +109,7 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
             if (tid == 0) s_phase[j] = ph;
         }
         if (tid < kTile) {
-            const size_t ti = (size_t)b * p.T_c + (size_t)tau * kTile + tid;
+            const size_t ti = (size_t)b * p.par_stride + (size_t)tau * kTile + tid;
             ks[tid] = a_ld16(p.k_scale, ti, p.dtype);
             kz[tid] = a_ld16(p.k_zero, ti, p.dtype);
             vs[tid] = a_ld16(p.v_scale, ti, p.dtype);
@@ -297,8 +299,8 @@ __device__ __forceinline__ void window_body(const AttnParams &p, uint8_t *lds, i
     for (int i = tid; i < G * kHeadDim; i += 256)
         qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
     __syncthreads();
-    const uint16_t *kbase = p.k_win + (((size_t)b * p.Hkv + h) * p.T_w + t0) * kHeadDim;
-    const uint16_t *vbase = p.v_win + (((size_t)b * p.Hkv + h) * p.T_w + t0) * kHeadDim;
+    const uint16_t *kbase = p.k_win + (((size_t)b * p.Hkv + h) * p.win_stride + t0) * kHeadDim;
+    const uint16_t *vbase = p.v_win + (((size_t)b * p.Hkv + h) * p.win_stride + t0) * kHeadDim;
     {   // scores: 16 tokens per pass, 16 threads per token, each with 8 channels of the row
         const int c = tid & 15;
         float qr[G][8];
@@ -527,7 +529,9 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
         PKV_REQUIRE(a->k_bytes > 0 && a->v_bytes > 0 && a->k_bytes < (1ull << 32) && a->v_bytes < (1ull << 32),
                     PKV_ERR_INVALID, "stream sizes must be in 1 .. 4 GiB - 1");
     }
-    PKV_REQUIRE((uint64_t)a->B * (uint64_t)a->T_c < (1ull << 28), PKV_ERR_UNSUPPORTED,
+    const int par_stride = a->par_stride ? a->par_stride : a->T_c, win_stride = a->win_stride ? a->win_stride : a->T_w;
+    PKV_REQUIRE(par_stride >= a->T_c && win_stride >= a->T_w, PKV_ERR_INVALID, "row stride shorter than the row");
+    PKV_REQUIRE((uint64_t)a->B * (uint64_t)par_stride < (1ull << 28), PKV_ERR_UNSUPPORTED,
                 "batch x compressed tokens above 2^28");
     PKV_REQUIRE((uint64_t)(a->T_c / 64) * (uint64_t)a->B * (uint64_t)a->Hkv < (1ull << 27), PKV_ERR_UNSUPPORTED,
                 "more than 2^27 blocks per stream");
@@ -547,6 +551,7 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     p.q = (const uint16_t *)a->q;
     p.k_win = (const uint16_t *)a->k_win; p.v_win = (const uint16_t *)a->v_win;
     p.B = a->B; p.Hq = a->Hq; p.Hkv = a->Hkv; p.T_c = a->T_c; p.T_w = a->T_w;
+    p.par_stride = par_stride; p.win_stride = win_stride;
     p.k_bits = a->k_bits; p.v_bits = a->v_bits; p.dtype = a->dtype; p.sm_scale = a->sm_scale;
     const int n_tiles = a->T_c / kTile;
     int nsplit = 0, tps = 0;

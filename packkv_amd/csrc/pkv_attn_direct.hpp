@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     const __amdgpu_buffer_rsrc_t v_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.v_stream), 0, (int)p.v_bytes, 0x00020000);
 
-    const int par_bytes = p.B * p.T_c * 2, info_bytes = (p.T_c / 64) * p.B * p.Hkv * 8;
+    const int par_bytes = p.B * p.par_stride * 2, info_bytes = (p.T_c / 64) * p.B * p.Hkv * 8;
     const __amdgpu_buffer_rsrc_t ks_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.k_scale), 0, par_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t kz_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.k_zero), 0, par_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.v_scale), 0, par_bytes, 0x00020000);
@@ -281,7 +281,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     // quantizer parameters of the two tokens (2*lane, 2*lane+1) this lane handles in the softmax stage
     struct QPar { uint32_t ks, kz, vs, vz; };
     auto qpar_issue = [&](int rel, QPar &q) {
-        const int tile_off = (b * p.T_c + (tile0 + min(rel, ntl - 1)) * kTile) * 2;     // bytes, wave-uniform
+        const int tile_off = (b * p.par_stride + (tile0 + min(rel, ntl - 1)) * kTile) * 2;     // bytes, wave-uniform
         q.ks = __builtin_amdgcn_raw_buffer_load_b32(ks_rsrc, 4 * lane, tile_off, 0);
         q.kz = __builtin_amdgcn_raw_buffer_load_b32(kz_rsrc, 4 * lane, tile_off, 0);
         q.vs = __builtin_amdgcn_raw_buffer_load_b32(vs_rsrc, 4 * lane, tile_off, 0);

@@ -175,7 +175,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
     // the stream this wave copies from, range-checked: block_info is never trusted with an address
     const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, wave < 2 ? p.k_bytes : p.v_bytes);
     const uint16_t *par_arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
-    const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.T_c * 2));
+    const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.par_stride * 2));
 
     // ---- prologue: split q into digits (through LDS, aliased onto the K tile) ----
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
             }
         }
         // parameter array `wave` of the tile: 128 tokens x 2 bytes = 64 lanes x 4 bytes
-        const int tile_off = (b * p.T_c + (tile0 + min(rel, ntl - 1)) * kTile) * 2;
+        const int tile_off = (b * p.par_stride + (tile0 + min(rel, ntl - 1)) * kTile) * 2;
         dma_b32(par_rsrc, ring_lds + (uint32_t)(slot * Geo::kSlot + Geo::kParOff + wave * 256), 4 * lane, (uint32_t)tile_off);
     };
 

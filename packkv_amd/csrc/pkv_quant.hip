@@ -361,7 +361,7 @@ template <bool IS_K, int DT>
 __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t nsub, uint32_t bound) {
+    ScanState *st, int W, uint32_t nsub, uint32_t bound, uint64_t base, int par_stride) {
     constexpr int CTX = IS_K ? 64 : 128;
     extern __shared__ __align__(16) uint8_t gbuf[];        // the sub-group's encoded bytes (8 x block bound)
     __shared__ uint32_t s_idx;
@@ -431,8 +431,8 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
             const float sc = round_t<DT>(range * rel);
             const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
             if (sg == 0) {
-                scale[(size_t)b * T + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
-                zero[(size_t)b * T + tok0 + tt] = (uint16_t)zb;
+                scale[(size_t)b * par_stride + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[(size_t)b * par_stride + tok0 + tt] = (uint16_t)zb;
                 if (SG > 1)
                     __hip_atomic_store(tokw + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(sc) << 16) | (uint64_t)zb,
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -496,7 +496,7 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     // ---- 3. one look-back for the whole sub-group, then one contiguous copy ----
     const uint32_t bytes = blk_off[nb];
     if (tid < 64) {
-        const uint64_t off = lookback_offset(st, sidx, bytes);
+        const uint64_t off = base + lookback_offset(st, sidx, bytes);
         if (tid == 0) {
             s_off = off;
             if (sidx == nsub - 1) st->total = off + bytes;
@@ -545,7 +545,7 @@ template <int DT>
 __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t bound) {
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -586,8 +586,8 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
                 const float range = round_t<DT>(mx - mn);
                 const float sc = round_t<DT>(range * rel);
                 const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-                scale[(size_t)b * T + tok0 + 16 * r + tt] = (uint16_t)T16<DT>::to_bits(sc);
-                zero[(size_t)b * T + tok0 + 16 * r + tt] = (uint16_t)zb;
+                scale[(size_t)b * par_stride + tok0 + 16 * r + tt] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[(size_t)b * par_stride + tok0 + 16 * r + tt] = (uint16_t)zb;
                 s_par[tt] = token_par<DT>(sc, zb);
             }
         }
@@ -621,7 +621,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     __syncthreads();
     const uint32_t bytes = blk_off[H];
     if (tid < 64) {
-        const uint64_t off = lookback_offset(st, gidx, bytes);
+        const uint64_t off = base + lookback_offset(st, gidx, bytes);
         if (tid == 0) {
             s_off = off;
             if (gidx == ngroups - 1) st->total = off + bytes;
@@ -673,8 +673,8 @@ static int check_xshape(const void *x, int dtype, int B, int H, int T) {
 
 template <bool IS_K>
 static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits,
-                            uint8_t *stream, uint64_t capacity, uint32_t *info, void *scale, void *zero,
-                            uint64_t *size_out, float *ms_out, hipStream_t s) {
+                            uint8_t *stream, uint64_t capacity, uint64_t base, uint32_t *info, void *scale,
+                            void *zero, int par_stride, uint64_t *size_out, float *ms_out, hipStream_t s) {
     int rc = check_xshape(x, dtype, B, H, T);
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
@@ -683,6 +683,8 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
+    PKV_REQUIRE(par_stride >= T, PKV_ERR_INVALID, "parameter row stride shorter than the token count");
+    PKV_REQUIRE(base <= capacity, PKV_ERR_INVALID, "stream offset beyond the buffer");
     ScanState *st = nullptr;
     // One workgroup per sub-group of up to eight consecutive blocks that share (context block, sequence).
     {
@@ -701,19 +703,19 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             if (dtype == PKV_F16)
                 k_quant_encode_rounds_kernel<PKV_F16><<<nsub, 256, lds, s>>>(
                     (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                    bits, nsub, slot);
+                    bits, nsub, slot, base, par_stride);
             else
                 k_quant_encode_rounds_kernel<PKV_BF16><<<nsub, 256, lds, s>>>(
                     (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                    bits, nsub, slot);
+                    bits, nsub, slot, base, par_stride);
         } else if (dtype == PKV_F16)
             quant_encode_group_kernel<IS_K, PKV_F16><<<nsub, 256, gbytes, s>>>(
                 (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                bits, nsub, bound);
+                bits, nsub, bound, base, par_stride);
         else
             quant_encode_group_kernel<IS_K, PKV_BF16><<<nsub, 256, gbytes, s>>>(
                 (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                bits, nsub, bound);
+                bits, nsub, bound, base, par_stride);
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
         return finish_encode(st, size_out, bits, s);
@@ -788,15 +790,33 @@ int pkv_dequantize(const uint8_t *codes, int dtype, int B, int H, int T, const v
 int pkv_k_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *stream,
                        uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
                        uint64_t *size_out, float *ms_out, pkv_stream_t s) {
-    return pkv::run_quant_encode<true>(x, dtype, B, H, T, rel, bits, stream, capacity, block_info, scale,
-                                       zero, size_out, ms_out, (hipStream_t)s);
+    return pkv::run_quant_encode<true>(x, dtype, B, H, T, rel, bits, stream, capacity, 0, block_info, scale,
+                                       zero, T, size_out, ms_out, (hipStream_t)s);
 }
 
 int pkv_v_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *stream,
                        uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
                        uint64_t *size_out, float *ms_out, pkv_stream_t s) {
-    return pkv::run_quant_encode<false>(x, dtype, B, H, T, rel, bits, stream, capacity, block_info, scale,
-                                        zero, size_out, ms_out, (hipStream_t)s);
+    return pkv::run_quant_encode<false>(x, dtype, B, H, T, rel, bits, stream, capacity, 0, block_info, scale,
+                                        zero, T, size_out, ms_out, (hipStream_t)s);
+}
+
+int pkv_k_quant_encode_append(const void *x, int dtype, int B, int H, int T_new, float rel, int bits,
+                               uint8_t *stream, uint64_t capacity, uint64_t stream_used, uint32_t *block_info_tail,
+                               void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
+                               float *ms_out, pkv_stream_t s) {
+    return pkv::run_quant_encode<true>(x, dtype, B, H, T_new, rel, bits, stream, capacity, stream_used,
+                                       block_info_tail, scale_tail, zero_tail, par_stride, size_out, ms_out,
+                                       (hipStream_t)s);
+}
+
+int pkv_v_quant_encode_append(const void *x, int dtype, int B, int H, int T_new, float rel, int bits,
+                               uint8_t *stream, uint64_t capacity, uint64_t stream_used, uint32_t *block_info_tail,
+                               void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
+                               float *ms_out, pkv_stream_t s) {
+    return pkv::run_quant_encode<false>(x, dtype, B, H, T_new, rel, bits, stream, capacity, stream_used,
+                                        block_info_tail, scale_tail, zero_tail, par_stride, size_out, ms_out,
+                                        (hipStream_t)s);
 }
 
 }  // extern "C"

@@ -267,6 +267,35 @@ def v_quant_encode(x, rel, bits=None, stream=None, info=None, want_size=True, ti
     return _quant_encode(False, x, rel, bits or bits_for_rel(rel), stream, info, want_size, timed)
 
 
+def quant_encode_append(is_k, x, rel, bits, stream, used, info, tokens, scale, zero):
+    """Append the tokens x [B, H, n, 128] (n a multiple of 64 for K, 128 for V) to a stream that holds
+    ``tokens`` tokens in its first ``used`` bytes.  ``info`` [blocks, 2] and ``scale`` / ``zero``
+    [B, row] are allocated for the cache's full length and filled behind what is there; the new blocks'
+    offsets count from the start of ``stream``.  Returns the bytes in use afterwards."""
+    B, H, n = _check_x(x)
+    ctx_blk, hid_blk = (64, 128) if is_k else (128, 64)
+    per_row = B * H * 128 // hid_blk
+    _require(n % ctx_blk == 0 and tokens % ctx_blk == 0, "token counts must be multiples of the block length")
+    nblk_done, nblk_new = tokens // ctx_blk * per_row, n // ctx_blk * per_row
+    _require(info.is_cuda and info.dtype == torch.uint32 and info.is_contiguous()
+             and info.numel() >= 2 * (nblk_done + nblk_new), "block_info_buffer too small")
+    _require(scale.shape == zero.shape and scale.dim() == 2 and scale.size(0) == B and scale.dtype == x.dtype
+             and zero.dtype == x.dtype and scale.is_contiguous() and zero.is_contiguous()
+             and scale.size(1) >= tokens + n, "scale / zero must be contiguous [B, row] with room for the new tokens")
+    _require(stream.is_cuda and stream.dtype == torch.uint8 and stream.is_contiguous() and 0 <= used <= stream.numel(),
+             "compressed_buffer must be a contiguous device UInt8 tensor holding the bytes in use")
+    es = scale.element_size()
+    size = ctypes.c_uint64(0)
+    fn = _lib.load().pkv_k_quant_encode_append if is_k else _lib.load().pkv_v_quant_encode_append
+    with torch.cuda.device(x.device):
+        rc = fn(_ptr(x), _dtype_code(x), B, H, n, float(rel), int(bits), _ptr(stream), stream.numel(), int(used),
+                ctypes.c_void_p(info.data_ptr() + 8 * nblk_done), ctypes.c_void_p(scale.data_ptr() + es * tokens),
+                ctypes.c_void_p(zero.data_ptr() + es * tokens), scale.size(1), ctypes.byref(size), None,
+                _stream(x.device))
+    _lib.check(rc)
+    return int(size.value)
+
+
 # ------------------------------------------------------- reference GEMV surface ------
 
 def _require_cuda(*ts):
@@ -384,12 +413,16 @@ def fused_wv(our_wv, w, v_quant_zero, v_quant_scale, term1):
 
 # ------------------------------------------------- fused decompress-attention --------
 
-def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False):
+def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False, win_len=None):
     """One decode step over a compressed cache.
 
     q [B, Hq, 128]; k and v are the dicts returned by k_quant_encode / v_quant_encode (stream,
     info, scale, zero, bits) or None when only the 16-bit window exists; k_win / v_win are
-    optional [B, Hkv, T_w, 128] tails.  Returns out [B, Hq, 128] (and ms when timed)."""
+    optional [B, Hkv, T_w, 128] tails.  Returns out [B, Hq, 128] (and ms when timed).
+
+    Buffers allocated for a cache that grows: the dicts may carry ``tokens`` (compressed tokens in use;
+    scale / zero rows and block_info are then longer than that) and ``heads`` (KV heads); ``win_len``
+    gives the window rows in use when k_win / v_win are allocated longer."""
     _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
              "q must be a contiguous device tensor [B, Hq, 128]")
     B, Hq, _ = q.shape
@@ -398,12 +431,18 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
     Hkv = None
     keep = [q]
     if k is not None:
-        T_c = k["scale"].size(1)
+        T_c = int(k.get("tokens", k["scale"].size(1)))
+        _require(int(v.get("tokens", v["scale"].size(1))) == T_c, "K and V hold different token counts")
+        _require(0 < T_c <= k["scale"].size(1) and k["scale"].shape == v["scale"].shape,
+                 "scale / zero rows shorter than the token count")
+        a.par_stride = k["scale"].size(1)
         for name, d in (("k", k), ("v", v)):
             for f in ("stream", "info", "scale", "zero"):
                 _require(d[f].is_cuda and d[f].is_contiguous(), "%s.%s must be a contiguous device tensor" % (name, f))
         nblk_k = k["info"].numel() // 2
-        Hkv = nblk_k // (T_c // 64) // B
+        Hkv = int(k["heads"]) if "heads" in k else nblk_k // (T_c // 64) // B
+        _require(nblk_k >= (T_c // 64) * B * Hkv and v["info"].numel() // 2 >= (T_c // 128) * B * Hkv * 2,
+                 "block_info_buffer block num mismatch")
         a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
         a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
         # readable bytes of each buffer: pack words are fetched as whole 8-byte words, so the last
@@ -421,7 +460,9 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
                  and k_win.shape == v_win.shape and k_win.dim() == 4 and k_win.size(3) == 128
                  and k_win.dtype == q.dtype and v_win.dtype == q.dtype,
                  "window tensors must be contiguous [B, Hkv, T_w, 128] of q's dtype")
-        T_w = k_win.size(2)
+        T_w = k_win.size(2) if win_len is None else int(win_len)
+        _require(0 < T_w <= k_win.size(2), "win_len outside the window tensors")
+        a.win_stride = k_win.size(2)
         _require(Hkv is None or Hkv == k_win.size(1), "window head count mismatch")
         Hkv = k_win.size(1)
         a.k_win, a.v_win = _ptr(k_win), _ptr(v_win)

@@ -1,0 +1,132 @@
+"""The compressed cache that grows (packkv_amd/cache.py) against the restated reference cache
+(oracle/cache.py): dense view bit-exact, decode step within the attention tolerance, streams equal to a
+one-shot encode."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cache as oc
+from oracle import quant as oq
+from packkv_amd import ops, synth
+from packkv_amd.cache import PackKVCacheConfig, PackKVCompressedCache
+
+pytestmark = pytest.mark.gpu
+
+ABS_TOL = 2e-3     # contract for fp16: |err| <= 2e-3 + 1e-3 |ref| against decompress-then-attend
+REL_TOL = 1e-3
+# A few hundred tokens with x10 outlier channels make a peaky softmax: the reference path's own rounding of the
+# dequantised K to 16 bits (logits move by ~1e-3 in fp16, ~8e-3 in bf16) then shows undamped in the output, while
+# the fused kernel keeps (code + zero) * scale in fp32.  Same widened absolute term as the short cases of
+# tests/test_gpu_attn.py.
+SHORT_ABS_TOL = {torch.float16: 8e-3, torch.bfloat16: 6e-2}
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _rope_tables(B, pos0, n, dtype):
+    pos = torch.arange(pos0, pos0 + n, dtype=torch.float32)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    f = torch.outer(pos, inv)
+    emb = torch.cat((f, f), dim=-1)
+    return emb.cos().to(dtype).expand(B, n, 128).contiguous(), emb.sin().to(dtype).expand(B, n, 128).contiguous()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rope", [False, True])
+def test_cache_matches_restated_reference(cuda, dtype, rope):
+    B, Hq, H, T0, steps = 2, 8, 4, 300, 200
+    k, v = synth.make_kv(B, H, T0 + steps, seed=90, dtype=dtype)
+    want = oc.SimulatedCache(1, 64, 192, 0.1, 0.1)
+    got = PackKVCompressedCache(B, H, 128, 1, PackKVCacheConfig(64, 192, 0.1, 0.1), max_tokens=1024, dtype=dtype,
+                                device=cuda)
+    check_at = {0, 1, 18, 19, 20, 82, 83, 84, 146, 147, 148, 199}   # around the cuts at steps 19, 83, 147
+    pos, tok = 0, 0
+    for step in range(-1, steps):
+        n = T0 if step < 0 else 1
+        ks, vs = k[:, :, tok:tok + n], v[:, :, tok:tok + n]
+        cos = sin = None
+        if rope:
+            cos, sin = _rope_tables(B, pos, n, dtype)
+        wk, wv = want.update(ks, vs, 0, cos, sin)
+        kw = {"cos": cos.to(cuda), "sin": sin.to(cuda)} if rope else None
+        got.update(ks.to(cuda), vs.to(cuda), 0, kw)
+        tok += n
+        pos += n
+        assert got.get_seq_length(0) == want.get_seq_length(0) == tok
+        if step in check_at or step < 0:
+            _say("cache case", dtype, "rope" if rope else "plain", "step", step, "tokens", tok,
+                 "compressed", got.layers[0].k.tokens, "window", got.layers[0].win_len)
+            gk, gv = got.materialize(0)
+            assert torch.equal(gk.cpu().view(torch.int16), wk.view(torch.int16))
+            assert torch.equal(gv.cpu().view(torch.int16), wv.view(torch.int16))
+            q = synth.make_q(B, Hq, seed=300 + step, dtype=dtype)
+            ref = oq.attention_f32(q.unsqueeze(2), wk, wv).squeeze(2).double().numpy()
+            out = got.attend(q.to(cuda), 0).double().cpu().numpy()
+            kk = 8.0 if dtype == torch.bfloat16 else 1.0     # bf16 keeps 3 fewer mantissa bits
+            err = np.abs(out - ref)
+            _say("   max|err| = %.3e" % err.max())
+            assert (err <= SHORT_ABS_TOL[dtype] + kk * REL_TOL * np.abs(ref)).all()
+    L = got.layers[0]
+    # 500 tokens: 320 have been cut (128 at the prefill, then at steps 19, 83, 147) = 2 tiles + one pending cut
+    assert L.k.tokens == L.v.tokens == 256 and L.pend == 64 and L.win_len == T0 + steps - 256
+
+
+def test_append_equals_one_shot_encode(cuda):
+    """Chunk-by-chunk append (K in cuts of 64 and 128 tokens, V of 128 and 256) gives the stream, block_info and
+    parameters of one encode over all tokens."""
+    B, H, T = 2, 4, 512
+    k, v = synth.make_kv(B, H, T, seed=95, device=cuda)
+    for is_k, x, chunks in ((True, k, (64, 128, 64, 256)), (False, v, (128, 256, 128))):
+        one = ops.k_quant_encode(x, 0.1) if is_k else ops.v_quant_encode(x, 0.1)
+        per_tok = (B * H) if is_k else (B * H * 2)
+        nblk = T // (64 if is_k else 128) * per_tok
+        stream = torch.zeros(one["size"] + 64, dtype=torch.uint8, device=cuda)
+        info = torch.zeros(nblk, 2, dtype=torch.uint32, device=cuda)
+        scale = torch.zeros(B, T + 128, dtype=x.dtype, device=cuda)     # rows longer than the token count
+        zero = torch.zeros_like(scale)
+        used, tok = 0, 0
+        for n in chunks:
+            _say("append case", "K" if is_k else "V", "tokens", tok, "+", n)
+            used = ops.quant_encode_append(is_k, x[:, :, tok:tok + n].contiguous(), 0.1, one["bits"], stream, used,
+                                           info, tok, scale, zero)
+            tok += n
+        assert tok == T and used == one["size"]
+        assert torch.equal(stream[:used], one["stream"][:used])
+        assert torch.equal(info.view(torch.int32), one["info"].view(torch.int32))
+        assert torch.equal(scale[:, :T].view(torch.int16), one["scale"].view(torch.int16))
+        assert torch.equal(zero[:, :T].view(torch.int16), one["zero"].view(torch.int16))
+
+
+def test_append_reports_a_full_buffer(cuda):
+    B, H = 1, 2
+    k, _ = synth.make_kv(B, H, 128, seed=96, device=cuda)
+    stream = torch.zeros(256, dtype=torch.uint8, device=cuda)
+    info = torch.zeros(4, 2, dtype=torch.uint32, device=cuda)
+    scale = torch.zeros(B, 128, dtype=k.dtype, device=cuda)
+    with pytest.raises(RuntimeError):
+        ops.quant_encode_append(True, k, 0.1, 4, stream, 0, info, 0, scale, torch.zeros_like(scale))
+
+
+def test_cache_bytes_and_prefill_only(cuda):
+    """A prompt below buffer_size stays uncompressed (utils/compute.py:54-67); a long prefill compresses all but
+    128..191 tokens, in whole tiles."""
+    B, H = 1, 8
+    k, v = synth.make_kv(B, H, 1000, seed=97, device=cuda)
+    c = PackKVCompressedCache(B, H, 128, 2, max_tokens=2048, device=cuda)
+    c.update(k[:, :, :191], v[:, :, :191], 0)
+    assert c.layers[0].k.tokens == 0 and c.layers[0].win_len == 191
+    assert c.cache_bytes(0) == 2 * B * H * 191 * 128 * 2
+    c.update(k, v, 1)                     # 1000 tokens: 832 cut = 6 tiles + one pending cut of 64, 168 buffered
+    L = c.layers[1]
+    assert L.k.tokens == 768 and L.pend == 64 and L.win_len == 64 + 168 and c.get_seq_length(1) == 1000
+    fp16_bytes = 2 * B * H * 1000 * 128 * 2
+    assert c.cache_bytes(1) < 0.45 * fp16_bytes
+    q = synth.make_q(B, 32, seed=98, device=cuda)
+    gk, gv = c.materialize(1)
+    ref = oq.attention_f32(q.cpu().unsqueeze(2), gk.cpu(), gv.cpu()).squeeze(2).double().numpy()
+    out = c.attend(q.unsqueeze(2), 1)
+    assert out.shape == (B, 32, 1, 128)
+    err = np.abs(out[:, :, 0].double().cpu().numpy() - ref)
+    assert (err <= SHORT_ABS_TOL[torch.float16] + REL_TOL * np.abs(ref)).all()

@@ -85,3 +85,33 @@ def test_attention_versions_agree_with_fp64():
     got16 = oq.eager_attention(q, kd, vd).double().numpy()
     assert np.abs(got32 - want).max() < 1e-5
     assert np.abs(got16 - want).max() < 5e-3
+
+
+def test_simulated_cache_follows_the_cut_policy():
+    """The restated cache against facts that do not depend on it: (i) the lengths follow cut_tensor's
+    closed form (prefix = cut tokens, buffer cycles 128..191); (ii) quantisation is per token, so the
+    dequantised prefix equals a one-shot quantise -> dequantise of the same tokens however they were
+    chunked; (iii) the buffer is the untouched tail; (iv) rotary embedding with cos = 1, sin = 0 is the
+    identity and with cos = 0, sin = 1 is rotate_half."""
+    from oracle import cache as oc
+    B, H, T0, steps = 1, 2, 300, 150
+    k, v = synth.make_kv(B, H, T0 + steps, seed=9)
+    c = oc.SimulatedCache(1, 64, 192, 0.1, 0.2)
+    kk, vv = c.update(k[:, :, :T0], v[:, :, :T0], 0)
+    n_pref, n_buf = oq.cut_counts(0, T0, 64, 192)
+    assert (n_pref, n_buf) == (128, 172) and kk.shape[2] == T0
+    for i in range(steps):
+        kk, vv = c.update(k[:, :, T0 + i:T0 + i + 1], v[:, :, T0 + i:T0 + i + 1], 0)
+        cut, n_buf = oq.cut_counts(n_buf, 1, 64, 192)
+        n_pref += cut
+        assert c.ck[0].shape[2] == n_pref and c.bk[0].shape[2] == n_buf and 128 <= n_buf <= 191
+    T = T0 + steps
+    assert c.get_seq_length(0) == T and kk.shape[2] == T
+    for got, x, rel in ((kk, k, 0.1), (vv, v, 0.2)):
+        want = oq.dequant(*oq.quant_ints(x[:, :, :n_pref], 64, rel))
+        assert torch.equal(got[:, :, :n_pref], want)
+        assert torch.equal(got[:, :, n_pref:], x[:, :, n_pref:T])
+    t = k[:, :, :8]
+    one, nil = torch.ones(B, 8, 128, dtype=t.dtype), torch.zeros(B, 8, 128, dtype=t.dtype)
+    assert torch.equal(oc.apply_rotary_pos_emb_single(t, one, nil), t)
+    assert torch.equal(oc.apply_rotary_pos_emb_single(t, nil, one), torch.cat((-t[..., 64:], t[..., :64]), dim=-1))
