@@ -394,20 +394,47 @@ __global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
     window_body<G>(p, lds, blockIdx.x, blockIdx.y, 0, p.T_w, p.nparts - 1);
 }
 
-// ---- merge of the per-split partials: grid (Hq, B), 128 threads ---------------------------
-__global__ void attn_merge_kernel(const float *__restrict__ part, uint16_t *__restrict__ out, int Hq,
-                                  int nparts, int dtype) {
+// ---- merge of the per-split partials: grid (Hq, B), 256 threads, nparts floats of dynamic LDS ----
+// Partials are read in parallel: thread <-> partial for the maxima and weights, then thread <-> (parity of the
+// partial, channel) for the weighted sum, four rows in flight.
+__global__ void __launch_bounds__(256) attn_merge_kernel(const float *__restrict__ part, uint16_t *__restrict__ out,
+                                                         int Hq, int nparts, int dtype) {
+    extern __shared__ float w_s[];                   // weight of every partial
+    __shared__ float red[8], half_num[kHeadDim];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t hq = (size_t)blockIdx.y * Hq + blockIdx.x;
     const float *base = part + hq * nparts * kPartStride;
-    float M = -INFINITY;
-    for (int s = 0; s < nparts; s++) M = fmaxf(M, base[s * kPartStride]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < nparts; s++) {
-        const float w = __expf(base[s * kPartStride] - M);
-        den += w * base[s * kPartStride + 1];
-        num += w * base[s * kPartStride + 2 + threadIdx.x];
+    float mx = -INFINITY;
+    for (int s = tid; s < nparts; s += 256) mx = fmaxf(mx, base[(size_t)s * kPartStride]);
+    mx = wave_max(mx);
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float den = 0.f;
+    for (int s = tid; s < nparts; s += 256) {
+        const float w = __expf(base[(size_t)s * kPartStride] - M);
+        w_s[s] = w;
+        den += w * base[(size_t)s * kPartStride + 1];
     }
-    out[hq * kHeadDim + threadIdx.x] = a_st16(num / den, dtype);
+    den = wave_sum(den);
+    if (lane == 0) red[4 + wave] = den;
+    __syncthreads();
+    den = (red[4] + red[5]) + (red[6] + red[7]);
+    const int half = tid >> 7, ch = tid & (kHeadDim - 1);
+    const float *col = base + 2 + ch;
+    float num = 0.f;
+    int s = half;
+    for (; s + 6 < nparts; s += 8) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = col[(size_t)(s + 2 * u) * kPartStride];
+#pragma unroll
+        for (int u = 0; u < 4; u++) num += w_s[s + 2 * u] * v[u];
+    }
+    for (; s < nparts; s += 2) num += w_s[s] * col[(size_t)s * kPartStride];
+    if (half) half_num[ch] = num;
+    __syncthreads();
+    if (!half) out[hq * kHeadDim + ch] = a_st16((num + half_num[ch]) / den, dtype);
 }
 
 }  // namespace pkv
@@ -500,8 +527,8 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_
         attn_window_kernel<G><<<dim3((unsigned)p.Hkv, (unsigned)p.B), 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
-    attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), kHeadDim, 0, s>>>(p.part, out, p.Hq, p.nparts,
-                                                                              p.dtype);
+    attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), 256, (size_t)p.nparts * sizeof(float), s>>>(
+        p.part, out, p.Hq, p.nparts, p.dtype);
     PKV_HIP_CHECK(hipGetLastError());
     return PKV_OK;
 }
