@@ -663,6 +663,198 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     }
 }
 
+// Copy n bytes (even) from LDS (src 4-byte aligned, readable up to 20 bytes past n) to global memory (dst 2-byte
+// aligned) with the 32 lanes of a half-wavefront: head to the first 16-byte boundary and tail in 2-byte pieces, the
+// body as aligned 16-byte stores fed by aligned LDS reads and byte funnel shifts.
+__device__ __forceinline__ void copy_out32(uint8_t *dst, const uint8_t *src, uint32_t n, int t) {
+    const uint32_t head = min(n, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
+    const uint32_t nq = (n - head) >> 4;
+    for (uint32_t i = t; i < (head >> 1); i += 32)
+        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(src)[i];
+    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(src + (head & ~3u));
+    for (uint32_t i = t; i < nq; i += 32) {
+        const uint32_t *q = src32 + 4 * i;
+        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+        uint4 v;
+        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
+        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
+        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
+        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+        *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
+    }
+    const uint32_t done = head + 16u * nq;
+    for (uint32_t i = t; i < ((n - done) >> 1); i += 32)
+        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(src + done)[i];
+}
+
+// OR the FB-bit fields f[0..3] of four adjacent lanes 4m..4m+3, slot i, into a unit's LSB-first metadata array
+// (field of lane c, slot i at bit (4c + i) * FB).  The 16 * FB bits of the four lanes start at byte 2 * FB * m.
+__device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, const uint32_t f[4]) {
+    uint64_t v = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) v |= (uint64_t)f[k] << (4 * FB * k + FB * i);
+    const uint32_t byte = 2u * (uint32_t)FB * (uint32_t)m;
+    uint32_t *w = reinterpret_cast<uint32_t *>(arr + (byte & ~3u));
+    v <<= 8u * (byte & 3u);                       // FB = 3 puts odd m two bytes into the word; 48 + 16 bits still fit
+    atomicOr(w, (uint32_t)v);
+    if (FB > 2) atomicOr(w + 1, (uint32_t)(v >> 32));
+}
+
+// ---- V, all heads in one workgroup: round-major single trip over x --------------------------
+// For H <= 8 one workgroup of 512 threads owns the 2 H blocks of a (128-token context block, sequence) group and
+// goes through it 32 tokens (two rounds) at a time: read the rows of all heads for the token parameters, then at
+// once re-read them as cells -- still in L2 -- quantize and append.  Thread = (round parity rp, head j, cell lane t):
+// its cell (round 2 it + rp, channels 4t..4t+3 of head j) holds slot (2 it + rp) % 4 of lanes 4m..4m+3, m = t % 8, of
+// unit (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight
+// threads of a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed
+// in with LDS atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.
+template <int DT>
+__global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride) {
+    extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[17];                       // byte offset of each block inside the group's bytes
+    __shared__ uint32_t s_tot[2][8][4];                    // payload bytes the two rounds of an iteration append per unit
+    __shared__ uint16_t s_usz[16][4];                      // bytes of every unit (block, unit index 2 w + sg)
+    __shared__ __attribute__((aligned(16))) TokPar s_par[32];
+    const int tid = threadIdx.x;
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = s_idx;
+    if (gidx >= ngroups) return;
+    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * 128;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31;
+    const bool active = j < H;
+    const int jc = min(j, H - 1);
+    const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
+    // metadata areas start as zeros (fields are OR-ed in)
+    for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)
+        reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
+    uint32_t run_off = 0;                                  // payload bytes of the thread's current unit so far
+    uint32_t cmax_all = 0;
+    for (int it = 0; it < 4; it++) {
+        // token parameters of the 32 tokens: 16 lanes x 8 channels per token, all heads
+        {
+            const int tt = tid >> 4, l16 = tid & 15;
+            float mn = INFINITY, mx = -INFINITY;
+            uint4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                v[i] = *reinterpret_cast<const uint4 *>(
+                    x + (((size_t)b * H + min(i, H - 1)) * T + tok0 + 32 * it + tt) * kHeadDim + l16 * 8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+#pragma unroll
+            for (int d = 8; d >= 1; d >>= 1) {
+                mn = fminf(mn, __shfl_xor(mn, d, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, d, 16));
+            }
+            if (l16 == 0) {
+                const float range = round_t<DT>(mx - mn);
+                const float sc = round_t<DT>(range * rel);
+                const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+                scale[(size_t)b * par_stride + tok0 + 32 * it + tt] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[(size_t)b * par_stride + tok0 + 32 * it + tt] = (uint16_t)zb;
+                s_par[tt] = token_par<DT>(sc, zb);
+            }
+        }
+        // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
+        uint2 xr[16];
+        cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
+        __syncthreads();
+        UnitPacks u;
+        uint32_t cmax;
+        cell_packs<DT>(xr, s_par + 16 * rp, u, cmax);
+        // bytes of the thread's four packs, their offsets inside the (unit, slot) and the slot's total
+        const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
+        uint32_t inc = pb;
+#pragma unroll
+        for (int d = 1; d < 8; d <<= 1) {
+            const uint32_t up = __shfl_up(inc, d, 8);
+            if (m >= d) inc += up;
+        }
+        const uint32_t tot = __shfl(inc, 7, 8);
+        if (m == 0) s_tot[rp][j][t >> 3] = tot;
+        __syncthreads();                                  // s_par is rewritten by the next iteration; s_tot is published
+        const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            const int sg = it >> 1, slot = 2 * (it & 1) + rp;
+            uint8_t *unit = gbuf + (size_t)(blkid * 4 + 2 * w + sg) * unit_slot;
+            meta_or4(unit, m, g.W, slot, u.mn);
+            meta_or4(unit + g.mins_bytes, m, g.LB, slot, u.len);
+            uint32_t o = meta + run_off + (rp ? tot_even : 0u) + (inc - pb);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                uint16_t *dst = reinterpret_cast<uint16_t *>(unit + o);
+                uint64_t wd = u.word[k];
+                for (uint32_t q = 0; q < u.len[k]; q++) {
+                    dst[q] = (uint16_t)wd;
+                    wd >>= 16;
+                }
+                o += 2u * u.len[k];
+            }
+        }
+        run_off += tot_even + tot_odd;                    // both rounds of the iteration are behind the unit now
+        if (it & 1) {                                     // the unit (w, it / 2) is complete
+            if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + (it >> 1)] = (uint16_t)(meta + run_off);
+            run_off = 0;
+        }
+    }
+    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+    __syncthreads();
+    const int nblk = 2 * H;
+    if (tid == 0) {
+        uint32_t run = 0;
+        for (int q = 0; q < nblk; q++) {
+            blk_off[q] = run;
+            run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
+        }
+        blk_off[nblk] = run;
+    }
+    __syncthreads();
+    const uint32_t bytes = blk_off[nblk];
+    if (tid < 64) {
+        const uint64_t off = base + lookback_offset(st, gidx, bytes);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < nblk) {
+        const uint32_t first = cb * (uint32_t)(B * nblk) + b * (uint32_t)nblk;
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    // half-wavefront q copies block q: the header of cumulative unit sizes, then its four units one after another
+    const int q = tid >> 5;
+    if (q < nblk) {
+        uint8_t *dst = stream + off + blk_off[q];
+        uint32_t cum = 0;
+#pragma unroll
+        for (int un = 0; un < 4; un++) {
+            const uint32_t n = s_usz[q][un];
+            copy_out32(dst + 8 + cum, gbuf + (size_t)(q * 4 + un) * unit_slot, n, t);
+            cum += n;
+            if (t == un) reinterpret_cast<uint16_t *>(dst)[un] = (uint16_t)cum;
+        }
+    }
+}
+
 static int check_xshape(const void *x, int dtype, int B, int H, int T) {
     PKV_REQUIRE(x != nullptr, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(dtype == PKV_F16 || dtype == PKV_BF16, PKV_ERR_UNSUPPORTED, "Unsupported data type");
@@ -697,7 +889,16 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
         if ((rc = prepare_scan_state(nsub + (shared_params ? (uint32_t)B * (uint32_t)T : 0u), &st, s))) return rc;   // status words, then one word per token
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
-        if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
+        if (!IS_K && H <= 8) {               // one workgroup per group of 2 H blocks
+            const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
+            const uint32_t lds = 64u * unit_slot + 64u;
+            const uint32_t ngroups = (uint32_t)(T / ctx_blk) * (uint32_t)B;
+            auto kern = dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16> : v_quant_encode_rounds_kernel<PKV_BF16>;
+            PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
+                                           stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride);
+        } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
             const uint32_t lds = (uint32_t)H * slot + 32u;
             if (dtype == PKV_F16)
