@@ -181,3 +181,34 @@ def test_attn_decode_full_size_property(cuda):
     err = (got.float() - want).abs().max().item()
     _say("   zero-query mean-of-V check: err %.3e, max|ref| %.3e" % (err, want.abs().max().item()))
     assert err <= 1e-3 * want.abs().max().item() + 2 ** -11 * want.abs().max().item() + 2e-5
+
+
+def test_attn_decode_replays_in_a_hip_graph(cuda):
+    """A decode step launches only kernels on the caller's stream (no allocation once the library's scratch exists,
+    no memset nodes), so a serving loop can capture it: four layers' worth of calls in one graph, replayed with new
+    queries and eager work in between, must reproduce the eager results every time."""
+    B, Hq, Hkv, T, Tw = 2, 16, 4, 1024, 150
+    layers = []
+    for i in range(4):
+        k, v = synth.make_kv(B, Hkv, T + Tw, seed=110 + i, device=cuda)
+        layers.append((ops.k_quant_encode(k[:, :, :T].contiguous(), 0.1), ops.v_quant_encode(v[:, :, :T].contiguous(), 0.1),
+                       k[:, :, T:].contiguous(), v[:, :, T:].contiguous()))
+    q = synth.make_q(B, Hq, seed=120, device=cuda)
+    outs = [torch.empty_like(q) for _ in layers]
+    for (ke, ve, kw, vw), o in zip(layers, outs):       # warm-up: sizes the library's scratch outside the capture
+        ops.attn_decode(q, ke, ve, kw, vw, out=o)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for (ke, ve, kw, vw), o in zip(layers, outs):
+            ops.attn_decode(q, ke, ve, kw, vw, out=o)
+    for rep in range(3):
+        q.copy_(synth.make_q(B, Hq, seed=121 + rep, device=cuda))
+        want = [ops.attn_decode(q, ke, ve, kw, vw) for (ke, ve, kw, vw) in layers]     # eager, own outputs
+        torch.cuda.synchronize()
+        for o in outs:
+            o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, w in zip(outs, want):
+            assert torch.equal(o, w)
