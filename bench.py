@@ -200,7 +200,17 @@ def main():
         codes = torch.empty(Tc, hidden, dtype=torch.uint8, device=dev)
         uk_ms = event_time_ms(torch, lambda: ops.k_decode(ke["stream"], ke["info"], codes, 64, 128, bits), 5)
         uv_ms = event_time_ms(torch, lambda: ops.v_decode(ve["stream"], ve["info"], codes, 128, 64, bits), 5)
-        del codes
+        # token repacking + analytic size on the code matrices (K codes in `codes`, V codes beside them)
+        codes_v = torch.empty(Tc, hidden, dtype=torch.uint8, device=dev)
+        ops.k_decode(ke["stream"], ke["info"], codes, 64, 128, bits)
+        ops.v_decode(ve["stream"], ve["info"], codes_v, 128, 64, bits)
+        rp_ms = event_time_ms(torch, lambda: ops.median_repacking(codes, codes_v, 64), 3)
+        bp_ms = event_time_ms(torch, lambda: ops.bit_pack_bytes(codes, 16), 3)
+        result["repack"] = {
+            "median_repack_ms": rp_ms, "median_repack_gbs": 5 * Tc * hidden / (rp_ms * 1e-3) / 1e9,   # V read twice, K once, both written
+            "bit_pack_size_ms": bp_ms, "bit_pack_size_gbs": Tc * hidden / (bp_ms * 1e-3) / 1e9,
+        }
+        del codes, codes_v
         enc_algo_k = x_bytes + ke["size"] + 8 * nblk_k + 4 * B * Tc
         enc_algo_v = x_bytes + ve["size"] + 8 * nblk_v + 4 * B * Tc
         result["encode"] = {

@@ -117,6 +117,22 @@ int pkv_v_quant_encode_append(const void *x, int dtype, int B, int H, int T_new,
                                void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
                                float *ms_out, pkv_stream_t s);
 
+/* ---- token repacking and the analytic pack-size model ---------------------------------
+ * On the uint8 code matrix [ctx_len, hidden_dim] (channel = (b * H + h) * 128 + d).
+ * pkv_bit_pack_size (utils/compute.py:272-297, `bit_pack`, one of its two halves): packs are
+ *   `pack_len` consecutive tokens of one channel; returns  len_sum = sum over packs of
+ *   bit_length(max - min)  and the number of distinct code values, from which the caller forms
+ *   bytes = (len_sum * pack_len + n_packs * (W + ceil(log2(W + 1)))) / 8,  W = ceil(log2(n_unique)).
+ * pkv_median_repack (utils/compute.py:262-270, `median_repacking`): inside every block of
+ *   `block_size` tokens the tokens of K and V are reordered together by descending lower median
+ *   of the token's V codes over all hidden_dim channels.  Equal medians keep their original order
+ *   (the reference leaves that order to torch.sort's backend).  perm[blk * block_size + r] is
+ *   the index inside the block of the token that moves to position r. */
+int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pack_len, uint64_t *len_sum_out,
+                      uint32_t *n_unique_out, float *ms_out, pkv_stream_t s);
+int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,
+                      int ctx_len, int hidden_dim, int block_size, float *ms_out, pkv_stream_t s);
+
 /* ---- the reference's GEMV surface -----------------------------------------------------
  * kq_mat_vec_mul (packkv_cuda.pyi:26-36, src/kernels.cu:611-630):
  *     kq_out[h, tok] = sum_d q[h, d] * code[tok, h*128 + d]        (dtype, [H, ctx_len])

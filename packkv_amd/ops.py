@@ -8,6 +8,7 @@ for device memory and the current stream only; every computation happens in
 libpackkv_hip.so.
 """
 import ctypes
+import math
 
 import torch
 
@@ -294,6 +295,69 @@ def quant_encode_append(is_k, x, rel, bits, stream, used, info, tokens, scale, z
                 _stream(x.device))
     _lib.check(rc)
     return int(size.value)
+
+
+# ------------------------------------------------- repacking and analytic size ------
+
+def _check_code_matrix(c, name):
+    _require(c.is_cuda and c.dim() == 2 and c.dtype == torch.uint8 and c.is_contiguous(),
+             "%s must be a contiguous device UInt8 code matrix [ctx_len, hidden]" % name)
+
+
+def bit_pack_bytes(codes, pack_len, timed=False):
+    """Analytic size of ONE code matrix [ctx_len, hidden] in bytes, as `bit_pack` prices each half
+    (utils/compute.py:272-297): packs of `pack_len` consecutive tokens of one channel cost
+    pack_len * bit_length(max - min) payload bits + W + ceil(log2(W + 1)) metadata bits, W = ceil(log2(#codes))."""
+    _check_code_matrix(codes, "codes")
+    ctx, hidden = codes.shape
+    len_sum, n_unique, ms = ctypes.c_uint64(0), ctypes.c_uint32(0), ctypes.c_float(0.0)
+    with torch.cuda.device(codes.device):
+        rc = _lib.load().pkv_bit_pack_size(_ptr(codes), ctx, hidden, int(pack_len), ctypes.byref(len_sum),
+                                           ctypes.byref(n_unique), ctypes.byref(ms) if timed else None,
+                                           _stream(codes.device))
+    _lib.check(rc)
+    w = math.ceil(math.log2(n_unique.value))
+    n_packs = (ctx // pack_len) * hidden
+    size = (int(len_sum.value) * pack_len + n_packs * (w + math.ceil(math.log2(w + 1)))) // 8
+    return (size, float(ms.value)) if timed else size
+
+
+def bit_pack(k_codes, v_codes, pack_len):
+    """(k_bytes, v_bytes) of `bit_pack(blocks, pack_len)` (utils/compute.py:272-297) for blocks = K and V codes
+    side by side."""
+    return bit_pack_bytes(k_codes, pack_len), bit_pack_bytes(v_codes, pack_len)
+
+
+def median_repacking(k_codes, v_codes, block_size=64, timed=False):
+    """`median_repacking` (utils/compute.py:262-270) on the device: inside every block of `block_size` tokens, K and
+    V rows are reordered together by descending median of the token's V codes; equal medians keep their order.
+    Returns (k_repacked, v_repacked, perm) with perm [ctx_len] int32: perm[blk * block_size + r] = position inside the
+    block the token at r came from."""
+    _check_code_matrix(k_codes, "k_codes")
+    _check_code_matrix(v_codes, "v_codes")
+    _require(k_codes.shape == v_codes.shape, "K and V code matrices must have one shape")
+    ctx, hidden = k_codes.shape
+    k_out, v_out = torch.empty_like(k_codes), torch.empty_like(v_codes)
+    perm = torch.empty(ctx, dtype=torch.int32, device=k_codes.device)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(k_codes.device):
+        rc = _lib.load().pkv_median_repack(_ptr(k_codes), _ptr(v_codes), _ptr(k_out), _ptr(v_out), _ptr(perm), ctx,
+                                           hidden, int(block_size), ctypes.byref(ms) if timed else None,
+                                           _stream(k_codes.device))
+    _lib.check(rc)
+    return (k_out, v_out, perm, float(ms.value)) if timed else (k_out, v_out, perm)
+
+
+def repack_and_encode(k_codes, v_codes, pack_size, repack_method="none", block_size=64):
+    """`repack_and_encode` (utils/compute.py:329-357) on code matrices: (k_size_pre, v_size_pre, k_size_aft,
+    v_size_aft) in bytes.  repack_method: "none" or "median" (the greedy method is not built)."""
+    k_pre, v_pre = bit_pack(k_codes, v_codes, pack_size)
+    if repack_method == "median":
+        k_codes, v_codes, _ = median_repacking(k_codes, v_codes, block_size)
+    elif repack_method != "none":
+        raise ValueError("repack_method must be one of none, median")
+    k_aft, v_aft = bit_pack(k_codes, v_codes, pack_size)
+    return k_pre, v_pre, k_aft, v_aft
 
 
 # ------------------------------------------------------- reference GEMV surface ------

@@ -1,0 +1,94 @@
+"""Token repacking and the analytic size model on the device against the NumPy restatement (oracle/repack.py):
+integers throughout, so everything is compared exactly."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from oracle import repack as orp
+from packkv_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _codes(B, H, T, rel, seed, k_mode="outliers"):
+    k, v = synth.make_kv(B, H, T, seed=seed, k_mode=k_mode)
+    ck, _, _ = oq.quant_ints(k, 64, rel)
+    cv, _, _ = oq.quant_ints(v, 64, rel)
+    return oq.code_matrix(ck), oq.code_matrix(cv)
+
+
+@pytest.mark.parametrize("rel", [0.1, 0.05, 0.02])
+def test_bit_pack_sizes_match_for_every_pack_length(cuda, rel):
+    """rel 0.05 / 0.02 give code widths up to 6 / 7 bits: the size model has no width limit."""
+    kc, vc = _codes(1, 8, 2048, rel, seed=130, k_mode="channel_scale")
+    kd, vd = kc.to(cuda), vc.to(cuda)
+    blocks = orp.blocks_from_code_matrices(kc.numpy(), vc.numpy(), 64)
+    for pack_len in (16, 32, 64, 128, 256):
+        want = orp.bit_pack(blocks, pack_len)
+        got = ops.bit_pack(kd, vd, pack_len)
+        _say("bit_pack case rel", rel, "pack", pack_len, "->", got, "max code", int(kc.max()), int(vc.max()))
+        assert got == want
+
+
+def test_median_repacking_matches_restatement(cuda):
+    for (B, H, T, bs) in ((1, 2, 256, 64), (2, 8, 512, 64), (1, 1, 384, 128), (3, 2, 128, 16)):
+        _say("repack case", B, H, T, bs)
+        kc, vc = _codes(B, H, T, 0.1, seed=140 + B)
+        blocks = orp.blocks_from_code_matrices(kc.numpy(), vc.numpy(), bs)
+        want, order = orp.median_repacking(blocks)
+        k_out, v_out, perm = ops.median_repacking(kc.to(cuda), vc.to(cuda), bs)
+        hid = kc.shape[1]
+        assert (perm.cpu().numpy().reshape(-1, bs) == order).all()
+        assert (k_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, :hid]).all()
+        assert (v_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, hid:]).all()
+        for pack in (16, 64):
+            assert ops.repack_and_encode(kc.to(cuda), vc.to(cuda), pack, "median", bs) == \
+                   orp.repack_and_encode(kc.numpy(), vc.numpy(), pack, "median", bs)
+            assert ops.repack_and_encode(kc.to(cuda), vc.to(cuda), pack, "none", bs) == \
+                   orp.repack_and_encode(kc.numpy(), vc.numpy(), pack, "none", bs)
+
+
+def test_repacked_codes_encode_and_round_trip(cuda):
+    """Repacked code matrices go through the codecs like any other: stream decodes to the repacked codes, and the
+    real K stream of 16-token packs is priced by bit_pack up to the block headers."""
+    B, H, T = 1, 8, 512
+    kc, vc = _codes(B, H, T, 0.1, seed=150)
+    k_rep, v_rep, _ = ops.median_repacking(kc.to(cuda), vc.to(cuda), 64)
+    hid = kc.shape[1]
+    stream = torch.empty(T * hid, dtype=torch.uint8, device=cuda)
+    info = torch.empty((T // 64) * (hid // 128), 2, dtype=torch.uint32, device=cuda)
+    size = ops.k_encode(k_rep, stream, info, bits=4)
+    back = torch.empty_like(k_rep)
+    ops.k_decode(stream, info, back, bits=4)
+    assert torch.equal(back, k_rep)
+    # real stream = analytic payload and metadata (4 + 3 bits per pack at W = 4) + 8 header bytes per block
+    n_packs = (T // 16) * hid
+    analytic_bits = ops.bit_pack_bytes(k_rep, 16) * 8
+    w = int(np.ceil(np.log2(len(torch.unique(k_rep)))))
+    payload_bits = analytic_bits - n_packs * (w + int(np.ceil(np.log2(w + 1))))
+    assert abs(size - ((payload_bits + n_packs * 7) // 8 + 8 * info.size(0))) <= 1
+
+
+def test_full_size_properties(cuda):
+    """configs[2] shape (8 KV heads x 128 x 16384 tokens): the oracle is slow there, so check what must hold:
+    perm is a permutation inside every block, rows move with it, medians come out non-increasing, and repacking
+    leaves the multiset of codes (hence the histogram and W) unchanged."""
+    T, hid, bs = 16384, 1024, 64
+    g = torch.Generator(device="cpu").manual_seed(160)
+    kc = torch.randint(0, 16, (T, hid), dtype=torch.uint8, generator=g).to(cuda)
+    vc = (torch.randn(T, 1, generator=g).mul(2).add(8).round().clamp(0, 15) +
+          torch.randint(-2, 3, (T, hid), generator=g)).clamp(0, 15).to(torch.uint8).to(cuda)
+    k_out, v_out, perm = ops.median_repacking(kc, vc, bs)
+    p = perm.view(-1, bs).long()
+    assert torch.equal(torch.sort(p, dim=1).values, torch.arange(bs, device=cuda).expand_as(p))
+    src = (torch.arange(T, device=cuda).view(-1, bs)[:, :1] + p).view(-1)
+    assert torch.equal(k_out, kc[src]) and torch.equal(v_out, vc[src])
+    med = torch.median(v_out.view(-1, bs, hid).to(torch.int16), dim=2).values
+    assert (med[:, :-1] >= med[:, 1:]).all()
+    assert torch.equal(torch.bincount(v_out.view(-1).long(), minlength=16), torch.bincount(vc.view(-1).long(), minlength=16))
+    assert ops.bit_pack_bytes(v_out, 16) <= ops.bit_pack_bytes(vc, 16)     # sorting by level helps this input

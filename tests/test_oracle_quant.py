@@ -115,3 +115,32 @@ def test_simulated_cache_follows_the_cut_policy():
     one, nil = torch.ones(B, 8, 128, dtype=t.dtype), torch.zeros(B, 8, 128, dtype=t.dtype)
     assert torch.equal(oc.apply_rotary_pos_emb_single(t, one, nil), t)
     assert torch.equal(oc.apply_rotary_pos_emb_single(t, nil, one), torch.cat((-t[..., 64:], t[..., :64]), dim=-1))
+
+
+def test_repack_restatement_against_library_routines():
+    """median = torch.median (lower median on even counts), order = torch.sort(descending, stable); bit_pack =
+    the single-tensor closed form; a hand-made block where the answer is known."""
+    from oracle import repack as orp
+    rng = np.random.default_rng(3)
+    blocks = rng.integers(0, 6, size=(5, 64, 2 * 96))
+    med = orp.token_medians(blocks)
+    want = torch.median(torch.from_numpy(blocks[:, :, 96:]), dim=2).values.numpy()
+    assert (med == want).all()
+    rep, order = orp.median_repacking(blocks)
+    _, idx = torch.sort(torch.from_numpy(med), dim=1, descending=True, stable=True)
+    assert (order == idx.numpy()).all()
+    assert (rep == np.take_along_axis(blocks, idx.numpy()[:, :, None], axis=1)).all()
+    m2 = orp.token_medians(rep)
+    assert (m2[:, :-1] >= m2[:, 1:]).all()                       # descending medians
+    assert (np.sort(rep, axis=1) == np.sort(blocks, axis=1)).all()   # same tokens
+    for pack_len in (16, 32, 64):
+        kb, vb = orp.bit_pack(blocks, pack_len)
+        flat = blocks.reshape(-1, 192)
+        assert kb == oq.bit_pack_bytes(flat[:, :96], pack_len) and vb == oq.bit_pack_bytes(flat[:, 96:], pack_len)
+    # 2 tokens-blocks of 4 tokens, 1 K + 1 V channel... token medians 3, 9, 9, 1 -> order 1, 2, 0, 3 (tie keeps 1 before 2)
+    b = np.array([[[10, 3], [11, 9], [12, 9], [13, 1]]])
+    rep, order = orp.median_repacking(b)
+    assert order.tolist() == [[1, 2, 0, 3]] and rep[0, :, 0].tolist() == [11, 12, 10, 13]
+    # packs of 2 tokens: K (11,12) (10,13) -> ranges 1, 3 -> 1 + 2 bits; 4 distinct values -> W = 2, 2 + 2 metadata bits
+    kb, vb = orp.bit_pack(rep, 2)
+    assert kb == ((1 + 2) * 2 + 2 * (2 + 2)) // 8
