@@ -32,11 +32,15 @@ __global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t
     // coalesced write-back: rows of hid_blk bytes, as dwords
     const int row_dw = hid_blk >> 2;
     const uint32_t *t4 = reinterpret_cast<const uint32_t *>(tile);
+    // (row, column) advance by the workgroup size without a division per element
+    const int step_row = (int)blockDim.x / row_dw, step_c = (int)blockDim.x % row_dw;
+    int row = (int)threadIdx.x / row_dw, c = (int)threadIdx.x % row_dw;
+    uint8_t *base = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
     for (int i = threadIdx.x; i < ctx_blk * row_dw; i += blockDim.x) {
-        const int row = i / row_dw, c = i % row_dw;
-        uint32_t *dst = reinterpret_cast<uint32_t *>(
-            codes + ((size_t)cb * ctx_blk + row) * hidden_dim + (size_t)hb * hid_blk);
-        dst[c] = t4[i];
+        reinterpret_cast<uint32_t *>(base + (size_t)row * hidden_dim)[c] = t4[i];
+        row += step_row;
+        c += step_c;
+        if (c >= row_dw) { c -= row_dw; row++; }
     }
 }
 
@@ -59,11 +63,24 @@ __global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restri
     const uint32_t cb = b / n_hid, hb = b % n_hid;
     const int row_dw = hid_blk >> 2;
     uint32_t *t4 = reinterpret_cast<uint32_t *>(tile);
-    for (int i = threadIdx.x; i < ctx_blk * row_dw; i += blockDim.x) {
-        const int row = i / row_dw, c = i % row_dw;
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(
-            codes + ((size_t)cb * ctx_blk + row) * hidden_dim + (size_t)hb * hid_blk);
-        t4[i] = src[c];
+    {   // (row, column) advance by the workgroup size without a division per element; four loads in flight
+        const int step_row = (int)blockDim.x / row_dw, step_c = (int)blockDim.x % row_dw;
+        int row = (int)threadIdx.x / row_dw, c = (int)threadIdx.x % row_dw;
+        const uint8_t *base = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+        const int n = ctx_blk * row_dw;
+        for (int i = threadIdx.x; i < n; i += 4 * (int)blockDim.x) {
+            uint32_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                v[u] = i + u * (int)blockDim.x < n ? reinterpret_cast<const uint32_t *>(base + (size_t)row * hidden_dim)[c] : 0u;
+                row += step_row;
+                c += step_c;
+                if (c >= row_dw) { c -= row_dw; row++; }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * (int)blockDim.x < n) t4[i + u * (int)blockDim.x] = v[u];
+        }
     }
     __syncthreads();
     block_finish<IS_K>(tile, blk, unit_bytes, &s_off, st, b, nblocks, stream, capacity, info, hid_blk,

@@ -135,7 +135,20 @@ __device__ __forceinline__ uint32_t stage_to_lds(const uint8_t *src, uint32_t nb
     const uint32_t *s4 = reinterpret_cast<const uint32_t *>(src - phase);
     uint32_t *d4 = reinterpret_cast<uint32_t *>(dst);
     const uint32_t ndw = (phase + nbytes + 3u) >> 2;
-    for (uint32_t i = tid; i < ndw; i += nthreads) d4[i] = s4[i];
+    // four loads in flight per thread before the first LDS store: the copy is latency-bound otherwise
+    for (uint32_t i = tid; i < ndw; i += 4u * (uint32_t)nthreads) {
+        uint32_t v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t idx = i + (uint32_t)u * (uint32_t)nthreads;
+            v[u] = idx < ndw ? s4[idx] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t idx = i + (uint32_t)u * (uint32_t)nthreads;
+            if (idx < ndw) d4[idx] = v[u];
+        }
+    }
     return phase;
 }
 
