@@ -44,6 +44,45 @@ __global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t
     }
 }
 
+// V blocks of 64 channels, two adjacent ones (the two halves of a head) per workgroup of 256 threads: the pair
+// decodes into one tile of 128 tokens x 128 channels, so the write-back stores whole 128-byte lines.  In tile
+// addressing the pair is a V block of 128 channels whose units 4 j + u are the units u of block j.
+__global__ void __launch_bounds__(256) unpack_v_pair_kernel(const uint8_t *__restrict__ stream,
+                                                            const uint32_t *__restrict__ info,
+                                                            uint8_t *__restrict__ codes, int hidden_dim, int W,
+                                                            uint32_t blk_cap) {
+    constexpr int kCtx = 128, kPairHid = 128;
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t *tile = lds;
+    const uint32_t blk_stride = round_up16(blk_cap) + 32u;
+    const int n_pair = hidden_dim / kPairHid;
+    const uint32_t cb = blockIdx.x / n_pair, hp = blockIdx.x % n_pair;
+    const uint32_t b0 = cb * (uint32_t)(2 * n_pair) + 2u * hp;
+    const int tid = threadIdx.x;
+    const int j = tid >> 7;                                   // which block of the pair this half of the workgroup serves
+    uint8_t *blk = lds + kCtx * kPairHid + j * blk_stride;
+    const uint32_t off = info[2 * (b0 + j)];
+    uint32_t size = info[2 * (b0 + j) + 1];
+    if (size > blk_cap) size = blk_cap;   // corrupt block_info must not overrun LDS
+    const uint32_t phase = stage_to_lds(stream + off, size, blk, tid & 127, 128);
+    __syncthreads();
+    {
+        const UnitGeom g = unit_geom(W);
+        const int t = tid & 31, u = (tid >> 5) & 3;
+        const uint16_t *cum = reinterpret_cast<const uint16_t *>(blk + phase);
+        const uint32_t start = phase + 8u + (u ? (uint32_t)cum[u - 1] : 0u);
+        unit_decode<false>(blk, min(start, blk_cap), 4 * j + u, t, g, tile, kPairHid);
+    }
+    __syncthreads();
+    const uint4 *t16 = reinterpret_cast<const uint4 *>(tile);
+    uint8_t *base = codes + (size_t)cb * kCtx * hidden_dim + (size_t)hp * kPairHid;
+#pragma unroll
+    for (int i = 0; i < kCtx * kPairHid / 16 / 256; i++) {     // 8 rows of 128 bytes per step, 16 bytes per thread
+        const int idx = tid + 256 * i;
+        *reinterpret_cast<uint4 *>(base + (size_t)(idx >> 3) * hidden_dim + 16 * (idx & 7)) = t16[idx];
+    }
+}
+
 template <bool IS_K>
 __global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                             uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
@@ -137,6 +176,9 @@ static int run_unpack(bool is_k, const uint8_t *stream, const uint32_t *info, ui
     if (is_k)
         unpack_kernel<true><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
             stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
+    else if (hid_blk == 64 && hidden_dim % 128 == 0 && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0)
+        unpack_v_pair_kernel<<<cs.nblocks / 2, 256, 128 * 128 + 2 * (round_up16(cs.blk_cap) + 32u), s>>>(
+            stream, info, codes, hidden_dim, bits, cs.blk_cap);
     else
         unpack_kernel<false><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
             stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
