@@ -176,7 +176,15 @@ __global__ void dequantize_kernel(const uint8_t *__restrict__ codes, int H, int 
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-struct TokPar { float s, r; uint32_t neg_zero2, pad; };   // scale, 1 / scale, (-zero, -zero) as two fp16 (or zero as fp32 bits for bf16)
+// Per-token constants: scale, 1 / scale, and for fp16 either
+//   sub2 != 0 (zero in [-500, 3000], the usual case): add2 = (c, c) with c = 1536 + (zero & 1) - zero as fp16 and
+//             sub2 = (0x6600 + (zero & 1)) in both halves.  h + c is then one correctly rounded fp16 addition whose
+//             result lies in [1535.5, 2048), where the spacing is 1: it rounds h - zero to an integer, and because
+//             c - zero is even a tie goes to the same side as in rint(h).  The code is the result's bit pattern
+//             minus sub2 -- no separate rounding instruction;
+//   sub2 == 0: add2 = (-zero, -zero) for the general sequence rint(h) + (-zero).
+// bf16: add2 = zero as fp32 bits.
+struct TokPar { float s, r; uint32_t add2, sub2; };
 
 __device__ __forceinline__ uint32_t pk_u16(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
@@ -193,13 +201,20 @@ __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01,
             return (_Float16)__fmaf_rn(e, tp.r, q0);
         };
         const f16x2 h01 = {quot(x01[0]), quot(x01[1])}, h23 = {quot(x23[0]), quot(x23[1])};
-        const f16x2 nz = __builtin_bit_cast(f16x2, tp.neg_zero2);
-        const f16x2 magic = {(_Float16)1024.f, (_Float16)1024.f};    // 1024 + c has c in its low mantissa bits
-        const f16x2 d01 = __builtin_elementwise_roundeven(h01) + nz, d23 = __builtin_elementwise_roundeven(h23) + nz;
-        c01 = __builtin_bit_cast(uint32_t, (f16x2)(d01 + magic)) & 0x00FF00FFu;
-        c23 = __builtin_bit_cast(uint32_t, (f16x2)(d23 + magic)) & 0x00FF00FFu;
+        const f16x2 add = __builtin_bit_cast(f16x2, tp.add2);
+        // every lane of the wavefront holds the same token constants: a uniform branch
+        if (__builtin_amdgcn_readfirstlane(tp.sub2) != 0u) {
+            const u16x2 sub = as_u16x2(tp.sub2);
+            c01 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h01 + add)) - sub));
+            c23 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h23 + add)) - sub));
+        } else {
+            const f16x2 magic = {(_Float16)1024.f, (_Float16)1024.f};    // 1024 + c has c in its low mantissa bits
+            const f16x2 d01 = __builtin_elementwise_roundeven(h01) + add, d23 = __builtin_elementwise_roundeven(h23) + add;
+            c01 = __builtin_bit_cast(uint32_t, (f16x2)(d01 + magic)) & 0x00FF00FFu;
+            c23 = __builtin_bit_cast(uint32_t, (f16x2)(d23 + magic)) & 0x00FF00FFu;
+        }
     } else {
-        const float z = __uint_as_float(tp.neg_zero2);
+        const float z = __uint_as_float(tp.add2);
         const uint32_t a = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.x & 0xFFFFu), tp.s, z) & 0xFFu;
         const uint32_t b = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.x >> 16), tp.s, z) & 0xFFu;
         const uint32_t c = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.y & 0xFFFFu), tp.s, z) & 0xFFu;
@@ -287,8 +302,19 @@ __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
     TokPar tp;
     tp.s = sc;
     tp.r = r;
-    tp.neg_zero2 = DT == PKV_F16 ? ((zero_bits ^ 0x8000u) * 0x00010001u) : __float_as_uint(T16<DT>::from_bits(zero_bits));
-    tp.pad = 0;
+    tp.sub2 = 0;
+    if (DT == PKV_F16) {
+        const float z = T16<DT>::from_bits(zero_bits);        // an integer (or inf / nan for degenerate tokens)
+        if (z >= -500.f && z <= 3000.f) {
+            const int zi = (int)z, odd = zi & 1;
+            tp.add2 = (uint32_t)__half_as_ushort(__float2half_rn((float)(1536 + odd - zi))) * 0x00010001u;   // exact: |c| < 2048
+            tp.sub2 = (uint32_t)(0x6600 + odd) * 0x00010001u;
+        } else {
+            tp.add2 = (zero_bits ^ 0x8000u) * 0x00010001u;
+        }
+    } else {
+        tp.add2 = __float_as_uint(T16<DT>::from_bits(zero_bits));
+    }
     return tp;
 }
 
