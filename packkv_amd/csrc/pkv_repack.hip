@@ -13,33 +13,71 @@
 
 namespace pkv {
 
-// ---- lower median of every token row: one wavefront per token, 256-bin histogram in LDS ----
+// ---- lower median of every token row: one wavefront per token ----
+// Rows of up to 16384 codes below 128 stay in registers (16 bytes x 16 per lane) and the median is found by
+// bisection on the value: a step counts the bytes above the probe with three word-wide instructions per four codes
+// ((x | 0x80) - (probe + 1) keeps bit 7 of a byte exactly when the byte is above the probe; no borrow crosses bytes
+// while both are at most 128).  Other rows use a 256-bin histogram in LDS (slow when few values dominate: equal
+// addresses serialise the LDS atomics).
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
+    return x;
+}
+
 __global__ void __launch_bounds__(256) token_median_kernel(const uint8_t *__restrict__ codes, int ctx_len, int hidden,
                                                            uint8_t *__restrict__ median) {
     __shared__ uint32_t hist[4][256];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int tok = blockIdx.x * 4 + wave;
+    if (tok >= ctx_len) return;                                   // whole wavefronts leave; no workgroup barrier below
+    const uint4 *row = reinterpret_cast<const uint4 *>(codes + (size_t)tok * hidden);
+    const int nchunks = hidden / 16;
+    const uint32_t k = (uint32_t)(hidden - 1) / 2u;               // torch.median: the lower of the two middle values
+    if (nchunks <= 16 * 64) {
+        uint32_t w[64];
+        uint32_t high = 0u;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int c = lane + 64 * i;
+            const uint4 v = c < nchunks ? row[c] : make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+            high |= v.x | v.y | v.z | v.w;
+        }
+        if (__ballot((high & 0x80808080u) != 0u) == 0ull) {
+            const uint32_t n_pad = (uint32_t)(16 * 64 * 16 - hidden);   // padding bytes hold 127: above every probe
+            uint32_t lo = 0u, hi = 127u;
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi) >> 1;
+                const uint32_t cmpw = (mid + 1u) * 0x01010101u;
+                uint32_t above = 0u;
+#pragma unroll
+                for (int i = 0; i < 64; i++)
+                    above += (uint32_t)__builtin_popcount(((w[i] | 0x80808080u) - cmpw) & 0x80808080u);
+                above = wave_sum_u32(above) - n_pad;
+                if ((uint32_t)hidden - above >= k + 1u) hi = mid; else lo = mid + 1u;   // codes <= mid reach rank k
+            }
+            if (lane == 0) median[tok] = (uint8_t)lo;
+            return;
+        }
+    }
     uint32_t *h = hist[wave];
     for (int i = lane; i < 256; i += 64) h[i] = 0u;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (tok < ctx_len) {
-        const uint4 *row = reinterpret_cast<const uint4 *>(codes + (size_t)tok * hidden);   // hidden % 128 == 0
-        for (int c = lane; c < hidden / 16; c += 64) {
-            const uint4 v = row[c];
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int c = lane; c < nchunks; c += 64) {
+        const uint4 v = row[c];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int k = 0; k < 4; k++) atomicAdd(&h[(w[i] >> (8 * k)) & 0xFFu], 1u);
-        }
+            for (int kk = 0; kk < 4; kk++) atomicAdd(&h[(w[i] >> (8 * kk)) & 0xFFu], 1u);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (tok >= ctx_len) return;
-    // lane l owns bins 4l..4l+3; torch.median returns the lower of the two middle values: rank (n - 1) / 2
+    // lane l owns bins 4l..4l+3
     const uint32_t c0 = h[4 * lane], c1 = h[4 * lane + 1], c2 = h[4 * lane + 2], c3 = h[4 * lane + 3];
     const uint32_t mine = c0 + c1 + c2 + c3;
     uint32_t inc = mine;
@@ -48,13 +86,13 @@ __global__ void __launch_bounds__(256) token_median_kernel(const uint8_t *__rest
         const uint32_t up = __shfl_up(inc, d, 64);
         if (lane >= d) inc += up;
     }
-    const uint32_t before = inc - mine, k = (uint32_t)(hidden - 1) / 2u;
+    const uint32_t before = inc - mine;
     if (before <= k && k < inc) {
-        uint32_t b = 4 * lane, run = before + c0;
-        if (k >= run) { b++; run += c1; }
-        if (k >= run) { b++; run += c2; }
-        if (k >= run) b++;
-        median[tok] = (uint8_t)b;
+        uint32_t bin = 4 * lane, run = before + c0;
+        if (k >= run) { bin++; run += c1; }
+        if (k >= run) { bin++; run += c2; }
+        if (k >= run) bin++;
+        median[tok] = (uint8_t)bin;
     }
 }
 

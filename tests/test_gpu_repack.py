@@ -92,3 +92,20 @@ def test_full_size_properties(cuda):
     assert (med[:, :-1] >= med[:, 1:]).all()
     assert torch.equal(torch.bincount(v_out.view(-1).long(), minlength=16), torch.bincount(vc.view(-1).long(), minlength=16))
     assert ops.bit_pack_bytes(v_out, 16) <= ops.bit_pack_bytes(vc, 16)     # sorting by level helps this input
+
+
+def test_median_repacking_wide_codes_and_wide_rows(cuda):
+    """Codes of 128 and above and rows longer than 16384 channels take the kernel's histogram path; a row of
+    exactly 16384 codes below 128 fills the register path completely."""
+    g = torch.Generator(device="cpu").manual_seed(170)
+    for (T, hid, top, bs) in ((128, 256, 256, 64), (64, 32768, 16, 64), (64, 16384, 128, 32), (128, 1040, 100, 64)):
+        _say("repack wide case", T, hid, top, bs)
+        kc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
+        vc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
+        vc[::3] //= 2                                   # spread the medians
+        blocks = orp.blocks_from_code_matrices(kc.numpy(), vc.numpy(), bs)
+        want, order = orp.median_repacking(blocks)
+        k_out, v_out, perm = ops.median_repacking(kc.to(cuda), vc.to(cuda), bs)
+        assert (perm.cpu().numpy().reshape(-1, bs) == order).all()
+        assert (v_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, hid:]).all()
+        assert (k_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, :hid]).all()
