@@ -56,8 +56,12 @@ uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits);
  * (packkv_cuda_ext/packkv_cuda.pyi:4-24, :38-58; src/k_encode_cpu.cpp:286-331,
  * src/v_encode_cpu.cpp:301-346, src/k_decode_cpu.cpp:281-326, src/v_decode_cpu.cpp:258-303).
  * Generalised from the reference's dispatch table to any hidden_dim that is a multiple of
- * the block width, bits in {2,3,4}; K blocks are ctx_blk x 128 (ctx_blk a multiple of 16,
+ * the block width, bits in 2..8; K blocks are ctx_blk x 128 (ctx_blk a multiple of 16,
  * at most 256), V blocks are 128 x hid_blk (hid_blk a multiple of 32, at most 256).
+ * bits 5..8 are an extension of the format: the reference stops at 16 * bits <= 64 bits per
+ * pack word (src/k_encode_cpu.cpp:211); here the same layout rules run on with pack words of
+ * up to 128 bits and a 4-bit length field at bits = 8.  A stream of such codes can be larger
+ * than the code matrix: size the buffer with pkv_block_bound.
  * `capacity` = bytes available at `stream`; `size_out` (host, may be NULL) receives the
  * stream size and makes the call synchronous. */
 int pkv_k_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,

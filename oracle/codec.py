@@ -42,12 +42,19 @@ class _Codec:
         self.enc.argtypes = [ctypes.c_int, _u8p, _u8p, _u32p] + [ctypes.c_int] * 5
         self.dec.restype = ctypes.c_int
         self.dec.argtypes = [ctypes.c_int, _u8p, _u32p, _u8p] + [ctypes.c_int] * 5
+        self.bound = getattr(self.lib, prefix + "_block_bound", None)     # the restated codec only
+        if self.bound is not None:
+            self.bound.restype = ctypes.c_uint64
+            self.bound.argtypes = [ctypes.c_int] * 4
 
     def encode(self, is_k, codes, ctx_blk, hid_blk, W):
         codes = np.ascontiguousarray(codes, dtype=np.uint8)
         ctx_len, hidden = codes.shape
         nblk = (ctx_len // ctx_blk) * (hidden // hid_blk)
-        stream = np.zeros(ctx_len * hidden, dtype=np.uint8)
+        # the reference sizes the buffer like the code matrix (evaluation/evaluation.py:426); widths above 4
+        # (this build's extension) can exceed that, so take the worst case when it is larger
+        bound = int(self.bound(int(is_k), ctx_blk, hid_blk, W)) if self.bound is not None else 0
+        stream = np.zeros(max(ctx_len * hidden, nblk * bound), dtype=np.uint8)
         info = np.zeros((nblk, 2), dtype=np.uint32)
         size = self.enc(int(is_k), codes.ctypes.data_as(_u8p), stream.ctypes.data_as(_u8p),
                         info.ctypes.data_as(_u32p), ctx_len, hidden, ctx_blk, hid_blk, W)

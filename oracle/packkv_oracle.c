@@ -20,6 +20,12 @@
  * stream + block_info for W in {2,3,4}), the committed golden vectors made
  * from that build, and closed-form block sizes / byte patterns in the tests.
  *
+ * W in 5..8 is a FORMAT EXTENSION of this build (the reference stops at 16 * W <= 64 bits
+ * per pack word, k_encode_cpu.cpp:211): the same layout rules with pack words of up to 128
+ * bits.  No reference exists for it -- parity unpinned; it is pinned by encode -> decode round
+ * trips, by the closed-form block sizes and by the reference's analytic size model
+ * (utils/compute.py:272-297), which has no width limit.
+ *
  * Layout facts restated here:
  *   - a pack is 16 consecutive tokens of one channel; min, len = bit_length(max-min);
  *     word = sum_k (code_k - min) << ((15-k)*len); stored as the low 2*len bytes, LE.
@@ -36,6 +42,7 @@
 #include <string.h>
 
 #define PACK_TOK 16
+typedef unsigned __int128 pkv_word;   /* 16 fields of up to 8 bits */
 #define LANES 32
 
 static int len_field_bits(int W) { /* include/utils.h:24-36 with n = W */
@@ -67,7 +74,7 @@ static unsigned get_bits(const uint8_t *base, size_t bitpos, int nbits) {
 
 /* min, len and word of the pack holding tokens tok0..tok0+15 of channel ch. */
 static void pack_stats(const uint8_t *codes, size_t row_stride, size_t tok0, size_t ch,
-                       unsigned *mn_out, int *len_out, uint64_t *word_out) {
+                       unsigned *mn_out, int *len_out, pkv_word *word_out) {
     unsigned mn = 255, mx = 0;
     for (int k = 0; k < PACK_TOK; k++) {
         unsigned c = codes[(tok0 + k) * row_stride + ch];
@@ -75,32 +82,32 @@ static void pack_stats(const uint8_t *codes, size_t row_stride, size_t tok0, siz
         if (c > mx) mx = c;
     }
     int len = bit_length(mx - mn);
-    uint64_t word = 0;
+    pkv_word word = 0;
     for (int k = 0; k < PACK_TOK; k++) {
         unsigned c = codes[(tok0 + k) * row_stride + ch];
-        word = (len ? (word << len) : 0) | (uint64_t)(c - mn);
+        word = (len ? (word << len) : 0) | (pkv_word)(c - mn);
     }
     *mn_out = mn; *len_out = len; *word_out = word;
 }
 
-static size_t put_word(uint8_t *dst, uint64_t word, int len) {
+static size_t put_word(uint8_t *dst, pkv_word word, int len) {
     size_t n = (size_t)len * PACK_TOK / 8;
     for (size_t i = 0; i < n; i++) { dst[i] = (uint8_t)(word & 0xFF); word >>= 8; }
     return n;
 }
 
-static uint64_t get_word(const uint8_t *src, int len) {
+static pkv_word get_word(const uint8_t *src, int len) {
     size_t n = (size_t)len * PACK_TOK / 8;
-    uint64_t w = 0;
-    for (size_t i = 0; i < n; i++) w |= (uint64_t)src[i] << (8 * i);
+    pkv_word w = 0;
+    for (size_t i = 0; i < n; i++) w |= (pkv_word)src[i] << (8 * i);
     return w;
 }
 
 static void unpack_word(uint8_t *codes, size_t row_stride, size_t tok0, size_t ch,
-                        uint64_t word, int len, unsigned mn) {
-    uint64_t mask = len ? ((1ull << len) - 1) : 0;
+                        pkv_word word, int len, unsigned mn) {
+    unsigned mask = len ? ((1u << len) - 1) : 0;
     for (int k = PACK_TOK - 1; k >= 0; k--) {
-        codes[(tok0 + k) * row_stride + ch] = (uint8_t)((word & mask) + mn);
+        codes[(tok0 + k) * row_stride + ch] = (uint8_t)(((unsigned)word & mask) + mn);
         word = len ? (word >> len) : 0;
     }
 }
@@ -124,7 +131,7 @@ size_t pkv_oracle_k_block_encode(const uint8_t *codes, size_t row_stride, int ct
         size_t pay = 0;
         for (int j = 0; j < hid_blk; j++) {
             int ch = (j % LANES) * per_lane + j / LANES;
-            unsigned mn; int len; uint64_t word;
+            unsigned mn; int len; pkv_word word;
             pack_stats(codes, row_stride, (size_t)r * PACK_TOK, (size_t)ch, &mn, &len, &word);
             put_bits(mins, (size_t)ch * W, W, mn);
             put_bits(lens, (size_t)ch * LB, LB, (unsigned)len);
@@ -158,7 +165,7 @@ void pkv_oracle_k_block_decode(const uint8_t *in, int ctx_blk, int hid_blk, int 
             int ch = (j % LANES) * per_lane + j / LANES;
             unsigned mn = get_bits(mins, (size_t)ch * W, W);
             int len = (int)get_bits(lens, (size_t)ch * LB, LB);
-            uint64_t word = get_word(payload + pay, len);
+            pkv_word word = get_word(payload + pay, len);
             pay += (size_t)len * PACK_TOK / 8;
             unpack_word(codes, row_stride, (size_t)r * PACK_TOK, (size_t)ch, word, len, mn);
         }
@@ -190,7 +197,7 @@ size_t pkv_oracle_v_block_encode(const uint8_t *codes, size_t row_stride, int ct
             size_t pay = 0;
             for (int i = 0; i < V_SLOTS; i++) {
                 for (int t = 0; t < LANES; t++) {
-                    unsigned mn; int len; uint64_t word;
+                    unsigned mn; int len; pkv_word word;
                     pack_stats(codes, row_stride, (size_t)(s * V_SLOTS + i) * PACK_TOK,
                                (size_t)(w * LANES + t), &mn, &len, &word);
                     put_bits(mins, (size_t)(t * V_SLOTS + i) * W, W, mn);
@@ -227,7 +234,7 @@ void pkv_oracle_v_block_decode(const uint8_t *in, int ctx_blk, int hid_blk, int 
                 for (int t = 0; t < LANES; t++) {
                     unsigned mn = get_bits(mins, (size_t)(t * V_SLOTS + i) * W, W);
                     int len = (int)get_bits(lens, (size_t)(t * V_SLOTS + i) * LB, LB);
-                    uint64_t word = get_word(payload + pay, len);
+                    pkv_word word = get_word(payload + pay, len);
                     pay += (size_t)len * PACK_TOK / 8;
                     unpack_word(codes, row_stride, (size_t)(s * V_SLOTS + i) * PACK_TOK,
                                 (size_t)(w * LANES + t), word, len, mn);
@@ -241,7 +248,7 @@ void pkv_oracle_v_block_decode(const uint8_t *in, int ctx_blk, int hid_blk, int 
 /* ------------------------------------------------- whole-tensor drivers -- */
 
 static int check_shape(int is_k, int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int W) {
-    if (W < 2 || W > 4) return -1;
+    if (W < 2 || W > 8) return -1;
     if (ctx_len <= 0 || hidden_dim <= 0 || ctx_blk <= 0 || hid_blk <= 0) return -1;
     if (ctx_len % ctx_blk || hidden_dim % hid_blk || ctx_blk % PACK_TOK) return -1;
     if (is_k) { if (hid_blk != 128) return -1; }

@@ -551,8 +551,8 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
         PKV_REQUIRE(a->k_stream && a->k_info && a->v_stream && a->v_info && a->k_scale && a->k_zero &&
                         a->v_scale && a->v_zero,
                     PKV_ERR_INVALID, "null pointer argument");
-        PKV_REQUIRE(a->k_bits >= 2 && a->k_bits <= 4 && a->v_bits >= 2 && a->v_bits <= 4, PKV_ERR_UNSUPPORTED,
-                    "not supported: bits_len outside 2..4");
+        PKV_REQUIRE(a->k_bits >= 2 && a->k_bits <= kMaxBits && a->v_bits >= 2 && a->v_bits <= kMaxBits, PKV_ERR_UNSUPPORTED,
+                    "not supported: bits_len outside 2..8");
         PKV_REQUIRE(a->k_bytes > 0 && a->v_bytes > 0 && a->k_bytes < (1ull << 32) && a->v_bytes < (1ull << 32),
                     PKV_ERR_INVALID, "stream sizes must be in 1 .. 4 GiB - 1");
     }
@@ -595,7 +595,9 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     // The async-copy kernel spreads the tail window over its splits (each takes win_piece tokens after its
     // tiles and writes one more partial), so the window costs no launch and no idle tail; other paths
     // give the window a kernel of its own.
-    const bool aligned16 = ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
+    // the matrix-core kernels are built for the reference's widths; the extension widths 5..8 run the plain kernel
+    const bool narrow = a->T_c == 0 || (a->k_bits <= 4 && a->v_bits <= 4);
+    const bool aligned16 = narrow && ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
     p.win_piece = 0;
     if (a->T_w > 0 && nsplit > 0 && a->variant == 0 && aligned16) {
         const int piece = (a->T_w + nsplit - 1) / nsplit;
@@ -615,11 +617,12 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
 
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
+    const int variant = narrow ? a->variant : 1;
     switch (G) {
-        case 1: rc = launch_attn<1>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
-        case 2: rc = launch_attn<2>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
-        case 4: rc = launch_attn<4>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
-        default: rc = launch_attn<8>(p, a->variant, aligned16, (uint16_t *)a->out, s); break;
+        case 1: rc = launch_attn<1>(p, variant, aligned16, (uint16_t *)a->out, s); break;
+        case 2: rc = launch_attn<2>(p, variant, aligned16, (uint16_t *)a->out, s); break;
+        case 4: rc = launch_attn<4>(p, variant, aligned16, (uint16_t *)a->out, s); break;
+        default: rc = launch_attn<8>(p, variant, aligned16, (uint16_t *)a->out, s); break;
     }
     if (rc) return rc;
     return tm.end(ms_out);

@@ -85,6 +85,33 @@ __device__ __forceinline__ void unit_parse2(const uint8_t *blk_a, uint32_t off_a
     }
 }
 
+// ---- widths 5..8 (format extension): pack words of up to 128 bits, plain field-by-field code ----
+typedef unsigned __int128 word128;
+
+template <bool IS_K>
+__device__ __forceinline__ void unit_decode_wide(const uint8_t *blk, uint32_t unit_off, int unit, int t,
+                                                 const UnitGeom g, uint8_t *tile, int hid_blk) {
+    const uint32_t minsw = lds_meta_word(blk + unit_off, t, g.W);
+    const uint32_t lensw = lds_meta_word(blk + unit_off + g.mins_bytes, t, g.LB);
+    const uint32_t pay0 = unit_off + g.mins_bytes + g.lens_bytes;
+    uint32_t len[4], mn[4], off[4], payload;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        len[i] = (lensw >> (i * g.LB)) & ((1u << g.LB) - 1u);
+        mn[i] = (minsw >> (i * g.W)) & ((1u << g.W) - 1u);
+    }
+    pack_offsets(len, off, payload);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const word128 w = ((word128)lds_load64(blk, pay0 + off[i] + 8u) << 64) | lds_load64(blk, pay0 + off[i]);
+        const uint32_t mask = (1u << len[i]) - 1u;
+        for (int k = 0; k < kPackTok; k++) {
+            const uint32_t code = ((uint32_t)(w >> ((uint32_t)(kPackTok - 1 - k) * len[i])) & mask) + mn[i];
+            tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] = (uint8_t)code;
+        }
+    }
+}
+
 // Decode one unit whose bytes start at blk[unit_off] into the LDS tile.
 // The four pack words are cut into 16-bit windows of four tokens (packs 0|1 and 2|3 share a
 // register), so one packed 16-bit shift moves two packs at a time and a byte permute gathers the
@@ -93,6 +120,10 @@ template <bool IS_K>
 __device__ __forceinline__ void unit_decode(const uint8_t *blk, uint32_t unit_off, int unit, int t,
                                             const UnitGeom g, uint8_t *tile, int hid_blk) {
     typedef unsigned short u16pair __attribute__((ext_vector_type(2)));
+    if (g.W > 4) {      // uniform
+        unit_decode_wide<IS_K>(blk, unit_off, unit, t, g, tile, hid_blk);
+        return;
+    }
     UnitPacks u;
     unit_parse(blk, unit_off, t, g, u);
     uint32_t hlf[4][2];
@@ -200,6 +231,66 @@ __device__ __forceinline__ void unit_emit(uint8_t *blk, uint32_t unit_off, int t
     }
 }
 
+// Widths 5..8: analyse lane t's four packs of `unit` and write them at blk[unit_off] (the unit's size is
+// known from a first call with blk == nullptr, which only returns it).  The metadata fields do not fall on byte
+// boundaries for every width, so the unit's metadata area is cleared and the fields are OR-ed in.
+template <bool IS_K>
+__device__ __forceinline__ uint32_t unit_encode_wide(const uint8_t *tile, int hid_blk, int unit, int t,
+                                                     const UnitGeom g, uint8_t *blk, uint32_t unit_off) {
+    word128 word[4];
+    uint32_t len[4], mn[4], off[4], payload;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t lo = 255u, hi = 0u;
+        for (int k = 0; k < kPackTok; k++) {
+            const uint32_t c = tile[tile_index<IS_K>(unit, i, k, t, hid_blk)];
+            lo = min(lo, c);
+            hi = max(hi, c);
+        }
+        len[i] = (uint32_t)bit_length_u32(hi - lo);
+        mn[i] = lo;
+        word128 w = 0;
+        for (int k = 0; k < kPackTok; k++)
+            w = (w << len[i]) | (word128)(tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] - lo);
+        word[i] = w;
+    }
+    pack_offsets(len, off, payload);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    if (blk == nullptr) return meta + payload;
+    uint16_t *m16 = reinterpret_cast<uint16_t *>(blk + unit_off);
+    for (uint32_t i = t; i < meta / 2u; i += 32) m16[i] = 0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // LDS serves a wavefront's accesses in order
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    uint32_t minsw = 0, lensw = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        minsw |= mn[i] << (i * g.W);
+        lensw |= len[i] << (i * g.LB);
+    }
+    auto or_field = [&](uint8_t *arr, int nbits, uint32_t v) {       // 4 * nbits bits at bit 4 * t * nbits of arr
+        const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>(arr);
+        const uint32_t bit = (addr & 3u) * 8u + (uint32_t)t * 4u * (uint32_t)nbits;
+        uint32_t *p = reinterpret_cast<uint32_t *>(arr - (addr & 3u)) + (bit >> 5);
+        const uint64_t wide = (uint64_t)v << (bit & 31u);
+        atomicOr(p, (uint32_t)wide);
+        if ((uint32_t)(wide >> 32)) atomicOr(p + 1, (uint32_t)(wide >> 32));
+    };
+    or_field(blk + unit_off, g.W, minsw);
+    or_field(blk + unit_off + g.mins_bytes, g.LB, lensw);
+    uint8_t *pay = blk + unit_off + meta;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(pay + off[i]);
+        word128 w = word[i];
+        for (uint32_t b = 0; b < len[i]; b++) {
+            dst[b] = (uint16_t)w;
+            w >>= 16;
+        }
+    }
+    return meta + payload;
+}
+
 // Encode the LDS code tile of one block into the LDS buffer `blk`; every thread of the
 // workgroup must call it, and the workgroup must hold at least one half-wavefront per unit
 // (blockDim.x >= 32 * nunits).  `unit_bytes` is an LDS array of >= nunits uint32.  Returns
@@ -213,9 +304,15 @@ __device__ __forceinline__ uint32_t block_encode(const uint8_t *tile, int hid_bl
     const bool active = unit < nunits;
     const uint32_t hdr = 2u * (uint32_t)nunits;
     UnitPacks u;
+    const bool wide = W > 4;
     if (active) {
-        unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
-        if (t == 0) unit_bytes[unit] = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        if (wide) {
+            const uint32_t usz = unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, nullptr, 0u);
+            if (t == 0) unit_bytes[unit] = usz;
+        } else {
+            unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
+            if (t == 0) unit_bytes[unit] = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        }
     }
     __syncthreads();
     uint32_t total = hdr;
@@ -224,7 +321,8 @@ __device__ __forceinline__ uint32_t block_encode(const uint8_t *tile, int hid_bl
         uint32_t base = hdr;
         for (int q = 0; q < unit; q++) base += unit_bytes[q];
         if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - hdr + unit_bytes[unit]);
-        unit_emit(blk, base, t, g, u);
+        if (wide) unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, blk, base);
+        else unit_emit(blk, base, t, g, u);
     }
     __syncthreads();
     return total;

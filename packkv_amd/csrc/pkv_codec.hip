@@ -138,7 +138,7 @@ struct CodecShape {
 
 static int codec_shape(bool is_k, int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits,
                        CodecShape *o) {
-    PKV_REQUIRE(bits >= 2 && bits <= 4, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (need 2..4)", bits);
+    PKV_REQUIRE(bits >= 2 && bits <= kMaxBits, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (need 2..8)", bits);
     PKV_REQUIRE(ctx_len > 0 && hidden_dim > 0 && ctx_blk > 0 && hid_blk > 0, PKV_ERR_INVALID,
                 "sizes must be positive");
     PKV_REQUIRE(ctx_len % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");

@@ -23,9 +23,10 @@ constexpr int kPackTok = 16;    // tokens per pack        (static_def.h:6)
 constexpr int kLanes = 32;      // format lanes per round (static_def.h:4)
 constexpr int kHeadDim = 128;   // K block width          (static_def.h:5)
 
-__host__ __device__ constexpr int len_field_bits(int W) {  // include/utils.h:24-36
-    return W >= 4 ? 3 : (W >= 2 ? 2 : 1);
+__host__ __device__ constexpr int len_field_bits(int W) {  // include/utils.h:24-36: bits that hold 0..W
+    return W >= 8 ? 4 : (W >= 4 ? 3 : (W >= 2 ? 2 : 1));
 }
+constexpr int kMaxBits = 8;     // widths 5..8 are this library's extension of the format (pack words up to 128 bits)
 __host__ __device__ constexpr int k_block_bound(int ctx_blk, int W) {
     return 2 * (ctx_blk / kPackTok) +
            (ctx_blk / kPackTok) * kHeadDim * (W + len_field_bits(W)) / 8 +
@@ -115,7 +116,7 @@ __device__ __forceinline__ uint64_t lds_load64(const uint8_t *lds, uint32_t off)
 }
 
 // The 4*nbits-bit metadata word of format lane t from an LSB-first bit array in LDS (4 fields
-// of nbits each; nbits in {2,3,4}; `arr` 2-byte aligned).  Reads the two aligned dwords around
+// of nbits each; nbits in 2..8; `arr` 2-byte aligned).  Reads the two aligned dwords around
 // the field and funnel-shifts: adjacent byte reads would be merged into misaligned 16-bit DS
 // reads, which stall the LDS pipeline.
 __device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int nbits) {
@@ -123,7 +124,7 @@ __device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int
     const uint32_t bit = (addr & 3u) * 8u + (uint32_t)t * 4u * (uint32_t)nbits;
     const uint32_t *p = reinterpret_cast<const uint32_t *>(arr - (addr & 3u)) + (bit >> 5);
     const uint32_t v = __builtin_amdgcn_alignbit(p[1], p[0], bit & 31u);
-    return v & ((1u << (4 * nbits)) - 1u);
+    return nbits >= 8 ? v : v & ((1u << (4 * nbits)) - 1u);
 }
 
 // Copy `nbytes` from global `src` (any alignment) into LDS `dst` (4-byte aligned) so that

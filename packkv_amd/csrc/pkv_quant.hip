@@ -897,7 +897,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
-    PKV_REQUIRE(bits >= 2 && bits <= 4, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (need 2..4)", bits);
+    PKV_REQUIRE(bits >= 2 && bits <= 4, PKV_ERR_UNSUPPORTED,
+                "not supported: bits_len %d (the fused encoders take 2..4; wider codes go through pkv_quant_params, "
+                "pkv_quantize and pkv_{k,v}_encode)", bits);
     PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");

@@ -71,7 +71,7 @@ def bits_for_rel(rel):
 
 # ------------------------------------------------------------------ codec ------------
 
-def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k):
+def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k, max_bits=4):
     # mirrors k_encode_cpu_assert / v_encode_cpu_assert (src/k_encode_cpu.cpp:247-284,
     # src/v_encode_cpu.cpp:262-299); raises instead of aborting the process
     _require(codes.dim() == 2 and codes.size(0) == ctx_len, "ctx_len mismatch")
@@ -83,7 +83,7 @@ def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk
     nblk = (ctx_len // ctx_blk) * (hidden_dim // hid_blk)
     _require(info.dim() == 2 and info.size(0) == nblk, "block_info_buffer block num mismatch")
     _require(info.size(1) == 2, "block_info_buffer.size(1) must be 2")
-    _require(bits <= 4, "bits_len must be less than or equal to 4")
+    _require(bits <= max_bits, "bits_len must be less than or equal to %d" % max_bits)
     _require(ctx_blk % 16 == 0, "ctx_len_block_size must be divisible by PACK_ELE_NUM")
     if is_k:
         _require(hid_blk == 128, "hidden_dim_block_size must be 128, because this is most common head dim")
@@ -96,8 +96,8 @@ def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk
 
 
 def _encode(is_k, codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, want_size=True,
-            timed=False):
-    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k)
+            timed=False, max_bits=4):
+    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k, max_bits)
     lib = _lib.load()
     dev = _device_of(codes, stream, info)
     on_host = not codes.is_cuda
@@ -120,8 +120,8 @@ def _encode(is_k, codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bi
     return (int(size.value), float(ms.value)) if timed else int(size.value)
 
 
-def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, timed=False):
-    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k)
+def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, timed=False, max_bits=4):
+    _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, is_k, max_bits)
     lib = _lib.load()
     dev = _device_of(codes, stream, info)
     on_host = not codes.is_cuda
@@ -170,23 +170,26 @@ def v_decode_cpu(compressed_buffer, block_info_buffer, quant_ints_tensor, ctx_le
             ctx_len_block_size, hidden_dim_block_size, bits_len)
 
 
+MAX_BITS = 8     # widths 5..8 are this library's extension of the format (the reference stops at 4)
+
+
 def k_encode(codes, stream, info, ctx_blk=64, hid_blk=128, bits=4, want_size=True, timed=False):
-    """Device encode of a uint8 code matrix [ctx_len, hidden]; returns the stream size (and ms)."""
+    """Device encode of a uint8 code matrix [ctx_len, hidden]; returns the stream size (and ms).  bits 2..8."""
     return _encode(True, codes, stream, info, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits,
-                   want_size, timed)
+                   want_size, timed, MAX_BITS)
 
 
 def v_encode(codes, stream, info, ctx_blk=128, hid_blk=64, bits=4, want_size=True, timed=False):
     return _encode(False, codes, stream, info, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits,
-                   want_size, timed)
+                   want_size, timed, MAX_BITS)
 
 
 def k_decode(stream, info, codes, ctx_blk=64, hid_blk=128, bits=4, timed=False):
-    return _decode(True, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed)
+    return _decode(True, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed, MAX_BITS)
 
 
 def v_decode(stream, info, codes, ctx_blk=128, hid_blk=64, bits=4, timed=False):
-    return _decode(False, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed)
+    return _decode(False, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed, MAX_BITS)
 
 
 # --------------------------------------------------------------- quantizer -----------
@@ -239,11 +242,23 @@ def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed):
     hidden = B * H * 128
     ctx_blk, hid_blk = (64, 128) if is_k else (128, 64)
     nblk = (T // ctx_blk) * (hidden // hid_blk)
-    if stream is None:
-        stream = torch.empty(T * hidden, dtype=torch.uint8, device=x.device)
+    if stream is None:     # sized like the code matrix as the reference does; the extension widths can need more
+        stream = torch.empty(max(T * hidden, nblk * block_bound(is_k, ctx_blk, hid_blk, bits) + 16) if bits > 4
+                             else T * hidden, dtype=torch.uint8, device=x.device)
     if info is None:
         info = torch.empty(nblk, 2, dtype=torch.uint32, device=x.device)
     _require(info.numel() == 2 * nblk and info.dtype == torch.uint32, "block_info_buffer block num mismatch")
+    if bits > 4:
+        # widths 5..8 (format extension): quantize to the code matrix, then the block codec -- three kernels
+        # instead of the fused one
+        scale, zero = quant_params(x, rel)
+        codes, mx = quantize(x, scale, zero)
+        if mx >= (1 << bits):
+            raise PackKVError(1, "not supported: code %d does not fit bits_len %d" % (mx, bits))
+        res = _encode(is_k, codes, stream, info, T, hidden, ctx_blk, hid_blk, bits, want_size, timed, MAX_BITS)
+        size, ms = res if timed else (res, 0.0)
+        return {"stream": stream, "info": info, "scale": scale, "zero": zero, "size": int(size), "ms": float(ms),
+                "bits": bits}
     scale = torch.empty(B, T, dtype=x.dtype, device=x.device)
     zero = torch.empty(B, T, dtype=x.dtype, device=x.device)
     size = ctypes.c_uint64(0)

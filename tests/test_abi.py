@@ -35,7 +35,7 @@ def test_version_bounds_and_error_text():
     assert rc == _lib.ERR_INVALID
     assert b"null" in lib.pkv_last_error()
     one = ctypes.c_void_p(16)
-    rc = lib.pkv_k_encode(one, one, 1, one, 64, 128, 64, 128, 7, None, None, None)
+    rc = lib.pkv_k_encode(one, one, 1, one, 64, 128, 64, 128, 9, None, None, None)
     assert rc == _lib.ERR_UNSUPPORTED and b"not supported" in lib.pkv_last_error()
     rc = lib.pkv_k_encode(one, one, 1, one, 64, 128, 64, 64, 4, None, None, None)
     assert rc == _lib.ERR_UNSUPPORTED

@@ -212,3 +212,22 @@ def test_attn_decode_replays_in_a_hip_graph(cuda):
         torch.cuda.synchronize()
         for o, w in zip(outs, want):
             assert torch.equal(o, w)
+
+
+def test_attn_decode_five_bit_codes(cuda):
+    """rel 0.05 gives 22 code levels: 5-bit codes, outside the reference's format and inside this build's extension
+    (three-kernel encode, plain attention kernel).  Same contract against decompress-then-attend."""
+    B, Hq, Hkv, T = 2, 16, 4, 512
+    k, v = synth.make_kv(B, Hkv, T, seed=180)
+    q = synth.make_q(B, Hq, seed=181)
+    want = _reference(q, k, v, 0.05, 0.05)
+    exact = _exact(q, k, v, 0.05, 0.05)
+    ke = ops.k_quant_encode(k.to(cuda), 0.05)
+    ve = ops.v_quant_encode(v.to(cuda), 0.05)
+    assert ke["bits"] == 5 and ve["bits"] == 5
+    ck, _, _ = oq.quant_ints(k, 64, 0.05)
+    codes = torch.empty(T, B * Hkv * 128, dtype=torch.uint8, device=cuda)
+    ops.k_decode(ke["stream"], ke["info"], codes, bits=5)
+    assert torch.equal(codes.cpu(), oq.code_matrix(ck))
+    got = ops.attn_decode(q.to(cuda), ke, ve)
+    _check(got, want, torch.float16, exact, abs_tol=STRESS_ABS_TOL[torch.float16], variant=1)

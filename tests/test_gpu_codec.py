@@ -108,7 +108,9 @@ def test_error_conventions(cuda):
     with pytest.raises(RuntimeError, match="not supported"):
         ops.k_encode(c, s, i, 64, 128, 1)
     with pytest.raises(RuntimeError, match="bits_len"):
-        ops.k_encode(c, s, i, 64, 128, 5)
+        ops.k_encode(c, s, i, 64, 128, 9)
+    with pytest.raises(RuntimeError, match="bits_len"):        # the drop-in functions keep the reference's limit
+        ops.k_encode_cpu(c, s, i, 64, 128, 64, 128, 5)
     with pytest.raises(RuntimeError, match="block num mismatch"):
         ops.k_encode(c, s, torch.zeros(2, 2, dtype=torch.uint32, device=cuda), 64, 128, 4)
     with pytest.raises(RuntimeError, match="UInt8"):
@@ -142,3 +144,33 @@ def test_round_trip_at_bench_scale(cuda):
         (ops.k_decode if is_k else ops.v_decode)(stream, info, out, cb, hb, 4)
         assert torch.equal(out, codes)
         _say("bench-scale", "K" if is_k else "V", "ratio uint8/stream = %.3f" % (T * H / size))
+
+
+@pytest.mark.parametrize("W", [5, 6, 7, 8])
+def test_wide_codes_stream_matches_restatement(cuda, oracle_codec, W):
+    """Widths 5..8 are this build's extension of the format (pack words of up to 128 bits; the reference's
+    templates stop at 4).  There is no reference for them: the device codec is held to the restated C codec byte for
+    byte, to an exact round trip, and the stream size to the closed form (payload 2 * len bytes per pack, W + LB bits
+    of metadata per pack, 8 header bytes per block)."""
+    rng = np.random.default_rng(40 + W)
+    for is_k, (cb, hb), (T, H) in ((1, (64, 128), (128, 256)), (0, (128, 64), (256, 192)), (1, (32, 128), (96, 128))):
+        codes = rng.integers(0, 2 ** W, size=(T, H), dtype=np.uint8)
+        codes[: T // 2, ::2] //= 8                 # mixed widths: some packs narrow, some constant
+        codes[:16, :32] = 7
+        _say("wide codec case W", W, "K" if is_k else "V", cb, hb, T, H)
+        so, io, zo = oracle_codec.encode(is_k, codes, cb, hb, W)
+        nblk = (T // cb) * (H // hb)
+        LB = int(np.ceil(np.log2(W + 1)))
+        packs = codes.reshape(T // 16, 16, H)
+        lens = np.ceil(np.log2(packs.max(1).astype(np.int64) - packs.min(1) + 1)).astype(np.int64)
+        assert zo == int(lens.sum()) * 2 + lens.size * (W + LB) // 8 + (2 * (cb // 16) if is_k else 4 * (hb // 32)) * nblk
+        d = torch.from_numpy(codes).to(cuda)
+        stream = torch.zeros(nblk * ops.block_bound(is_k, cb, hb, W) + 16, dtype=torch.uint8, device=cuda)
+        info = torch.zeros(nblk, 2, dtype=torch.uint32, device=cuda)
+        size = (ops.k_encode if is_k else ops.v_encode)(d, stream, info, cb, hb, W)
+        assert size == zo
+        assert np.array_equal(info.cpu().numpy(), io)
+        assert np.array_equal(stream[:zo].cpu().numpy(), so[:zo])
+        back = torch.zeros_like(d)
+        (ops.k_decode if is_k else ops.v_decode)(stream, info, back, cb, hb, W)
+        assert torch.equal(back, d)

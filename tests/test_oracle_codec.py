@@ -115,7 +115,7 @@ def test_sizes_offsets_and_bit_pack_parity(oracle_codec):
 def test_unsupported_shapes_raise(oracle_codec):
     c = np.zeros((64, 128), dtype=np.uint8)
     with pytest.raises(RuntimeError):
-        oracle_codec.encode(1, c, 64, 128, 5)
+        oracle_codec.encode(1, c, 64, 128, 9)
     with pytest.raises(RuntimeError):
         oracle_codec.encode(1, c, 64, 64, 4)
     with pytest.raises(RuntimeError):
