@@ -23,11 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the decode kernel on the default workload, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 208450 and WRITE_SIZE 2176 per dispatch), each scaled by what the same counter read
-# for a plain 256 MiB device copy in the same run (131088 -> factor 1.99976; 262144 -> factor 1.0);
+# (FETCH_SIZE 208470 and WRITE_SIZE 2176 per dispatch), each scaled by what the same counter read
+# for a plain 256 MiB device copy in the same run (131086 -> factor 1.99979; 262144 -> factor 1.0);
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
-DEFAULT_TRAFFIC_BYTES = int((208450 * (262144 / 131088) + 2176 * 1.0) * 1024)
+DEFAULT_TRAFFIC_BYTES = int((208470 * (262144 / 131086) + 2176 * 1.0) * 1024)
 
 
 def parse():
@@ -44,6 +44,9 @@ def parse():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip encode / unpack timing")
+    ap.add_argument("--layers", type=int, default=0,
+                    help="instead of the single-layer step: a decode loop over this many layers through the growing "
+                         "compressed cache (configs[4] is --layers 32 --batch 4 --ctx 131072); prints its own JSON line")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -111,6 +114,68 @@ def cpu_encoder(torch, args, k1):
             "sample": "K codes of 1 sequence x %d tokens (%d channels), bit-pack only" % (T, cm.shape[1])}
 
 
+def decode_loop(torch, args, dev):
+    """Every layer's cache is prefilled with --ctx tokens through PackKVCompressedCache.update (residual window
+    policy of the reference: all but 128..191 tokens are compressed), then a decode step = for every layer: append
+    one token, attend.  Reports us per token over all layers, the share of HBM peak on the algorithmic bytes, the
+    bytes the caches hold and the peak device memory."""
+    from packkv_amd import synth
+    from packkv_amd.cache import PackKVCacheConfig, PackKVCompressedCache
+    B, Hq, Hkv, T, L = args.batch, args.hq, args.hkv, args.ctx, args.layers
+    cfg = PackKVCacheConfig(64, 192, args.rel, args.rel)
+    cache = PackKVCompressedCache(B, Hkv, 128, L, cfg, max_tokens=T + 1024, device=dev)
+    torch.cuda.reset_peak_memory_stats()
+    for layer in range(L):
+        k, v = synth.make_kv(B, Hkv, T, seed=layer, device=dev)
+        cache.update(k, v, layer)
+        del k, v
+    torch.cuda.synchronize()
+    q = synth.make_q(B, Hq, seed=1, device=dev)
+    kn, vn = synth.make_kv(B, Hkv, 1, seed=7, device=dev)
+    outs = [torch.empty_like(q) for _ in range(L)]
+
+    def token():
+        for layer in range(L):
+            cache.update(kn, vn, layer)
+            cache.attend(q, layer, out=outs[layer])
+
+    def algo_bytes():
+        n = 0
+        for lay in cache.layers:
+            for side in (lay.k, lay.v):
+                n += side.used + side.tokens // 128 * side.blocks_per_tile * 8 + 4 * B * side.tokens
+            n += 2 * 2 * B * Hkv * lay.win_len * 128 + 2 * 2 * B * Hq * 128
+        return n
+
+    for _ in range(args.warmup):
+        token()
+    torch.cuda.synchronize()
+    bytes_step = algo_bytes()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        token()
+    torch.cuda.synchronize()
+    us_token = (time.perf_counter() - t0) * 1e6 / args.steps
+    lay0 = cache.layers[0]
+    result = {
+        "metric": "compressed-cache decode us/token over all layers", "value": us_token, "unit": "us/token",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": us_token / 1e3,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "%d layers, batch %d, %d q / %d KV heads, head_dim 128, %d cached tokens per sequence "
+                               "(%d compressed + %d in the 16-bit window at the start of timing), rel %.3g; a step appends "
+                               "one token to every layer and attends" % (L, B, Hq, Hkv, T, lay0.k.tokens,
+                                                                         T - lay0.k.tokens, args.rel)},
+        "tokens_per_s": B / (us_token * 1e-6),
+        "roofline": {"bound": "hbm", "achieved": bytes_step / (us_token * 1e-6) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": bytes_step / (us_token * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": bytes_step},
+        "kv_bytes": cache.cache_bytes(), "fp16_kv_bytes": L * 2 * B * Hkv * cache.get_seq_length(0) * 128 * 2,
+        "peak_device_bytes": torch.cuda.max_memory_allocated(),
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -125,6 +190,9 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.layers > 0:
+        decode_loop(torch, args, dev)
+        return
     B, Hq, Hkv, T, Tw = args.batch, args.hq, args.hkv, args.ctx, args.window
     Tc = T - Tw
     assert Tc % 128 == 0, "compressed tokens must be a multiple of 128"
