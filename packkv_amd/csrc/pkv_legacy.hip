@@ -95,42 +95,65 @@ __global__ void wv_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
     atomicAdd(wv_out + (size_t)hb * hid_blk + ch, acc);
 }
 
-// grid = M, 256 threads.
-__global__ void fused_kq_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
-                                const uint16_t *__restrict__ zero, const uint16_t *__restrict__ scale,
-                                const uint16_t *__restrict__ t, int K, int N, int dtype) {
-    __shared__ float red[256];
-    const int m = blockIdx.x;
+__device__ __forceinline__ float wave_sum_f32(float x) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
+    return x;
+}
+
+// grid = (ceil(N / 2048), M), 256 threads: every workgroup forms the row's sum of q itself (K values) and then
+// finishes 2048 columns, eight per thread.
+__global__ void __launch_bounds__(256) fused_kq_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
+                                                       const uint16_t *__restrict__ zero, const uint16_t *__restrict__ scale,
+                                                       const uint16_t *__restrict__ t, int K, int N, int dtype) {
+    __shared__ float red[4];
+    const int m = blockIdx.y;
     float s = 0.f;
     for (int d = threadIdx.x; d < K; d += 256) s += ld16(q, (size_t)m * K + d, dtype);
-    red[threadIdx.x] = s;
+    s = wave_sum_f32(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
     __syncthreads();
-    for (int stride = 128; stride > 0; stride >>= 1) {
-        if ((int)threadIdx.x < stride) red[threadIdx.x] += red[threadIdx.x + stride];
-        __syncthreads();
-    }
-    const float sm = red[0];
-    for (int n = threadIdx.x; n < N; n += 256) {
-        const float u = sm * ld16(zero, n, dtype) + ld16(t, (size_t)m * N + n, dtype);
-        out[(size_t)m * N + n] = st16(u * ld16(scale, n, dtype), dtype);
+    const float sm = (red[0] + red[1]) + (red[2] + red[3]);
+    const int n0 = blockIdx.x * 2048;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int n = n0 + threadIdx.x + 256 * i;
+        if (n < N) {
+            const float u = sm * ld16(zero, n, dtype) + ld16(t, (size_t)m * N + n, dtype);
+            out[(size_t)m * N + n] = st16(u * ld16(scale, n, dtype), dtype);
+        }
     }
 }
 
-__global__ void fused_wv_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ w,
-                                const uint16_t *__restrict__ zero, const uint16_t *__restrict__ scale,
-                                const uint16_t *__restrict__ term1, int N, int D, int dtype) {
-    __shared__ float red[256];
+// Row sums of w * zero * scale in two steps: grid (ceil(N / 4096), M) partial sums, then one workgroup per row
+// adds the partials and finishes the D outputs.
+__global__ void __launch_bounds__(256) fused_wv_partial_kernel(const uint16_t *__restrict__ w, const uint16_t *__restrict__ zero,
+                                                               const uint16_t *__restrict__ scale, float *__restrict__ part,
+                                                               int N, int dtype) {
+    __shared__ float red[4];
+    const int m = blockIdx.y, n0 = blockIdx.x * 4096;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int n = n0 + threadIdx.x + 256 * i;
+        if (n < N) s += ld16(w, (size_t)m * N + n, dtype) * ld16(zero, n, dtype) * ld16(scale, n, dtype);
+    }
+    s = wave_sum_f32(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) part[(size_t)m * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ void __launch_bounds__(256) fused_wv_kernel(uint16_t *__restrict__ out, const float *__restrict__ part, int nparts,
+                                                       const uint16_t *__restrict__ term1, int D, int dtype) {
+    __shared__ float red[4];
     const int m = blockIdx.x;
     float s = 0.f;
-    for (int n = threadIdx.x; n < N; n += 256)
-        s += ld16(w, (size_t)m * N + n, dtype) * ld16(zero, n, dtype) * ld16(scale, n, dtype);
-    red[threadIdx.x] = s;
+    for (int i = threadIdx.x; i < nparts; i += 256) s += part[(size_t)m * nparts + i];
+    s = wave_sum_f32(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
     __syncthreads();
-    for (int stride = 128; stride > 0; stride >>= 1) {
-        if ((int)threadIdx.x < stride) red[threadIdx.x] += red[threadIdx.x + stride];
-        __syncthreads();
-    }
-    const float c = red[0];
+    const float c = (red[0] + red[1]) + (red[2] + red[3]);
     for (int d = threadIdx.x; d < D; d += 256)
         out[(size_t)m * D + d] = st16(c + ld16(term1, (size_t)m * D + d, dtype), dtype);
 }
@@ -201,10 +224,12 @@ int pkv_fused_kq(void *our_kq, const void *q, const void *k_zero, const void *k_
     if (rc) return rc;
     PKV_REQUIRE(our_kq && q && k_zero && k_scale && t, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(M > 0 && K > 0 && N > 0, PKV_ERR_INVALID, "sizes must be positive");
+    PKV_REQUIRE(M <= 65535, PKV_ERR_UNSUPPORTED, "more than 65535 rows");
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    fused_kq_kernel<<<M, 256, 0, s>>>((uint16_t *)our_kq, (const uint16_t *)q, (const uint16_t *)k_zero,
-                                      (const uint16_t *)k_scale, (const uint16_t *)t, K, N, dtype);
+    fused_kq_kernel<<<dim3((unsigned)((N + 2047) / 2048), (unsigned)M), 256, 0, s>>>(
+        (uint16_t *)our_kq, (const uint16_t *)q, (const uint16_t *)k_zero, (const uint16_t *)k_scale,
+        (const uint16_t *)t, K, N, dtype);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
@@ -217,10 +242,16 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
     if (rc) return rc;
     PKV_REQUIRE(our_wv && w && v_zero && v_scale && term1, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(M > 0 && N > 0 && D > 0, PKV_ERR_INVALID, "sizes must be positive");
+    PKV_REQUIRE(M <= 65535, PKV_ERR_UNSUPPORTED, "more than 65535 rows");
+    const int nparts = (N + 4095) / 4096;
+    void *scratch = nullptr;
+    if ((rc = scratch_get((size_t)M * nparts * sizeof(float), &scratch))) return rc;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    fused_wv_kernel<<<M, 256, 0, s>>>((uint16_t *)our_wv, (const uint16_t *)w, (const uint16_t *)v_zero,
-                                      (const uint16_t *)v_scale, (const uint16_t *)term1, N, D, dtype);
+    fused_wv_partial_kernel<<<dim3((unsigned)nparts, (unsigned)M), 256, 0, s>>>(
+        (const uint16_t *)w, (const uint16_t *)v_zero, (const uint16_t *)v_scale, (float *)scratch, N, dtype);
+    fused_wv_kernel<<<M, 256, 0, s>>>((uint16_t *)our_wv, (const float *)scratch, nparts, (const uint16_t *)term1,
+                                      D, dtype);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
