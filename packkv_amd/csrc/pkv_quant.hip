@@ -183,7 +183,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 //             c - zero is even a tie goes to the same side as in rint(h).  The code is the result's bit pattern
 //             minus sub2 -- no separate rounding instruction;
 //   sub2 == 0: add2 = (-zero, -zero) for the general sequence rint(h) + (-zero).
-// bf16: add2 = zero as fp32 bits.
+// bf16: sub2 != 0 (|zero| <= 2^20): add2 = 2^23 - zero as fp32 bits; sub2 == 0: add2 = zero as fp32 bits.
 struct TokPar { float s, r; uint32_t add2, sub2; };
 
 __device__ __forceinline__ uint32_t pk_u16(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
@@ -213,6 +213,29 @@ __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01,
             c01 = __builtin_bit_cast(uint32_t, (f16x2)(d01 + magic)) & 0x00FF00FFu;
             c23 = __builtin_bit_cast(uint32_t, (f16x2)(d23 + magic)) & 0x00FF00FFu;
         }
+    } else if (__builtin_amdgcn_readfirstlane(tp.sub2) != 0u) {
+        // bf16, zero point of moderate size: the same three-instruction quotient (a quotient of two 8-bit
+        // significands is either exactly a bf16 rounding midpoint or at least 2^-17 away from every one), rounded to
+        // bf16 by the hardware conversion; rint(h) and rint(h) - zero are then exact in fp32 (bf16 values of 256 and
+        // above are integers already), so adding 2^23 - zero leaves the code in the low mantissa bits.
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        auto quot = [&](float f) -> float {
+            const float q0 = __fmul_rn(f, tp.r);
+            const float e = __fmaf_rn(-tp.s, q0, f);
+            return __fmaf_rn(e, tp.r, q0);
+        };
+        const f32x2 q01 = {quot(__uint_as_float(xw.x << 16)), quot(__uint_as_float(xw.x & 0xFFFF0000u))};
+        const f32x2 q23 = {quot(__uint_as_float(xw.y << 16)), quot(__uint_as_float(xw.y & 0xFFFF0000u))};
+        const uint32_t h01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(q01, bf16x2));
+        const uint32_t h23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(q23, bf16x2));
+        const float mz = __uint_as_float(tp.add2);                        // 2^23 - zero
+        const uint32_t a = __float_as_uint(rintf(__uint_as_float(h01 << 16)) + mz) & 0xFFu;
+        const uint32_t b = __float_as_uint(rintf(__uint_as_float(h01 & 0xFFFF0000u)) + mz) & 0xFFu;
+        const uint32_t c = __float_as_uint(rintf(__uint_as_float(h23 << 16)) + mz) & 0xFFu;
+        const uint32_t d = __float_as_uint(rintf(__uint_as_float(h23 & 0xFFFF0000u)) + mz) & 0xFFu;
+        c01 = a | (b << 16);
+        c23 = c | (d << 16);
     } else {
         const float z = __uint_as_float(tp.add2);
         const uint32_t a = (uint32_t)(int)quant_code<DT>(T16<DT>::from_bits(xw.x & 0xFFFFu), tp.s, z) & 0xFFu;
@@ -313,7 +336,13 @@ __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
             tp.add2 = (zero_bits ^ 0x8000u) * 0x00010001u;
         }
     } else {
-        tp.add2 = __float_as_uint(T16<DT>::from_bits(zero_bits));
+        const float z = T16<DT>::from_bits(zero_bits);        // an integer (or inf / nan for degenerate tokens)
+        if (fabsf(z) <= 1048576.f) {       // 2^23 - zero and the sums below stay exact
+            tp.add2 = __float_as_uint(8388608.f - z);
+            tp.sub2 = 1u;
+        } else {
+            tp.add2 = __float_as_uint(z);
+        }
     }
     return tp;
 }

@@ -56,23 +56,28 @@ def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
             assert torch.equal(r["zero"].cpu().view(torch.int16), z.reshape(B, T).view(torch.int16))
 
 
-def test_fused_quant_encode_offset_rows_bit_exact(cuda, oracle_codec):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_quant_encode_offset_rows_bit_exact(cuda, oracle_codec, dtype):
     """Rows far from zero: the zero point is large (here about -750 and +750, and a few hundred for the smaller
     shift), which takes the encoders' general rounding sequence for some tokens and the short one for others;
     ties (quotients at exactly k + 0.5) are common because the shifted fp16 values are multiples of 0.5."""
     B, H, T, rel = 2, 4, 256, 0.1
     k, v = synth.make_kv(B, H, T, seed=77)
     shift = torch.zeros(B, 1, T, 1)
-    shift[:, :, 0:128:3] = -600.0        # first half: every 16-token round holds tokens of both kinds
-    shift[:, :, 1:128:3] = 600.0
-    shift[:, :, 2:128:6] = 150.0
-    shift[:, :, 128::2] = 600.0          # second half: large positive zero points only (the short sequence)
-    shift[:, :, 129::4] = 150.0
+    big, small = (600.0, 150.0) if dtype == torch.float16 else (48.0, 12.0)    # bf16 keeps 8 bits: stay where it resolves the rows
+    shift[:, :, 0:128:3] = -big          # first half: every 16-token round holds tokens of both kinds
+    shift[:, :, 1:128:3] = big
+    shift[:, :, 2:128:6] = small
+    shift[:, :, 128::2] = big            # second half: large positive zero points only (the short sequence)
+    shift[:, :, 129::4] = small
     for is_k, x0 in ((1, v), (0, v)):          # unit-variance rows, so that the codes stay within 4 bits
-        x = (x0.float() + shift).to(torch.float16)
+        x = (x0.float() + shift).to(dtype)
         c, z, s = oq.quant_ints(x, 64, rel)
         zi = z.float().flatten()
-        assert (zi.abs() > 600).any() and (zi.abs() < 400).any()
+        if dtype == torch.float16:
+            assert (zi.abs() > 600).any() and (zi.abs() < 400).any()
+        else:
+            assert (zi.abs() > 40).any()
         cm = oq.code_matrix(c).numpy()
         assert int(cm.max()) <= 15
         cb, hb = (64, 128) if is_k else (128, 64)
