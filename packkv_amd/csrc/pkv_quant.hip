@@ -121,7 +121,10 @@ __global__ void quantize_kernel(const uint16_t *__restrict__ x, int H, int T,
     if (max_code_out) {
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) cmax = max(cmax, __shfl_xor(cmax, d, 64));
-        if ((threadIdx.x & 63) == 0 && cmax) atomicMax(max_code_out, cmax);
+        // a read first: once the largest code has been seen nobody writes any more (a million atomics on one
+        // address would cost milliseconds)
+        if ((threadIdx.x & 63) == 0 && cmax > __hip_atomic_load(max_code_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax(max_code_out, cmax);
     }
 }
 
