@@ -102,6 +102,7 @@ class _Layer:
         self.win_len = 0
         self.pend = 0                      # 0 or 64: tokens at the head of the window that are a quantised cut
         self.k_pend = self.v_pend = None   # their original values
+        self.plan = None                   # checked arguments of the decode step, valid until the next cut
 
 
 class PackKVCompressedCache:
@@ -162,6 +163,7 @@ class PackKVCompressedCache:
             L.k_win[:, :, L.pend:L.pend + left] = kbuf[:, :, n_cut:]
             L.v_win[:, :, L.pend:L.pend + left] = vbuf[:, :, n_cut:]
             L.win_len = L.pend + left
+            L.plan = None                  # token counts (and possibly the stream buffers) changed
         if return_dense:
             return self.materialize(layer_idx)
         return None
@@ -180,10 +182,19 @@ class PackKVCompressedCache:
         if squeeze:
             q = q[:, :, 0]
         q = q.contiguous()
-        k = L.k.as_dict() if L.k.tokens else None
-        v = L.v.as_dict() if L.v.tokens else None
-        res = ops.attn_decode(q, k, v, L.k_win if L.win_len else None, L.v_win if L.win_len else None,
-                              sm_scale=sm_scale, out=out, win_len=L.win_len)
+        if out is None:
+            out = torch.empty_like(q)
+        plan = L.plan
+        if plan is None or plan.sm_scale_arg != sm_scale or not L.win_len or plan._shape != q.shape or plan._dtype != q.dtype:
+            k = L.k.as_dict() if L.k.tokens else None
+            v = L.v.as_dict() if L.v.tokens else None
+            plan = ops.AttnPlan(q, k, v, L.k_win if L.win_len else None, L.v_win if L.win_len else None,
+                                sm_scale=sm_scale, out=out, win_len=L.win_len)
+            plan.sm_scale_arg = sm_scale
+            L.plan = plan if L.win_len else None      # between cuts only the window rows in use change
+        else:
+            plan.set_window_rows(L.win_len)
+        res = plan(q=q, out=out)
         return res.unsqueeze(2) if squeeze else res
 
     # -- dense view and accounting ---------------------------------------------------------------------

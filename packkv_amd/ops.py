@@ -20,7 +20,7 @@ __all__ = [
     "kq_mat_vec_mul", "wv_mat_vec_mul", "fused_kq", "fused_wv",
     "k_encode", "v_encode", "k_decode", "v_decode",
     "quant_params", "quantize", "dequantize", "k_quant_encode", "v_quant_encode",
-    "attn_decode", "block_bound", "bits_for_rel",
+    "attn_decode", "AttnPlan", "block_bound", "bits_for_rel",
 ]
 
 
@@ -492,6 +492,92 @@ def fused_wv(our_wv, w, v_quant_zero, v_quant_scale, term1):
 
 # ------------------------------------------------- fused decompress-attention --------
 
+class AttnPlan:
+    """The checked, filled-in arguments of one decode step, kept for callers that repeat it (a decode loop over the
+    same layer): ``plan()`` launches again without re-validating; ``plan(q=..., out=...)`` swaps the query / output
+    tensors (same shape and dtype).  The tensors given at construction must stay alive and in place; build a new
+    plan when a buffer is reallocated or the token counts change."""
+
+    def __init__(self, q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, win_len=None):
+        _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
+                 "q must be a contiguous device tensor [B, Hq, 128]")
+        B, Hq, _ = q.shape
+        a = AttnArgs()
+        T_c = 0
+        Hkv = None
+        if k is not None:
+            T_c = int(k.get("tokens", k["scale"].size(1)))
+            _require(int(v.get("tokens", v["scale"].size(1))) == T_c, "K and V hold different token counts")
+            _require(0 < T_c <= k["scale"].size(1) and k["scale"].shape == v["scale"].shape,
+                     "scale / zero rows shorter than the token count")
+            a.par_stride = k["scale"].size(1)
+            for name, d in (("k", k), ("v", v)):
+                for f in ("stream", "info", "scale", "zero"):
+                    _require(d[f].is_cuda and d[f].is_contiguous(), "%s.%s must be a contiguous device tensor" % (name, f))
+            nblk_k = k["info"].numel() // 2
+            Hkv = int(k["heads"]) if "heads" in k else nblk_k // (T_c // 64) // B
+            _require(nblk_k >= (T_c // 64) * B * Hkv and v["info"].numel() // 2 >= (T_c // 128) * B * Hkv * 2,
+                     "block_info_buffer block num mismatch")
+            a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
+            a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
+            # readable bytes of each buffer: pack words are fetched as whole 8-byte words, so the last
+            # block needs 7 bytes of readable slack behind the encoded size
+            for d in (k, v):
+                _require(not d.get("size") or d["stream"].numel() >= int(d["size"]) + 7,
+                         "stream buffers need 7 readable bytes behind the encoded size")
+            a.k_bytes, a.v_bytes = k["stream"].numel(), v["stream"].numel()
+            a.k_scale, a.k_zero = _ptr(k["scale"]), _ptr(k["zero"])
+            a.v_scale, a.v_zero = _ptr(v["scale"]), _ptr(v["zero"])
+            a.k_bits, a.v_bits = int(k["bits"]), int(v["bits"])
+        T_w = 0
+        if k_win is not None:
+            _require(k_win.is_cuda and v_win.is_cuda and k_win.is_contiguous() and v_win.is_contiguous()
+                     and k_win.shape == v_win.shape and k_win.dim() == 4 and k_win.size(3) == 128
+                     and k_win.dtype == q.dtype and v_win.dtype == q.dtype,
+                     "window tensors must be contiguous [B, Hkv, T_w, 128] of q's dtype")
+            T_w = k_win.size(2) if win_len is None else int(win_len)
+            _require(0 < T_w <= k_win.size(2), "win_len outside the window tensors")
+            a.win_stride = k_win.size(2)
+            _require(Hkv is None or Hkv == k_win.size(1), "window head count mismatch")
+            Hkv = k_win.size(1)
+            a.k_win, a.v_win = _ptr(k_win), _ptr(v_win)
+        _require(Hkv is not None, "empty cache")
+        if out is None:
+            out = torch.empty_like(q)
+        a.q, a.out = _ptr(q), _ptr(out)
+        a.B, a.Hq, a.Hkv, a.T_c, a.T_w = B, Hq, Hkv, T_c, T_w
+        a.dtype = _dtype_code(q)
+        a.sm_scale = float(sm_scale if sm_scale is not None else 128 ** -0.5)
+        a.variant = int(variant)
+        self.args, self.out, self.device = a, out, q.device
+        self._shape, self._dtype = q.shape, q.dtype
+        self._keep = (q, k, v, k_win, v_win, out)          # the buffers the pointers refer to
+        self._fn = _lib.load().pkv_attn_decode
+        self._ref = ctypes.byref(a)
+
+    def set_window_rows(self, win_len):
+        """Window rows in use (the window tensors are allocated longer and fill up between cuts)."""
+        self.args.T_w = int(win_len)
+
+    def __call__(self, q=None, out=None, timed=False):
+        a = self.args
+        if q is not None:
+            _require(q.is_cuda and q.shape == self._shape and q.dtype == self._dtype and q.is_contiguous(),
+                     "q must match the plan's query tensor")
+            a.q = _ptr(q)
+        if out is not None:
+            _require(out.is_cuda and out.shape == self._shape and out.dtype == self._dtype and out.is_contiguous(),
+                     "out must match the plan's output tensor")
+            a.out = _ptr(out)
+            self.out = out
+        ms = ctypes.c_float(0.0)
+        with torch.cuda.device(self.device):
+            rc = self._fn(self._ref, ctypes.byref(ms) if timed else None, _stream(self.device))
+        if rc:
+            _lib.check(rc)
+        return (self.out, float(ms.value)) if timed else self.out
+
+
 def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False, win_len=None):
     """One decode step over a compressed cache.
 
@@ -501,61 +587,6 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
 
     Buffers allocated for a cache that grows: the dicts may carry ``tokens`` (compressed tokens in use;
     scale / zero rows and block_info are then longer than that) and ``heads`` (KV heads); ``win_len``
-    gives the window rows in use when k_win / v_win are allocated longer."""
-    _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
-             "q must be a contiguous device tensor [B, Hq, 128]")
-    B, Hq, _ = q.shape
-    a = AttnArgs()
-    T_c = 0
-    Hkv = None
-    keep = [q]
-    if k is not None:
-        T_c = int(k.get("tokens", k["scale"].size(1)))
-        _require(int(v.get("tokens", v["scale"].size(1))) == T_c, "K and V hold different token counts")
-        _require(0 < T_c <= k["scale"].size(1) and k["scale"].shape == v["scale"].shape,
-                 "scale / zero rows shorter than the token count")
-        a.par_stride = k["scale"].size(1)
-        for name, d in (("k", k), ("v", v)):
-            for f in ("stream", "info", "scale", "zero"):
-                _require(d[f].is_cuda and d[f].is_contiguous(), "%s.%s must be a contiguous device tensor" % (name, f))
-        nblk_k = k["info"].numel() // 2
-        Hkv = int(k["heads"]) if "heads" in k else nblk_k // (T_c // 64) // B
-        _require(nblk_k >= (T_c // 64) * B * Hkv and v["info"].numel() // 2 >= (T_c // 128) * B * Hkv * 2,
-                 "block_info_buffer block num mismatch")
-        a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
-        a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
-        # readable bytes of each buffer: pack words are fetched as whole 8-byte words, so the last
-        # block needs 7 bytes of readable slack behind the encoded size
-        for d in (k, v):
-            _require(not d.get("size") or d["stream"].numel() >= int(d["size"]) + 7,
-                     "stream buffers need 7 readable bytes behind the encoded size")
-        a.k_bytes, a.v_bytes = k["stream"].numel(), v["stream"].numel()
-        a.k_scale, a.k_zero = _ptr(k["scale"]), _ptr(k["zero"])
-        a.v_scale, a.v_zero = _ptr(v["scale"]), _ptr(v["zero"])
-        a.k_bits, a.v_bits = int(k["bits"]), int(v["bits"])
-    T_w = 0
-    if k_win is not None:
-        _require(k_win.is_cuda and v_win.is_cuda and k_win.is_contiguous() and v_win.is_contiguous()
-                 and k_win.shape == v_win.shape and k_win.dim() == 4 and k_win.size(3) == 128
-                 and k_win.dtype == q.dtype and v_win.dtype == q.dtype,
-                 "window tensors must be contiguous [B, Hkv, T_w, 128] of q's dtype")
-        T_w = k_win.size(2) if win_len is None else int(win_len)
-        _require(0 < T_w <= k_win.size(2), "win_len outside the window tensors")
-        a.win_stride = k_win.size(2)
-        _require(Hkv is None or Hkv == k_win.size(1), "window head count mismatch")
-        Hkv = k_win.size(1)
-        a.k_win, a.v_win = _ptr(k_win), _ptr(v_win)
-    _require(Hkv is not None, "empty cache")
-    if out is None:
-        out = torch.empty_like(q)
-    a.q, a.out = _ptr(q), _ptr(out)
-    a.B, a.Hq, a.Hkv, a.T_c, a.T_w = B, Hq, Hkv, T_c, T_w
-    a.dtype = _dtype_code(q)
-    a.sm_scale = float(sm_scale if sm_scale is not None else 128 ** -0.5)
-    a.variant = int(variant)
-    ms = ctypes.c_float(0.0)
-    with torch.cuda.device(q.device):
-        rc = _lib.load().pkv_attn_decode(ctypes.byref(a), ctypes.byref(ms) if timed else None,
-                                         _stream(q.device))
-    _lib.check(rc)
-    return (out, float(ms.value)) if timed else out
+    gives the window rows in use when k_win / v_win are allocated longer.  AttnPlan keeps the checked
+    arguments for callers that repeat the step."""
+    return AttnPlan(q, k, v, k_win, v_win, sm_scale, out, variant, win_len)(timed=timed)
