@@ -40,6 +40,7 @@ struct AttnParams {
     const uint16_t *q;
     const uint16_t *k_win, *v_win;
     float *part;          // [B, Hq, nparts, kPartStride]
+    uint16_t *out;        // [B, Hq, 128]: written directly by the attention kernel when there is a single partial
     int B, Hq, Hkv, T_c, T_w;
     int par_stride;       // tokens per sequence row of the scale / zero arrays (>= T_c)
     int win_stride;       // tokens per (sequence, KV head) row of k_win / v_win (>= T_w)
@@ -527,9 +528,12 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_
         attn_window_kernel<G><<<dim3((unsigned)p.Hkv, (unsigned)p.B), 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
-    attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), 256, (size_t)p.nparts * sizeof(float), s>>>(
-        p.part, out, p.Hq, p.nparts, p.dtype);
-    PKV_HIP_CHECK(hipGetLastError());
+    const bool dma_path = p.T_c > 0 && variant == 0 && aligned16;
+    if (!(dma_path && p.nparts == 1)) {      // a single partial is the result: the async-copy kernel wrote it out itself
+        attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), 256, (size_t)p.nparts * sizeof(float), s>>>(
+            p.part, out, p.Hq, p.nparts, p.dtype);
+        PKV_HIP_CHECK(hipGetLastError());
+    }
     return PKV_OK;
 }
 
@@ -614,6 +618,7 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     int rc = scratch_get(part_bytes, &scratch);
     if (rc) return rc;
     p.part = (float *)scratch;
+    p.out = (uint16_t *)a->out;
 
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;

@@ -532,9 +532,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 #pragma unroll
         for (int g = 0; g < G; g++) {
             const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
-            float *dst = p.part + (hq * p.nparts + split) * kPartStride;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
-            dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
+            const float val = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
+            if (p.nparts == 1) {               // one split and no window: this is the result, no merge launch follows
+                p.out[hq * kHeadDim + ch] = a_st16(val / st_l[g], p.dtype);
+                continue;
+            }
+            float *dst = p.part + (hq * p.nparts + split) * kPartStride;
+            dst[2 + ch] = val;
             if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
         }
     }
