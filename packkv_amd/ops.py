@@ -20,7 +20,7 @@ __all__ = [
     "kq_mat_vec_mul", "wv_mat_vec_mul", "fused_kq", "fused_wv",
     "k_encode", "v_encode", "k_decode", "v_decode",
     "quant_params", "quantize", "dequantize", "k_quant_encode", "v_quant_encode",
-    "attn_decode", "AttnPlan", "block_bound", "bits_for_rel",
+    "attn_decode", "AttnPlan", "block_bound", "bits_for_rel", "repack_quant_encode",
 ]
 
 
@@ -373,6 +373,45 @@ def repack_and_encode(k_codes, v_codes, pack_size, repack_method="none", block_s
         raise ValueError("repack_method must be one of none, median")
     k_aft, v_aft = bit_pack(k_codes, v_codes, pack_size)
     return k_pre, v_pre, k_aft, v_aft
+
+
+def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=64, k_bits=None, v_bits=None):
+    """Quantize K and V [B, H, T, 128], reorder the tokens of every quantisation block (jointly for K and V, as the
+    reference's repacking does before it prices the packs, utils/compute.py:329-357) and encode.  Returns (k, v,
+    perm): dicts like k_quant_encode / v_quant_encode -- stream, info, scale, zero in the REPACKED token order, so
+    attn_decode takes them as they are (attention does not depend on the order of the cached tokens) -- and the
+    permutation [T] int32 (perm[blk * block_size + r] = position inside the block the token at r came from)."""
+    B, H, T = _check_x(k)
+    _require(v.shape == k.shape and v.dtype == k.dtype and v.is_cuda and v.is_contiguous(), "K and V must have one shape")
+    _require(T % 128 == 0 and 128 % block_size == 0 or block_size % 128 == 0, "token count / block size mismatch")
+    k_bits, v_bits = k_bits or bits_for_rel(k_rel), v_bits or bits_for_rel(v_rel)
+    ks, kz = quant_params(k, k_rel)
+    vs, vz = quant_params(v, v_rel)
+    kc, kmx = quantize(k, ks, kz)
+    vc, vmx = quantize(v, vs, vz)
+    for mx, bits in ((kmx, k_bits), (vmx, v_bits)):
+        if mx >= (1 << bits):
+            raise PackKVError(1, "not supported: code %d does not fit bits_len %d" % (mx, bits))
+    if repack_method == "median":
+        kc, vc, perm = median_repacking(kc, vc, block_size)
+        src = (torch.arange(T, device=k.device, dtype=torch.int64) // block_size) * block_size + perm.to(torch.int64)
+        ks, kz, vs, vz = (p[:, src].contiguous() for p in (ks, kz, vs, vz))
+    elif repack_method == "none":
+        perm = (torch.arange(T, device=k.device, dtype=torch.int32) % block_size)
+    else:
+        raise ValueError("repack_method must be one of none, median")
+    hidden = B * H * 128
+    out = []
+    for is_k, codes, scale, zero, bits in ((True, kc, ks, kz, k_bits), (False, vc, vs, vz, v_bits)):
+        ctx_blk, hid_blk = (64, 128) if is_k else (128, 64)
+        nblk = (T // ctx_blk) * (hidden // hid_blk)
+        stream = torch.empty(max(T * hidden, nblk * block_bound(is_k, ctx_blk, hid_blk, bits) + 16) if bits > 4
+                             else T * hidden, dtype=torch.uint8, device=k.device)
+        info = torch.empty(nblk, 2, dtype=torch.uint32, device=k.device)
+        size = _encode(is_k, codes, stream, info, T, hidden, ctx_blk, hid_blk, bits, True, False, MAX_BITS)
+        out.append({"stream": stream, "info": info, "scale": scale, "zero": zero, "size": int(size), "ms": 0.0,
+                    "bits": bits})
+    return out[0], out[1], perm
 
 
 # ------------------------------------------------------- reference GEMV surface ------

@@ -109,3 +109,39 @@ def test_median_repacking_wide_codes_and_wide_rows(cuda):
         assert (perm.cpu().numpy().reshape(-1, bs) == order).all()
         assert (v_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, hid:]).all()
         assert (k_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, :hid]).all()
+
+
+def test_repacked_cache_attends_like_the_original(cuda):
+    """Attention does not depend on the order of the cached tokens, so a cache whose 64-token blocks were reordered
+    by median repacking (K, V and their per-token parameters together) must give the output of the cache in natural
+    order, and both must meet the contract against decompress-then-attend."""
+    B, Hq, Hkv, T = 2, 16, 4, 1024
+    k, v = synth.make_kv(B, Hkv, T, seed=190)
+    g = torch.Generator().manual_seed(191)
+    v = (v.float() * 0.3 + torch.randn(1, 1, T, 1, generator=g) * 2.0).to(torch.float16)   # token-wise level shift
+    q = synth.make_q(B, Hq, seed=192)
+    ck, zk, sk = oq.quant_ints(k, 64, 0.1)
+    cv, zv, sv = oq.quant_ints(v, 64, 0.1)
+    want = oq.attention_f32(q.unsqueeze(2), oq.dequant(ck, zk, sk), oq.dequant(cv, zv, sv)).squeeze(2).double().numpy()
+    kd, vd, qd = k.to(cuda), v.to(cuda), q.to(cuda)
+    kr, vr, perm = ops.repack_quant_encode(kd, vd, 0.1, 0.1, "median")
+    kn, vn, ident = ops.repack_quant_encode(kd, vd, 0.1, 0.1, "none")
+    assert torch.equal(ident.view(-1, 64), torch.arange(64, dtype=torch.int32, device=cuda).expand(T // 64, 64))
+    plain_k = ops.k_quant_encode(kd, 0.1)
+    assert kn["size"] == plain_k["size"] and torch.equal(kn["stream"][:kn["size"]], plain_k["stream"][:kn["size"]])
+    # the repacked streams hold the oracle's repacked codes
+    blocks = orp.blocks_from_code_matrices(oq.code_matrix(ck).numpy(), oq.code_matrix(cv).numpy(), 64)
+    rep, order = orp.median_repacking(blocks)
+    assert (perm.cpu().numpy().reshape(-1, 64) == order).all()
+    hid = B * Hkv * 128
+    codes = torch.empty(T, hid, dtype=torch.uint8, device=cuda)
+    ops.v_decode(vr["stream"], vr["info"], codes, bits=vr["bits"])
+    assert (codes.cpu().numpy().reshape(-1, 64, hid) == rep[:, :, hid:]).all()
+    assert vr["size"] <= vn["size"]                      # tokens of similar level side by side: no wider packs
+    out_r = ops.attn_decode(qd, kr, vr).double().cpu().numpy()
+    out_n = ops.attn_decode(qd, kn, vn).double().cpu().numpy()
+    _say("repacked cache: V bytes %d -> %d, max|out_r - out_n| = %.2e" % (vn["size"], vr["size"], np.abs(out_r - out_n).max()))
+    for out in (out_r, out_n):
+        assert (np.abs(out - want) <= 8e-3 + 1e-3 * np.abs(want)).all()
+    # the two orders add the same terms in a different sequence: at most an output rounding apart
+    assert np.abs(out_r - out_n).max() <= 2 ** -10 * np.abs(out_n).max()
