@@ -103,11 +103,17 @@ __device__ __forceinline__ void unit_decode_wide(const uint8_t *blk, uint32_t un
     pack_offsets(len, off, payload);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const word128 w = ((word128)lds_load64(blk, pay0 + off[i] + 8u) << 64) | lds_load64(blk, pay0 + off[i]);
-        const uint32_t mask = (1u << len[i]) - 1u;
-        for (int k = 0; k < kPackTok; k++) {
-            const uint32_t code = ((uint32_t)(w >> ((uint32_t)(kPackTok - 1 - k) * len[i])) & mask) + mn[i];
-            tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] = (uint8_t)code;
+        // the word as four dwords, shifted down one field at a time (token 15 sits in the lowest field)
+        const uint64_t lo = lds_load64(blk, pay0 + off[i]), hi = lds_load64(blk, pay0 + off[i] + 8u);
+        uint32_t d0 = (uint32_t)lo, d1 = (uint32_t)(lo >> 32), d2 = (uint32_t)hi, d3 = (uint32_t)(hi >> 32);
+        const uint32_t mask = (1u << len[i]) - 1u, sh = len[i];
+#pragma unroll
+        for (int k = kPackTok - 1; k >= 0; k--) {
+            tile[tile_index<IS_K>(unit, i, k, t, hid_blk)] = (uint8_t)((d0 & mask) + mn[i]);
+            d0 = __builtin_amdgcn_alignbit(d1, d0, sh);
+            d1 = __builtin_amdgcn_alignbit(d2, d1, sh);
+            d2 = __builtin_amdgcn_alignbit(d3, d2, sh);
+            d3 >>= sh;
         }
     }
 }
