@@ -33,8 +33,12 @@ DEFAULT_TRAFFIC_BYTES = int((208470 * (262144 / 131086) + 2176 * 1.0) * 1024)
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--preheat-ms", type=float, default=300.0,
+                    help="run the step untimed for this long before the warmup steps, so that the GPU's power "
+                         "management has reached its sustained state (the first ~10 ms after a quiet period run at "
+                         "lower clocks: 50 steps measured cold give 172 us/layer, 1000 steps 146 us); 0 switches it off")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--hq", type=int, default=32)
@@ -224,6 +228,13 @@ def main():
     def step():
         ops.attn_decode(q, ke, ve, kw, vw, out=out, variant=args.variant)
 
+    preheat_steps = 0
+    t_end = time.perf_counter() + args.preheat_ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        preheat_steps += 20
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -244,7 +255,7 @@ def main():
         "metric": "fused decompress-attn decode us/layer",
         "value": ms_step * 1e3, "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic", "preheat": {"ms": args.preheat_ms, "steps": preheat_steps},
         "config": {"workload": "configs[1]: GQA decode, batch %d, %d q / %d KV heads, head_dim 128, %d tokens"
                                " (%d compressed + %d fp16 tail), rel %.3g, %d-bit codes"
                                % (B, Hq, Hkv, T, Tc, Tw, args.rel, bits),
