@@ -415,6 +415,15 @@ __device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane
 // So x crosses HBM once, and the ordered-ticket / look-back traffic shrinks eightfold.
 constexpr int kSubBlocks = 8;
 
+// Wave priorities (s_setprio) of the round-major encoders' phases: the parameter pass goes first, so that its rows
+// are requested from HBM as early as possible; forming the packs, the long arithmetic phase, yields to everything
+// else.  Worth 3-4 % (0.392 -> 0.377 ms for K, 0.431 -> 0.414 ms for V on 1 GiB of input).
+#ifndef PKV_EPRIO_STAT
+#define PKV_EPRIO_STAT 3
+#define PKV_EPRIO_PACK 0
+#define PKV_EPRIO_EMIT 2
+#endif
+
 template <bool IS_K, int DT>
 __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
@@ -625,6 +634,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     uint32_t cmax_all = 0;
     for (int r = 0; r < 4; r++) {
         // token parameters of the round: 16 lanes x 8 channels per token, all heads
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
             float mn = INFINITY, mx = -INFINITY;
@@ -653,10 +663,12 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         uint2 xr[16];
         cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
         __syncthreads();
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         UnitPacks u;
         uint32_t cmax;
         cell_packs<DT>(xr, s_par, u, cmax);
         __syncthreads();                                  // s_par is rewritten by the next round
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
         if (active) {
             cmax_all = max(cmax_all, cmax);
@@ -798,6 +810,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     uint32_t cmax_all = 0;
     for (int it = 0; it < 4; it++) {
         // token parameters of the 32 tokens: 16 lanes x 8 channels per token, all heads
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
             float mn = INFINITY, mx = -INFINITY;
@@ -826,6 +839,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         uint2 xr[16];
         cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
         __syncthreads();
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         UnitPacks u;
         uint32_t cmax;
         cell_packs<DT>(xr, s_par + 16 * rp, u, cmax);
@@ -840,6 +854,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         const uint32_t tot = __shfl(inc, 7, 8);
         if (m == 0) s_tot[rp][j][t >> 3] = tot;
         __syncthreads();                                  // s_par is rewritten by the next iteration; s_tot is published
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
         if (active) {
             cmax_all = max(cmax_all, cmax);
