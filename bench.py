@@ -23,11 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the decode kernel on the default workload, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 208470 and WRITE_SIZE 2176 per dispatch), each scaled by what the same counter read
-# for a plain 256 MiB device copy in the same run (131086 -> factor 1.99979; 262144 -> factor 1.0);
+# (FETCH_SIZE 208383 and WRITE_SIZE 2176 per dispatch), each scaled by what the same counter read
+# for a plain 256 MiB device copy in the same run (131088 -> factor 1.99976; 262144 -> factor 1.0);
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
-DEFAULT_TRAFFIC_BYTES = int((208470 * (262144 / 131086) + 2176 * 1.0) * 1024)
+DEFAULT_TRAFFIC_BYTES = int((208383 * (262144 / 131088) + 2176 * 1.0) * 1024)
 
 
 def parse():

@@ -13,6 +13,10 @@
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
 
+#ifndef PKV_SPLIT_TARGET
+#define PKV_SPLIT_TARGET 1024
+#endif
+
 namespace pkv {
 
 constexpr int kTile = 128;              // tokens per super-tile
@@ -588,7 +592,7 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     int nsplit = 0, tps = 0;
     if (n_tiles > 0) {
         const int pairs = a->B * a->Hkv;
-        const int target = 1024;                   // four resident workgroups on each of 256 CUs
+        const int target = PKV_SPLIT_TARGET;       // four resident workgroups on each of 256 CUs
         int want = (target + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
         if (want < 1) want = 1;
         if (want > n_tiles) want = n_tiles;
