@@ -85,6 +85,10 @@ __device__ __forceinline__ uint32_t pk_mask16(uint32_t len_pair) {   // (1 << le
     return __builtin_bit_cast(uint32_t, (ushort2v)((ushort2v)(one << __builtin_bit_cast(ushort2v, len_pair)) - one));
 }
 
+__device__ __forceinline__ int4v pair128(long a, long b) {
+    return (int4v){(int)a, (int)(a >> 32), (int)b, (int)(b >> 32)};
+}
+
 // 64 bits at byte offset `off` (even) of an LDS array whose base is 4-byte aligned: the three
 // aligned dwords that cover it, funnel-shifted by bytes (a misaligned DS read stalls the LDS pipe).
 __device__ __forceinline__ uint64_t lds_word64(const uint8_t *base, uint32_t off) {
@@ -362,8 +366,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 #pragma unroll
             for (int s = 0; s < NSETS; s++) {
                 int4v d = {0, 0, 0, 0};
+                // two K = 64 products: which 64 channels an instruction contracts does not matter as long
+                // as A and B pair up the same ones, and both operands were loaded in the same pattern
+                // (the 8 channels at 32 sl + 8 (lane / 16)), so slices (0, 1) and (2, 3) simply concatenate
 #pragma unroll
-                for (int sl = 0; sl < 4; sl++) d = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[s][sl], bop[sl], d, 0, 0, 0);
+                for (int sl = 0; sl < 4; sl += 2)
+                    d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pair128(aop[s][sl], aop[s][sl + 1]), pair128(bop[sl], bop[sl + 1]), d, 0, 0, 0);
                 // row-major [m][token]; odd rounds sit 16 banks further so the softmax reads spread over all banks
                 // (the four rows one instruction writes, m = 4 (lane / 16) + jj, are stored as 4 jj + lane / 16:
                 // adjacent, so they alternate between the two halves of the banks)
