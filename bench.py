@@ -285,7 +285,10 @@ def main():
         ops.v_decode(ve["stream"], ve["info"], codes_v, 128, 64, bits)
         rp_ms = event_time_ms(torch, lambda: ops.median_repacking(codes, codes_v, 64), 3)
         bp_ms = event_time_ms(torch, lambda: ops.bit_pack_bytes(codes, 16), 3)
+        g_rows = min(Tc, 8192)      # the greedy order re-reads a block once per pick: a slice of the workload is enough
+        gr_ms = event_time_ms(torch, lambda: ops.greedy_repacking(codes[:g_rows], codes_v[:g_rows], 16, 64), 2)
         result["repack"] = {
+            "greedy_repack_ms": gr_ms, "greedy_repack_rows": g_rows,
             "median_repack_ms": rp_ms, "median_repack_gbs": 5 * Tc * hidden / (rp_ms * 1e-3) / 1e9,   # V read twice, K once, both written
             "bit_pack_size_ms": bp_ms, "bit_pack_size_gbs": Tc * hidden / (bp_ms * 1e-3) / 1e9,
         }

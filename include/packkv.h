@@ -136,6 +136,15 @@ int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pac
                       uint32_t *n_unique_out, float *ms_out, pkv_stream_t s);
 int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,
                       int ctx_len, int hidden_dim, int block_size, float *ms_out, pkv_stream_t s);
+/* pkv_greedy_repack (utils/compute.py:210-260, `greedy_repacking`, with `_batched_pick` :186-208): every block of
+ *   `block_size` tokens (at most 256, a multiple of pack_len) is rebuilt pack by pack -- a pack starts from the
+ *   remaining token with the largest cosine to the rounded mean of the remaining tokens (rows = K codes then V
+ *   codes of all channels) and then takes, pack_len - 1 times, the remaining token that adds the fewest payload
+ *   bits, sum over channels of bit_length(max - min).  Integer arithmetic throughout, cosines compared exactly,
+ *   every tie to the earlier token (the reference computes both criteria in fp32 and leaves ties to the backend).
+ *   Same outputs as pkv_median_repack.  hidden_dim <= 32768. */
+int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,
+                      int ctx_len, int hidden_dim, int block_size, int pack_len, float *ms_out, pkv_stream_t s);
 
 /* ---- the reference's GEMV surface -----------------------------------------------------
  * kq_mat_vec_mul (packkv_cuda.pyi:26-36, src/kernels.cu:611-630):

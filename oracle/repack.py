@@ -2,12 +2,24 @@
 
 Follows utils/compute.py:262-270 (``median_repacking``), :272-297 (``bit_pack``) and :329-357
 (``repack_and_encode``: K and V codes side by side, ``blocks`` [n_blocks, block tokens, 2 * B * H * D]).
-``greedy_repacking`` (:210-260) is not restated.
+``greedy_repacking`` (:210-260, with ``_batched_pick`` :186-208) is restated in integers, see below.
 
 Tie order.  The reference sorts the per-token medians with ``torch.sort(descending=True)`` without
 ``stable=True``; the order of equal medians is then whatever the backend does (medians of small integer codes tie
 constantly), so repacked sizes are not uniquely defined by the reference: **parity unpinned** for
 ``RepackMethod.MEDIAN``.  This restatement, like the device kernels, keeps ties in their original order.
+
+Greedy method.  Every pack starts from the remaining token most similar (cosine) to the rounded mean of the
+remaining tokens and then takes, pack_len - 1 times, the remaining token that adds the fewest payload bits
+(sum over channels of bit_length(max - min)).  The reference computes both criteria in fp32 and leaves ties to
+``torch.argmax`` / ``torch.argmin``.  The bit counts are small integers, exact in fp32, so only the tie order of
+the second criterion is open; the cosine, however, is a rounded fp32 quotient whose near-ties depend on the
+backend's reduction order: **parity unpinned** for ``RepackMethod.GREEDY`` as well.  This restatement (and the
+device kernel) compares the cosines exactly -- codes are non-negative integers, the mean is common to all
+candidates, so cos_a > cos_b  <=>  dot_a^2 * |b|^2 > dot_b^2 * |a|^2 in integers -- and resolves every tie to the
+token that comes first in the block.  Pinned by: a brute-force fp64 recomputation of both criteria on small random
+blocks away from ties, the invariant that the result is a permutation that never raises the seed's own cost, and
+the hand-built cases of tests/test_oracle_quant.py.
 
 Pinned by (tests/test_oracle_quant.py): the median against ``torch.median`` (library routine: lower median on an
 even count) and the order against ``torch.sort(descending=True, stable=True)``; ``bit_pack`` against the closed
@@ -44,6 +56,50 @@ def median_repacking(blocks):
     return np.take_along_axis(blocks, order[:, :, None], axis=1), order
 
 
+def _bit_length(a):
+    """bit_length of non-negative integers below 2**16, elementwise (= ceil(log2(a + 1)))."""
+    return np.frexp(np.asarray(a, dtype=np.float64))[1].astype(np.int64)    # a = m * 2**e, m in [0.5, 1): e = bit_length
+
+
+def greedy_order(block, pack_len):
+    """Order of ``greedy_repacking`` (utils/compute.py:210-260) for ONE block [N, D] of non-negative integer codes:
+    order[r] = original position of the token picked r-th.  Ties go to the earlier token (see the module text)."""
+    x = np.asarray(block, dtype=np.int64)
+    n, _ = x.shape
+    assert n % pack_len == 0, "the reference drops the tokens of an incomplete last pack"
+    alive = list(range(n))          # _batched_pick keeps the remaining tokens in their original order
+    order = []
+    for _ in range(n // pack_len):
+        rem = x[alive]
+        # mean(dim=1).round() in fp32: sum / count, round half to even (compute.py:219)
+        mean = np.rint(rem.sum(axis=0).astype(np.float32) / np.float32(len(alive))).astype(np.int64)
+        dot = [int(v) for v in rem @ mean]
+        nx = [int(v) for v in (rem * rem).sum(axis=1)]
+        best = 0
+        for i in range(1, len(alive)):   # cos_i > cos_best, exactly; a zero vector has cosine 0
+            if nx[i] == 0:
+                continue
+            if (dot[i] > 0) if nx[best] == 0 else (dot[i] * dot[i] * nx[best] > dot[best] * dot[best] * nx[i]):
+                best = i
+        seed = alive.pop(best)
+        order.append(seed)
+        mn, mx = x[seed].copy(), x[seed].copy()
+        for _ in range(pack_len - 1):
+            rem = x[alive]
+            # the bits before the pick are common to all candidates (compute.py:235-243): argmin of the new total
+            cost = _bit_length(np.maximum(rem, mx) - np.minimum(rem, mn)).sum(axis=1)
+            pick = alive.pop(int(np.argmin(cost)))          # np.argmin: first minimum
+            order.append(pick)
+            mn, mx = np.minimum(mn, x[pick]), np.maximum(mx, x[pick])
+    return np.asarray(order, dtype=np.int64)
+
+
+def greedy_repacking(blocks, pack_len):
+    """utils/compute.py:210-260 on blocks [n_blocks, N, D].  Returns (repacked blocks, order)."""
+    order = np.stack([greedy_order(b, pack_len) for b in blocks])
+    return np.take_along_axis(blocks, order[:, :, None], axis=1), order
+
+
 def bit_pack(blocks, pack_len):
     """utils/compute.py:272-297: (k_bytes, v_bytes)."""
     half = blocks.shape[2] // 2
@@ -65,7 +121,9 @@ def repack_and_encode(k_codes, v_codes, pack_size, method="none", block_size=64)
     k_pre, v_pre = bit_pack(blocks, pack_size)
     if method == "median":
         blocks, _ = median_repacking(blocks)
+    elif method == "greedy":
+        blocks, _ = greedy_repacking(blocks, pack_size)
     elif method != "none":
-        raise ValueError("repack_method must be one of none, median")
+        raise ValueError("repack_method must be one of none, median, greedy")
     k_aft, v_aft = bit_pack(blocks, pack_size)
     return k_pre, v_pre, k_aft, v_aft

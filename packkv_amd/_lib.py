@@ -51,6 +51,7 @@ SIGNATURES = {
     "pkv_v_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),
     "pkv_bit_pack_size": (_i, [_vp, _i, _i, _i, _u64p, ctypes.POINTER(ctypes.c_uint32), _fp, _vp]),
     "pkv_median_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _fp, _vp]),
+    "pkv_greedy_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_kq_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_wv_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_fused_kq": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),

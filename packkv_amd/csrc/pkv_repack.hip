@@ -13,6 +13,8 @@
 
 namespace pkv {
 
+typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
+
 // ---- lower median of every token row: one wavefront per token ----
 // Rows of up to 16384 codes below 128 stay in registers (16 bytes x 16 per lane) and the median is found by
 // bisection on the value: a step counts the bytes above the probe with three word-wide instructions per four codes
@@ -112,6 +114,190 @@ __global__ void block_order_kernel(const uint8_t *__restrict__ median, int block
         rank += (o > mine) || (o == mine && j < i);
     }
     perm[base + rank] = (uint32_t)i;
+}
+
+// ---- greedy order of the tokens of every block: one workgroup of 1024 threads per block ----
+// `greedy_repacking` (utils/compute.py:210-260): a block's N tokens are rows of D2 = 2 * hidden codes (K half, then
+// V half).  Every pack starts from the remaining token with the largest cosine to the rounded mean of the remaining
+// tokens and then takes, pack_len - 1 times, the remaining token whose addition costs the fewest payload bits,
+// sum over channels of bit_length(max - min).  All of it is integer work here: the bit counts are exact, the
+// bits already spent are common to all candidates (so the new total decides), and the cosines are compared exactly
+// (codes are non-negative and the mean is common: cos_a > cos_b  <=>  dot_a^2 |b|^2 > dot_b^2 |a|^2, 128-bit
+// products).  Ties go to the earlier token -- the order the reference's argmax / argmin see on a CPU backend;
+// the reference itself leaves them, and fp32 near-ties of the cosine, to the backend.
+//
+// LDS: running minimum and maximum per channel (D2 bytes each; the mean borrows the maximum's array), one cost or
+// one (dot, norm) pair per token, and the alive flags.  A wavefront prices whole tokens (tokens wave, wave + 16, ..),
+// its lanes stride over the row 16 channels at a time; every wavefront then finds the winner for itself from the
+// LDS array, so a pick costs two barriers.
+constexpr int kGreedyThreads = 1024;
+constexpr int kGreedyMaxTokens = 256;
+
+__device__ __forceinline__ uint32_t bytes_even(uint32_t x) { return x & 0x00FF00FFu; }          // bytes 0, 2 -> 16-bit lanes
+__device__ __forceinline__ uint32_t bytes_odd(uint32_t x) { return (x >> 8) & 0x00FF00FFu; }    // bytes 1, 3
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ushort2v, a), __builtin_bit_cast(ushort2v, b)));
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(ushort2v, a), __builtin_bit_cast(ushort2v, b)));
+}
+// bit_length of a value below 256 held in byte `B` of x: the exponent of its float (frexp: 0 -> 0, 1 -> 1, 2..3 -> 2, ..)
+template <int B>
+__device__ __forceinline__ uint32_t byte_bit_length(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_frexp_expf((float)((x >> (8 * B)) & 0xFFu));
+}
+// sum over the four bytes of bit_length(max(x, mx) - min(x, mn))
+__device__ __forceinline__ uint32_t range_bits4(uint32_t x, uint32_t mn, uint32_t mx) {
+    const uint32_t re = pk_max_u16(bytes_even(x), bytes_even(mx)) - pk_min_u16(bytes_even(x), bytes_even(mn));
+    const uint32_t ro = pk_max_u16(bytes_odd(x), bytes_odd(mx)) - pk_min_u16(bytes_odd(x), bytes_odd(mn));
+    return byte_bit_length<0>(re) + byte_bit_length<2>(re) + byte_bit_length<0>(ro) + byte_bit_length<2>(ro);
+}
+__device__ __forceinline__ uint32_t bytes_min4(uint32_t a, uint32_t b) {
+    return pk_min_u16(bytes_even(a), bytes_even(b)) | (pk_min_u16(bytes_odd(a), bytes_odd(b)) << 8);
+}
+__device__ __forceinline__ uint32_t bytes_max4(uint32_t a, uint32_t b) {
+    return pk_max_u16(bytes_even(a), bytes_even(b)) | (pk_max_u16(bytes_odd(a), bytes_odd(b)) << 8);
+}
+__device__ __forceinline__ uint32_t dot_bytes4(uint32_t a, uint32_t b) {      // sum of the four byte products
+    return (a & 0xFFu) * (b & 0xFFu) + ((a >> 8) & 0xFFu) * ((b >> 8) & 0xFFu) + ((a >> 16) & 0xFFu) * ((b >> 16) & 0xFFu) +
+           (a >> 24) * (b >> 24);
+}
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long x) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
+    return x;
+}
+// cos_a > cos_b for non-negative vectors with a common second operand: (dot, squared norm) pairs, exact
+__device__ __forceinline__ bool cos_greater(unsigned long long dot_a, unsigned long long nx_a, unsigned long long dot_b,
+                                            unsigned long long nx_b) {
+    if (nx_a == 0) return false;                 // a is the zero vector: cosine 0, never above a non-negative cosine
+    if (nx_b == 0) return dot_a > 0;
+    const unsigned long long pa = dot_a * dot_a, pb = dot_b * dot_b;          // < 2^63 for rows of up to 2^16 bytes
+    const unsigned long long lhs_hi = __umul64hi(pa, nx_b), lhs_lo = pa * nx_b;
+    const unsigned long long rhs_hi = __umul64hi(pb, nx_a), rhs_lo = pb * nx_a;
+    return lhs_hi > rhs_hi || (lhs_hi == rhs_hi && lhs_lo > rhs_lo);
+}
+
+__global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint8_t *__restrict__ k_codes,
+                                                                      const uint8_t *__restrict__ v_codes, int hidden,
+                                                                      int block_size, int pack_len,
+                                                                      uint32_t *__restrict__ perm) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t g_lds[];
+    const int D2 = 2 * hidden, n16 = D2 / 16, h16 = hidden / 16;
+    uint4 *mn = reinterpret_cast<uint4 *>(g_lds), *mx = mn + n16;                 // [D2] bytes each
+    unsigned long long *key_dot = reinterpret_cast<unsigned long long *>(mx + n16);   // [256]
+    unsigned long long *key_nx = key_dot + kGreedyMaxTokens;                           // [256]
+    uint32_t *cost = reinterpret_cast<uint32_t *>(key_nx + kGreedyMaxTokens);        // [2][256]
+    uint8_t *alive = reinterpret_cast<uint8_t *>(cost + 2 * kGreedyMaxTokens);        // [256]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int N = block_size;
+    const size_t row0 = (size_t)blockIdx.x * N;
+    // 16 channels `c16` of token `tok`: K half first, then V half
+    auto row16 = [&](int tok, int c16) -> uint4 {
+        const uint8_t *base = c16 < h16 ? k_codes + (row0 + tok) * (size_t)hidden + 16 * (size_t)c16
+                                        : v_codes + (row0 + tok) * (size_t)hidden + 16 * (size_t)(c16 - h16);
+        return *reinterpret_cast<const uint4 *>(base);
+    };
+    if (tid < kGreedyMaxTokens) alive[tid] = tid < N;
+    __syncthreads();
+
+    int n_alive = N, picked = 0, flip = 0;
+    for (int pk = 0; pk < N / pack_len; pk++) {
+        // ---- seed: rounded mean of the remaining tokens (into mx), then the best cosine ----
+        for (int c16 = tid; c16 < n16; c16 += kGreedyThreads) {
+            uint32_t sum[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) sum[i] = 0;
+            for (int tok = 0; tok < N; tok++) {
+                if (!alive[tok]) continue;
+                const uint4 x = row16(tok, c16);
+                const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int i = 0; i < 16; i++) sum[i] += (w[i >> 2] >> (8 * (i & 3))) & 0xFFu;
+            }
+            uint32_t m[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < 16; i++)      // mean(dim=1).round(): fp32 quotient, round half to even
+                m[i >> 2] |= (uint32_t)rintf((float)sum[i] / (float)n_alive) << (8 * (i & 3));
+            mx[c16] = make_uint4(m[0], m[1], m[2], m[3]);
+        }
+        __syncthreads();
+        for (int tok = wave; tok < N; tok += kGreedyThreads / 64) {
+            if (!alive[tok]) continue;
+            unsigned long long dot = 0, nx = 0;
+            for (int c16 = lane; c16 < n16; c16 += 64) {
+                const uint4 x = row16(tok, c16), m = mx[c16];
+                dot += dot_bytes4(x.x, m.x) + dot_bytes4(x.y, m.y) + dot_bytes4(x.z, m.z) + dot_bytes4(x.w, m.w);
+                nx += dot_bytes4(x.x, x.x) + dot_bytes4(x.y, x.y) + dot_bytes4(x.z, x.z) + dot_bytes4(x.w, x.w);
+            }
+            dot = wave_sum_u64(dot);
+            nx = wave_sum_u64(nx);
+            if (lane == 0) { key_dot[tok] = dot; key_nx[tok] = nx; }
+        }
+        __syncthreads();
+        int sel = -1;
+        {   // every wavefront finds the winner itself: lane-local scan in token order, then a reduction that
+            // prefers the earlier token on equal cosines
+            unsigned long long bd = 0, bn = 0;
+            for (int tok = lane; tok < N; tok += 64) {
+                if (!alive[tok]) continue;
+                if (sel < 0 || cos_greater(key_dot[tok], key_nx[tok], bd, bn)) { sel = tok; bd = key_dot[tok]; bn = key_nx[tok]; }
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                const int os = __shfl_xor(sel, d, 64);
+                const unsigned long long od = __shfl_xor(bd, d, 64), on = __shfl_xor(bn, d, 64);
+                if (os >= 0 && (sel < 0 || cos_greater(od, on, bd, bn) || (!cos_greater(bd, bn, od, on) && os < sel))) {
+                    sel = os; bd = od; bn = on;
+                }
+            }
+        }
+        __syncthreads();                          // everyone has read the mean and the alive flags
+        for (int c16 = tid; c16 < n16; c16 += kGreedyThreads) {
+            const uint4 x = row16(sel, c16);
+            mn[c16] = x;
+            mx[c16] = x;
+        }
+        if (tid == 0) { alive[sel] = 0; perm[row0 + picked] = (uint32_t)sel; }
+        picked++;
+        n_alive--;
+        __syncthreads();
+
+        // ---- the pack's other tokens: fewest bits after the pick ----
+        for (int j = 1; j < pack_len; j++) {
+            uint32_t *cst = cost + flip * kGreedyMaxTokens;
+            flip ^= 1;
+            for (int tok = wave; tok < N; tok += kGreedyThreads / 64) {
+                if (!alive[tok]) continue;
+                uint32_t bits = 0;
+                for (int c16 = lane; c16 < n16; c16 += 64) {
+                    const uint4 x = row16(tok, c16), lo = mn[c16], hi = mx[c16];
+                    bits += range_bits4(x.x, lo.x, hi.x) + range_bits4(x.y, lo.y, hi.y) + range_bits4(x.z, lo.z, hi.z) +
+                            range_bits4(x.w, lo.w, hi.w);
+                }
+                bits = wave_sum_u32(bits);
+                if (lane == 0) cst[tok] = bits;
+            }
+            __syncthreads();
+            uint32_t best = 0xFFFFFFFFu;           // (cost, token) in one word: the minimum is the first cheapest token
+            for (int tok = lane; tok < N; tok += 64)
+                if (alive[tok]) best = min(best, (cst[tok] << 8) | (uint32_t)tok);
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) best = min(best, (uint32_t)__shfl_xor(best, d, 64));
+            sel = (int)(best & 0xFFu);
+            __syncthreads();                      // everyone has read the alive flags
+            for (int c16 = tid; c16 < n16; c16 += kGreedyThreads) {
+                const uint4 x = row16(sel, c16), lo = mn[c16], hi = mx[c16];
+                mn[c16] = make_uint4(bytes_min4(lo.x, x.x), bytes_min4(lo.y, x.y), bytes_min4(lo.z, x.z), bytes_min4(lo.w, x.w));
+                mx[c16] = make_uint4(bytes_max4(hi.x, x.x), bytes_max4(hi.y, x.y), bytes_max4(hi.z, x.z), bytes_max4(hi.w, x.w));
+            }
+            if (tid == 0) { alive[sel] = 0; perm[row0 + picked] = (uint32_t)sel; }
+            picked++;
+            n_alive--;
+            __syncthreads();
+        }
+    }
 }
 
 // ---- out row r = in row perm[r], for K and V at once: grid (ctx_len), 256 threads ----
@@ -253,6 +439,37 @@ int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
     token_median_kernel<<<(unsigned)((ctx_len + 3) / 4), 256, 0, s>>>(v_codes, ctx_len, hidden_dim, median);
     const int threads = (block_size + 63) / 64 * 64;
     block_order_kernel<<<(unsigned)(ctx_len / block_size), threads, (size_t)block_size, s>>>(median, block_size, perm);
+    gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
+    PKV_HIP_CHECK(hipGetLastError());
+    return tm.end(ms_out);
+}
+
+int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,
+                      int ctx_len, int hidden_dim, int block_size, int pack_len, float *ms_out, pkv_stream_t s_) {
+    using namespace pkv;
+    hipStream_t s = (hipStream_t)s_;
+    PKV_REQUIRE(k_codes && v_codes && k_out && v_out && perm, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(k_codes != k_out && v_codes != v_out, PKV_ERR_INVALID, "repacking cannot run in place");
+    PKV_REQUIRE(ctx_len > 0 && hidden_dim > 0 && block_size > 0 && pack_len > 0, PKV_ERR_INVALID, "sizes must be positive");
+    PKV_REQUIRE(hidden_dim % 16 == 0 && ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes) |
+                                          reinterpret_cast<uintptr_t>(k_out) | reinterpret_cast<uintptr_t>(v_out)) & 15u) == 0,
+                PKV_ERR_INVALID, "hidden_dim must be a multiple of 16 and the code matrices 16-byte aligned");
+    PKV_REQUIRE(block_size <= kGreedyMaxTokens && ctx_len % block_size == 0, PKV_ERR_INVALID,
+                "ctx_len must be divisible by a block size of at most 256 tokens");
+    PKV_REQUIRE(block_size % pack_len == 0, PKV_ERR_INVALID,
+                "block_size must be a multiple of pack_len (the reference drops the tokens of an incomplete pack)");
+    // the cost word holds (bits << 8 | token): bits <= 8 * 2 * hidden_dim must stay below 2^24
+    const size_t lds = 4 * (size_t)hidden_dim + kGreedyMaxTokens * (8 + 8 + 8 + 1);
+    PKV_REQUIRE(hidden_dim <= 32768 && lds <= 160 * 1024, PKV_ERR_UNSUPPORTED,
+                "not supported: the greedy order keeps 4 * hidden_dim bytes in LDS (hidden_dim <= 32768)");
+    if (lds > 48 * 1024)
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(greedy_order_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    LaunchTimer tm(s, ms_out != nullptr);
+    int rc;
+    if ((rc = tm.begin())) return rc;
+    greedy_order_kernel<<<(unsigned)(ctx_len / block_size), kGreedyThreads, lds, s>>>(k_codes, v_codes, hidden_dim, block_size,
+                                                                                    pack_len, perm);
     gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);

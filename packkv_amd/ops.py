@@ -363,14 +363,36 @@ def median_repacking(k_codes, v_codes, block_size=64, timed=False):
     return (k_out, v_out, perm, float(ms.value)) if timed else (k_out, v_out, perm)
 
 
+def greedy_repacking(k_codes, v_codes, pack_len=16, block_size=64, timed=False):
+    """`greedy_repacking` (utils/compute.py:210-260) on the device: every block of `block_size` tokens is rebuilt pack
+    by pack -- seed = the remaining token closest (cosine) to the rounded mean of the remaining tokens, then
+    pack_len - 1 times the remaining token that adds the fewest payload bits -- jointly for K and V.  Exact integer
+    arithmetic; ties go to the earlier token.  Returns (k_repacked, v_repacked, perm) like median_repacking."""
+    _check_code_matrix(k_codes, "k_codes")
+    _check_code_matrix(v_codes, "v_codes")
+    _require(k_codes.shape == v_codes.shape, "K and V code matrices must have one shape")
+    ctx, hidden = k_codes.shape
+    k_out, v_out = torch.empty_like(k_codes), torch.empty_like(v_codes)
+    perm = torch.empty(ctx, dtype=torch.int32, device=k_codes.device)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(k_codes.device):
+        rc = _lib.load().pkv_greedy_repack(_ptr(k_codes), _ptr(v_codes), _ptr(k_out), _ptr(v_out), _ptr(perm), ctx,
+                                           hidden, int(block_size), int(pack_len), ctypes.byref(ms) if timed else None,
+                                           _stream(k_codes.device))
+    _lib.check(rc)
+    return (k_out, v_out, perm, float(ms.value)) if timed else (k_out, v_out, perm)
+
+
 def repack_and_encode(k_codes, v_codes, pack_size, repack_method="none", block_size=64):
     """`repack_and_encode` (utils/compute.py:329-357) on code matrices: (k_size_pre, v_size_pre, k_size_aft,
-    v_size_aft) in bytes.  repack_method: "none" or "median" (the greedy method is not built)."""
+    v_size_aft) in bytes.  repack_method: "none", "median" or "greedy"."""
     k_pre, v_pre = bit_pack(k_codes, v_codes, pack_size)
     if repack_method == "median":
         k_codes, v_codes, _ = median_repacking(k_codes, v_codes, block_size)
+    elif repack_method == "greedy":
+        k_codes, v_codes, _ = greedy_repacking(k_codes, v_codes, pack_size, block_size)
     elif repack_method != "none":
-        raise ValueError("repack_method must be one of none, median")
+        raise ValueError("repack_method must be one of none, median, greedy")
     k_aft, v_aft = bit_pack(k_codes, v_codes, pack_size)
     return k_pre, v_pre, k_aft, v_aft
 
@@ -392,14 +414,17 @@ def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=6
     for mx, bits in ((kmx, k_bits), (vmx, v_bits)):
         if mx >= (1 << bits):
             raise PackKVError(1, "not supported: code %d does not fit bits_len %d" % (mx, bits))
-    if repack_method == "median":
-        kc, vc, perm = median_repacking(kc, vc, block_size)
+    if repack_method in ("median", "greedy"):
+        if repack_method == "median":
+            kc, vc, perm = median_repacking(kc, vc, block_size)
+        else:
+            kc, vc, perm = greedy_repacking(kc, vc, 16, block_size)      # the codecs' packs are 16 tokens
         src = (torch.arange(T, device=k.device, dtype=torch.int64) // block_size) * block_size + perm.to(torch.int64)
         ks, kz, vs, vz = (p[:, src].contiguous() for p in (ks, kz, vs, vz))
     elif repack_method == "none":
         perm = (torch.arange(T, device=k.device, dtype=torch.int32) % block_size)
     else:
-        raise ValueError("repack_method must be one of none, median")
+        raise ValueError("repack_method must be one of none, median, greedy")
     hidden = B * H * 128
     out = []
     for is_k, codes, scale, zero, bits in ((True, kc, ks, kz, k_bits), (False, vc, vs, vz, v_bits)):

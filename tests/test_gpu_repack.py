@@ -111,6 +111,54 @@ def test_median_repacking_wide_codes_and_wide_rows(cuda):
         assert (k_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, :hid]).all()
 
 
+def test_greedy_repacking_matches_restatement(cuda):
+    """The greedy order (seed by cosine to the rounded mean, then fewest added bits) on the device against the
+    integer restatement: same permutation, same rows, same priced sizes; quantised K/V and plain random codes
+    (which tie often: ties must go to the earlier token on both sides)."""
+    cases = []
+    for (B, H, T, bs, pack) in ((1, 2, 256, 64, 16), (2, 4, 256, 64, 16), (1, 1, 128, 32, 8), (1, 2, 128, 64, 64)):
+        kc, vc = _codes(B, H, T, 0.1, seed=240 + B + H)
+        cases.append((kc, vc, bs, pack, "quantised %dx%dx%d" % (B, H, T)))
+    g = torch.Generator(device="cpu").manual_seed(241)
+    for (T, hid, top, bs, pack) in ((64, 16, 4, 16, 4), (128, 48, 2, 64, 16), (256, 2064, 200, 256, 32), (64, 32768, 16, 64, 16)):
+        kc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
+        vc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
+        cases.append((kc, vc, bs, pack, "random %dx%d below %d" % (T, hid, top)))
+    zero = torch.zeros(64, 128, dtype=torch.uint8)
+    cases.append((zero, zero.clone(), 64, 16, "all zero"))
+    for kc, vc, bs, pack, name in cases:
+        _say("greedy case", name, "block", bs, "pack", pack)
+        hid = kc.shape[1]
+        blocks = orp.blocks_from_code_matrices(kc.numpy(), vc.numpy(), bs)
+        want, order = orp.greedy_repacking(blocks, pack)
+        k_out, v_out, perm = ops.greedy_repacking(kc.to(cuda), vc.to(cuda), pack, bs)
+        assert (perm.cpu().numpy().reshape(-1, bs) == order).all()
+        assert (k_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, :hid]).all()
+        assert (v_out.cpu().numpy().reshape(-1, bs, hid) == want[:, :, hid:]).all()
+        if kc.max() > 0:
+            assert ops.repack_and_encode(kc.to(cuda), vc.to(cuda), pack, "greedy", bs) == \
+                   orp.repack_and_encode(kc.numpy(), vc.numpy(), pack, "greedy", bs)
+
+
+def test_greedy_repacking_shrinks_shifted_tokens_and_feeds_attention(cuda):
+    """Tokens with a token-wise level shift: grouping similar tokens must shrink the priced V size, and the cache
+    encoded in greedy order must attend like the cache in natural order (attention ignores token order)."""
+    B, Hq, Hkv, T = 1, 8, 2, 512
+    k, v = synth.make_kv(B, Hkv, T, seed=250)
+    g = torch.Generator().manual_seed(251)
+    v = (v.float() * 0.3 + torch.randn(1, 1, T, 1, generator=g) * 2.0).to(torch.float16)
+    q = synth.make_q(B, Hq, seed=252)
+    kd, vd = k.to(cuda), v.to(cuda)
+    ke, ve, perm = ops.repack_quant_encode(kd, vd, 0.1, 0.1, "greedy")
+    kn, vn, _ = ops.repack_quant_encode(kd, vd, 0.1, 0.1, "none")
+    assert sorted(perm.cpu().numpy().reshape(-1, 64)[0].tolist()) == list(range(64))
+    _say("greedy sizes", ke["size"], ve["size"], "natural", kn["size"], vn["size"])
+    assert ve["size"] < vn["size"]
+    out_g = ops.attn_decode(q.to(cuda), ke, ve).float().cpu()
+    out_n = ops.attn_decode(q.to(cuda), kn, vn).float().cpu()
+    assert (out_g - out_n).abs().max().item() < 2e-3
+
+
 def test_repacked_cache_attends_like_the_original(cuda):
     """Attention does not depend on the order of the cached tokens, so a cache whose 64-token blocks were reordered
     by median repacking (K, V and their per-token parameters together) must give the output of the cache in natural

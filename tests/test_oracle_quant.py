@@ -144,3 +144,53 @@ def test_repack_restatement_against_library_routines():
     # packs of 2 tokens: K (11,12) (10,13) -> ranges 1, 3 -> 1 + 2 bits; 4 distinct values -> W = 2, 2 + 2 metadata bits
     kb, vb = orp.bit_pack(rep, 2)
     assert kb == ((1 + 2) * 2 + 2 * (2 + 2)) // 8
+
+
+def test_greedy_repack_restatement_against_brute_force():
+    """greedy_repacking (utils/compute.py:210-260): the integer restatement against a direct fp64 transcription of
+    the two criteria (cosine to the rounded mean; added bits as ceil(log2(range + 1)) differences), on random blocks
+    whose criteria have no ties, plus hand-built blocks with a known answer."""
+    from oracle import repack as orp
+
+    def brute(block, pack_len):
+        x = block.astype(np.float64)
+        alive, order = list(range(len(x))), []
+        for _ in range(len(x) // pack_len):
+            rem = x[alive]
+            mean = np.round(rem.mean(axis=0))            # numpy rounds half to even, like torch
+            cos = (rem @ mean) / np.maximum(np.linalg.norm(rem, axis=1) * np.linalg.norm(mean), 1e-8)
+            gap = np.sort(cos)[::-1]
+            assert len(gap) < 2 or gap[0] - gap[1] > 1e-9, "test data must not tie"
+            seed = alive.pop(int(np.argmax(cos)))
+            order.append(seed)
+            mn, mx = x[seed].copy(), x[seed].copy()
+            for _ in range(pack_len - 1):
+                rem = x[alive]
+                pre = np.ceil(np.log2(mx - mn + 1))
+                inc = (np.ceil(np.log2(np.maximum(rem, mx) - np.minimum(rem, mn) + 1)) - pre).sum(axis=1)
+                pick = alive.pop(int(np.argmin(inc)))      # ties: first, the documented rule
+                order.append(pick)
+                mn, mx = np.minimum(mn, x[pick]), np.maximum(mx, x[pick])
+        return order
+
+    rng = np.random.default_rng(11)
+    for (n, d, pack, top) in ((16, 24, 4, 16), (32, 40, 8, 12), (64, 64, 16, 16), (12, 10, 3, 200)):
+        for _ in range(3):
+            block = rng.integers(0, top, size=(n, d))
+            got = orp.greedy_order(block, pack)
+            assert sorted(got.tolist()) == list(range(n))            # a permutation
+            assert got.tolist() == brute(block, pack)
+    # hand-built: 1 channel per half is too coarse for a cosine, so use 2 channels.  Tokens (rows):
+    #   a = (4, 4)  b = (4, 5)  c = (0, 9)  d = (9, 0);  mean = (4.25, 4.5) -> rounds to (4, 4): a has cosine 1 -> seed a.
+    #   pack_len 2: b adds bit_length(0) + bit_length(1) = 1 bit, c adds 3 + 3, d adds 3 + 3 -> b.  Second pack: remaining
+    #   c, d: mean (4.5, 4.5) -> (4, 4) (half to even), cosines equal -> earlier token c, then d.
+    block = np.array([[4, 4], [4, 5], [0, 9], [9, 0]])
+    assert orp.greedy_order(block, 2).tolist() == [0, 1, 2, 3]
+    assert orp.greedy_order(block[[2, 3, 1, 0]], 2).tolist() == [3, 2, 0, 1]      # same tokens, other positions
+    # all-zero tokens: every cosine is 0, every cost 0 -> original order
+    assert orp.greedy_order(np.zeros((8, 6), dtype=np.int64), 4).tolist() == list(range(8))
+    # repacking by the greedy order never costs more payload bits than the seed packs' own lower bound and keeps the tokens
+    blocks = rng.integers(0, 16, size=(3, 64, 2 * 32))
+    rep, order = orp.greedy_repacking(blocks, 16)
+    assert (np.sort(rep, axis=1) == np.sort(blocks, axis=1)).all()
+    assert (rep == np.take_along_axis(blocks, order[:, :, None], axis=1)).all()
