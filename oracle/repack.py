@@ -127,3 +127,23 @@ def repack_and_encode(k_codes, v_codes, pack_size, method="none", block_size=64)
         raise ValueError("repack_method must be one of none, median, greedy")
     k_aft, v_aft = bit_pack(blocks, pack_size)
     return k_pre, v_pre, k_aft, v_aft
+
+
+def crs_record(k, v, block_size, pack_size, k_rel, v_rel, method="none"):
+    """One layer of ``crs_evaluation_with_data`` (evaluation/evaluation.py:188-250) for K, V torch tensors
+    [B, H, T, D]: the sizes in bytes that the reference appends to its record, as a dict (the ratios are
+    original / size and are left to the caller)."""
+    import torch
+    from oracle import quant as oq
+    out, mats = {}, {}
+    for side, x, rel in (("k", k, k_rel), ("v", v, v_rel)):
+        codes, zero, scale = oq.quant_ints(x, block_size, rel)
+        bit_num = math.ceil(math.log2(int(torch.unique(codes).numel())))
+        out[side + "_original_size"] = x.numel() * x.element_size()
+        out[side + "_quant_size"] = (codes.numel() * bit_num // 8 + zero.numel() * zero.element_size() +
+                                     scale.numel() * scale.element_size())
+        mats[side] = oq.code_matrix(codes).numpy()
+    pre_k, pre_v, aft_k, aft_v = repack_and_encode(mats["k"], mats["v"], pack_size, method, block_size)
+    out.update(k_encode_size_before_repack=pre_k, v_encode_size_before_repack=pre_v,
+               k_encode_size_after_repack=aft_k, v_encode_size_after_repack=aft_v)
+    return out

@@ -319,10 +319,10 @@ def _check_code_matrix(c, name):
              "%s must be a contiguous device UInt8 code matrix [ctx_len, hidden]" % name)
 
 
-def bit_pack_bytes(codes, pack_len, timed=False):
-    """Analytic size of ONE code matrix [ctx_len, hidden] in bytes, as `bit_pack` prices each half
-    (utils/compute.py:272-297): packs of `pack_len` consecutive tokens of one channel cost
-    pack_len * bit_length(max - min) payload bits + W + ceil(log2(W + 1)) metadata bits, W = ceil(log2(#codes))."""
+def code_stats(codes, pack_len, timed=False):
+    """(sum over packs of bit_length(max - min), number of distinct code values) of a code matrix [ctx_len, hidden]
+    for packs of `pack_len` consecutive tokens of one channel: the two data-dependent terms of `bit_pack`
+    (utils/compute.py:272-297)."""
     _check_code_matrix(codes, "codes")
     ctx, hidden = codes.shape
     len_sum, n_unique, ms = ctypes.c_uint64(0), ctypes.c_uint32(0), ctypes.c_float(0.0)
@@ -331,10 +331,20 @@ def bit_pack_bytes(codes, pack_len, timed=False):
                                            ctypes.byref(n_unique), ctypes.byref(ms) if timed else None,
                                            _stream(codes.device))
     _lib.check(rc)
-    w = math.ceil(math.log2(n_unique.value))
+    out = (int(len_sum.value), int(n_unique.value))
+    return out + (float(ms.value),) if timed else out
+
+
+def bit_pack_bytes(codes, pack_len, timed=False):
+    """Analytic size of ONE code matrix [ctx_len, hidden] in bytes, as `bit_pack` prices each half
+    (utils/compute.py:272-297): packs of `pack_len` consecutive tokens of one channel cost
+    pack_len * bit_length(max - min) payload bits + W + ceil(log2(W + 1)) metadata bits, W = ceil(log2(#codes))."""
+    len_sum, n_unique, ms = code_stats(codes, pack_len, timed=True)
+    ctx, hidden = codes.shape
+    w = math.ceil(math.log2(n_unique))
     n_packs = (ctx // pack_len) * hidden
-    size = (int(len_sum.value) * pack_len + n_packs * (w + math.ceil(math.log2(w + 1)))) // 8
-    return (size, float(ms.value)) if timed else size
+    size = (len_sum * pack_len + n_packs * (w + math.ceil(math.log2(w + 1)))) // 8
+    return (size, ms) if timed else size
 
 
 def bit_pack(k_codes, v_codes, pack_len):
