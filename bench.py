@@ -51,6 +51,13 @@ def parse():
     ap.add_argument("--layers", type=int, default=0,
                     help="instead of the single-layer step: a decode loop over this many layers through the growing "
                          "compressed cache (configs[4] is --layers 32 --batch 4 --ctx 131072); prints its own JSON line")
+    ap.add_argument("--e2e", action="store_true",
+                    help="instead of the single-layer step: greedy decoding on a random-init decoder of Qwen3-8B shape "
+                         "through the compressed cache (configs[3]: --e2e --batch 32 --ctx 8192 --steps 256); --e2e-layers "
+                         "and --e2e-dense-steps scale it; prints its own JSON line")
+    ap.add_argument("--e2e-layers", type=int, default=36)
+    ap.add_argument("--e2e-dense-steps", type=int, default=4,
+                    help="steps of the decompress-then-attend path timed beside the fused one (on a copy of the run)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -180,6 +187,64 @@ def decode_loop(torch, args, dev):
     print(json.dumps(result))
 
 
+def e2e_decode(torch, args, dev):
+    """configs[3]: a random-init decoder of Qwen3-8B shape (bf16 weights ~ N(0, 0.02)), a random-token prompt of
+    --ctx tokens per sequence, --steps greedy tokens; the cache compresses a 64-token cut whenever its 16-bit buffer
+    reaches 192 tokens.  Reports decode tokens/s of the fused path, the prompt pass, the bytes the caches hold, and
+    a few steps of the reference's decompress-then-attend on the same cache for scale."""
+    from packkv_amd.cache import PackKVCacheConfig
+    from packkv_amd.decoder import DecoderShape, ShapedDecoder
+    B, T, steps = args.batch, args.ctx, args.steps
+    shape = DecoderShape(layers=args.e2e_layers, q_heads=args.hq, kv_heads=args.hkv)
+    t0 = time.perf_counter()
+    model = ShapedDecoder(shape, dtype=torch.bfloat16, device=dev, seed=0)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    ids = torch.randint(0, shape.vocab, (B, T), generator=torch.Generator().manual_seed(1)).to(dev)
+    cache = model.new_cache(B, T + steps + args.e2e_dense_steps + 256, PackKVCacheConfig(64, 192, args.rel, args.rel))
+    torch.cuda.reset_peak_memory_stats()
+    t0 = time.perf_counter()
+    logits = model.prefill(ids, cache)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    for _ in range(args.warmup):               # untimed steps (they stay in the cache; the timed ones follow)
+        logits = model.forward(logits.argmax(dim=-1, keepdim=True), cache, attention="fused")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        logits = model.forward(logits.argmax(dim=-1, keepdim=True), cache, attention="fused")
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) * 1e3 / steps
+    kv_bytes, seq = cache.cache_bytes(), cache.get_seq_length(0)
+    lay0 = cache.layers[0]
+    dense_ms = None
+    if args.e2e_dense_steps > 0:
+        nxt = logits.argmax(dim=-1, keepdim=True)
+        model.forward(nxt, cache, attention="dense")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.e2e_dense_steps):
+            model.forward(nxt, cache, attention="dense")
+        torch.cuda.synchronize()
+        dense_ms = (time.perf_counter() - t0) * 1e3 / args.e2e_dense_steps
+    result = {
+        "metric": "end-to-end greedy decode tokens/s with the compressed cache", "value": B / (step_ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": step_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "random-init decoder, %d layers, hidden %d, %d q / %d KV heads, head_dim 128, vocabulary %d; "
+                               "batch %d, %d-token random prompt, %d greedy tokens (+%d untimed), rel %.3g, 64-token cuts, "
+                               "16-bit buffer 128..191 tokens" % (shape.layers, shape.hidden, shape.q_heads, shape.kv_heads,
+                                                                  shape.vocab, B, T, steps, args.warmup, args.rel)},
+        "prefill_s": prefill_s, "prefill_tokens_per_s": B * T / prefill_s, "model_build_s": build_s,
+        "cached_tokens": seq, "compressed_tokens": lay0.k.tokens,
+        "kv_bytes": kv_bytes, "fp16_kv_bytes": shape.layers * 2 * B * shape.kv_heads * seq * 128 * 2,
+        "decompress_then_attend_ms_per_step": dense_ms,
+        "peak_device_bytes": torch.cuda.max_memory_allocated(),
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -196,6 +261,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.layers > 0:
         decode_loop(torch, args, dev)
+        return
+    if args.e2e:
+        e2e_decode(torch, args, dev)
         return
     B, Hq, Hkv, T, Tw = args.batch, args.hq, args.hkv, args.ctx, args.window
     Tc = T - Tw
