@@ -374,6 +374,15 @@ def main():
             "k_gbs": (ke["size"] + 8 * nblk_k + Tc * hidden) / (uk_ms * 1e-3) / 1e9,
             "v_gbs": (ve["size"] + 8 * nblk_v + Tc * hidden) / (uv_ms * 1e-3) / 1e9,
         }
+        # what this GPU sustains on plain traffic, beside the published 8 TB/s the roofline is priced against:
+        # a 1 GiB device-to-device copy (read + write) and the read-only parameter pass over the same 1 GiB
+        src = kc.view(torch.uint8).reshape(-1)
+        dst = torch.empty_like(src)
+        cp_ms = event_time_ms(torch, lambda: dst.copy_(src), 5)
+        rd_ms = event_time_ms(torch, lambda: ops.quant_params(kc, args.rel), 5)
+        result["hbm_probe"] = {"copy_gbs": 2 * src.numel() / (cp_ms * 1e-3) / 1e9,
+                               "read_gbs": src.numel() / (rd_ms * 1e-3) / 1e9, "bytes": src.numel()}
+        del dst
 
     if not args.no_cpu:
         k1, v1, q1 = kc[:1].cpu(), vc[:1].cpu(), q[:1].cpu()

@@ -415,7 +415,7 @@ def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=6
     permutation [T] int32 (perm[blk * block_size + r] = position inside the block the token at r came from)."""
     B, H, T = _check_x(k)
     _require(v.shape == k.shape and v.dtype == k.dtype and v.is_cuda and v.is_contiguous(), "K and V must have one shape")
-    _require(T % 128 == 0 and 128 % block_size == 0 or block_size % 128 == 0, "token count / block size mismatch")
+    _require(T % 128 == 0 and T % block_size == 0, "the token count must be a multiple of 128 and of block_size")
     k_bits, v_bits = k_bits or bits_for_rel(k_rel), v_bits or bits_for_rel(v_rel)
     ks, kz = quant_params(k, k_rel)
     vs, vz = quant_params(v, v_rel)
