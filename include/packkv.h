@@ -121,6 +121,18 @@ int pkv_v_quant_encode_append(const void *x, int dtype, int B, int H, int T_new,
                                void *scale_tail, void *zero_tail, int par_stride, uint64_t *size_out,
                                float *ms_out, pkv_stream_t s);
 
+/* ---- the decode step's write into a cache's 16-bit window ------------------------------
+ * pkv_window_append: rows win_pos .. win_pos + n - 1 of the windows k_win / v_win [B, H, win_stride, 128] receive the
+ * new tokens k_new / v_new [B, H, n, 128] (element strides stride_b / stride_h / stride_t, channels contiguous; the
+ * same for both).  With cos / sin [B, n, 128] (batch stride rot_stride_b elements, 0 for one shared table) the K rows
+ * get the rotary embedding first, rounded like the reference's chain of 16-bit elementwise kernels
+ * (`apply_rotary_pos_emb_single`, utils/compute.py:35-43, applied by the cache itself,
+ * models/cache/packkv_quant.py:59-60); cos = sin = NULL copies K as it is.  Stands in for that embedding plus the
+ * torch.cat growth of the reference's buffer (packkv_quant.py:62-83) on a decode step that cuts nothing. */
+int pkv_window_append(const void *k_new, const void *v_new, const void *cos, const void *sin, int dtype, int B, int H,
+                      int n, int64_t stride_b, int64_t stride_h, int64_t stride_t, int64_t rot_stride_b, void *k_win,
+                      void *v_win, int win_pos, int win_stride, pkv_stream_t s);
+
 /* ---- token repacking and the analytic pack-size model ---------------------------------
  * On the uint8 code matrix [ctx_len, hidden_dim] (channel = (b * H + h) * 128 + d).
  * pkv_bit_pack_size (utils/compute.py:272-297, `bit_pack`, one of its two halves): packs are

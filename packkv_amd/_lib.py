@@ -49,6 +49,8 @@ SIGNATURES = {
     "pkv_v_quant_encode": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
     "pkv_k_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),
     "pkv_v_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),
+    "pkv_window_append": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                               ctypes.c_int64, _vp, _vp, _i, _i, _vp]),
     "pkv_bit_pack_size": (_i, [_vp, _i, _i, _i, _u64p, ctypes.POINTER(ctypes.c_uint32), _fp, _vp]),
     "pkv_median_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _fp, _vp]),
     "pkv_greedy_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),

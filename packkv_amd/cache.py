@@ -129,18 +129,19 @@ class PackKVCompressedCache:
         (K, V) [B, H, T, 128] the reference returns (packkv_quant.py:84-85)."""
         L = self._layer(layer_idx)
         cfg = self.config
-        if cache_kwargs and cache_kwargs.get("cos") is not None:
-            key_states = apply_rotary_pos_emb_single(key_states, cache_kwargs["cos"], cache_kwargs["sin"])
+        rotary = bool(cache_kwargs) and cache_kwargs.get("cos") is not None
         n = key_states.size(2)
         buf_len = L.win_len - L.pend
         total = buf_len + n
         n_blk = max((total + cfg.block_size - total % cfg.block_size - cfg.buffer_size) // cfg.block_size, 0)
         n_cut = n_blk * cfg.block_size
-        if n_cut == 0 and L.win_len + n <= L.cap:                 # the common decode step: one more row
-            L.k_win[:, :, L.win_len:L.win_len + n] = key_states
-            L.v_win[:, :, L.win_len:L.win_len + n] = value_states
+        if n_cut == 0 and L.win_len + n <= L.cap:                 # the common decode step: rotary + the new rows, one launch
+            ops.window_append(key_states, value_states, cache_kwargs["cos"] if rotary else None,
+                              cache_kwargs["sin"] if rotary else None, L.k_win, L.v_win, L.win_len)
             L.win_len += n
         else:
+            if rotary:
+                key_states = apply_rotary_pos_emb_single(key_states, cache_kwargs["cos"], cache_kwargs["sin"])
             kbuf = torch.cat([L.k_win[:, :, L.pend:L.win_len], key_states], dim=2)
             vbuf = torch.cat([L.v_win[:, :, L.pend:L.win_len], value_states], dim=2)
             k_cut, v_cut = kbuf[:, :, :n_cut], vbuf[:, :, :n_cut]

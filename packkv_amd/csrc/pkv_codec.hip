@@ -225,6 +225,8 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
                     float *ms_out, hipStream_t s) {
     PKV_REQUIRE(stream && info && codes, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
+    // block_info holds 32-bit byte offsets: a stream past 4 GiB is reported as a full buffer, never wrapped
+    if (capacity > (1ull << 32)) capacity = 1ull << 32;
     CodecShape cs;
     int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
     if (rc) return rc;

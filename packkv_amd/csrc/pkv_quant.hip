@@ -952,6 +952,10 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
     PKV_REQUIRE(par_stride >= T, PKV_ERR_INVALID, "parameter row stride shorter than the token count");
     PKV_REQUIRE(base <= capacity, PKV_ERR_INVALID, "stream offset beyond the buffer");
+    // block_info holds 32-bit byte offsets (uint32 in the reference too, evaluation/evaluation.py:420-426): a stream
+    // that would grow past 4 GiB is reported as a full buffer instead of wrapping its offsets
+    if (capacity > (1ull << 32)) capacity = 1ull << 32;
+    PKV_REQUIRE(base <= capacity, PKV_ERR_CAPACITY, "stream offset beyond 4 GiB: block_info offsets are 32 bits");
     ScanState *st = nullptr;
     // One workgroup per sub-group of up to eight consecutive blocks that share (context block, sequence).
     {

@@ -312,6 +312,34 @@ def quant_encode_append(is_k, x, rel, bits, stream, used, info, tokens, scale, z
     return int(size.value)
 
 
+def window_append(k_new, v_new, cos, sin, k_win, v_win, win_pos):
+    """Write the new tokens k_new / v_new [B, H, n, 128] into rows win_pos.. of the 16-bit windows k_win / v_win
+    [B, H, cap, 128]; with cos / sin [B, n, 128] the keys get the rotary embedding first, rounded like the reference's
+    chain of 16-bit elementwise ops (utils/compute.py:35-43).  One launch; strided views (a transposed projection
+    output, an expanded cos / sin table) are read in place."""
+    B, H, n, D = k_new.shape
+    _require(D == 128 and v_new.shape == k_new.shape and k_new.is_cuda and v_new.dtype == k_new.dtype,
+             "K and V must be device tensors [B, H, n, 128] of one dtype")
+    _require(k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape and k_win.dim() == 4
+             and k_win.size(0) == B and k_win.size(1) == H and k_win.size(3) == 128 and k_win.dtype == k_new.dtype,
+             "windows must be contiguous [B, H, cap, 128] of the tokens' dtype")
+    if k_new.stride(3) != 1 or k_new.stride() != v_new.stride():
+        k_new, v_new = k_new.contiguous(), v_new.contiguous()
+    rot_sb = 0
+    if cos is not None:
+        _require(cos.shape == (B, n, 128) and sin.shape == (B, n, 128) and cos.dtype == k_new.dtype
+                 and sin.dtype == k_new.dtype, "cos / sin must be [B, n, 128] of the tokens' dtype")
+        if cos.stride(2) != 1 or (n > 1 and cos.stride(1) != 128) or cos.stride() != sin.stride():
+            cos, sin = cos.contiguous(), sin.contiguous()
+        rot_sb = cos.stride(0) if B > 1 else 0
+    with torch.cuda.device(k_new.device):
+        rc = _lib.load().pkv_window_append(_ptr(k_new), _ptr(v_new), _ptr(cos) if cos is not None else None,
+                                           _ptr(sin) if cos is not None else None, _dtype_code(k_new), B, H, n,
+                                           k_new.stride(0), k_new.stride(1), k_new.stride(2), rot_sb, _ptr(k_win),
+                                           _ptr(v_win), int(win_pos), k_win.size(2), _stream(k_new.device))
+    _lib.check(rc)
+
+
 # ------------------------------------------------- repacking and analytic size ------
 
 def _check_code_matrix(c, name):

@@ -130,3 +130,37 @@ def test_cache_bytes_and_prefill_only(cuda):
     assert out.shape == (B, 32, 1, 128)
     err = np.abs(out[:, :, 0].double().cpu().numpy() - ref)
     assert (err <= SHORT_ABS_TOL[torch.float16] + REL_TOL * np.abs(ref)).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_window_append_is_the_reference_chain_bit_for_bit(cuda, dtype):
+    """Rotary embedding of the new keys + append, one launch, against the reference's chain of 16-bit elementwise ops
+    (utils/compute.py:35-43, restated in oracle/cache.py) evaluated by torch on the device: equal bits; contiguous
+    and strided inputs (a transposed projection output, an expanded cos / sin table), one and several new tokens,
+    with and without the embedding."""
+    from oracle import cache as oc
+    g = torch.Generator().manual_seed(400)
+    B, H, cap = 3, 4, 40
+    for n, pos, strided in ((1, 0, False), (1, 17, True), (5, 30, True), (8, 32, False)):
+        _say("append case", dtype, n, pos, strided)
+        if strided:     # [B, n, H, 128] storage seen as [B, H, n, 128], like a projection output after transpose(1, 2)
+            k = (torch.randn(B, n, H, 128, generator=g) * 3).to(dtype).to(cuda).transpose(1, 2)
+            v = torch.randn(B, n, H, 128, generator=g).to(dtype).to(cuda).transpose(1, 2)
+            cos1, sin1 = _rope_tables(1, 100 + pos, n, dtype)
+            cos, sin = cos1.to(cuda).expand(B, n, 128), sin1.to(cuda).expand(B, n, 128)
+        else:
+            k = (torch.randn(B, H, n, 128, generator=g) * 3).to(dtype).to(cuda)
+            v = torch.randn(B, H, n, 128, generator=g).to(dtype).to(cuda)
+            cos, sin = (t.to(cuda) for t in _rope_tables(B, 100 + pos, n, dtype))
+        for rotary in (True, False):
+            k_win = torch.full((B, H, cap, 128), 7.0, dtype=dtype, device=cuda)
+            v_win = torch.full((B, H, cap, 128), 7.0, dtype=dtype, device=cuda)
+            ops.window_append(k, v, cos if rotary else None, sin if rotary else None, k_win, v_win, pos)
+            want_k = oc.apply_rotary_pos_emb_single(k, cos, sin) if rotary else k
+            assert torch.equal(k_win[:, :, pos:pos + n].view(torch.int16), want_k.contiguous().view(torch.int16))
+            assert torch.equal(v_win[:, :, pos:pos + n], v)
+            rest = torch.ones(cap, dtype=torch.bool)
+            rest[pos:pos + n] = False
+            assert (k_win[:, :, rest] == 7.0).all() and (v_win[:, :, rest] == 7.0).all()     # nothing else written
+    with pytest.raises(Exception):
+        ops.window_append(k, v, None, None, k_win, v_win, cap - 2)                           # 8 rows do not fit
