@@ -208,7 +208,10 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *   variant           0 = default (asynchronous-copy matrix-core kernel; streams must be 16-byte
  *                     aligned, otherwise variant 2 runs); 1 = plain VALU kernel; 2 = matrix-core
  *                     kernel that gathers straight from global memory.  All three implement the
- *                     same contract; tests cross-check them.
+ *                     same contract; tests cross-check them.  The matrix-core kernels take the reference's
+ *                     widths (k_bits, v_bits in 2..4, any mix); variant 0 also takes the extension widths 5
+ *                     and 6 when K and V share one.  Any other extension width runs the plain kernel whatever
+ *                     `variant` says.
  */
 typedef struct pkv_attn_args {
     const uint8_t *k_stream;

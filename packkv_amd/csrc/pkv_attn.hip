@@ -486,6 +486,8 @@ static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
         case 3 * 8 + 4: return launch_dma<G, 3, 4>(p, s);
         case 4 * 8 + 2: return launch_dma<G, 4, 2>(p, s);
         case 4 * 8 + 3: return launch_dma<G, 4, 3>(p, s);
+        case 5 * 8 + 5: return launch_dma<G, 5, 5>(p, s);       // the extension widths, K and V alike
+        case 6 * 8 + 6: return launch_dma<G, 6, 6>(p, s);
         default: return launch_dma<G, 4, 4>(p, s);
     }
 }
@@ -603,9 +605,12 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     // The async-copy kernel spreads the tail window over its splits (each takes win_piece tokens after its
     // tiles and writes one more partial), so the window costs no launch and no idle tail; other paths
     // give the window a kernel of its own.
-    // the matrix-core kernels are built for the reference's widths; the extension widths 5..8 run the plain kernel
+    // the matrix-core kernels take the reference's widths and, in the asynchronous-copy kernel, the extension widths
+    // 5 and 6 when K and V share one; any other extension width runs the plain kernel
     const bool narrow = a->T_c == 0 || (a->k_bits <= 4 && a->v_bits <= 4);
-    const bool aligned16 = narrow && ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
+    const bool wide_fast = !narrow && a->k_bits == a->v_bits && a->k_bits <= 6 && a->variant == 0;
+    const bool aligned16 = (narrow || wide_fast) &&
+                           ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
     p.win_piece = 0;
     if (a->T_w > 0 && nsplit > 0 && a->variant == 0 && aligned16) {
         const int piece = (a->T_w + nsplit - 1) / nsplit;
@@ -626,7 +631,7 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
 
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    const int variant = narrow ? a->variant : 1;
+    const int variant = narrow || (wide_fast && aligned16) ? a->variant : 1;
     switch (G) {
         case 1: rc = launch_attn<1>(p, variant, aligned16, (uint16_t *)a->out, s); break;
         case 2: rc = launch_attn<2>(p, variant, aligned16, (uint16_t *)a->out, s); break;

@@ -103,14 +103,15 @@ template <int NB>
 __device__ __forceinline__ uint32_t lds_meta(const uint8_t *base, uint32_t off, int t) {
     if (NB == 4) return *reinterpret_cast<const uint16_t *>(base + off + 2 * t);
     if (NB == 2) return base[off + t];
-    const uint32_t a = off + ((uint32_t)(t * 12) >> 3);          // NB == 3: 12 bits at bit 12 t
+    // 4 NB bits at bit 4 NB t: byte (4 NB t) / 8, then 0 or 4 bits further (4 NB + 4 <= 32 for NB <= 7)
+    const uint32_t bit = (uint32_t)(t * 4 * NB), a = off + (bit >> 3);
     const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (a & ~3u));
     const uint32_t v = __builtin_amdgcn_alignbyte(q[1], q[0], a);
-    return (v >> ((t & 1) * 4)) & 0xFFFu;
+    return (v >> (bit & 7u)) & ((1u << (4 * NB)) - 1u);
 }
 
-template <int W>
-__device__ __forceinline__ void meta_pairs(uint32_t minsw, uint32_t lensw, UnitPairs &u) {
+template <int W, typename U>
+__device__ __forceinline__ void meta_pairs(uint32_t minsw, uint32_t lensw, U &u) {
     constexpr int LB = len_field_bits(W);
     u.len01 = __builtin_amdgcn_ubfe(lensw, 0, LB) | (__builtin_amdgcn_ubfe(lensw, LB, LB) << 16);
     u.len23 = __builtin_amdgcn_ubfe(lensw, 2 * LB, LB) | (__builtin_amdgcn_ubfe(lensw, 3 * LB, LB) << 16);
@@ -146,6 +147,51 @@ __device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[
     }
 }
 
+// Widths 5 and 6 (this build's extension of the format): a quarter of a pack no longer fits a 16-bit lane, so the
+// windows hold TWO tokens each.  e01[e] = tokens 2e, 2e+1 of packs 0 and 1 in the low / high 16 bits (token 2e on
+// top), e23 likewise; bits above 2*len in a half are other tokens' fields, every consumer masks.
+struct UnitWide {
+    uint32_t e01[8], e23[8];
+    uint32_t len01, len23;
+    uint32_t mins;
+};
+
+// The eight two-token windows of the four packs whose words start at byte pay0 + 2 * off2[i] of `base`.  A word is
+// up to 12 bytes long, so it is not assembled: each quarter (four tokens, 4 * len bits starting (3 - q) * 4 * len
+// bits into the word, i.e. at a byte or a nibble boundary) is fetched on its own as the 32 bits at its byte
+// address -- two aligned dwords and a byte funnel shift -- and moved down by the odd nibble.
+__device__ __forceinline__ void wide_windows(const uint8_t *base, uint32_t pay0, const uint32_t off2[4], UnitWide &u) {
+    const uint32_t len[4] = {u.len01 & 0xFFFFu, u.len01 >> 16, u.len23 & 0xFFFFu, u.len23 >> 16};
+    uint32_t hi[4][4], lo[4][4];       // [pack][quarter]: tokens 4q, 4q+1 and 4q+2, 4q+3
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t a = pay0 + 2u * off2[i], L = len[i], nib = (L & 1u) * 4u;
+        const uint32_t at[4] = {a + ((3u * L) >> 1), a + L, a + (L >> 1), a};      // byte address of quarter q
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t *dq = reinterpret_cast<const uint32_t *>(base + (at[q] & ~3u));
+            uint32_t v = __builtin_amdgcn_alignbyte(dq[1], dq[0], at[q]);
+            if (q == 0 || q == 2) v >>= nib;
+            lo[i][q] = v;
+            hi[i][q] = v >> (2u * L);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        u.e01[2 * q] = __builtin_amdgcn_perm(hi[1][q], hi[0][q], 0x05040100u);
+        u.e01[2 * q + 1] = __builtin_amdgcn_perm(lo[1][q], lo[0][q], 0x05040100u);
+        u.e23[2 * q] = __builtin_amdgcn_perm(hi[3][q], hi[2][q], 0x05040100u);
+        u.e23[2 * q + 1] = __builtin_amdgcn_perm(lo[3][q], lo[2][q], 0x05040100u);
+    }
+}
+
+// Wavefronts per SIMD the register allocation aims for: four workgroups per CU for the reference's widths (three for
+// groups of 8 query heads); the two-token windows of widths 5 and 6 need about 210 VGPRs, two workgroups per CU
+// (at three, 168 VGPRs, the compiler spills 47 of them and the kernel is 2.4 times slower).
+#define PKV_DMA_WAVES(KW, G) ((KW) > 4 ? ((G) <= 4 ? 2 : 1) : ((G) <= 4 ? 4 : 3))
+template <bool WIDE> struct UnitOf { typedef UnitPairs type; };
+template <> struct UnitOf<true> { typedef UnitWide type; };
+
 template <int G, int KW, int VW>
 constexpr int dma_lds_bytes() {          // static LDS of attn_dma_kernel: two slots, weights, round sums, state
     constexpr int GP = (G + 3) / 4 * 4;
@@ -153,8 +199,13 @@ constexpr int dma_lds_bytes() {          // static LDS of attn_dma_kernel: two s
 }
 
 template <int G, int KW, int VW, bool BF>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 3, 4))) attn_dma_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DMA_WAVES(KW, G), 4))) attn_dma_kernel(const AttnParams p) {
     using Geo = DmaGeom<KW, VW>;
+    constexpr bool WIDE = KW > 4;                // widths 5, 6: two-token windows
+    static_assert((KW > 4) == (VW > 4) && KW <= 6 && VW <= 6, "K and V are both reference widths or both 5..6");
+    constexpr int TPW = WIDE ? 2 : 4;            // tokens per window
+    constexpr int NWIN = 16 / TPW;
+    typedef typename UnitOf<WIDE>::type Unit;
     constexpr int ROWS = 3 * G;
     constexpr int NSETS = (ROWS + 15) / 16;
     constexpr int NG4 = (G + 3) / 4;
@@ -286,7 +337,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 
     // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
     const int ku = hw & 3;
-    auto parse = [&](int slot, const TileInfo &ti, UnitPairs &kr, UnitPairs &vr) {
+    auto parse = [&](int slot, const TileInfo &ti, Unit &kr, Unit &vr) {
         const uint8_t *kb = ring + slot * Geo::kSlot + kj * Geo::kRegion;
         const uint8_t *vb = ring + slot * Geo::kSlot + (2 + kj) * Geo::kRegion;
         const uint32_t kph = ti.k_off & 15u, vph = ti.v_off & 15u;
@@ -309,10 +360,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
         pack_offsets8(__builtin_amdgcn_perm(kr.len23, kr.len01, 0x06040200u), koff);
         pack_offsets8(__builtin_amdgcn_perm(vr.len23, vr.len01, 0x06040200u), voff);
         const uint32_t kpay0 = k_unit + K_META, vpay0 = v_unit + V_META;
+        if constexpr (WIDE) {
+            wide_windows(kb, kpay0, koff, kr);
+            wide_windows(vb, vpay0, voff, vr);
+        } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
-            vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
+            for (int i = 0; i < 4; i++) {
+                kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
+                vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
+            }
         }
     };
 
@@ -334,20 +390,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
     for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
 
     // ---- stage 1: K round hw -> int8 tile rows [hw*16, hw*16+16), then scores on the matrix cores ----
-    auto k_stage = [&](const UnitPairs &kr, uint8_t *kt) {
+    auto k_stage = [&](const Unit &kr, uint8_t *kt) {
         {
-            uint32_t w01[4], w23[4];
-            pair_windows(kr, w01, w23);
+            uint32_t w01[NWIN], w23[NWIN];
+            if constexpr (WIDE) {
+#pragma unroll
+                for (int e = 0; e < NWIN; e++) { w01[e] = kr.e01[e]; w23[e] = kr.e23[e]; }
+            } else {
+                pair_windows(kr, w01, w23);
+            }
             const uint32_t len01 = kr.len01, len23 = kr.len23;
             const uint32_t mq = __builtin_amdgcn_perm(pk_mask16(len23), pk_mask16(len01), 0x06040200u);   // byte masks
             uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
+            for (int q = 0; q < NWIN; q++) {
 #pragma unroll
-                for (int pp = 0; pp < 4; pp++) {
-                    const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
-                    const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
-                    dst[(q * 4 + pp) * kKtDw] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + kr.mins;
+                for (int pp = 0; pp < TPW; pp++) {
+                    const uint32_t x01 = pp == TPW - 1 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(TPW - 1 - pp));
+                    const uint32_t x23 = pp == TPW - 1 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(TPW - 1 - pp));
+                    dst[(q * TPW + pp) * kKtDw] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + kr.mins;
                 }
             }
         }
@@ -442,10 +503,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
         for (int pp = 0; pp < 4; pp++) a_w[pp][i4] = (half4v){0, 0, 0, 0};
     }
     const bool a_loader = (lane & 31) < 4;
-    auto v_stage = [&](const UnitPairs &vr) {
+    auto v_stage = [&](const Unit &vr) {
         const int seg = hw & 1;
-        uint32_t w01[4], w23[4];
-        pair_windows(vr, w01, w23);
+        uint32_t w01[NWIN], w23[NWIN];
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int e = 0; e < NWIN; e++) { w01[e] = vr.e01[e]; w23[e] = vr.e23[e]; }
+        } else {
+            pair_windows(vr, w01, w23);
+        }
         const uint32_t len01 = vr.len01, len23 = vr.len23;
         const uint32_t m01 = pk_mask16(len01), m23 = pk_mask16(len23);
         // rescale the accumulators only when some head's running maximum moved (alpha <= 1, so the
@@ -489,8 +555,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
             }
 #pragma unroll
             for (int pp = 0; pp < 4; pp++) {
-                const uint32_t x01 = pp == 3 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(3 - pp));
-                const uint32_t x23 = pp == 3 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(3 - pp));
+                constexpr int SH_MAX = TPW - 1;
+                const int wi = (4 * q + pp) / TPW, ps = (4 * q + pp) % TPW;      // window and position of token 4q + pp
+                const uint32_t x01 = ps == SH_MAX ? w01[wi] : pk_shr16(w01[wi], len01 * (uint32_t)(SH_MAX - ps));
+                const uint32_t x23 = ps == SH_MAX ? w23[wi] : pk_shr16(w23[wi], len23 * (uint32_t)(SH_MAX - ps));
                 const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
 #pragma unroll
                 for (int i4 = 0; i4 < NG4; i4++)
@@ -501,7 +569,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
 
     // ---- pipeline ----
     TileInfo i0 = load_info(0), i1 = load_info(1), i2 = load_info(2);
-    UnitPairs kcur, vcur;
+    Unit kcur, vcur;
     dma_issue(0, 0, i0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     PKV_LDS_BARRIER();
@@ -519,7 +587,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(G <= 4
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
         PKV_LDS_BARRIER();                                    // publishes the scores and tile s+1
-        UnitPairs knext, vnext;
+        Unit knext, vnext;
         __builtin_amdgcn_s_setprio(PKV_PRIO_S);
         parse(slot ^ 1, i1, knext, vnext);
         softmax_stage(slot, kt);

@@ -214,20 +214,32 @@ def test_attn_decode_replays_in_a_hip_graph(cuda):
             assert torch.equal(o, w)
 
 
-def test_attn_decode_five_bit_codes(cuda):
-    """rel 0.05 gives 22 code levels: 5-bit codes, outside the reference's format and inside this build's extension
-    (three-kernel encode, plain attention kernel).  Same contract against decompress-then-attend."""
-    B, Hq, Hkv, T = 2, 16, 4, 512
-    k, v = synth.make_kv(B, Hkv, T, seed=180)
-    q = synth.make_q(B, Hq, seed=181)
-    want = _reference(q, k, v, 0.05, 0.05)
-    exact = _exact(q, k, v, 0.05, 0.05)
-    ke = ops.k_quant_encode(k.to(cuda), 0.05)
-    ve = ops.v_quant_encode(v.to(cuda), 0.05)
-    assert ke["bits"] == 5 and ve["bits"] == 5
-    ck, _, _ = oq.quant_ints(k, 64, 0.05)
+@pytest.mark.parametrize("rel,bits", [(0.05, 5), (0.03, 6)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attn_decode_wide_codes(cuda, rel, bits, dtype):
+    """rel 0.05 gives 22 code levels, rel 0.03 gives 35: 5- and 6-bit codes, outside the reference's format and
+    inside this build's extension (three-kernel encode).  The asynchronous-copy kernel takes them with two-token
+    windows (variant 0); the plain kernel (variant 1) is the cross-check.  Same contract against
+    decompress-then-attend, with a tail window and a context that is not a multiple of the split size."""
+    B, Hq, Hkv, T, Tw = 2, 16, 4, 1152, 70
+    k, v = synth.make_kv(B, Hkv, T + Tw, seed=180, dtype=dtype)
+    q = synth.make_q(B, Hq, seed=181, dtype=dtype)
+    k_c, v_c, k_w, v_w = k[:, :, :T].contiguous(), v[:, :, :T].contiguous(), k[:, :, T:].contiguous(), v[:, :, T:].contiguous()
+    want = _reference(q, k_c, v_c, rel, rel, k_w, v_w)
+    exact = _exact(q, k_c, v_c, rel, rel, k_w, v_w)
+    kc, vc = k_c.to(cuda), v_c.to(cuda)
+    ke = ops.k_quant_encode(kc, rel)
+    ve = ops.v_quant_encode(vc, rel)
+    assert ke["bits"] == bits and ve["bits"] == bits
+    ck, _, _ = oq.quant_ints(k_c, 64, rel)
     codes = torch.empty(T, B * Hkv * 128, dtype=torch.uint8, device=cuda)
-    ops.k_decode(ke["stream"], ke["info"], codes, bits=5)
+    ops.k_decode(ke["stream"], ke["info"], codes, bits=bits)
     assert torch.equal(codes.cpu(), oq.code_matrix(ck))
-    got = ops.attn_decode(q.to(cuda), ke, ve)
-    _check(got, want, torch.float16, exact, abs_tol=STRESS_ABS_TOL[torch.float16], variant=1)
+    kw, vw = k_w.to(cuda), v_w.to(cuda)
+    outs = []
+    for variant in (0, 1):
+        _say("wide attention case", dtype, "bits", bits, "variant", variant)
+        got = ops.attn_decode(q.to(cuda), ke, ve, kw, vw, variant=variant)
+        _check(got, want, dtype, exact, abs_tol=STRESS_ABS_TOL[dtype], variant=variant)
+        outs.append(got.float())
+    _say("  fast vs plain kernel: max diff", (outs[0] - outs[1]).abs().max().item())
