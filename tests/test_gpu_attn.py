@@ -243,3 +243,19 @@ def test_attn_decode_wide_codes(cuda, rel, bits, dtype):
         _check(got, want, dtype, exact, abs_tol=STRESS_ABS_TOL[dtype], variant=variant)
         outs.append(got.float())
     _say("  fast vs plain kernel: max diff", (outs[0] - outs[1]).abs().max().item())
+
+
+@pytest.mark.parametrize("hq", [4, 8, 32])
+def test_attn_decode_wide_codes_group_sizes(cuda, hq):
+    """The 5-bit path for groups of 1, 2 and 8 query heads per KV head (the case above has 4), no tail window."""
+    B, Hkv, T = 1, 4, 640
+    k, v = synth.make_kv(B, Hkv, T, seed=185)
+    q = synth.make_q(B, hq, seed=186)
+    want = _reference(q, k, v, 0.05, 0.05)
+    exact = _exact(q, k, v, 0.05, 0.05)
+    ke = ops.k_quant_encode(k.to(cuda), 0.05)
+    ve = ops.v_quant_encode(v.to(cuda), 0.05)
+    assert ke["bits"] == 5 and ve["bits"] == 5
+    _say("wide attention case: group of", hq // Hkv)
+    got = ops.attn_decode(q.to(cuda), ke, ve)
+    _check(got, want, torch.float16, exact, abs_tol=STRESS_ABS_TOL[torch.float16])
