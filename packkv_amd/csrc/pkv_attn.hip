@@ -21,6 +21,7 @@ namespace pkv {
 
 constexpr int kTile = 128;              // tokens per super-tile
 constexpr int kPartStride = 2 + kHeadDim;  // floats per partial: m, l, acc[128]
+typedef float float2v __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float a_ld16(const uint16_t *p, size_t i, int dtype) {
     const uint32_t u = p[i];
@@ -405,7 +406,8 @@ __global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
 __global__ void __launch_bounds__(256) attn_merge_kernel(const float *__restrict__ part, uint16_t *__restrict__ out,
                                                          int Hq, int nparts, int dtype) {
     extern __shared__ float w_s[];                   // weight of every partial
-    __shared__ float red[8], half_num[kHeadDim];
+    __shared__ float red[8];
+    __shared__ __attribute__((aligned(8))) float part_num[3 * kHeadDim];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t hq = (size_t)blockIdx.y * Hq + blockIdx.x;
     const float *base = part + hq * nparts * kPartStride;
@@ -425,21 +427,39 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float *__restrict
     if (lane == 0) red[4 + wave] = den;
     __syncthreads();
     den = (red[4] + red[5]) + (red[6] + red[7]);
-    const int half = tid >> 7, ch = tid & (kHeadDim - 1);
-    const float *col = base + 2 + ch;
-    float num = 0.f;
-    int s = half;
-    for (; s + 6 < nparts; s += 8) {
-        float v[4];
+    // weighted sum: wavefront = every fourth partial, lane = two adjacent channels (rows are 8-byte aligned), eight
+    // loads in flight per lane -- a long list of partials (small batches spread one head over many splits) is a
+    // chain of dependent round trips otherwise
+    const float2v *col = reinterpret_cast<const float2v *>(base + 2) + lane;
+    float2v num = {0.f, 0.f};
+    int s = wave;
+    for (; s + 28 < nparts; s += 32) {
+        float2v v[8];
 #pragma unroll
-        for (int u = 0; u < 4; u++) v[u] = col[(size_t)(s + 2 * u) * kPartStride];
+        for (int u = 0; u < 8; u++) v[u] = col[(size_t)(s + 4 * u) * (kPartStride / 2)];
 #pragma unroll
-        for (int u = 0; u < 4; u++) num += w_s[s + 2 * u] * v[u];
+        for (int u = 0; u < 8; u++) num += w_s[s + 4 * u] * v[u];
     }
-    for (; s < nparts; s += 2) num += w_s[s] * col[(size_t)s * kPartStride];
-    if (half) half_num[ch] = num;
+    if (s < nparts) {                                  // the last, partial batch: still one round trip
+        float2v v[8];
+        float w[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int idx = min(s + 4 * u, nparts - 1);
+            v[u] = col[(size_t)idx * (kPartStride / 2)];
+            w[u] = s + 4 * u < nparts ? w_s[idx] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) num += w[u] * v[u];
+    }
+    if (wave) reinterpret_cast<float2v *>(part_num + (wave - 1) * kHeadDim)[lane] = num;
     __syncthreads();
-    if (!half) out[hq * kHeadDim + ch] = a_st16((num + half_num[ch]) / den, dtype);
+    if (wave == 0) {
+#pragma unroll
+        for (int w = 0; w < 3; w++) num += reinterpret_cast<const float2v *>(part_num + w * kHeadDim)[lane];
+        const uint32_t lo = a_st16(num[0] / den, dtype), hi = a_st16(num[1] / den, dtype);
+        reinterpret_cast<uint32_t *>(out + hq * kHeadDim)[lane] = lo | (hi << 16);
+    }
 }
 
 }  // namespace pkv
