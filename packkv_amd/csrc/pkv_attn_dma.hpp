@@ -27,16 +27,18 @@
 
 namespace pkv {
 
-// Wave priorities of the pipeline stages (s_setprio): the further a wavefront is in its tile, the sooner it issues,
-// so the four resident workgroups of a CU drift apart instead of competing stage for stage -- wavefronts reach
-// their barriers earlier and the vector ALUs idle less.  Measured on the 16 x 8 x 32768-token workload: 142.5 us
-// with equal priorities, 129.5 us with these (a sweep over the 2-bit range; copy issue lowest was best).
-#ifndef PKV_PRIO_K
-#define PKV_PRIO_K 1     /* K stage */
-#define PKV_PRIO_S 2     /* parse of the next tile + softmax */
-#define PKV_PRIO_D 0     /* issue of the asynchronous copies, and every barrier wait */
-#define PKV_PRIO_V 3     /* V stage */
-#endif
+// Wave priorities of the pipeline stages (s_setprio).  With four workgroups per CU (groups of up to 4 query heads,
+// the reference's widths) the further a wavefront is in its tile the sooner it issues, so the resident workgroups
+// drift apart instead of competing stage for stage -- wavefronts reach their barriers earlier and the vector ALUs
+// idle less: 142.5 us with equal priorities, 129.5 us with (K 1, softmax 2, copy issue 0, V 3) on the 16 x 8 x
+// 32768-token workload (a sweep over the 2-bit range; copy issue lowest was best).  The setting does not carry over
+// to fewer resident workgroups: with three (groups of 8) equal priorities are best (197 us against 218), with two
+// (widths 5 and 6) the K stage first (211 us against 218).
+template <int G, bool WIDE> struct StagePrio {                       // 4 workgroups per CU
+    static constexpr int K = 1, S = 2, D = 0, V = 3;                 // K stage, parse + softmax, copy issue and waits, V stage
+};
+template <int G> struct StagePrio<G, true> { static constexpr int K = 2, S = 1, D = 0, V = 0; };
+template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 0, V = 0; };
 #define PKV_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -206,6 +208,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     constexpr int TPW = WIDE ? 2 : 4;            // tokens per window
     constexpr int NWIN = 16 / TPW;
     typedef typename UnitOf<WIDE>::type Unit;
+    typedef StagePrio<G, WIDE> Prio;
     constexpr int ROWS = 3 * G;
     constexpr int NSETS = (ROWS + 15) / 16;
     constexpr int NG4 = (G + 3) / 4;
@@ -582,20 +585,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         const int slot = s & 1;
         uint8_t *kt = ring + slot * Geo::kSlot;
         const TileInfo i3 = load_info(s + 3);
-        __builtin_amdgcn_s_setprio(PKV_PRIO_K);
+        __builtin_amdgcn_s_setprio(Prio::K);
         k_stage(kcur, kt);
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
         PKV_LDS_BARRIER();                                    // publishes the scores and tile s+1
         Unit knext, vnext;
-        __builtin_amdgcn_s_setprio(PKV_PRIO_S);
+        __builtin_amdgcn_s_setprio(Prio::S);
         parse(slot ^ 1, i1, knext, vnext);
         softmax_stage(slot, kt);
         __builtin_amdgcn_s_setprio(0);
         PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile s+1 is parsed
-        __builtin_amdgcn_s_setprio(PKV_PRIO_D);
+        __builtin_amdgcn_s_setprio(Prio::D);
         dma_issue(slot, s + 2, i2);
-        __builtin_amdgcn_s_setprio(PKV_PRIO_V);
+        __builtin_amdgcn_s_setprio(Prio::V);
         v_stage(vcur);
         __builtin_amdgcn_s_setprio(0);
         kcur = knext;
