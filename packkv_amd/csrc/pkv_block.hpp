@@ -202,7 +202,7 @@ __device__ __forceinline__ void lds_put_meta(uint8_t *arr, int t, int nbits, uin
         reinterpret_cast<uint16_t *>(arr)[t] = (uint16_t)w;
     } else if (nbits == 2) {
         arr[t] = (uint8_t)w;
-    } else {  // 12 bits per lane: an even/odd lane pair shares three bytes
+    } else if (nbits == 3) {  // 12 bits per lane: an even/odd lane pair shares three bytes
         const uint32_t hi = __shfl_down(w, 1, 32);
         if ((t & 1) == 0) {
             const uint32_t v = w | (hi << 12);
@@ -210,6 +210,19 @@ __device__ __forceinline__ void lds_put_meta(uint8_t *arr, int t, int nbits, uin
             p[0] = (uint8_t)v;
             p[1] = (uint8_t)(v >> 8);
             p[2] = (uint8_t)(v >> 16);
+        }
+    } else if (nbits == 6) {  // 24 bits per lane: three bytes of its own
+        uint8_t *p = arr + t * 3;
+        p[0] = (uint8_t)w;
+        p[1] = (uint8_t)(w >> 8);
+        p[2] = (uint8_t)(w >> 16);
+    } else {                  // nbits == 5: 20 bits per lane, an even/odd lane pair shares five bytes
+        const uint32_t hi = __shfl_down(w, 1, 32);
+        if ((t & 1) == 0) {
+            const uint64_t v = (uint64_t)w | ((uint64_t)hi << 20);
+            uint8_t *p = arr + (t >> 1) * 5;
+#pragma unroll
+            for (int i = 0; i < 5; i++) p[i] = (uint8_t)(v >> (8 * i));
         }
     }
 }

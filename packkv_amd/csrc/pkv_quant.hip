@@ -365,6 +365,105 @@ __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par
     u.len[0] = len01 & 0xFFFFu; u.len[1] = len01 >> 16; u.len[2] = len23 & 0xFFFFu; u.len[3] = len23 >> 16;
 }
 
+// ---- widths 5 and 6 (extension of the format) in the round-major encoders ------------------------------------
+// A pack word grows to 16 * len <= 96 bits.  It is kept as two halves of 8 * len bits -- `hi` tokens 0..7, `lo`
+// tokens 8..15 -- and since 8 * len bits are len whole bytes, the word's 2 * len bytes in the stream are simply the
+// bytes of `lo` followed by the bytes of `hi`.  The halves are assembled from windows of TWO tokens (2 * len <= 12
+// bits fit the packed 16-bit arithmetic the quarter windows of the reference's widths use).
+struct UnitPacksW {
+    uint64_t lo[4], hi[4];
+    uint32_t len[4];
+    uint32_t mn[4];
+    uint32_t off[4];
+    uint32_t payload;
+};
+
+// bit_length of both 16-bit halves, clamped to 6
+__device__ __forceinline__ uint32_t pk_bitlen6(uint32_t d) {
+    const u16x2 v = as_u16x2(d), one = {1, 1};
+    u16x2 l = __builtin_elementwise_min(v, one);
+#pragma unroll
+    for (int k = 1; k < 6; k++) l += __builtin_elementwise_min((u16x2)(v >> (uint16_t)k), one);
+    return pk_u16(l);
+}
+
+__device__ __forceinline__ uint64_t join4(uint32_t e0, uint32_t e1, uint32_t e2, uint32_t e3, uint32_t l2) {
+    return ((((((uint64_t)e0 << l2) | e1) << l2) | e2) << l2) | e3;      // l2 = 2 * len
+}
+
+__device__ __forceinline__ void build_pair_wide(const uint32_t c[16], uint32_t &mn2, uint32_t &len2, uint32_t &mx2,
+                                                uint64_t &lo_a, uint64_t &hi_a, uint64_t &lo_b, uint64_t &hi_b) {
+    u16x2 mn = as_u16x2(c[0]), mx = as_u16x2(c[0]);
+#pragma unroll
+    for (int k = 1; k < 16; k++) {
+        mn = __builtin_elementwise_min(mn, as_u16x2(c[k]));
+        mx = __builtin_elementwise_max(mx, as_u16x2(c[k]));
+    }
+    mn2 = pk_u16(mn);
+    mx2 = pk_u16(mx);
+    len2 = pk_bitlen6(pk_u16((u16x2)(mx - mn)));
+    const u16x2 one = {1, 1};
+    const u16x2 p = one << as_u16x2(len2);                       // 2^len per half
+    const u16x2 mnrep = mn * (p + one);
+    uint32_t ew[8];                                              // tokens 2j, 2j+1: (c - min) p + (c' - min) < 2^12
+#pragma unroll
+    for (int j = 0; j < 8; j++) ew[j] = pk_u16((u16x2)(as_u16x2(c[2 * j]) * p + as_u16x2(c[2 * j + 1]) - mnrep));
+    const uint32_t l0 = 2u * (len2 & 0xFFFFu), l1 = 2u * (len2 >> 16);
+    hi_a = join4(ew[0] & 0xFFFFu, ew[1] & 0xFFFFu, ew[2] & 0xFFFFu, ew[3] & 0xFFFFu, l0);
+    lo_a = join4(ew[4] & 0xFFFFu, ew[5] & 0xFFFFu, ew[6] & 0xFFFFu, ew[7] & 0xFFFFu, l0);
+    hi_b = join4(ew[0] >> 16, ew[1] >> 16, ew[2] >> 16, ew[3] >> 16, l1);
+    lo_b = join4(ew[4] >> 16, ew[5] >> 16, ew[6] >> 16, ew[7] >> 16, l1);
+}
+
+template <int DT>
+__device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par, UnitPacksW &u, uint32_t &cmax) {
+    uint32_t c01[16], c23[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+    uint32_t mn01, mn23, len01, len23, mx01, mx23;
+    build_pair_wide(c01, mn01, len01, mx01, u.lo[0], u.hi[0], u.lo[1], u.hi[1]);
+    build_pair_wide(c23, mn23, len23, mx23, u.lo[2], u.hi[2], u.lo[3], u.hi[3]);
+    const u16x2 m = __builtin_elementwise_max(as_u16x2(mx01), as_u16x2(mx23));
+    cmax = max((uint32_t)m[0], (uint32_t)m[1]);
+    u.mn[0] = mn01 & 0xFFFFu; u.mn[1] = mn01 >> 16; u.mn[2] = mn23 & 0xFFFFu; u.mn[3] = mn23 >> 16;
+    u.len[0] = len01 & 0xFFFFu; u.len[1] = len01 >> 16; u.len[2] = len23 & 0xFFFFu; u.len[3] = len23 >> 16;
+}
+
+template <bool WIDE> struct PacksOf { typedef UnitPacks type; };
+template <> struct PacksOf<true> { typedef UnitPacksW type; };
+
+// the 2 * len bytes of pack k at dst (2-byte aligned)
+__device__ __forceinline__ void put_pack(uint16_t *dst, const UnitPacks &u, int k) {
+    uint64_t wd = u.word[k];
+    for (uint32_t q = 0; q < u.len[k]; q++) {
+        dst[q] = (uint16_t)wd;
+        wd >>= 16;
+    }
+}
+__device__ __forceinline__ void put_pack(uint16_t *dst, const UnitPacksW &u, int k) {
+    unsigned __int128 wd = ((unsigned __int128)u.hi[k] << (8u * u.len[k])) | u.lo[k];
+    for (uint32_t q = 0; q < u.len[k]; q++) {
+        dst[q] = (uint16_t)wd;
+        wd >>= 16;
+    }
+}
+
+// Emit one analysed unit at blk[unit_off] (the K layout: lane t's packs sit where they were computed).
+template <class U>
+__device__ __forceinline__ void unit_emit_any(uint8_t *blk, uint32_t unit_off, int t, const UnitGeom g, const U &u) {
+    uint32_t minsw = 0, lensw = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        minsw |= u.mn[i] << (i * g.W);
+        lensw |= u.len[i] << (i * g.LB);
+    }
+    lds_put_meta(blk + unit_off, t, g.W, minsw);
+    lds_put_meta(blk + unit_off + g.mins_bytes, t, g.LB, lensw);
+    uint8_t *pay = blk + unit_off + g.mins_bytes + g.lens_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) put_pack(reinterpret_cast<uint16_t *>(pay + u.off[i]), u, i);
+}
+
 // V blocks: a wavefront's 64 cells (round 4 sg + i, channels 4 g .. 4 g + 3; lane = 16 i + g) cover
 // one segment sg of the block; V units want lane c = channel c holding the packs of rounds
 // 4 sg .. 4 sg + 3.  The packs change lanes inside the wavefront through a 1 KiB LDS area, one
@@ -608,7 +707,7 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
 // workgroup), then at once re-read them as cells -- the lines are still in L2 -- quantize, and emit
 // unit `round` of every block behind the units already there.  x therefore crosses HBM once.
 // Blocks sit in worst-case slots in LDS and are compacted by the final copy.
-template <int DT>
+template <int DT, bool WIDE>
 __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
@@ -664,7 +763,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
-        UnitPacks u;
+        typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_packs<DT>(xr, s_par, u, cmax);
         __syncthreads();                                  // s_par is rewritten by the next round
@@ -674,7 +773,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
             cmax_all = max(cmax_all, cmax);
             const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
             if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
-            unit_emit(blk, my_off, t, g, u);
+            unit_emit_any(blk, my_off, t, g, u);
             my_off += usz;
         }
     }
@@ -760,6 +859,20 @@ __device__ __forceinline__ void copy_out32(uint8_t *dst, const uint8_t *src, uin
 // OR the FB-bit fields f[0..3] of four adjacent lanes 4m..4m+3, slot i, into a unit's LSB-first metadata array
 // (field of lane c, slot i at bit (4c + i) * FB).  The 16 * FB bits of the four lanes start at byte 2 * FB * m.
 __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, const uint32_t f[4]) {
+    if (FB > 4) {                                 // widths 5, 6: 80 / 96 bits of four lanes, plus up to 16 bits of phase
+        unsigned __int128 v = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) v |= (unsigned __int128)f[k] << (4 * FB * k + FB * i);
+        const uint32_t byte = 2u * (uint32_t)FB * (uint32_t)m;
+        uint32_t *w = reinterpret_cast<uint32_t *>(arr + (byte & ~3u));
+        v <<= 8u * (byte & 3u);
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t piece = (uint32_t)(v >> (32 * d));
+            if (piece) atomicOr(w + d, piece);
+        }
+        return;
+    }
     uint64_t v = 0;
 #pragma unroll
     for (int k = 0; k < 4; k++) v |= (uint64_t)f[k] << (4 * FB * k + FB * i);
@@ -778,7 +891,7 @@ __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, con
 // unit (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight
 // threads of a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed
 // in with LDS atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.
-template <int DT>
+template <int DT, bool WIDE>
 __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
@@ -840,7 +953,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
-        UnitPacks u;
+        typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_packs<DT>(xr, s_par + 16 * rp, u, cmax);
         // bytes of the thread's four packs, their offsets inside the (unit, slot) and the slot's total
@@ -865,12 +978,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
             uint32_t o = meta + run_off + (rp ? tot_even : 0u) + (inc - pb);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                uint16_t *dst = reinterpret_cast<uint16_t *>(unit + o);
-                uint64_t wd = u.word[k];
-                for (uint32_t q = 0; q < u.len[k]; q++) {
-                    dst[q] = (uint16_t)wd;
-                    wd >>= 16;
-                }
+                put_pack(reinterpret_cast<uint16_t *>(unit + o), u, k);
                 o += 2u * u.len[k];
             }
         }
@@ -944,9 +1052,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
-    PKV_REQUIRE(bits >= 2 && bits <= 4, PKV_ERR_UNSUPPORTED,
-                "not supported: bits_len %d (the fused encoders take 2..4; wider codes go through pkv_quant_params, "
-                "pkv_quantize and pkv_{k,v}_encode)", bits);
+    PKV_REQUIRE(bits >= 2 && (bits <= 4 || (bits <= 6 && H <= kSubBlocks)), PKV_ERR_UNSUPPORTED,
+                "not supported: bits_len %d with %d heads (the fused encoders take 2..4, and 5..6 for up to 8 heads; "
+                "other widths go through pkv_quant_params, pkv_quantize and pkv_{k,v}_encode)", bits, H);
     PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
@@ -972,7 +1080,10 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
             const uint32_t lds = 64u * unit_slot + 64u;
             const uint32_t ngroups = (uint32_t)(T / ctx_blk) * (uint32_t)B;
-            auto kern = dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16> : v_quant_encode_rounds_kernel<PKV_BF16>;
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true>)
+                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false>);
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
@@ -980,14 +1091,12 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
             const uint32_t lds = (uint32_t)H * slot + 32u;
-            if (dtype == PKV_F16)
-                k_quant_encode_rounds_kernel<PKV_F16><<<nsub, 256, lds, s>>>(
-                    (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                    bits, nsub, slot, base, par_stride);
-            else
-                k_quant_encode_rounds_kernel<PKV_BF16><<<nsub, 256, lds, s>>>(
-                    (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                    bits, nsub, slot, base, par_stride);
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true>)
+                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false>);
+            kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                        capacity, info, st, bits, nsub, slot, base, par_stride);
         } else if (dtype == PKV_F16)
             quant_encode_group_kernel<IS_K, PKV_F16><<<nsub, 256, gbytes, s>>>(
                 (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,

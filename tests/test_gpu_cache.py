@@ -164,3 +164,35 @@ def test_window_append_is_the_reference_chain_bit_for_bit(cuda, dtype):
             assert (k_win[:, :, rest] == 7.0).all() and (v_win[:, :, rest] == 7.0).all()     # nothing else written
     with pytest.raises(Exception):
         ops.window_append(k, v, None, None, k_win, v_win, cap - 2)                           # 8 rows do not fit
+
+
+def test_cache_with_five_bit_codes(cuda):
+    """rel 0.05 (5-bit codes, the format extension) through the growing cache: the fused encoders append, the
+    asynchronous-copy attention kernel reads; dense view bit-exact with the restated reference cache, the decode
+    step within the attention tolerance, across one cut."""
+    B, Hq, H, T0, steps = 2, 8, 4, 300, 40
+    dtype = torch.float16
+    k, v = synth.make_kv(B, H, T0 + steps, seed=96, dtype=dtype)
+    want = oc.SimulatedCache(1, 64, 192, 0.05, 0.05)
+    got = PackKVCompressedCache(B, H, 128, 1, PackKVCacheConfig(64, 192, 0.05, 0.05), max_tokens=1024, dtype=dtype,
+                                device=cuda)
+    assert got.config.k_bits == 5 and got.config.v_bits == 5
+    tok = 0
+    for step in range(-1, steps):
+        n = T0 if step < 0 else 1
+        ks, vs = k[:, :, tok:tok + n], v[:, :, tok:tok + n]
+        wk, wv = want.update(ks, vs, 0, None, None)
+        got.update(ks.to(cuda), vs.to(cuda), 0, None)
+        tok += n
+        if step in (-1, 0, 19, 20, 39):
+            _say("5-bit cache case step", step, "tokens", tok, "compressed", got.layers[0].k.tokens)
+            gk, gv = got.materialize(0)
+            assert torch.equal(gk.cpu().view(torch.int16), wk.view(torch.int16))
+            assert torch.equal(gv.cpu().view(torch.int16), wv.view(torch.int16))
+            q = synth.make_q(B, Hq, seed=500 + step, dtype=dtype)
+            ref = oq.attention_f32(q.unsqueeze(2), wk, wv).squeeze(2).double().numpy()
+            out = got.attend(q.to(cuda), 0).double().cpu().numpy()
+            err = np.abs(out - ref)
+            _say("   max|err| = %.3e" % err.max())
+            assert (err <= SHORT_ABS_TOL[dtype] + REL_TOL * np.abs(ref)).all()
+    assert got.layers[0].k.tokens == 128 and got.layers[0].pend == 64      # 128 at the prefill, one more cut waiting for its partner
