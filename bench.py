@@ -386,6 +386,31 @@ def main():
                                "read_gbs": src.numel() / (rd_ms * 1e-3) / 1e9, "bytes": src.numel()}
         del dst
 
+    if not args.no_extras and default_workload:
+        # configs[1] names three error bounds; the line above is the middle one.  The other two on the same tensors:
+        # fused encode, unpack and the decode step (5-bit codes at 0.05 are this build's extension of the format)
+        other = {}
+        for rel2 in (0.05, 0.2):
+            b2 = ops.bits_for_rel(rel2)
+            ke2, ve2 = ops.k_quant_encode(kc, rel2, b2), ops.v_quant_encode(vc, rel2, b2)
+            out2 = torch.empty_like(q)
+            f2 = lambda: ops.attn_decode(q, ke2, ve2, out=out2)
+            for _ in range(100):
+                f2()
+            a_ms = event_time_ms(torch, f2, 300)
+            k2 = event_time_ms(torch, lambda: ops.k_quant_encode(kc, rel2, b2, ke2["stream"], ke2["info"], want_size=False), 5)
+            v2 = event_time_ms(torch, lambda: ops.v_quant_encode(vc, rel2, b2, ve2["stream"], ve2["info"], want_size=False), 5)
+            codes2 = torch.empty(Tc, hidden, dtype=torch.uint8, device=dev)
+            uk2 = event_time_ms(torch, lambda: ops.k_decode(ke2["stream"], ke2["info"], codes2, 64, 128, b2), 5)
+            uv2 = event_time_ms(torch, lambda: ops.v_decode(ve2["stream"], ve2["info"], codes2, 128, 64, b2), 5)
+            bytes2 = ke2["size"] + ve2["size"] + 8 * (nblk_k + nblk_v) + 8 * B * Tc + 2 * 2 * B * Hq * 128
+            other["rel %.3g" % rel2] = {
+                "bits": b2, "attn_us": a_ms * 1e3, "attn_roofline_frac": bytes2 / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "encode_k_ms": k2, "encode_v_ms": v2, "unpack_k_ms": uk2, "unpack_v_ms": uv2,
+                "ratio_k": fp16_bytes / 2 / ke2["size"], "ratio_v": fp16_bytes / 2 / ve2["size"]}
+            del ke2, ve2, codes2
+        result["other_error_bounds"] = other
+
     if not args.no_cpu:
         ns = min(B, 16)
         k1, v1, q1 = kc[:ns].cpu(), vc[:ns].cpu(), q[:ns].cpu()
