@@ -93,10 +93,10 @@ int pkv_dequantize(const uint8_t *codes, int dtype, int B, int H, int T, const v
  * x [B, H, T, 128] `dtype` -> stream + block_info + scale/zero [B, T], never materialising
  * the code matrix.  Same stream as pkv_quant_params + pkv_quantize + pkv_{k,v}_encode.
  * K uses blocks of 64 x 128, V blocks of 128 x 64 (the shapes the reference's kernels
- * consume, src/kernels.cu:564-589, :795-818).  `bits` is the raw code width W: 2..4 for any
- * head count, and the extension widths 5 and 6 for up to eight heads (other shapes and widths
- * go through pkv_quant_params + pkv_quantize + pkv_{k,v}_encode); a code that does not fit W
- * bits raises PKV_ERR_UNSUPPORTED when size_out is requested. */
+ * consume, src/kernels.cu:564-589, :795-818).  `bits` is the raw code width W: 2..4, and the
+ * extension widths 5 and 6 (7 and 8 go through pkv_quant_params + pkv_quantize +
+ * pkv_{k,v}_encode); a code that does not fit W bits raises PKV_ERR_UNSUPPORTED when size_out
+ * is requested. */
 int pkv_k_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *stream,
                        uint64_t capacity, uint32_t *block_info, void *scale, void *zero,
                        uint64_t *size_out, float *ms_out, pkv_stream_t s);

@@ -500,6 +500,39 @@ __device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane
     }
 }
 
+// the same exchange for the two-halves pack words of widths 5 and 6
+__device__ __forceinline__ void v_exchange(UnitPacksW &u, uint8_t *area, int lane) {
+    uint32_t *a = reinterpret_cast<uint32_t *>(area);
+    uint32_t f[5][4];
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) {
+        f[0][sl] = (uint32_t)u.lo[sl];
+        f[1][sl] = (uint32_t)(u.lo[sl] >> 32);
+        f[2][sl] = (uint32_t)u.hi[sl];
+        f[3][sl] = (uint32_t)(u.hi[sl] >> 32);
+        f[4][sl] = u.mn[sl] | (u.len[sl] << 8);
+    }
+#pragma unroll
+    for (int kind = 0; kind < 5; kind++) {
+        *reinterpret_cast<uint4 *>(a + 4 * lane) = make_uint4(f[kind][0], f[kind][1], f[kind][2], f[kind][3]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[kind][i] = a[64 * i + lane];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) {
+        u.lo[sl] = ((uint64_t)f[1][sl] << 32) | f[0][sl];
+        u.hi[sl] = ((uint64_t)f[3][sl] << 32) | f[2][sl];
+        u.mn[sl] = f[4][sl] & 0xFFu;
+        u.len[sl] = f[4][sl] >> 8;
+    }
+}
+
 // ---- fused parameters + quantize + encode, one workgroup per sub-group ---------------------
 // A group is the run of blocks that share one (context block, sequence): H blocks for K, 2 H for
 // V, consecutive in stream order; a sub-group is up to eight consecutive blocks of a group.  One
@@ -523,7 +556,7 @@ constexpr int kSubBlocks = 8;
 #define PKV_EPRIO_EMIT 2
 #endif
 
-template <bool IS_K, int DT>
+template <bool IS_K, int DT, bool WIDE>
 __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
@@ -624,7 +657,7 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
         const int h = IS_K ? j : j >> 1, d0 = IS_K ? 0 : (j & 1) * 64;
         uint2 xr[16];
         cell_load(x + (((size_t)b * H + h) * T + tok0 + 16 * round) * kHeadDim + d0 + 4 * cgrp, xr);
-        UnitPacks u;
+        typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_packs<DT>(xr, s_par + 16 * round, u, cmax);
         if (active) {
@@ -649,7 +682,7 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
 #pragma unroll
             for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
             if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
-            unit_emit(blk, base, t, g, u);
+            unit_emit_any(blk, base, t, g, u);
         }
         __syncthreads();
     }
@@ -1052,9 +1085,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
-    PKV_REQUIRE(bits >= 2 && (bits <= 4 || (bits <= 6 && H <= kSubBlocks)), PKV_ERR_UNSUPPORTED,
-                "not supported: bits_len %d with %d heads (the fused encoders take 2..4, and 5..6 for up to 8 heads; "
-                "other widths go through pkv_quant_params, pkv_quantize and pkv_{k,v}_encode)", bits, H);
+    PKV_REQUIRE(bits >= 2 && bits <= 6, PKV_ERR_UNSUPPORTED,
+                "not supported: bits_len %d (the fused encoders take 2..6; wider codes go through pkv_quant_params, "
+                "pkv_quantize and pkv_{k,v}_encode)", bits);
     PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
@@ -1097,14 +1130,14 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
                                                       : k_quant_encode_rounds_kernel<PKV_BF16, false>);
             kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
                                         capacity, info, st, bits, nsub, slot, base, par_stride);
-        } else if (dtype == PKV_F16)
-            quant_encode_group_kernel<IS_K, PKV_F16><<<nsub, 256, gbytes, s>>>(
-                (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                bits, nsub, bound, base, par_stride);
-        else
-            quant_encode_group_kernel<IS_K, PKV_BF16><<<nsub, 256, gbytes, s>>>(
-                (const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream, capacity, info, st,
-                bits, nsub, bound, base, par_stride);
+        } else {
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, true>
+                                                      : quant_encode_group_kernel<IS_K, PKV_BF16, true>)
+                                 : (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, false>
+                                                      : quant_encode_group_kernel<IS_K, PKV_BF16, false>);
+            kern<<<nsub, 256, gbytes, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                           capacity, info, st, bits, nsub, bound, base, par_stride);
+        }
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
         return finish_encode(st, size_out, bits, s);

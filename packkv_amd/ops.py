@@ -248,9 +248,9 @@ def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed):
     if info is None:
         info = torch.empty(nblk, 2, dtype=torch.uint32, device=x.device)
     _require(info.numel() == 2 * nblk and info.dtype == torch.uint32, "block_info_buffer block num mismatch")
-    if bits > 6 or (bits > 4 and H > 8):
-        # widths 7..8 (and 5..6 with more than eight heads; format extension): quantize to the code matrix, then the
-        # block codec -- three kernels instead of the fused one
+    if bits > 6:
+        # widths 7..8 (format extension): quantize to the code matrix, then the block codec -- three kernels instead
+        # of the fused one
         scale, zero = quant_params(x, rel)
         codes, mx = quantize(x, scale, zero)
         if mx >= (1 << bits):
