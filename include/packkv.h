@@ -212,8 +212,8 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *                     kernel that gathers straight from global memory.  All three implement the
  *                     same contract; tests cross-check them.  The matrix-core kernels take the reference's
  *                     widths (k_bits, v_bits in 2..4, any mix); variant 0 also takes the extension widths 5
- *                     and 6 when K and V share one.  Any other extension width runs the plain kernel whatever
- *                     `variant` says.
+ *                     and 6 on either side with 4, 5 or 6 on the other.  Any other combination with an
+ *                     extension width runs the plain kernel whatever `variant` says.
  */
 typedef struct pkv_attn_args {
     const uint8_t *k_stream;

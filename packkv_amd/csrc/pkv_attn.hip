@@ -506,8 +506,14 @@ static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
         case 3 * 8 + 4: return launch_dma<G, 3, 4>(p, s);
         case 4 * 8 + 2: return launch_dma<G, 4, 2>(p, s);
         case 4 * 8 + 3: return launch_dma<G, 4, 3>(p, s);
-        case 5 * 8 + 5: return launch_dma<G, 5, 5>(p, s);       // the extension widths, K and V alike
+        case 5 * 8 + 5: return launch_dma<G, 5, 5>(p, s);       // the extension widths 5 and 6, for K, V or both
         case 6 * 8 + 6: return launch_dma<G, 6, 6>(p, s);
+        case 5 * 8 + 4: return launch_dma<G, 5, 4>(p, s);
+        case 4 * 8 + 5: return launch_dma<G, 4, 5>(p, s);
+        case 6 * 8 + 5: return launch_dma<G, 6, 5>(p, s);
+        case 5 * 8 + 6: return launch_dma<G, 5, 6>(p, s);
+        case 6 * 8 + 4: return launch_dma<G, 6, 4>(p, s);
+        case 4 * 8 + 6: return launch_dma<G, 4, 6>(p, s);
         default: return launch_dma<G, 4, 4>(p, s);
     }
 }
@@ -626,9 +632,9 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     // tiles and writes one more partial), so the window costs no launch and no idle tail; other paths
     // give the window a kernel of its own.
     // the matrix-core kernels take the reference's widths and, in the asynchronous-copy kernel, the extension widths
-    // 5 and 6 when K and V share one; any other extension width runs the plain kernel
+    // 5 and 6 (the other side then 4, 5 or 6); any other combination with an extension width runs the plain kernel
     const bool narrow = a->T_c == 0 || (a->k_bits <= 4 && a->v_bits <= 4);
-    const bool wide_fast = !narrow && a->k_bits == a->v_bits && a->k_bits <= 6 && a->variant == 0;
+    const bool wide_fast = !narrow && a->k_bits >= 4 && a->v_bits >= 4 && a->k_bits <= 6 && a->v_bits <= 6 && a->variant == 0;
     const bool aligned16 = (narrow || wide_fast) &&
                            ((reinterpret_cast<uintptr_t>(a->k_stream) | reinterpret_cast<uintptr_t>(a->v_stream)) & 15u) == 0;
     p.win_piece = 0;

@@ -201,13 +201,15 @@ constexpr int dma_lds_bytes() {          // static LDS of attn_dma_kernel: two s
 }
 
 template <int G, int KW, int VW, bool BF>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DMA_WAVES(KW, G), 4))) attn_dma_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DMA_WAVES((KW > VW ? KW : VW), G), 4))) attn_dma_kernel(const AttnParams p) {
     using Geo = DmaGeom<KW, VW>;
-    constexpr bool WIDE = KW > 4;                // widths 5, 6: two-token windows
-    static_assert((KW > 4) == (VW > 4) && KW <= 6 && VW <= 6, "K and V are both reference widths or both 5..6");
-    constexpr int TPW = WIDE ? 2 : 4;            // tokens per window
-    constexpr int NWIN = 16 / TPW;
-    typedef typename UnitOf<WIDE>::type Unit;
+    constexpr bool KWIDE = KW > 4, VWIDE = VW > 4;            // widths 5, 6: two-token windows (K and V independently)
+    constexpr bool WIDE = KWIDE || VWIDE;
+    static_assert(KW <= 6 && VW <= 6, "widths 2..6");
+    constexpr int KTPW = KWIDE ? 2 : 4, VTPW = VWIDE ? 2 : 4;  // tokens per window
+    constexpr int KNWIN = 16 / KTPW, VNWIN = 16 / VTPW;
+    typedef typename UnitOf<KWIDE>::type KUnit;
+    typedef typename UnitOf<VWIDE>::type VUnit;
     typedef StagePrio<G, WIDE> Prio;
     constexpr int ROWS = 3 * G;
     constexpr int NSETS = (ROWS + 15) / 16;
@@ -340,7 +342,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
 
     // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
     const int ku = hw & 3;
-    auto parse = [&](int slot, const TileInfo &ti, Unit &kr, Unit &vr) {
+    auto parse = [&](int slot, const TileInfo &ti, KUnit &kr, VUnit &vr) {
         const uint8_t *kb = ring + slot * Geo::kSlot + kj * Geo::kRegion;
         const uint8_t *vb = ring + slot * Geo::kSlot + (2 + kj) * Geo::kRegion;
         const uint32_t kph = ti.k_off & 15u, vph = ti.v_off & 15u;
@@ -363,15 +365,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         pack_offsets8(__builtin_amdgcn_perm(kr.len23, kr.len01, 0x06040200u), koff);
         pack_offsets8(__builtin_amdgcn_perm(vr.len23, vr.len01, 0x06040200u), voff);
         const uint32_t kpay0 = k_unit + K_META, vpay0 = v_unit + V_META;
-        if constexpr (WIDE) {
+        if constexpr (KWIDE) {
             wide_windows(kb, kpay0, koff, kr);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
+        }
+        if constexpr (VWIDE) {
             wide_windows(vb, vpay0, voff, vr);
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
-                vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
-            }
+            for (int i = 0; i < 4; i++) vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
         }
     };
 
@@ -393,10 +397,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
 
     // ---- stage 1: K round hw -> int8 tile rows [hw*16, hw*16+16), then scores on the matrix cores ----
-    auto k_stage = [&](const Unit &kr, uint8_t *kt) {
+    auto k_stage = [&](const KUnit &kr, uint8_t *kt) {
         {
+            constexpr int TPW = KTPW, NWIN = KNWIN;
             uint32_t w01[NWIN], w23[NWIN];
-            if constexpr (WIDE) {
+            if constexpr (KWIDE) {
 #pragma unroll
                 for (int e = 0; e < NWIN; e++) { w01[e] = kr.e01[e]; w23[e] = kr.e23[e]; }
             } else {
@@ -506,10 +511,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         for (int pp = 0; pp < 4; pp++) a_w[pp][i4] = (half4v){0, 0, 0, 0};
     }
     const bool a_loader = (lane & 31) < 4;
-    auto v_stage = [&](const Unit &vr) {
+    auto v_stage = [&](const VUnit &vr) {
+        constexpr int TPW = VTPW, NWIN = VNWIN;
         const int seg = hw & 1;
         uint32_t w01[NWIN], w23[NWIN];
-        if constexpr (WIDE) {
+        if constexpr (VWIDE) {
 #pragma unroll
             for (int e = 0; e < NWIN; e++) { w01[e] = vr.e01[e]; w23[e] = vr.e23[e]; }
         } else {
@@ -572,7 +578,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
 
     // ---- pipeline ----
     TileInfo i0 = load_info(0), i1 = load_info(1), i2 = load_info(2);
-    Unit kcur, vcur;
+    KUnit kcur;
+    VUnit vcur;
     dma_issue(0, 0, i0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     PKV_LDS_BARRIER();
@@ -590,7 +597,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
         PKV_LDS_BARRIER();                                    // publishes the scores and tile s+1
-        Unit knext, vnext;
+        KUnit knext;
+        VUnit vnext;
         __builtin_amdgcn_s_setprio(Prio::S);
         parse(slot ^ 1, i1, knext, vnext);
         softmax_stage(slot, kt);

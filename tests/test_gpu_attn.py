@@ -259,3 +259,24 @@ def test_attn_decode_wide_codes_group_sizes(cuda, hq):
     _say("wide attention case: group of", hq // Hkv)
     got = ops.attn_decode(q.to(cuda), ke, ve)
     _check(got, want, torch.float16, exact, abs_tol=STRESS_ABS_TOL[torch.float16])
+
+
+@pytest.mark.parametrize("rel_k,rel_v,bits", [(0.05, 0.1, (5, 4)), (0.1, 0.05, (4, 5)), (0.03, 0.05, (6, 5)), (0.03, 0.1, (6, 4))])
+def test_attn_decode_mixed_widths(cuda, rel_k, rel_v, bits):
+    """K and V at different error bounds, one of them (or both) at an extension width: the asynchronous-copy kernel
+    windows each side on its own.  Checked against decompress-then-attend and against the plain kernel."""
+    B, Hq, Hkv, T = 2, 16, 4, 896
+    k, v = synth.make_kv(B, Hkv, T, seed=187)
+    q = synth.make_q(B, Hq, seed=188)
+    want = _reference(q, k, v, rel_k, rel_v)
+    exact = _exact(q, k, v, rel_k, rel_v)
+    ke = ops.k_quant_encode(k.to(cuda), rel_k)
+    ve = ops.v_quant_encode(v.to(cuda), rel_v)
+    assert (ke["bits"], ve["bits"]) == bits
+    outs = []
+    for variant in (0, 1):
+        _say("mixed widths case", bits, "variant", variant)
+        got = ops.attn_decode(q.to(cuda), ke, ve, variant=variant)
+        _check(got, want, torch.float16, exact, abs_tol=STRESS_ABS_TOL[torch.float16], variant=variant)
+        outs.append(got.float())
+    assert (outs[0] - outs[1]).abs().max().item() < 4e-3
