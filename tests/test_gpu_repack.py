@@ -156,7 +156,9 @@ def test_greedy_repacking_shrinks_shifted_tokens_and_feeds_attention(cuda):
     assert ve["size"] < vn["size"]
     out_g = ops.attn_decode(q.to(cuda), ke, ve).float().cpu()
     out_n = ops.attn_decode(q.to(cuda), kn, vn).float().cpu()
-    assert (out_g - out_n).abs().max().item() < 2e-3
+    diff = (out_g - out_n).abs().max().item()
+    _say("greedy order vs natural order: max|diff| = %.2e, max|out| = %.2e" % (diff, out_n.abs().max().item()))
+    assert diff <= 2 ** -9 * max(out_n.abs().max().item(), 1.0)      # the same terms in another order: an output rounding or two apart
 
 
 def test_repacked_cache_attends_like_the_original(cuda):
