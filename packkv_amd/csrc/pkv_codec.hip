@@ -126,6 +126,119 @@ __global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restri
                        nunits, W);
 }
 
+// ---- the same encode, eight blocks per workgroup (blocks of four units, widths 2..4) ------------------------
+// With one ticket per block a launch has tens of thousands of status words in flight and a block's look-back walks
+// far before it meets an inclusive prefix: the per-block kernel spends most of its time there (vector ALUs 24 %
+// busy).  Here a workgroup of 256 threads takes eight consecutive blocks of the stream -- two at a time: load the
+// two code tiles with 16-byte loads, analyse, emit behind the blocks already in LDS -- and then asks ONE offset for
+// all of them and writes their bytes, contiguous in the stream, in one sweep of aligned 16-byte stores.
+constexpr int kPackGroup = 8;
+
+template <bool IS_K>
+__global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                                                         uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                                                         int hidden_dim, int ctx_blk, int hid_blk, int W, uint32_t nblocks,
+                                                         uint32_t ngroups) {
+    extern __shared__ __align__(16) uint8_t lds[];         // two code tiles | the group's bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t unit_bytes[2][4];
+    __shared__ uint32_t blk_off[kPackGroup + 1];
+    const int tid = threadIdx.x;
+    if (tid == 0) { s_idx = atomicAdd(&st->ticket, 1u); blk_off[0] = 0u; }
+    __syncthreads();
+    const uint32_t gidx = s_idx;
+    if (gidx >= ngroups) return;
+    const uint32_t b0 = gidx * (uint32_t)kPackGroup;
+    const int nb = (int)min((uint32_t)kPackGroup, nblocks - b0);
+    const int tile_bytes = ctx_blk * hid_blk;              // a multiple of 16
+    uint8_t *gbuf = lds + 2 * tile_bytes;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const int n_hid = hidden_dim / hid_blk;
+    const int jl = tid >> 7, lt = tid & 127, unit = lt >> 5, t = tid & 31;
+    const uint8_t *tile = lds + jl * tile_bytes;
+    const int row16 = hid_blk >> 4, n16 = ctx_blk * row16;
+    for (int j0 = 0; j0 < nb; j0 += 2) {
+        const int jj = j0 + jl;
+        const bool active = jj < nb;
+        const uint32_t b = b0 + (uint32_t)min(jj, nb - 1);            // clamped: the loads are unconditional
+        const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+        const uint8_t *src = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+        uint4 *t16 = reinterpret_cast<uint4 *>(lds + jl * tile_bytes);
+        for (int i = lt; i < n16; i += 4 * 128) {                     // four loads in flight
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int idx = min(i + 128 * u, n16 - 1);
+                v[u] = *reinterpret_cast<const uint4 *>(src + (size_t)(idx / row16) * hidden_dim + 16 * (idx % row16));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + 128 * u < n16) t16[i + 128 * u] = v[u];
+        }
+        __syncthreads();
+        UnitPacks u;
+        if (active) {
+            unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
+            if (t == 0) unit_bytes[jl][unit] = meta + u.payload;
+        }
+        __syncthreads();
+        if (tid == 0) {                                   // block sizes of this pair -> offsets inside the group
+            uint32_t off = blk_off[j0] + 8u + unit_bytes[0][0] + unit_bytes[0][1] + unit_bytes[0][2] + unit_bytes[0][3];
+            blk_off[j0 + 1] = off;
+            if (j0 + 1 < nb) blk_off[j0 + 2] = off + 8u + unit_bytes[1][0] + unit_bytes[1][1] + unit_bytes[1][2] + unit_bytes[1][3];
+        }
+        __syncthreads();
+        if (active) {
+            uint8_t *blk = gbuf + blk_off[jj];
+            uint32_t base = 8u;
+#pragma unroll
+            for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
+            if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
+            unit_emit(blk, base, t, g, u);
+        }
+        __syncthreads();
+    }
+    const uint32_t bytes = blk_off[nb];
+    if (tid < 64) {
+        const uint64_t off = lookback_offset(st, gidx, bytes);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < nb) {
+        info[2 * (size_t)(b0 + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(b0 + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    // head (to the first 16-byte boundary of the stream) and tail in 2-byte pieces, the body as aligned 16-byte
+    // stores fed by aligned LDS reads and byte funnel shifts
+    uint8_t *dst = stream + off;
+    const uint32_t head = min(bytes, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
+    const uint32_t nq = (bytes - head) >> 4;
+    for (uint32_t i = tid; i < (head >> 1); i += 256)
+        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(gbuf)[i];
+    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(gbuf + (head & ~3u));
+    for (uint32_t i = tid; i < nq; i += 256) {
+        const uint32_t *q = src32 + 4 * i;
+        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+        uint4 v;
+        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
+        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
+        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
+        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+        *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
+    }
+    const uint32_t done = head + 16u * nq;
+    for (uint32_t i = tid; i < ((bytes - done) >> 1); i += 256)
+        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(gbuf + done)[i];
+}
+
 __global__ void zero_state_kernel(uint64_t *p, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -231,6 +344,24 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
     int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
     if (rc) return rc;
     ScanState *st = nullptr;
+    // blocks of four units at the reference's widths, 16-byte aligned rows: eight blocks per workgroup
+    const bool grouped = cs.nunits == 4 && bits <= 4 && hid_blk % 16 == 0 && hidden_dim % 16 == 0 &&
+                         (reinterpret_cast<uintptr_t>(codes) & 15u) == 0;
+    if (grouped) {
+        const uint32_t ngroups = ((uint32_t)cs.nblocks + kPackGroup - 1) / kPackGroup;
+        const uint32_t lds = 2u * (uint32_t)(ctx_blk * hid_blk) + (uint32_t)kPackGroup * cs.blk_cap + 32u;
+        if ((rc = prepare_scan_state(ngroups, &st, s))) return rc;
+        auto kern = is_k ? pack_group_kernel<true> : pack_group_kernel<false>;
+        if (lds > 48u * 1024u)
+            PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        LaunchTimer tm(s, ms_out != nullptr);
+        if ((rc = tm.begin())) return rc;
+        kern<<<ngroups, 256, lds, s>>>(codes, stream, capacity, info, st, hidden_dim, ctx_blk, hid_blk, bits,
+                                       (uint32_t)cs.nblocks, ngroups);
+        PKV_HIP_CHECK(hipGetLastError());
+        if ((rc = tm.end(ms_out))) return rc;
+        return finish_encode(st, size_out, 0, s);
+    }
     if ((rc = prepare_scan_state((uint32_t)cs.nblocks, &st, s))) return rc;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
