@@ -353,6 +353,9 @@ def main():
         codes_v = torch.empty(Tc, hidden, dtype=torch.uint8, device=dev)
         ops.k_decode(ke["stream"], ke["info"], codes, 64, 128, bits)
         ops.v_decode(ve["stream"], ve["info"], codes_v, 128, 64, bits)
+        # the block codec alone, code matrix -> stream (the reference's k_encode_cpu / v_encode_cpu on the device)
+        ck_ms = event_time_ms(torch, lambda: ops.k_encode(codes, ke["stream"], ke["info"], 64, 128, bits, want_size=False), 3)
+        cv_ms = event_time_ms(torch, lambda: ops.v_encode(codes_v, ve["stream"], ve["info"], 128, 64, bits, want_size=False), 3)
         rp_ms = event_time_ms(torch, lambda: ops.median_repacking(codes, codes_v, 64), 3)
         bp_ms = event_time_ms(torch, lambda: ops.bit_pack_bytes(codes, 16), 3)
         g_rows = min(Tc, 8192)      # the greedy order re-reads a block once per pick: a slice of the workload is enough
@@ -371,6 +374,8 @@ def main():
             "k_roofline_frac": enc_algo_k / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "v_roofline_frac": enc_algo_v / (v_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         }
+        result["codec_encode"] = {"k_ms": ck_ms, "v_ms": cv_ms, "k_gbs_codes": Tc * hidden / (ck_ms * 1e-3) / 1e9,
+                                  "v_gbs_codes": Tc * hidden / (cv_ms * 1e-3) / 1e9}
         result["unpack"] = {
             "k_ms": uk_ms, "v_ms": uv_ms,
             "k_gbs": (ke["size"] + 8 * nblk_k + Tc * hidden) / (uk_ms * 1e-3) / 1e9,
