@@ -368,7 +368,7 @@ __device__ __forceinline__ void block_decode(const uint8_t *blk, uint32_t phase,
 constexpr uint64_t kFlagAgg = 1ull << 62;
 constexpr uint64_t kFlagIncl = 2ull << 62;
 constexpr uint64_t kValueMask = (1ull << 62) - 1ull;
-constexpr int kSpinLimit = 1 << 20;
+constexpr int kSpinLimit = 1 << 18;          // polls before a wait gives up with PKV_ERR_INTERNAL: well under a second at the look-back's back-off
 
 struct ScanState {
     uint32_t ticket;      // next block index to hand out
