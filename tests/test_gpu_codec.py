@@ -36,10 +36,11 @@ def _gpu_encode(cuda, is_k, c, cb, hb, W):
     return d_stream, d_info, size
 
 
+# (192, 640) and (256, 320): 15 and 10 blocks, so the eight-blocks-per-workgroup encoder ends on a partial group
 SHAPES = {1: [(64, 128, 64, 128), (256, 512, 64, 128), (128, 4096, 64, 128), (64, 256, 32, 128),
-              (256, 128, 128, 128), (32, 128, 16, 128)],
+              (256, 128, 128, 128), (32, 128, 16, 128), (192, 640, 64, 128)],
           0: [(128, 64, 128, 64), (512, 512, 128, 64), (128, 4096, 128, 64), (256, 128, 128, 32),
-              (128, 256, 128, 128)]}
+              (128, 256, 128, 128), (256, 320, 128, 64)]}
 
 
 @pytest.mark.parametrize("is_k", [1, 0])
@@ -63,6 +64,24 @@ def test_encode_decode_bit_exact_vs_oracle(cuda, oracle_codec, is_k, W):
             s2 = torch.from_numpy(so[:zo].copy()).to(cuda)      # exactly-sized stream buffer
             (ops.k_decode if is_k else ops.v_decode)(s2, torch.from_numpy(io).to(cuda), d_out, cb, hb, W)
             assert np.array_equal(d_out.cpu().numpy(), c)
+
+
+def test_encode_from_a_misaligned_code_matrix(cuda, oracle_codec):
+    """A code matrix that does not start on a 16-byte boundary takes the one-block-per-workgroup encoder; same
+    stream."""
+    rng = np.random.default_rng(77)
+    for is_k, (T, H, cb, hb) in ((1, (128, 256, 64, 128)), (0, (128, 256, 128, 64))):
+        c = _rand_codes(rng, T, H, 4, "gauss")
+        so, io, zo = oracle_codec.encode(is_k, c, cb, hb, 4)
+        flat = torch.zeros(T * H + 16, dtype=torch.uint8, device=cuda)
+        d_codes = flat[3:3 + T * H].view(T, H)
+        d_codes.copy_(torch.from_numpy(c))
+        assert d_codes.data_ptr() % 16 != 0 and d_codes.is_contiguous()
+        d_stream = torch.zeros(T * H, dtype=torch.uint8, device=cuda)
+        d_info = torch.zeros((T // cb) * (H // hb), 2, dtype=torch.uint32, device=cuda)
+        size = (ops.k_encode if is_k else ops.v_encode)(d_codes, d_stream, d_info, cb, hb, 4)
+        assert size == zo and np.array_equal(d_info.cpu().numpy(), io)
+        assert np.array_equal(d_stream[:size].cpu().numpy(), so[:zo])
 
 
 def test_golden_vectors_from_reference_codec(cuda, golden):
