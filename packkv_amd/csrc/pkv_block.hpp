@@ -387,16 +387,23 @@ struct ScanState {
 #ifndef PKV_LOOKBACK_SLEEP
 #define PKV_LOOKBACK_SLEEP 100
 #endif
-__device__ __forceinline__ uint64_t lookback_offset(ScanState *st, uint32_t idx, uint32_t my_bytes) {
+// One thread may publish the size ahead of the look-back, as soon as it is known (the successors then wait less);
+// the look-back is told so and does not store it again.
+__device__ __forceinline__ void lookback_publish(ScanState *st, uint32_t idx, uint32_t my_bytes) {
+    __hip_atomic_store(&st->status[idx], (idx == 0 ? kFlagIncl : kFlagAgg) | (uint64_t)my_bytes, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint64_t lookback_offset(ScanState *st, uint32_t idx, uint32_t my_bytes, bool published = false) {
     const int lane = threadIdx.x & 63;
     uint64_t *status = st->status;
     if (idx == 0) {
-        if (lane == 0)
+        if (lane == 0 && !published)
             __hip_atomic_store(&status[0], kFlagIncl | (uint64_t)my_bytes, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
         return 0;
     }
-    if (lane == 0)
+    if (lane == 0 && !published)
         __hip_atomic_store(&status[idx], kFlagAgg | (uint64_t)my_bytes, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     uint64_t prefix = 0;

@@ -802,9 +802,20 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         __syncthreads();                                  // s_par is rewritten by the next round
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
+        const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        if (r == 3) {
+            // every block's final size is known before its last unit is written: the group's size is published
+            // now, so that the workgroups behind it in the stream wait that much less for it
+            if (active && t == 0) blk_off[j + 1] = my_off + usz;          // sizes first ...
+            if (tid == 0) blk_off[0] = 0;
+            __syncthreads();
+            if (tid == 0) {                                               // ... then their running sum
+                for (int q = 1; q <= H; q++) blk_off[q] += blk_off[q - 1];
+                lookback_publish(st, gidx, blk_off[H]);
+            }
+        }
         if (active) {
             cmax_all = max(cmax_all, cmax);
-            const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
             if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
             unit_emit_any(blk, my_off, t, g, u);
             my_off += usz;
@@ -815,15 +826,10 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
         if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
     }
-    if (active && t == 0) blk_off[j + 1] = my_off;          // sizes first ...
-    if (tid == 0) blk_off[0] = 0;
-    __syncthreads();
-    if (tid == 0)                                           // ... then their running sum
-        for (int q = 1; q <= H; q++) blk_off[q] += blk_off[q - 1];
     __syncthreads();
     const uint32_t bytes = blk_off[H];
     if (tid < 64) {
-        const uint64_t off = base + lookback_offset(st, gidx, bytes);
+        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
         if (tid == 0) {
             s_off = off;
             if (gidx == ngroups - 1) st->total = off + bytes;
@@ -1002,6 +1008,21 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         __syncthreads();                                  // s_par is rewritten by the next iteration; s_tot is published
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
+        if (it == 3) {
+            // the last units' sizes are known before their packs are written: the group's size is published now, so
+            // that the workgroups behind it in the stream wait that much less for it
+            if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
+            __syncthreads();
+            if (tid == 0) {
+                uint32_t run = 0;
+                for (int q = 0; q < 2 * H; q++) {
+                    blk_off[q] = run;
+                    run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
+                }
+                blk_off[2 * H] = run;
+                lookback_publish(st, gidx, run);
+            }
+        }
         if (active) {
             cmax_all = max(cmax_all, cmax);
             const int sg = it >> 1, slot = 2 * (it & 1) + rp;
@@ -1017,7 +1038,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         }
         run_off += tot_even + tot_odd;                    // both rounds of the iteration are behind the unit now
         if (it & 1) {                                     // the unit (w, it / 2) is complete
-            if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + (it >> 1)] = (uint16_t)(meta + run_off);
+            if (it == 1 && active && rp == 0 && m == 0) s_usz[blkid][2 * w] = (uint16_t)(meta + run_off);
             run_off = 0;
         }
     }
@@ -1028,18 +1049,9 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     }
     __syncthreads();
     const int nblk = 2 * H;
-    if (tid == 0) {
-        uint32_t run = 0;
-        for (int q = 0; q < nblk; q++) {
-            blk_off[q] = run;
-            run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
-        }
-        blk_off[nblk] = run;
-    }
-    __syncthreads();
     const uint32_t bytes = blk_off[nblk];
     if (tid < 64) {
-        const uint64_t off = base + lookback_offset(st, gidx, bytes);
+        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
         if (tid == 0) {
             s_off = off;
             if (gidx == ngroups - 1) st->total = off + bytes;
