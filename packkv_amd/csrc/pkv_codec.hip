@@ -1,5 +1,6 @@
-// Bit-unpack (stream -> uint8 codes) and bit-pack (uint8 codes -> stream) kernels, one
-// workgroup per block, one 32-lane half-wavefront per round (K) or segment (V).
+// Bit-unpack (stream -> uint8 codes) and bit-pack (uint8 codes -> stream) kernels: one 32-lane
+// half-wavefront per round (K) or segment (V); one workgroup per block, except the encoder of
+// the standard block shapes, which takes eight consecutive blocks per workgroup.
 //
 // Replaces the reference's scalar CPU codec on the device:
 //   packkv_cuda_ext/src/k_encode_cpu.cpp:203-231, v_encode_cpu.cpp:230-259  (encode drivers)
