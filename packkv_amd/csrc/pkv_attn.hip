@@ -230,8 +230,9 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
 // ---- matrix-core kernels (variants 0 and 2): shared arithmetic ----------------------------
 // K side: every half-wavefront unpacks one round (16 tokens x 128 channels, lane t = channels
 // 4t..4t+3) into an int8 tile in LDS laid out [token][channel]; the tile is read back in the
-// operand layout of v_mfma_i32_16x16x32_i8 (lane = token, 8 consecutive channels) and
-// contracted against q, which is split per query head into three signed 7-bit digits
+// operand layout of the 16x16 int8 MFMAs (lane = token, 8 consecutive channels per 8-byte read;
+// the staged kernel pairs two reads into one v_mfma_i32_16x16x64_i8 operand, the gather kernel
+// issues v_mfma_i32_16x16x32_i8 per read) and contracted against q, which is split per query head into three signed 7-bit digits
 // (q = qs * (d0 * 2^14 + d1 * 2^7 + d2)), one MFMA row per (digit, head).  Integer arithmetic
 // is exact, so the scores carry only the 2^-21 relative rounding of that split.
 // V side: lane = channel as in the stream, nothing is transposed.  MFMA number k of a segment

@@ -325,20 +325,26 @@ __global__ void pack_size_zero_kernel(PackSizeOut *out) {
     out->present[threadIdx.x] = 0u;
 }
 
-// grid (ceil(hidden / 4096), ctx_len / pack_len), 256 threads; thread = 16 adjacent channels of one pack, four rows
-// in flight; minima and maxima as packed 16-bit lanes (even and odd bytes of every dword apart)
+// 256 threads per workgroup, a grid-stride walk over the items (pack, 16 adjacent channels), the channel chunk
+// running fastest so that a wavefront reads whole rows; four rows in flight per thread; minima and maxima as packed
+// 16-bit lanes (even and odd bytes of every dword apart).  One atomic per workgroup: same-address atomics retire
+// one after the other, so their number, not the bytes, would set the time of a grid with a workgroup per pack.
+// Bound by instruction issue: 7 vector instructions per dword for the ranges and 8 for the presence flags (a
+// register bit mask for values below 32 instead of the LDS flags costs the same).
 typedef unsigned short pk_u16x2 __attribute__((ext_vector_type(2)));
 
 __global__ void __launch_bounds__(256) pack_size_kernel(const uint8_t *__restrict__ codes, int hidden, int pack_len,
-                                                        PackSizeOut *out) {
+                                                        size_t n_items, PackSizeOut *out) {
     __shared__ uint32_t seen[256];
-    __shared__ uint32_t wsum[4];
+    __shared__ unsigned long long wsum[4];
     seen[threadIdx.x] = 0u;
     __syncthreads();
-    const int ch = (blockIdx.x * 256 + threadIdx.x) * 16;
-    uint32_t lens = 0;
-    if (ch < hidden) {
-        const uint8_t *p = codes + (size_t)blockIdx.y * pack_len * hidden + ch;
+    const uint32_t chunks = (uint32_t)hidden / 16u;
+    unsigned long long lens = 0;
+    for (size_t item = (size_t)blockIdx.x * 256 + threadIdx.x; item < n_items; item += (size_t)gridDim.x * 256) {
+        const size_t pack = item / chunks;
+        const uint32_t chunk = (uint32_t)(item - pack * chunks);
+        const uint8_t *p = codes + pack * (size_t)pack_len * hidden + (size_t)chunk * 16;
         pk_u16x2 mn[8], mx[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) { mn[i] = (pk_u16x2){255, 255}; mx[i] = (pk_u16x2){0, 0}; }
@@ -367,19 +373,21 @@ __global__ void __launch_bounds__(256) pack_size_kernel(const uint8_t *__restric
             for (int u = 0; u < 4; u++) take(v[u]);
         }
         for (; k < pack_len; k++) take(*reinterpret_cast<const uint4 *>(p + (size_t)k * hidden));
+        uint32_t l = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const pk_u16x2 r = mx[i] - mn[i];
 #pragma unroll
             for (int hlf = 0; hlf < 2; hlf++)
-                lens += r[hlf] ? 32u - (uint32_t)__builtin_clz((uint32_t)r[hlf]) : 0u;   // bit_length = ceil(log2(range + 1))
+                l += r[hlf] ? 32u - (uint32_t)__builtin_clz((uint32_t)r[hlf]) : 0u;   // bit_length = ceil(log2(range + 1))
         }
+        lens += l;
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) lens += __shfl_xor(lens, d, 64);
     if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = lens;
     __syncthreads();
-    if (threadIdx.x == 0) atomicAdd(&out->len_sum, (unsigned long long)(wsum[0] + wsum[1] + wsum[2] + wsum[3]));
+    if (threadIdx.x == 0) atomicAdd(&out->len_sum, wsum[0] + wsum[1] + wsum[2] + wsum[3]);
     if (seen[threadIdx.x]) out->present[threadIdx.x] = 1u;
 }
 
@@ -396,7 +404,6 @@ int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pac
     PKV_REQUIRE(hidden_dim % 16 == 0 && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0, PKV_ERR_INVALID,
                 "hidden_dim must be a multiple of 16 and the code matrix 16-byte aligned");
     PKV_REQUIRE(ctx_len % pack_len == 0, PKV_ERR_INVALID, "ctx_len must be divisible by the pack length");
-    PKV_REQUIRE(ctx_len / pack_len <= 65535, PKV_ERR_UNSUPPORTED, "more than 65535 packs along the context");
     void *scratch = nullptr;
     int rc = scratch_get(sizeof(PackSizeOut), &scratch);
     if (rc) return rc;
@@ -404,8 +411,9 @@ int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pac
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     pack_size_zero_kernel<<<1, 256, 0, s>>>(out);
-    pack_size_kernel<<<dim3((unsigned)((hidden_dim + 4095) / 4096), (unsigned)(ctx_len / pack_len)), 256, 0, s>>>(
-        codes, hidden_dim, pack_len, out);
+    const size_t n_items = (size_t)(ctx_len / pack_len) * (size_t)(hidden_dim / 16);
+    const size_t wanted = (n_items + 255) / 256;
+    pack_size_kernel<<<(unsigned)(wanted < 2048 ? wanted : 2048), 256, 0, s>>>(codes, hidden_dim, pack_len, n_items, out);
     PKV_HIP_CHECK(hipGetLastError());
     if ((rc = tm.end(ms_out))) return rc;
     PackSizeOut h;

@@ -35,6 +35,21 @@ def test_bit_pack_sizes_match_for_every_pack_length(cuda, rel):
         assert got == want
 
 
+def test_code_stats_shapes_against_closed_forms(cuda):
+    """Narrow, wide and very long code matrices (more packs along the context than one grid dimension holds, fewer
+    items than one workgroup, 16 channels, byte values up to 255) against numpy on the same codes."""
+    rng = np.random.default_rng(77)
+    for (T, hid, top, pack) in ((65552 * 16, 16, 32, 16), (48, 16, 256, 16), (4096, 1024, 40, 32), (512, 16384, 6, 64),
+                                (640, 48, 256, 128)):
+        _say("code_stats case", T, hid, top, pack)
+        c = rng.integers(0, top, size=(T, hid), dtype=np.uint8)
+        c[T // 2, hid // 3] = top - 1
+        r = c.reshape(T // pack, pack, hid).astype(np.int64)
+        span = r.max(axis=1) - r.min(axis=1)
+        want = (int(np.where(span > 0, np.floor(np.log2(np.maximum(span, 1))) + 1, 0).sum()), int(np.unique(c).size))
+        assert ops.code_stats(torch.from_numpy(c).to(cuda), pack) == want
+
+
 def test_median_repacking_matches_restatement(cuda):
     for (B, H, T, bs) in ((1, 2, 256, 64), (2, 8, 512, 64), (1, 1, 384, 128), (3, 2, 128, 16)):
         _say("repack case", B, H, T, bs)
