@@ -66,6 +66,30 @@ def test_encode_decode_bit_exact_vs_oracle(cuda, oracle_codec, is_k, W):
             assert np.array_equal(d_out.cpu().numpy(), c)
 
 
+ODD_SHAPES = {1: [(96, 128, 48, 128), (160, 256, 80, 128), (512, 128, 256, 128), (112, 384, 112, 128)],
+              0: [(128, 96, 128, 96), (256, 320, 128, 160), (128, 512, 128, 256), (128, 448, 128, 224)]}
+
+
+@pytest.mark.parametrize("is_k", [1, 0])
+def test_block_shapes_off_the_beaten_track(cuda, oracle_codec, is_k):
+    """K blocks of 48, 80, 112 and 256 tokens and V blocks of 96, 160, 224 and 256 channels (3, 5, 7 and 8 units per
+    block), at every code width from 2 to 8 bits: stream, block_info and the decoded codes against the restatement."""
+    rng = np.random.default_rng(300 + is_k)
+    for (T, H, cb, hb) in ODD_SHAPES[is_k]:
+        for W in range(2, 9):
+            kind = ("uniform", "gauss", "narrow")[W % 3]
+            _say("odd block case", "K" if is_k else "V", T, H, cb, hb, W, kind)
+            c = _rand_codes(rng, T, H, W, kind)
+            so, io, zo = oracle_codec.encode(is_k, c, cb, hb, W)
+            d_stream, d_info, size = _gpu_encode(cuda, is_k, c, cb, hb, W)
+            assert size == zo
+            assert np.array_equal(d_info.cpu().numpy(), io)
+            assert np.array_equal(d_stream[:size].cpu().numpy(), so[:zo])
+            d_out = torch.zeros(T, H, dtype=torch.uint8, device=cuda)
+            (ops.k_decode if is_k else ops.v_decode)(d_stream, d_info, d_out, cb, hb, W)
+            assert np.array_equal(d_out.cpu().numpy(), c)
+
+
 def test_encode_from_a_misaligned_code_matrix(cuda, oracle_codec):
     """A code matrix that does not start on a 16-byte boundary takes the one-block-per-workgroup encoder; same
     stream."""
