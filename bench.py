@@ -248,6 +248,45 @@ def e2e_decode(torch, args, dev):
     print(json.dumps(result))
 
 
+def gemv_surface(torch, ops, synth, dev):
+    """The reference's own GPU ops at the shape its throughput script runs (one sequence of Llama-3.1-8B shape:
+    8 KV heads, 65536 cached tokens, K at rel 0.1 = 4-bit codes, V at rel 0.2 = 3-bit codes) and by its definition:
+    fp16 bytes of the uncompressed tensor / kernel time, K = kq_mat_vec_mul + fused_kq, V = wv_mat_vec_mul +
+    fused_wv, every op timed by the events inside its launcher (scripts/figure/throughput.py:124-138), beside
+    torch.matmul on the fp16 tensor."""
+    H, T = 8, 65536
+    hid = H * 128
+    k, v = synth.make_kv(1, H, T, seed=5, device=dev)
+    ke, ve = ops.k_quant_encode(k, 0.1, 4), ops.v_quant_encode(v, 0.2, 3)
+    q = torch.randn(H, 128, device=dev).half()
+    t = torch.zeros(H, T, dtype=torch.float16, device=dev)
+    w = torch.softmax(torch.randn(H, T, device=dev), dim=1).half()
+    term = torch.zeros(H, 128, dtype=torch.float32, device=dev)
+    our_kq, our_wv = torch.empty_like(t), torch.empty(H, 128, dtype=torch.float16, device=dev)
+    kz, ks = ke["zero"].reshape(-1), ke["scale"].reshape(-1)
+    vz, vs = ve["zero"].reshape(-1), ve["scale"].reshape(-1)
+    term16 = term.half()
+
+    def med(fn):
+        xs = sorted(fn() for _ in range(31))
+        return xs[15]
+
+    kq = med(lambda: ops.kq_mat_vec_mul(ke["stream"], ke["info"], q, t, T, hid, 64, 128, 4))
+    fkq = med(lambda: ops.fused_kq(our_kq, q, kz, ks, t))
+    wv = med(lambda: ops.wv_mat_vec_mul(ve["stream"], ve["info"], w, term, T, hid, 128, 64, 3))
+    fwv = med(lambda: ops.fused_wv(our_wv, w, vz, vs, term16))
+    k3, v3 = k[0], v[0]                                   # [H, T, 128]
+    mk = event_time_ms(torch, lambda: torch.matmul(k3, q.unsqueeze(2)), 30)
+    mv = event_time_ms(torch, lambda: torch.matmul(w.unsqueeze(1), v3), 30)
+    fp16 = T * hid * 2
+    gib = lambda ms: fp16 / 2 ** 30 / (ms * 1e-3)
+    return {"shape": "1 sequence, 8 KV heads x 128, 65536 tokens; K 4-bit (rel 0.1), V 3-bit (rel 0.2)",
+            "kq_ms": kq, "fused_kq_ms": fkq, "wv_ms": wv, "fused_wv_ms": fwv,
+            "k_gibs_of_fp16": gib(kq + fkq), "v_gibs_of_fp16": gib(wv + fwv),
+            "torch_matmul_k_ms": mk, "torch_matmul_v_ms": mv,
+            "torch_matmul_k_gibs": gib(mk), "torch_matmul_v_gibs": gib(mv)}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -416,6 +455,9 @@ def main():
                 "ratio_k": fp16_bytes / 2 / ke2["size"], "ratio_v": fp16_bytes / 2 / ve2["size"]}
             del ke2, ve2, codes2
         result["other_error_bounds"] = other
+
+    if not args.no_extras and default_workload:
+        result["gemv_surface"] = gemv_surface(torch, ops, synth, dev)
 
     if not args.no_cpu:
         ns = min(B, 16)

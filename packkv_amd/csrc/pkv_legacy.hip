@@ -23,7 +23,9 @@ __device__ __forceinline__ uint16_t st16(float x, int dtype) {
     return (uint16_t)(u >> 16);
 }
 
-// grid = number of K blocks, threads = 2 * ctx_blk (one half-wavefront per round).
+// grid = number of K blocks, threads = 2 * ctx_blk (one half-wavefront per round).  (Padding the tile rows so
+// that the dot product's reads spread over the LDS banks changes nothing measurable: the kernel's time is the
+// latency chain stage -> decode -> dot of many small workgroups.)
 __global__ void kq_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
                           const uint16_t *__restrict__ q, uint16_t *__restrict__ kq_out, int ctx_len,
                           int hidden_dim, int ctx_blk, int nunits, int W, uint32_t blk_cap, int dtype,
@@ -67,7 +69,7 @@ __global__ void kq_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
         kq_out[(size_t)hb * ctx_len + (size_t)cb * ctx_blk + r] = st16(acc, dtype);
 }
 
-// grid = number of V blocks, threads = 2 * hid_blk (one half-wavefront per segment).
+// grid = number of V blocks, threads = 2 * hid_blk (one half-wavefront per segment; 8 * hid_blk / 4 in the dot product).
 __global__ void wv_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
                           const uint16_t *__restrict__ w, float *__restrict__ wv_out, int ctx_len,
                           int hidden_dim, int hid_blk, int nunits, int W, uint32_t blk_cap, int dtype) {
@@ -88,11 +90,30 @@ __global__ void wv_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
     __syncthreads();
     block_decode<false>(blk, phase, nunits, W, tile, hid_blk);
     __syncthreads();
-    const int ch = threadIdx.x % hid_blk, half = threadIdx.x / hid_blk;
-    float acc = 0.f;
-#pragma unroll 8
-    for (int t = 0; t < 64; t++) acc += ws[half * 64 + t] * (float)tile[(half * 64 + t) * hid_blk + ch];
-    atomicAdd(wv_out + (size_t)hb * hid_blk + ch, acc);
+    // thread = 4 adjacent channels x 16 tokens (one dword of the tile per token); the eight token slices meet in
+    // LDS, over the staged block, which nobody reads any more (it holds at least 32 * hid_blk bytes at 2 bits)
+    const int ncg = hid_blk >> 2;
+    const int cg = threadIdx.x % ncg, ts = threadIdx.x / ncg;
+    const uint32_t *col = reinterpret_cast<const uint32_t *>(tile) + (ts * 16) * ncg + cg;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+        const uint32_t c = col[t * ncg];
+        const float wt = ws[ts * 16 + t];
+        a0 += wt * (float)(c & 0xFFu);
+        a1 += wt * (float)((c >> 8) & 0xFFu);
+        a2 += wt * (float)((c >> 16) & 0xFFu);
+        a3 += wt * (float)(c >> 24);
+    }
+    float *part = reinterpret_cast<float *>(blk);
+    *reinterpret_cast<float4 *>(part + ts * hid_blk + 4 * cg) = make_float4(a0, a1, a2, a3);
+    __syncthreads();
+    if ((int)threadIdx.x < hid_blk) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc += part[i * hid_blk + threadIdx.x];
+        atomicAdd(wv_out + (size_t)hb * hid_blk + threadIdx.x, acc);
+    }
 }
 
 __device__ __forceinline__ float wave_sum_f32(float x) {
