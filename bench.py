@@ -55,6 +55,10 @@ def parse():
                     help="instead of the single-layer step: greedy decoding on a random-init decoder of Qwen3-8B shape "
                          "through the compressed cache (configs[3]: --e2e --batch 32 --ctx 8192 --steps 256); --e2e-layers "
                          "and --e2e-dense-steps scale it; prints its own JSON line")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the single-layer step: the repack + bit-pack sweep of configs[2] (--sweep --hkv 8 "
+                         "--ctx 16384): compression ratios over pack sizes 16..256, code widths 2..8 bits and the three "
+                         "repacking methods, and the block codec's encode / decode rates per width; prints its own JSON line")
     ap.add_argument("--e2e-layers", type=int, default=36)
     ap.add_argument("--e2e-dense-steps", type=int, default=4,
                     help="steps of the decompress-then-attend path timed beside the fused one (on a copy of the run)")
@@ -248,6 +252,61 @@ def e2e_decode(torch, args, dev):
     print(json.dumps(result))
 
 
+SWEEP_RELS = (0.5, 0.2, 0.1, 0.05, 0.025, 0.0125, 0.00625)      # code widths 2, 3, 4, 5, 6, 7, 8 bits
+SWEEP_PACKS = (16, 32, 64, 128, 256)
+
+
+def pack_sweep(torch, H, T, dev, rels=SWEEP_RELS, packs=SWEEP_PACKS, time_codec=True, kv=None):
+    """configs[2]: one layer of H KV heads x 128 x T tokens, K with a per-channel scale drawn log-uniform in
+    [0.1, 10], V ~ N(0, 1).  For every error bound (one per code width) the tensors are quantised once; every
+    (pack size, repacking method) is then priced with the reference's size model (`repack_and_encode`,
+    utils/compute.py:329-357: integers, so the ratios are the reference's wherever its token order is defined),
+    and the real block codec (16-token packs) is timed on the same codes."""
+    from packkv_amd import ops, synth
+    hid = H * 128
+    k, v = kv if kv is not None else synth.make_kv(1, H, T, seed=2, device=dev, k_mode="channel_scale")
+    fp16 = T * hid * 2
+    rows, codec = [], []
+    for rel in rels:
+        bits = ops.bits_for_rel(rel)
+        mats = []
+        for x in (k, v):
+            scale, zero = ops.quant_params(x, rel)
+            mats.append(ops.quantize(x, scale, zero)[0])
+        kc, vc = mats
+        for pack in packs:
+            for method in ("none", "median", "greedy"):
+                bs = max(64, pack)
+                if method == "greedy" and bs > 256:
+                    continue
+                k_pre, v_pre, k_aft, v_aft = ops.repack_and_encode(kc, vc, pack, method, bs)
+                rows.append({"rel": rel, "bits": bits, "pack": pack, "method": method, "block": bs,
+                             "k_bytes": k_aft, "v_bytes": v_aft, "k_cr": fp16 / k_aft, "v_cr": fp16 / v_aft})
+        if time_codec:
+            stream = torch.empty(2 * T * hid + 4096, dtype=torch.uint8, device=dev)
+            ik = torch.empty((T // 64) * H, 2, dtype=torch.uint32, device=dev)
+            iv = torch.empty((T // 128) * H * 2, 2, dtype=torch.uint32, device=dev)
+            back = torch.empty_like(kc)
+            k_size = ops.k_encode(kc, stream, ik, 64, 128, bits)
+            ke = event_time_ms(torch, lambda: ops.k_encode(kc, stream, ik, 64, 128, bits, want_size=False), 10)
+            kd = event_time_ms(torch, lambda: ops.k_decode(stream, ik, back, 64, 128, bits), 10)
+            assert torch.equal(back, kc)
+            v_size = ops.v_encode(vc, stream, iv, 128, 64, bits)
+            ve = event_time_ms(torch, lambda: ops.v_encode(vc, stream, iv, 128, 64, bits, want_size=False), 10)
+            vd = event_time_ms(torch, lambda: ops.v_decode(stream, iv, back, 128, 64, bits), 10)
+            assert torch.equal(back, vc)
+            gbs = lambda ms: T * hid / (ms * 1e-3) / 1e9
+            codec.append({"rel": rel, "bits": bits, "k_stream_bytes": k_size, "v_stream_bytes": v_size,
+                          "k_cr": fp16 / k_size, "v_cr": fp16 / v_size,
+                          "k_encode_gbs_codes": gbs(ke), "v_encode_gbs_codes": gbs(ve),
+                          "k_decode_gbs_codes": gbs(kd), "v_decode_gbs_codes": gbs(vd)})
+    return {"metric": "repack + bit-pack sweep", "n_gpus": 1, "data": "synthetic", "dtype": "u8",
+            "config": {"workload": "configs[2]: %d KV heads x 128 x %d tokens, K per-channel scale log-uniform in "
+                                   "[0.1, 10], V ~ N(0, 1); sizes by the reference's size model (payload + pack "
+                                   "metadata, no quantiser parameters), ratios against fp16" % (H, T)},
+            "rows": rows, "codec_16_token_packs": codec}
+
+
 def gemv_surface(torch, ops, synth, dev):
     """The reference's own GPU ops at the shape its throughput script runs (one sequence of Llama-3.1-8B shape:
     8 KV heads, 65536 cached tokens, K at rel 0.1 = 4-bit codes, V at rel 0.2 = 3-bit codes) and by its definition:
@@ -306,6 +365,9 @@ def main():
         return
     if args.e2e:
         e2e_decode(torch, args, dev)
+        return
+    if args.sweep:
+        print(json.dumps(pack_sweep(torch, args.hkv, args.ctx, dev)))
         return
     B, Hq, Hkv, T, Tw = args.batch, args.hq, args.hkv, args.ctx, args.window
     Tc = T - Tw

@@ -20,5 +20,5 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_help_lists_the_other_workloads():
     r = _run("--help")
     assert r.returncode == 0
-    for flag in ("--layers", "--e2e", "--rel", "--window", "--no-cpu", "--preheat-ms"):
+    for flag in ("--layers", "--e2e", "--sweep", "--rel", "--window", "--no-cpu", "--preheat-ms"):
         assert flag in r.stdout
