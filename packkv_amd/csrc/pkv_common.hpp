@@ -127,27 +127,27 @@ __device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int
     return nbits >= 8 ? v : v & ((1u << (4 * nbits)) - 1u);
 }
 
-// Copy `nbytes` from global `src` (any alignment) into LDS `dst` (4-byte aligned) so that
-// dst[(src & 3) + i] == src[i]; touches only the aligned dwords that overlap the range.
-// Returns the phase (src & 3).
+// Copy `nbytes` from global `src` (any alignment) into LDS `dst` (16-byte aligned, room for nbytes + 30) so that
+// dst[(src & 15) + i] == src[i]; touches only the aligned 16-byte chunks that overlap the range (a chunk never
+// straddles a page, so the bytes around the range that come along are always mapped).  Returns the phase (src & 15).
 __device__ __forceinline__ uint32_t stage_to_lds(const uint8_t *src, uint32_t nbytes, uint8_t *dst,
                                                  int tid, int nthreads) {
-    const uint32_t phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 3u);
-    const uint32_t *s4 = reinterpret_cast<const uint32_t *>(src - phase);
-    uint32_t *d4 = reinterpret_cast<uint32_t *>(dst);
-    const uint32_t ndw = (phase + nbytes + 3u) >> 2;
+    const uint32_t phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
+    const uint4 *s16 = reinterpret_cast<const uint4 *>(src - phase);
+    uint4 *d16 = reinterpret_cast<uint4 *>(dst);
+    const uint32_t n16 = (phase + nbytes + 15u) >> 4;
     // four loads in flight per thread before the first LDS store: the copy is latency-bound otherwise
-    for (uint32_t i = tid; i < ndw; i += 4u * (uint32_t)nthreads) {
-        uint32_t v[4];
+    for (uint32_t i = tid; i < n16; i += 4u * (uint32_t)nthreads) {
+        uint4 v[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const uint32_t idx = i + (uint32_t)u * (uint32_t)nthreads;
-            v[u] = idx < ndw ? s4[idx] : 0u;
+            v[u] = idx < n16 ? s16[idx] : make_uint4(0u, 0u, 0u, 0u);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const uint32_t idx = i + (uint32_t)u * (uint32_t)nthreads;
-            if (idx < ndw) d4[idx] = v[u];
+            if (idx < n16) d16[idx] = v[u];
         }
     }
     return phase;
