@@ -127,7 +127,7 @@ __global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restri
                        nunits, W);
 }
 
-// ---- the same encode, eight blocks per workgroup (blocks of four units, widths 2..4) ------------------------
+// ---- the same encode, eight blocks per workgroup (blocks of four units) ----------------------------------------
 // With one ticket per block a launch has tens of thousands of status words in flight and a block's look-back walks
 // far before it meets an inclusive prefix: the per-block kernel spends most of its time there (vector ALUs 24 %
 // busy).  Here a workgroup of 256 threads takes eight consecutive blocks of the stream -- two at a time: load the
@@ -180,9 +180,15 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
         }
         __syncthreads();
         UnitPacks u;
+        const bool wide = W > 4;                          // uniform: the field-by-field code of the extension widths
         if (active) {
-            unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
-            if (t == 0) unit_bytes[jl][unit] = meta + u.payload;
+            if (wide) {
+                const uint32_t usz = unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, nullptr, 0u);
+                if (t == 0) unit_bytes[jl][unit] = usz;
+            } else {
+                unit_analyse<IS_K>(tile, hid_blk, unit, t, u);
+                if (t == 0) unit_bytes[jl][unit] = meta + u.payload;
+            }
         }
         __syncthreads();
         if (tid == 0) {                                   // block sizes of this pair -> offsets inside the group
@@ -197,7 +203,8 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
 #pragma unroll
             for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
             if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
-            unit_emit(blk, base, t, g, u);
+            if (wide) unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, blk, base);
+            else unit_emit(blk, base, t, g, u);
         }
         __syncthreads();
     }
@@ -345,8 +352,9 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
     int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
     if (rc) return rc;
     ScanState *st = nullptr;
-    // blocks of four units at the reference's widths, 16-byte aligned rows: eight blocks per workgroup
-    const bool grouped = cs.nunits == 4 && bits <= 4 && hid_blk % 16 == 0 && hidden_dim % 16 == 0 &&
+    // blocks of four units, 16-byte aligned rows: eight blocks per workgroup (not at 8 bits, where the group's 88 KB
+    // of LDS leave one workgroup per CU and the per-block kernel is 10 % faster)
+    const bool grouped = cs.nunits == 4 && bits <= 7 && hid_blk % 16 == 0 && hidden_dim % 16 == 0 &&
                          (reinterpret_cast<uintptr_t>(codes) & 15u) == 0;
     if (grouped) {
         const uint32_t ngroups = ((uint32_t)cs.nblocks + kPackGroup - 1) / kPackGroup;
