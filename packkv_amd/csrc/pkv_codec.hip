@@ -135,7 +135,7 @@ __global__ void pack_kernel(const uint8_t *__restrict__ codes, uint8_t *__restri
 // all of them and writes their bytes, contiguous in the stream, in one sweep of aligned 16-byte stores.
 constexpr int kPackGroup = 8;
 
-template <bool IS_K>
+template <bool IS_K, bool WIDE>
 __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                          uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
                                                          int hidden_dim, int ctx_blk, int hid_blk, int W, uint32_t nblocks,
@@ -180,9 +180,9 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
         }
         __syncthreads();
         UnitPacks u;
-        const bool wide = W > 4;                          // uniform: the field-by-field code of the extension widths
+        constexpr bool wide = WIDE;                       // the field-by-field code of the extension widths (W > 4)
         if (active) {
-            if (wide) {
+            if constexpr (wide) {
                 const uint32_t usz = unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, nullptr, 0u);
                 if (t == 0) unit_bytes[jl][unit] = usz;
             } else {
@@ -203,7 +203,7 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
 #pragma unroll
             for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
             if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
-            if (wide) unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, blk, base);
+            if constexpr (wide) unit_encode_wide<IS_K>(tile, hid_blk, unit, t, g, blk, base);
             else unit_emit(blk, base, t, g, u);
         }
         __syncthreads();
@@ -360,7 +360,8 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
         const uint32_t ngroups = ((uint32_t)cs.nblocks + kPackGroup - 1) / kPackGroup;
         const uint32_t lds = 2u * (uint32_t)(ctx_blk * hid_blk) + (uint32_t)kPackGroup * cs.blk_cap + 32u;
         if ((rc = prepare_scan_state(ngroups, &st, s))) return rc;
-        auto kern = is_k ? pack_group_kernel<true> : pack_group_kernel<false>;
+        auto kern = bits > 4 ? (is_k ? pack_group_kernel<true, true> : pack_group_kernel<false, true>)
+                             : (is_k ? pack_group_kernel<true, false> : pack_group_kernel<false, false>);
         if (lds > 48u * 1024u)
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         LaunchTimer tm(s, ms_out != nullptr);
