@@ -30,13 +30,20 @@ __global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t
     __syncthreads();
     block_decode<IS_K>(blk, phase, nunits, W, tile, hid_blk);
     __syncthreads();
-    // coalesced write-back: rows of hid_blk bytes, as dwords
+    uint8_t *base = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+    // coalesced write-back: rows of hid_blk bytes, 16 bytes per lane where rows start on 16-byte boundaries
+    if (((hid_blk | hidden_dim) & 15) == 0 && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0) {
+        const int row16 = hid_blk >> 4;
+        const uint4 *t16 = reinterpret_cast<const uint4 *>(tile);
+        for (int i = threadIdx.x; i < ctx_blk * row16; i += blockDim.x)
+            *reinterpret_cast<uint4 *>(base + (size_t)(i / row16) * hidden_dim + 16 * (i % row16)) = t16[i];
+        return;
+    }
     const int row_dw = hid_blk >> 2;
     const uint32_t *t4 = reinterpret_cast<const uint32_t *>(tile);
     // (row, column) advance by the workgroup size without a division per element
     const int step_row = (int)blockDim.x / row_dw, step_c = (int)blockDim.x % row_dw;
     int row = (int)threadIdx.x / row_dw, c = (int)threadIdx.x % row_dw;
-    uint8_t *base = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
     for (int i = threadIdx.x; i < ctx_blk * row_dw; i += blockDim.x) {
         reinterpret_cast<uint32_t *>(base + (size_t)row * hidden_dim)[c] = t4[i];
         row += step_row;
