@@ -202,6 +202,8 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
             uint32_t off = blk_off[j0] + 8u + unit_bytes[0][0] + unit_bytes[0][1] + unit_bytes[0][2] + unit_bytes[0][3];
             blk_off[j0 + 1] = off;
             if (j0 + 1 < nb) blk_off[j0 + 2] = off + 8u + unit_bytes[1][0] + unit_bytes[1][1] + unit_bytes[1][2] + unit_bytes[1][3];
+            // the group's size is known here, before its last pair is written: the successors' look-backs wait less
+            if (j0 + 2 >= nb) lookback_publish(st, gidx, blk_off[nb]);
         }
         __syncthreads();
         if (active) {
@@ -217,7 +219,7 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
     }
     const uint32_t bytes = blk_off[nb];
     if (tid < 64) {
-        const uint64_t off = lookback_offset(st, gidx, bytes);
+        const uint64_t off = lookback_offset(st, gidx, bytes, true);
         if (tid == 0) {
             s_off = off;
             if (gidx == ngroups - 1) st->total = off + bytes;
