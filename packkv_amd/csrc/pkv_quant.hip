@@ -674,6 +674,8 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
             off += 8u + unit_bytes[0][0] + unit_bytes[0][1] + unit_bytes[0][2] + unit_bytes[0][3];
             blk_off[j0 + 1] = off;
             if (j0 + 1 < nb) blk_off[j0 + 2] = off + 8u + unit_bytes[1][0] + unit_bytes[1][1] + unit_bytes[1][2] + unit_bytes[1][3];
+            // the sub-group's size is known here, before its last pair is written: the successors' look-backs wait less
+            if (j0 + 2 >= nb) lookback_publish(st, sidx, blk_off[nb]);
         }
         __syncthreads();
         if (active) {
@@ -695,7 +697,7 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     // ---- 3. one look-back for the whole sub-group, then one contiguous copy ----
     const uint32_t bytes = blk_off[nb];
     if (tid < 64) {
-        const uint64_t off = base + lookback_offset(st, sidx, bytes);
+        const uint64_t off = base + lookback_offset(st, sidx, bytes, true);
         if (tid == 0) {
             s_off = off;
             if (sidx == nsub - 1) st->total = off + bytes;
