@@ -314,9 +314,15 @@ __device__ __forceinline__ uint32_t unit_encode_wide(const uint8_t *tile, int hi
 // workgroup must call it, and the workgroup must hold at least one half-wavefront per unit
 // (blockDim.x >= 32 * nunits).  `unit_bytes` is an LDS array of >= nunits uint32.  Returns
 // the block size in bytes (uniform).  Contains __syncthreads().
+struct ScanState;
+__device__ __forceinline__ void lookback_publish(ScanState *st, uint32_t idx, uint32_t my_bytes);
+
+// With `st`, the block's size is published for the look-backs of its successors as soon as it is known, before the
+// units are written (the caller then tells lookback_offset that it is published).
 template <bool IS_K>
 __device__ __forceinline__ uint32_t block_encode(const uint8_t *tile, int hid_blk, int nunits, int W,
-                                                 uint8_t *blk, uint32_t *unit_bytes) {
+                                                 uint8_t *blk, uint32_t *unit_bytes, ScanState *st = nullptr,
+                                                 uint32_t idx = 0) {
     const UnitGeom g = unit_geom(W);
     const int t = threadIdx.x & 31;
     const int unit = threadIdx.x >> 5;
@@ -336,6 +342,7 @@ __device__ __forceinline__ uint32_t block_encode(const uint8_t *tile, int hid_bl
     __syncthreads();
     uint32_t total = hdr;
     for (int q = 0; q < nunits; q++) total += unit_bytes[q];
+    if (st && threadIdx.x == 0) lookback_publish(st, idx, total);
     if (active) {
         uint32_t base = hdr;
         for (int q = 0; q < unit; q++) base += unit_bytes[q];
@@ -449,9 +456,9 @@ __device__ __forceinline__ void block_finish(const uint8_t *tile, uint8_t *blk, 
                                              uint64_t *s_off, ScanState *st, uint32_t b, uint32_t nblocks,
                                              uint8_t *__restrict__ stream, uint64_t capacity,
                                              uint32_t *__restrict__ info, int hid_blk, int nunits, int W) {
-    const uint32_t bytes = block_encode<IS_K>(tile, hid_blk, nunits, W, blk, unit_bytes);
+    const uint32_t bytes = block_encode<IS_K>(tile, hid_blk, nunits, W, blk, unit_bytes, st, b);
     if (threadIdx.x < 64) {
-        const uint64_t off = lookback_offset(st, b, bytes);
+        const uint64_t off = lookback_offset(st, b, bytes, true);
         if (threadIdx.x == 0) {
             *s_off = off;
             info[2 * b] = (uint32_t)off;
