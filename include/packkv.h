@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PKV_ABI_VERSION 2
+#define PKV_ABI_VERSION 3
 
 #define PKV_F16 0
 #define PKV_BF16 1
@@ -214,7 +214,16 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *                     widths (k_bits, v_bits in 2..4, any mix); variant 0 also takes the extension widths 5
  *                     and 6 on either side with 4, 5 or 6 on the other.  Any other combination with an
  *                     extension width runs the plain kernel whatever `variant` says.
+ *   flags             PKV_ATTN_OUT_F32: `out` is [B, Hq, 128] fp32 instead of `dtype` (the result before its
+ *                     rounding to 16 bits).  PKV_ATTN_REF_ROUNDING (variant 1 only, otherwise PKV_ERR_INVALID):
+ *                     decompress-then-attend to the letter -- every K and V element is formed as the reference
+ *                     stores it, dtype(dtype(code + zero) * scale) (utils/compute.py:173-179), before the fp32
+ *                     dot products, instead of folding scale and zero into the scores and weights.  This is the
+ *                     checking mode: slow, and equal to the reference path up to fp32 summation order.
  */
+#define PKV_ATTN_REF_ROUNDING 1
+#define PKV_ATTN_OUT_F32 2
+
 typedef struct pkv_attn_args {
     const uint8_t *k_stream;
     const uint32_t *k_info;
@@ -231,6 +240,7 @@ typedef struct pkv_attn_args {
     float sm_scale;
     int variant;
     int par_stride, win_stride;
+    int flags;
 } pkv_attn_args;
 
 int pkv_attn_decode(const pkv_attn_args *args, float *ms_out, pkv_stream_t s);

@@ -42,16 +42,21 @@ class SimulatedCache:
     """One layer list of (dequantised prefix, 16-bit buffer) pairs; ``update`` returns what
     the reference's ``update`` returns: K and V [B, H, T, D] for decompress-then-attend."""
 
-    def __init__(self, layer_num, block_size=64, buffer_size=192, k_rel=0.1, v_rel=0.1):
+    def __init__(self, layer_num, block_size=64, buffer_size=192, k_rel=0.1, v_rel=0.1, track_exact=False):
         self.block_size, self.buffer_size = block_size, buffer_size
         self.k_rel, self.v_rel = k_rel, v_rel
+        # track_exact: also keep the quantised prefix BEFORE its rounding to 16 bits, (code + zero) * scale in fp64
+        # -- not something the reference holds; the tests use it to measure what that rounding moves
+        self.track_exact = track_exact
+        self.xk = [None] * layer_num
+        self.xv = [None] * layer_num
         self.ck = [None] * layer_num
         self.cv = [None] * layer_num
         self.bk = [None] * layer_num
         self.bv = [None] * layer_num
 
-    def _quant_error(self, done, buf, new, rel):
-        """utils/compute.py:149-181."""
+    def _quant_error(self, done, buf, new, rel, exact=None):
+        """utils/compute.py:149-181.  `exact` (a one-element list, or None) accumulates the unrounded prefix."""
         buf = _cat(buf, new)
         n_cut, _ = oq.cut_counts(0, buf.shape[2], self.block_size, self.buffer_size)
         to_compress = None
@@ -59,16 +64,29 @@ class SimulatedCache:
             to_compress, buf = buf[:, :, :n_cut], buf[:, :, n_cut:]
             codes, zero, scale = oq.quant_ints(to_compress, self.block_size, rel)
             to_compress = oq.dequant(codes, zero, scale)
+            if exact is not None:
+                x = (codes.double() + zero.double()) * scale.double()
+                exact[0] = _cat(exact[0], x.reshape(x.shape[0], x.shape[1], -1, x.shape[4]))
         return _cat(done, to_compress), buf
 
     def update(self, key_states, value_states, layer_idx, cos=None, sin=None):
         if cos is not None:
             key_states = apply_rotary_pos_emb_single(key_states, cos, sin)
+        xk = [self.xk[layer_idx]] if self.track_exact else None
+        xv = [self.xv[layer_idx]] if self.track_exact else None
         self.ck[layer_idx], self.bk[layer_idx] = self._quant_error(self.ck[layer_idx], self.bk[layer_idx],
-                                                                   key_states, self.k_rel)
+                                                                   key_states, self.k_rel, xk)
         self.cv[layer_idx], self.bv[layer_idx] = self._quant_error(self.cv[layer_idx], self.bv[layer_idx],
-                                                                   value_states, self.v_rel)
+                                                                   value_states, self.v_rel, xv)
+        if self.track_exact:
+            self.xk[layer_idx], self.xv[layer_idx] = xk[0], xv[0]
         return _cat(self.ck[layer_idx], self.bk[layer_idx]), _cat(self.cv[layer_idx], self.bv[layer_idx])
+
+    def exact(self, layer_idx):
+        """(K, V) [B, H, T, D] in fp64 with the quantised prefix unrounded (needs track_exact)."""
+        bk, bv = self.bk[layer_idx], self.bv[layer_idx]
+        return (_cat(self.xk[layer_idx], None if bk is None else bk.double()),
+                _cat(self.xv[layer_idx], None if bv is None else bv.double()))
 
     def get_seq_length(self, layer_idx=0):
         n = 0

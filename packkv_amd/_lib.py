@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libpackkv_hip.so")
 
 F16, BF16 = 0, 1
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_CAPACITY, ERR_INTERNAL = range(6)
+ATTN_REF_ROUNDING, ATTN_OUT_F32 = 1, 2
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -29,7 +30,7 @@ class AttnArgs(ctypes.Structure):
         ("q", _vp), ("out", _vp), ("k_win", _vp), ("v_win", _vp),
         ("B", _i), ("Hq", _i), ("Hkv", _i), ("T_c", _i), ("T_w", _i),
         ("k_bits", _i), ("v_bits", _i), ("dtype", _i), ("sm_scale", _f), ("variant", _i),
-        ("par_stride", _i), ("win_stride", _i),
+        ("par_stride", _i), ("win_stride", _i), ("flags", _i),
     ]
 
 

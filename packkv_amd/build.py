@@ -1,6 +1,7 @@
 """Builds libpackkv_hip.so (hand-written HIP for gfx950) in-tree with hipcc.
 
     python -m packkv_amd.build          # compile every kernel source and link
+    python -m packkv_amd.build --changed   # recompile only what is older than its sources
 
 The library has no PyTorch dependency: it is a plain C-ABI shared object (include/packkv.h)
 that takes raw device pointers and a hipStream_t.
@@ -30,8 +31,20 @@ def _hipcc():
     return "hipcc"
 
 
-def _compile(src):
+def _stale(src, obj):
+    """True when `obj` is older than the source, any header beside it or the public header."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [os.path.join(CSRC, src), os.path.join(HERE, "..", "include", "packkv.h"), os.path.abspath(__file__)]
+    deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _compile(src, only_stale=False):
     obj = os.path.join(OBJ, src.replace(".hip", ".o"))
+    if only_stale and not _stale(src, obj):
+        return obj
     cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines()
@@ -43,10 +56,12 @@ def _compile(src):
     return obj
 
 
-def build(verbose=True):
+def build(verbose=True, only_stale=False):
+    """Compile and link.  only_stale=True (``--changed`` on the command line) recompiles only the sources whose
+    object file is older than the source or a header."""
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        objs = list(ex.map(lambda src: _compile(src, only_stale), SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -57,4 +72,4 @@ def build(verbose=True):
 
 
 if __name__ == "__main__":
-    build()
+    build(only_stale="--changed" in sys.argv[1:])

@@ -174,15 +174,22 @@ class PackKVCompressedCache:
         return 0 if L is None else L.k.tokens + L.win_len
 
     # -- hot path ------------------------------------------------------------------------------------
-    def attend(self, query_states, layer_idx, sm_scale=None, out=None):
+    def attend(self, query_states, layer_idx, sm_scale=None, out=None, variant=0, ref_rounding=False, out_f32=False):
         """One decode step: query_states [B, Hq, 128] (or [B, Hq, 1, 128]) against everything cached in the
-        layer; returns [B, Hq, 128] (same rank as given)."""
+        layer; returns [B, Hq, 128] (same rank as given).  variant / ref_rounding / out_f32 select the checking
+        kernels of ops.attn_decode (not cached as a plan)."""
         L = self._layer(layer_idx)
         q = query_states
         squeeze = q.dim() == 4
         if squeeze:
             q = q[:, :, 0]
         q = q.contiguous()
+        if variant or ref_rounding or out_f32:
+            res = ops.attn_decode(q, L.k.as_dict() if L.k.tokens else None, L.v.as_dict() if L.v.tokens else None,
+                                  L.k_win if L.win_len else None, L.v_win if L.win_len else None, sm_scale=sm_scale,
+                                  out=out, variant=variant, win_len=L.win_len or None, ref_rounding=ref_rounding,
+                                  out_f32=out_f32)
+            return res.unsqueeze(2) if squeeze else res
         if out is None:
             out = torch.empty_like(q)
         plan = L.plan

@@ -56,11 +56,21 @@ struct AttnParams {
                           // writes partial nsplit + i; 0: the window has a kernel of its own (partial nparts - 1)
     uint32_t k_cap, v_cap, blk_stride;
     uint32_t k_bytes, v_bytes;   // valid bytes of the streams
+    int out_f32;          // `out` holds fp32 instead of the 16-bit storage type
+    int direct_out;       // a single partial and a 16-bit result: the async-copy kernel writes `out` itself
 };
+
+// x rounded to the 16-bit storage type (nearest even), as fp32.
+__device__ __forceinline__ float round16(float x, int dtype) {
+    const uint32_t u = a_st16(x, dtype);
+    return dtype == PKV_F16 ? __half2float(__ushort_as_half((unsigned short)u)) : __uint_as_float(u << 16);
+}
 
 // ---- variant 1: decode tiles into LDS, then plain VALU attention --------------------------
 // Straightforward and easy to audit; kept as the cross-check for the tuned kernel.
-template <int G>
+// REF: decompress-then-attend to the letter -- every element is formed as the reference stores it,
+// T(T(code + zero) * scale) (utils/compute.py:178), and the dot products run on those values.
+template <int G, bool REF>
 __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t *ktile = lds;                                   // [128 tok][128 ch]
@@ -145,11 +155,18 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
             float dot[G];
 #pragma unroll
             for (int g = 0; g < G; g++) dot[g] = 0.f;
+            const float s_tok = ks[tok], z_tok = kz[tok];
 #pragma unroll 4
             for (int i = 0; i < 16; i++) {
                 const uint32_t w = row[i];
-                const float c0 = (float)(w & 0xFFu), c1 = (float)((w >> 8) & 0xFFu),
-                            c2 = (float)((w >> 16) & 0xFFu), c3 = (float)(w >> 24);
+                float c0 = (float)(w & 0xFFu), c1 = (float)((w >> 8) & 0xFFu),
+                      c2 = (float)((w >> 16) & 0xFFu), c3 = (float)(w >> 24);
+                if (REF) {
+                    c0 = round16(round16(c0 + z_tok, p.dtype) * s_tok, p.dtype);
+                    c1 = round16(round16(c1 + z_tok, p.dtype) * s_tok, p.dtype);
+                    c2 = round16(round16(c2 + z_tok, p.dtype) * s_tok, p.dtype);
+                    c3 = round16(round16(c3 + z_tok, p.dtype) * s_tok, p.dtype);
+                }
 #pragma unroll
                 for (int g = 0; g < G; g++) {
                     const float *qq = qf + g * kHeadDim + half * 64 + 4 * i;
@@ -159,7 +176,7 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 const float d = dot[g] + __shfl_xor(dot[g], 1, 64);
-                if (half == 0) S[g * kTile + tok] = p.sm_scale * ks[tok] * (d + kz[tok] * qsum[g]);
+                if (half == 0) S[g * kTile + tok] = REF ? d * p.sm_scale : p.sm_scale * s_tok * (d + z_tok * qsum[g]);
             }
         }
         __syncthreads();
@@ -173,11 +190,11 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
             const float m_old = st_m[g];
             const float m_new = fmaxf(m_old, mx);
             const float p0 = __expf(s0 - m_new), p1 = __expf(s1 - m_new);
-            const float w0 = p0 * vs[lane], w1 = p1 * vs[64 + lane];
+            const float w0 = REF ? p0 : p0 * vs[lane], w1 = REF ? p1 : p1 * vs[64 + lane];
             P[g * kTile + lane] = w0;
             P[g * kTile + 64 + lane] = w1;
             float sum = p0 + p1;
-            float zs = w0 * vz[lane] + w1 * vz[64 + lane];
+            float zs = REF ? 0.f : w0 * vz[lane] + w1 * vz[64 + lane];
 #pragma unroll
             for (int d = 32; d >= 1; d >>= 1) {
                 sum += __shfl_xor(sum, d, 64);
@@ -200,7 +217,8 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
             for (int g = 0; g < G; g++) part[g] = 0.f;
 #pragma unroll 8
             for (int t = 0; t < 64; t++) {
-                const float c = (float)vtile[(half * 64 + t) * kHeadDim + ch];
+                float c = (float)vtile[(half * 64 + t) * kHeadDim + ch];
+                if (REF) c = round16(round16(c + vz[half * 64 + t], p.dtype) * vs[half * 64 + t], p.dtype);
 #pragma unroll
                 for (int g = 0; g < G; g++) part[g] += P[g * kTile + half * 64 + t] * c;
             }
@@ -405,7 +423,7 @@ __global__ void __launch_bounds__(256) attn_window_kernel(const AttnParams p) {
 // Partials are read in parallel: thread <-> partial for the maxima and weights, then thread <-> (parity of the
 // partial, channel) for the weighted sum, four rows in flight.
 __global__ void __launch_bounds__(256) attn_merge_kernel(const float *__restrict__ part, uint16_t *__restrict__ out,
-                                                         int Hq, int nparts, int dtype) {
+                                                         int Hq, int nparts, int dtype, int out_f32) {
     extern __shared__ float w_s[];                   // weight of every partial
     __shared__ float red[8];
     __shared__ __attribute__((aligned(8))) float part_num[3 * kHeadDim];
@@ -458,8 +476,12 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float *__restrict
     if (wave == 0) {
 #pragma unroll
         for (int w = 0; w < 3; w++) num += reinterpret_cast<const float2v *>(part_num + w * kHeadDim)[lane];
-        const uint32_t lo = a_st16(num[0] / den, dtype), hi = a_st16(num[1] / den, dtype);
-        reinterpret_cast<uint32_t *>(out + hq * kHeadDim)[lane] = lo | (hi << 16);
+        if (out_f32) {
+            reinterpret_cast<float2v *>(reinterpret_cast<float *>(out) + hq * kHeadDim)[lane] = num / den;
+        } else {
+            const uint32_t lo = a_st16(num[0] / den, dtype), hi = a_st16(num[1] / den, dtype);
+            reinterpret_cast<uint32_t *>(out + hq * kHeadDim)[lane] = lo | (hi << 16);
+        }
     }
 }
 
@@ -535,7 +557,7 @@ static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
 }
 
 template <int G>
-static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_t *out, hipStream_t s) {
+static int launch_attn(const AttnParams &p, int variant, bool aligned16, bool ref_rounding, uint16_t *out, hipStream_t s) {
     PKV_REQUIRE(variant >= 0 && variant <= 2, PKV_ERR_INVALID, "variant must be 0, 1 or 2");
     // variant 0: asynchronous-copy kernel (needs 16-byte aligned streams; otherwise, and as
     // variant 2, the kernel that gathers straight from global memory); variant 1: plain VALU kernel
@@ -549,9 +571,13 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_
         const uint32_t lds_bytes = 2u * kTile * kHeadDim + 4u * p.blk_stride +
                                    (uint32_t)sizeof(float) * (G * kHeadDim + 2 * G * kTile + 4 * kTile + 5 * G);
         const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
-        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_tiles_kernel<G>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attn_tiles_kernel<G><<<grid, 256, lds_bytes, s>>>(p);
+        const void *fn = ref_rounding ? reinterpret_cast<const void *>(attn_tiles_kernel<G, true>)
+                                      : reinterpret_cast<const void *>(attn_tiles_kernel<G, false>);
+        PKV_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        if (ref_rounding)
+            attn_tiles_kernel<G, true><<<grid, 256, lds_bytes, s>>>(p);
+        else
+            attn_tiles_kernel<G, false><<<grid, 256, lds_bytes, s>>>(p);
         PKV_HIP_CHECK(hipGetLastError());
     }
     if (p.T_w > 0 && p.win_piece == 0) {
@@ -562,9 +588,9 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, uint16_
         PKV_HIP_CHECK(hipGetLastError());
     }
     const bool dma_path = p.T_c > 0 && variant == 0 && aligned16;
-    if (!(dma_path && p.nparts == 1)) {      // a single partial is the result: the async-copy kernel wrote it out itself
+    if (!(dma_path && p.direct_out)) {       // a single partial is the result: the async-copy kernel wrote it out itself
         attn_merge_kernel<<<dim3((unsigned)p.Hq, (unsigned)p.B), 256, (size_t)p.nparts * sizeof(float), s>>>(
-            p.part, out, p.Hq, p.nparts, p.dtype);
+            p.part, out, p.Hq, p.nparts, p.dtype, p.out_f32);
         PKV_HIP_CHECK(hipGetLastError());
     }
     return PKV_OK;
@@ -584,6 +610,10 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     PKV_REQUIRE(a->T_c % kTile == 0, PKV_ERR_INVALID, "compressed length must be a multiple of 128 tokens");
     PKV_REQUIRE(a->T_w <= 2048, PKV_ERR_UNSUPPORTED, "tail window longer than 2048 tokens");
     PKV_REQUIRE(a->q && a->out, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE((a->flags & ~(PKV_ATTN_REF_ROUNDING | PKV_ATTN_OUT_F32)) == 0, PKV_ERR_INVALID, "unknown flag bits");
+    const bool ref_rounding = (a->flags & PKV_ATTN_REF_ROUNDING) != 0;
+    PKV_REQUIRE(!ref_rounding || a->variant == 1, PKV_ERR_INVALID,
+                "PKV_ATTN_REF_ROUNDING is a mode of the plain kernel (variant 1)");
     if (a->T_c > 0) {
         PKV_REQUIRE(a->k_stream && a->k_info && a->v_stream && a->v_info && a->k_scale && a->k_zero &&
                         a->v_scale && a->v_zero,
@@ -655,15 +685,17 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     if (rc) return rc;
     p.part = (float *)scratch;
     p.out = (uint16_t *)a->out;
+    p.out_f32 = (a->flags & PKV_ATTN_OUT_F32) ? 1 : 0;
+    p.direct_out = p.nparts == 1 && !p.out_f32;
 
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     const int variant = narrow || (wide_fast && aligned16) ? a->variant : 1;
     switch (G) {
-        case 1: rc = launch_attn<1>(p, variant, aligned16, (uint16_t *)a->out, s); break;
-        case 2: rc = launch_attn<2>(p, variant, aligned16, (uint16_t *)a->out, s); break;
-        case 4: rc = launch_attn<4>(p, variant, aligned16, (uint16_t *)a->out, s); break;
-        default: rc = launch_attn<8>(p, variant, aligned16, (uint16_t *)a->out, s); break;
+        case 1: rc = launch_attn<1>(p, variant, aligned16, ref_rounding, (uint16_t *)a->out, s); break;
+        case 2: rc = launch_attn<2>(p, variant, aligned16, ref_rounding, (uint16_t *)a->out, s); break;
+        case 4: rc = launch_attn<4>(p, variant, aligned16, ref_rounding, (uint16_t *)a->out, s); break;
+        default: rc = launch_attn<8>(p, variant, aligned16, ref_rounding, (uint16_t *)a->out, s); break;
     }
     if (rc) return rc;
     return tm.end(ms_out);

@@ -638,7 +638,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
             const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
             const float val = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
-            if (p.nparts == 1) {               // one split and no window: this is the result, no merge launch follows
+            if (p.direct_out) {                // one split and no window: this is the result, no merge launch follows
                 p.out[hq * kHeadDim + ch] = a_st16(val / st_l[g], p.dtype);
                 continue;
             }

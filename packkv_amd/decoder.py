@@ -94,7 +94,8 @@ class ShapedDecoder:
     @torch.no_grad()
     def forward(self, ids, cache, attention="fused", taps=None):
         """ids [B, n] continue the sequences held in `cache`; returns the logits of the last position [B, vocab]
-        (fp32).  `taps`, a list, receives every layer's attention output [B, Hq, n, 128] when given."""
+        (fp32).  `taps`, a list, receives every layer's (rotated query, attention output), both [B, Hq, n, 128],
+        when given."""
         s = self.shape
         B, n = ids.shape
         pos0 = cache.get_seq_length(0)
@@ -118,7 +119,7 @@ class ShapedDecoder:
                 kd, vd = cache.update(k, v, li, kw, return_dense=True)
                 a = self._dense_attention(q, kd, vd, scaling)
             if taps is not None:
-                taps.append(a)
+                taps.append((q, a))
             h = h + F.linear(a.transpose(1, 2).reshape(B, n, s.q_heads * s.head_dim), blk["o"])
             x = _rms(h, blk["post_norm"], s.rms_eps)
             h = h + F.linear(F.silu(F.linear(x, blk["gate"])) * F.linear(x, blk["up"]), blk["down"])

@@ -600,7 +600,8 @@ class AttnPlan:
     tensors (same shape and dtype).  The tensors given at construction must stay alive and in place; build a new
     plan when a buffer is reallocated or the token counts change."""
 
-    def __init__(self, q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, win_len=None):
+    def __init__(self, q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, win_len=None,
+                 ref_rounding=False, out_f32=False):
         _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
                  "q must be a contiguous device tensor [B, Hq, 128]")
         B, Hq, _ = q.shape
@@ -644,15 +645,19 @@ class AttnPlan:
             Hkv = k_win.size(1)
             a.k_win, a.v_win = _ptr(k_win), _ptr(v_win)
         _require(Hkv is not None, "empty cache")
+        out_dtype = torch.float32 if out_f32 else q.dtype
         if out is None:
-            out = torch.empty_like(q)
+            out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+        _require(out.is_cuda and out.shape == q.shape and out.dtype == out_dtype and out.is_contiguous(),
+                 "out must be a contiguous device tensor of q's shape (fp32 with out_f32, else q's dtype)")
+        a.flags = (_lib.ATTN_REF_ROUNDING if ref_rounding else 0) | (_lib.ATTN_OUT_F32 if out_f32 else 0)
         a.q, a.out = _ptr(q), _ptr(out)
         a.B, a.Hq, a.Hkv, a.T_c, a.T_w = B, Hq, Hkv, T_c, T_w
         a.dtype = _dtype_code(q)
         a.sm_scale = float(sm_scale if sm_scale is not None else 128 ** -0.5)
         a.variant = int(variant)
         self.args, self.out, self.device = a, out, q.device
-        self._shape, self._dtype = q.shape, q.dtype
+        self._shape, self._dtype, self._out_dtype = q.shape, q.dtype, out_dtype
         self._keep = (q, k, v, k_win, v_win, out)          # the buffers the pointers refer to
         self._fn = _lib.load().pkv_attn_decode
         self._ref = ctypes.byref(a)
@@ -668,7 +673,7 @@ class AttnPlan:
                      "q must match the plan's query tensor")
             a.q = _ptr(q)
         if out is not None:
-            _require(out.is_cuda and out.shape == self._shape and out.dtype == self._dtype and out.is_contiguous(),
+            _require(out.is_cuda and out.shape == self._shape and out.dtype == self._out_dtype and out.is_contiguous(),
                      "out must match the plan's output tensor")
             a.out = _ptr(out)
             self.out = out
@@ -680,7 +685,8 @@ class AttnPlan:
         return (self.out, float(ms.value)) if timed else self.out
 
 
-def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False, win_len=None):
+def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False, win_len=None,
+                ref_rounding=False, out_f32=False):
     """One decode step over a compressed cache.
 
     q [B, Hq, 128]; k and v are the dicts returned by k_quant_encode / v_quant_encode (stream,
@@ -690,5 +696,9 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
     Buffers allocated for a cache that grows: the dicts may carry ``tokens`` (compressed tokens in use;
     scale / zero rows and block_info are then longer than that) and ``heads`` (KV heads); ``win_len``
     gives the window rows in use when k_win / v_win are allocated longer.  AttnPlan keeps the checked
-    arguments for callers that repeat the step."""
-    return AttnPlan(q, k, v, k_win, v_win, sm_scale, out, variant, win_len)(timed=timed)
+    arguments for callers that repeat the step.
+
+    out_f32: the result as fp32, before its rounding to q's dtype.  ref_rounding (variant 1 only): the checking
+    mode -- every K and V element is formed as the reference stores it, dtype(dtype(code + zero) * scale)
+    (utils/compute.py:173-179), before the fp32 dot products."""
+    return AttnPlan(q, k, v, k_win, v_win, sm_scale, out, variant, win_len, ref_rounding, out_f32)(timed=timed)

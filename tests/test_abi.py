@@ -27,7 +27,7 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_version_bounds_and_error_text():
     lib = _lib.load()
-    assert lib.pkv_abi_version() == 2
+    assert lib.pkv_abi_version() == 3
     assert lib.pkv_block_bound(1, 64, 128, 4) == 4552      # 8 + 4*112 + 512*8
     assert lib.pkv_block_bound(0, 128, 64, 3) == 3400      # 8 + 4*80 + 512*6
     # argument validation happens before any GPU call: a bad width is reported, not crashed on

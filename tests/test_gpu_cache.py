@@ -9,20 +9,24 @@ from oracle import cache as oc
 from oracle import quant as oq
 from packkv_amd import ops, synth
 from packkv_amd.cache import PackKVCacheConfig, PackKVCompressedCache
+from attn_bounds import check_fast, check_reference_mode, say as _say
 
 pytestmark = pytest.mark.gpu
 
-ABS_TOL = 2e-3     # contract for fp16: |err| <= 2e-3 + 1e-3 |ref| against decompress-then-attend
-REL_TOL = 1e-3
-# A few hundred tokens with x10 outlier channels make a peaky softmax: the reference path's own rounding of the
-# dequantised K to 16 bits (logits move by ~1e-3 in fp16, ~8e-3 in bf16) then shows undamped in the output, while
-# the fused kernel keeps (code + zero) * scale in fp32.  Same widened absolute term as the short cases of
-# tests/test_gpu_attn.py.
-SHORT_ABS_TOL = {torch.float16: 8e-3, torch.bfloat16: 6e-2}
 
-
-def _say(*a):
-    print(*a, flush=True)
+def _attend_parity(cache, layer, q, wk, wv, ek, ev, dtype, cuda, label):
+    """cache.attend in the checking mode against the reference path at the contract, and the fast decode step
+    against exact arithmetic / the reference path within the bound the oracle gives (tests/attn_bounds.py).
+    wk, wv: what the reference's update returns; ek, ev: the same tokens before their rounding to 16 bits (fp64).
+    Only the tokens already in the streams are attended unrounded: a pending 64-token cut sits in the 16-bit window
+    in dequantised form, like the buffer."""
+    n = cache.layers[layer].k.tokens
+    ek, ev = torch.cat([ek[:, :, :n], wk[:, :, n:].double()], dim=2), torch.cat([ev[:, :, :n], wv[:, :, n:].double()], dim=2)
+    ref = oq.attention_f32(q.unsqueeze(2), wk, wv).squeeze(2)
+    exact = oq.attention_f64_np(q.unsqueeze(2), ek, ev).squeeze(2)
+    chk = cache.attend(q.to(cuda), layer, variant=1, ref_rounding=True, out_f32=True)
+    check_reference_mode(chk, ref, label)
+    check_fast(cache.attend(q.to(cuda), layer), ref, exact, dtype, label=label)
 
 
 def _rope_tables(B, pos0, n, dtype):
@@ -38,7 +42,7 @@ def _rope_tables(B, pos0, n, dtype):
 def test_cache_matches_restated_reference(cuda, dtype, rope):
     B, Hq, H, T0, steps = 2, 8, 4, 300, 200
     k, v = synth.make_kv(B, H, T0 + steps, seed=90, dtype=dtype)
-    want = oc.SimulatedCache(1, 64, 192, 0.1, 0.1)
+    want = oc.SimulatedCache(1, 64, 192, 0.1, 0.1, track_exact=True)
     got = PackKVCompressedCache(B, H, 128, 1, PackKVCacheConfig(64, 192, 0.1, 0.1), max_tokens=1024, dtype=dtype,
                                 device=cuda)
     check_at = {0, 1, 18, 19, 20, 82, 83, 84, 146, 147, 148, 199}   # around the cuts at steps 19, 83, 147
@@ -62,12 +66,8 @@ def test_cache_matches_restated_reference(cuda, dtype, rope):
             assert torch.equal(gk.cpu().view(torch.int16), wk.view(torch.int16))
             assert torch.equal(gv.cpu().view(torch.int16), wv.view(torch.int16))
             q = synth.make_q(B, Hq, seed=300 + step, dtype=dtype)
-            ref = oq.attention_f32(q.unsqueeze(2), wk, wv).squeeze(2).double().numpy()
-            out = got.attend(q.to(cuda), 0).double().cpu().numpy()
-            kk = 8.0 if dtype == torch.bfloat16 else 1.0     # bf16 keeps 3 fewer mantissa bits
-            err = np.abs(out - ref)
-            _say("   max|err| = %.3e" % err.max())
-            assert (err <= SHORT_ABS_TOL[dtype] + kk * REL_TOL * np.abs(ref)).all()
+            ek, ev = want.exact(0)
+            _attend_parity(got, 0, q, wk, wv, ek, ev, dtype, cuda, "step %d" % step)
     L = got.layers[0]
     # 500 tokens: 320 have been cut (128 at the prefill, then at steps 19, 83, 147) = 2 tiles + one pending cut
     assert L.k.tokens == L.v.tokens == 256 and L.pend == 64 and L.win_len == T0 + steps - 256
@@ -125,11 +125,19 @@ def test_cache_bytes_and_prefill_only(cuda):
     assert c.cache_bytes(1) < 0.45 * fp16_bytes
     q = synth.make_q(B, 32, seed=98, device=cuda)
     gk, gv = c.materialize(1)
-    ref = oq.attention_f32(q.cpu().unsqueeze(2), gk.cpu(), gv.cpu()).squeeze(2).double().numpy()
+    ref = oq.attention_f32(q.cpu().unsqueeze(2), gk.cpu(), gv.cpu()).squeeze(2)
     out = c.attend(q.unsqueeze(2), 1)
     assert out.shape == (B, 32, 1, 128)
-    err = np.abs(out[:, :, 0].double().cpu().numpy() - ref)
-    assert (err <= SHORT_ABS_TOL[torch.float16] + REL_TOL * np.abs(ref)).all()
+    # the reference path on the dense view: the checking mode at the contract; the fast step within the bound the
+    # oracle gives (exact arithmetic = the restated quantiser's unrounded values for the 832 cut tokens)
+    sim = oc.SimulatedCache(1, 64, 192, 0.1, 0.1, track_exact=True)
+    wk, wv = sim.update(k.cpu(), v.cpu(), 0)
+    assert torch.equal(gk.cpu().view(torch.int16), wk.view(torch.int16))
+    ek, ev = sim.exact(0)
+    ek, ev = torch.cat([ek[:, :, :768], wk[:, :, 768:].double()], dim=2), torch.cat([ev[:, :, :768], wv[:, :, 768:].double()], dim=2)
+    exact = oq.attention_f64_np(q.cpu().unsqueeze(2), ek, ev).squeeze(2)
+    check_reference_mode(c.attend(q, 1, variant=1, ref_rounding=True, out_f32=True), ref, "prefill 1000")
+    check_fast(out[:, :, 0], ref, exact, torch.float16, label="prefill 1000")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -173,7 +181,7 @@ def test_cache_with_five_bit_codes(cuda):
     B, Hq, H, T0, steps = 2, 8, 4, 300, 40
     dtype = torch.float16
     k, v = synth.make_kv(B, H, T0 + steps, seed=96, dtype=dtype)
-    want = oc.SimulatedCache(1, 64, 192, 0.05, 0.05)
+    want = oc.SimulatedCache(1, 64, 192, 0.05, 0.05, track_exact=True)
     got = PackKVCompressedCache(B, H, 128, 1, PackKVCacheConfig(64, 192, 0.05, 0.05), max_tokens=1024, dtype=dtype,
                                 device=cuda)
     assert got.config.k_bits == 5 and got.config.v_bits == 5
@@ -190,9 +198,6 @@ def test_cache_with_five_bit_codes(cuda):
             assert torch.equal(gk.cpu().view(torch.int16), wk.view(torch.int16))
             assert torch.equal(gv.cpu().view(torch.int16), wv.view(torch.int16))
             q = synth.make_q(B, Hq, seed=500 + step, dtype=dtype)
-            ref = oq.attention_f32(q.unsqueeze(2), wk, wv).squeeze(2).double().numpy()
-            out = got.attend(q.to(cuda), 0).double().cpu().numpy()
-            err = np.abs(out - ref)
-            _say("   max|err| = %.3e" % err.max())
-            assert (err <= SHORT_ABS_TOL[dtype] + REL_TOL * np.abs(ref)).all()
+            ek, ev = want.exact(0)
+            _attend_parity(got, 0, q, wk, wv, ek, ev, dtype, cuda, "5-bit step %d" % step)
     assert got.layers[0].k.tokens == 128 and got.layers[0].pend == 64      # 128 at the prefill, one more cut waiting for its partner

@@ -8,6 +8,8 @@ from oracle import quant as oq
 from oracle import repack as orp
 from packkv_amd import ops, synth
 
+from attn_bounds import check_fast, check_reference_mode
+
 pytestmark = pytest.mark.gpu
 
 
@@ -206,8 +208,12 @@ def test_repacked_cache_attends_like_the_original(cuda):
     out_r = ops.attn_decode(qd, kr, vr).double().cpu().numpy()
     out_n = ops.attn_decode(qd, kn, vn).double().cpu().numpy()
     _say("repacked cache: V bytes %d -> %d, max|out_r - out_n| = %.2e" % (vn["size"], vr["size"], np.abs(out_r - out_n).max()))
-    for out in (out_r, out_n):
-        assert (np.abs(out - want) <= 8e-3 + 1e-3 * np.abs(want)).all()
+    exact = oq.attention_f64_np(q.unsqueeze(2), ((ck.double() + zk.double()) * sk.double()).reshape(k.shape),
+                                ((cv.double() + zv.double()) * sv.double()).reshape(v.shape)).squeeze(2)
+    for name, (ke_, ve_), out in (("repacked", (kr, vr), out_r), ("natural order", (kn, vn), out_n)):
+        chk = ops.attn_decode(qd, ke_, ve_, variant=1, ref_rounding=True, out_f32=True)
+        check_reference_mode(chk, want, name)          # the contract, on the checking mode
+        check_fast(out, want, exact, torch.float16, label=name)
     # the two orders add the same terms in a different sequence: at most an output rounding apart
     assert np.abs(out_r - out_n).max() <= 2 ** -10 * np.abs(out_n).max()
 
