@@ -13,6 +13,8 @@
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
 
+#include <mutex>
+
 #ifndef PKV_SPLIT_TARGET
 #define PKV_SPLIT_TARGET 1024
 #endif
@@ -598,9 +600,48 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, bool re
 
 }  // namespace pkv
 
+// ---- partials without an allocation --------------------------------------------------------------
+// pkv_attn_decode_noalloc keeps the per-split partials in this array instead of library-allocated memory.  Every
+// GPU the library runs on holds its own copy, at its own address, until the process ends.  In host code the name
+// below is only a handle for hipGetSymbolAddress: the device address it yields (per device) is what kernels get.
+#define PKV_ATTN_STATIC_SCRATCH_BYTES (8u << 20)
+static __device__ __align__(256) unsigned char scratch[PKV_ATTN_STATIC_SCRATCH_BYTES];
+
+namespace pkv {
+namespace {
+constexpr int kStaticMaxDevices = 16;
+void *g_static_part[kStaticMaxDevices];          // device address of `scratch` on each device, once looked up
+std::mutex g_static_mu;
+
+// Device address of this device's copy of `scratch` (looked up once per device, with that device current).
+int static_scratch_ptr(void **out) {
+    int dev = 0;
+    PKV_HIP_CHECK(hipGetDevice(&dev));
+    PKV_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, PKV_ERR_INVALID, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    if (!g_static_part[dev]) {
+        void *ptr = nullptr;
+        PKV_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        PKV_REQUIRE(ptr != nullptr, PKV_ERR_HIP, "hipGetSymbolAddress returned a null address");
+        g_static_part[dev] = ptr;
+    }
+    *out = g_static_part[dev];
+    return PKV_OK;
+}
+
+}  // namespace
+static int attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, bool static_partials);
+}  // namespace pkv
+
 extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream_t s_) {
-    using namespace pkv;
-    hipStream_t s = (hipStream_t)s_;
+    return pkv::attn_decode_impl(a, ms_out, (hipStream_t)s_, false);
+}
+
+extern "C" int pkv_attn_decode_noalloc(const pkv_attn_args *a, pkv_stream_t s_) {
+    return pkv::attn_decode_impl(a, nullptr, (hipStream_t)s_, true);
+}
+
+int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, bool static_partials) {
     PKV_REQUIRE(a != nullptr, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(a->dtype == PKV_F16 || a->dtype == PKV_BF16, PKV_ERR_UNSUPPORTED, "Unsupported data type");
     PKV_REQUIRE(a->B > 0 && a->Hq > 0 && a->Hkv > 0 && a->Hq % a->Hkv == 0, PKV_ERR_INVALID,
@@ -679,11 +720,20 @@ extern "C" int pkv_attn_decode(const pkv_attn_args *a, float *ms_out, pkv_stream
     const uint32_t cap = p.k_cap > p.v_cap ? p.k_cap : p.v_cap;
     p.blk_stride = ((cap + 14u + 15u) & ~15u) + 32u;
     p.k_bytes = (uint32_t)a->k_bytes; p.v_bytes = (uint32_t)a->v_bytes;   // up to 14 bytes of phase in front, slack behind
-    void *scratch = nullptr;
+    void *part = nullptr;
     const size_t part_bytes = (size_t)a->B * a->Hq * p.nparts * kPartStride * sizeof(float);
-    int rc = scratch_get(part_bytes, &scratch);
+    int rc;
+    if (static_partials) {
+        PKV_REQUIRE(part_bytes <= (size_t)PKV_ATTN_STATIC_SCRATCH_BYTES, PKV_ERR_UNSUPPORTED,
+                    "pkv_attn_decode_noalloc: %zu bytes of partials (batch %d x %d query heads x %d partials) exceed the "
+                    "%u-byte static buffer; use pkv_attn_decode", part_bytes, a->B, a->Hq, p.nparts,
+                    (unsigned)PKV_ATTN_STATIC_SCRATCH_BYTES);
+        rc = static_scratch_ptr(&part);
+    } else {
+        rc = scratch_get(part_bytes, &part);
+    }
     if (rc) return rc;
-    p.part = (float *)scratch;
+    p.part = (float *)part;
     p.out = (uint16_t *)a->out;
     p.out_f32 = (a->flags & PKV_ATTN_OUT_F32) ? 1 : 0;
     p.direct_out = p.nparts == 1 && !p.out_f32;

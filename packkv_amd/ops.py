@@ -601,7 +601,7 @@ class AttnPlan:
     plan when a buffer is reallocated or the token counts change."""
 
     def __init__(self, q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, win_len=None,
-                 ref_rounding=False, out_f32=False):
+                 ref_rounding=False, out_f32=False, noalloc=False):
         _require(q.is_cuda and q.dim() == 3 and q.size(2) == 128 and q.is_contiguous(),
                  "q must be a contiguous device tensor [B, Hq, 128]")
         B, Hq, _ = q.shape
@@ -660,6 +660,7 @@ class AttnPlan:
         self._shape, self._dtype, self._out_dtype = q.shape, q.dtype, out_dtype
         self._keep = (q, k, v, k_win, v_win, out)          # the buffers the pointers refer to
         self._fn = _lib.load().pkv_attn_decode
+        self._fn_noalloc = _lib.load().pkv_attn_decode_noalloc if noalloc else None
         self._ref = ctypes.byref(a)
 
     def set_window_rows(self, win_len):
@@ -679,14 +680,18 @@ class AttnPlan:
             self.out = out
         ms = ctypes.c_float(0.0)
         with torch.cuda.device(self.device):
-            rc = self._fn(self._ref, ctypes.byref(ms) if timed else None, _stream(self.device))
+            if self._fn_noalloc is not None:
+                _require(not timed, "the entry point that allocates nothing does not time its launch")
+                rc = self._fn_noalloc(self._ref, _stream(self.device))
+            else:
+                rc = self._fn(self._ref, ctypes.byref(ms) if timed else None, _stream(self.device))
         if rc:
             _lib.check(rc)
         return (self.out, float(ms.value)) if timed else self.out
 
 
 def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, variant=0, timed=False, win_len=None,
-                ref_rounding=False, out_f32=False):
+                ref_rounding=False, out_f32=False, noalloc=False):
     """One decode step over a compressed cache.
 
     q [B, Hq, 128]; k and v are the dicts returned by k_quant_encode / v_quant_encode (stream,
@@ -700,5 +705,6 @@ def attn_decode(q, k, v, k_win=None, v_win=None, sm_scale=None, out=None, varian
 
     out_f32: the result as fp32, before its rounding to q's dtype.  ref_rounding (variant 1 only): the checking
     mode -- every K and V element is formed as the reference stores it, dtype(dtype(code + zero) * scale)
-    (utils/compute.py:173-179), before the fp32 dot products."""
-    return AttnPlan(q, k, v, k_win, v_win, sm_scale, out, variant, win_len, ref_rounding, out_f32)(timed=timed)
+    (utils/compute.py:173-179), before the fp32 dot products.  noalloc: go through pkv_attn_decode_noalloc (the
+    partial results in the library's fixed 8 MiB device array; the caller passes `out`, or torch allocates it)."""
+    return AttnPlan(q, k, v, k_win, v_win, sm_scale, out, variant, win_len, ref_rounding, out_f32, noalloc)(timed=timed)

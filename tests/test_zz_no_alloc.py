@@ -1,0 +1,50 @@
+"""pkv_attn_decode_noalloc (partials in the library's fixed device array, no allocation) against pkv_attn_decode:
+same kernels, so the same bits -- on two calls in a row, the second with a smaller input (which leaves the first
+call's partials behind it in the shared array), and the size limit is reported."""
+import pytest
+import torch
+
+from packkv_amd import _lib, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(cuda, B, Hq, Hkv, T, Tw, seed, dtype=torch.float16):
+    k, v = synth.make_kv(B, Hkv, T + Tw, seed=seed, dtype=dtype, device=cuda)
+    q = synth.make_q(B, Hq, seed=seed + 1, dtype=dtype, device=cuda)
+    ke = ops.k_quant_encode(k[:, :, :T].contiguous(), 0.1)
+    ve = ops.v_quant_encode(v[:, :, :T].contiguous(), 0.1)
+    kw = k[:, :, T:].contiguous() if Tw else None
+    vw = v[:, :, T:].contiguous() if Tw else None
+    return q, ke, ve, kw, vw
+
+
+def test_noalloc_entry_point_matches_the_allocating_one(cuda):
+    big = _case(cuda, 4, 32, 8, 4096, 150, seed=700)
+    small = _case(cuda, 1, 8, 2, 512, 3, seed=710, dtype=torch.bfloat16)
+    want = [ops.attn_decode(*c) for c in (big, small)]
+    torch.cuda.synchronize()
+    for variant in (0, 1, 2):
+        for c, w in zip((big, small), want):
+            print("no-alloc case: variant", variant, "batch", c[0].shape[0], "tokens", c[1]["scale"].shape[1], flush=True)
+            out = torch.full_like(c[0], 7.0)
+            got = ops.attn_decode(*c, out=out, variant=variant, noalloc=True)
+            ref = ops.attn_decode(*c, variant=variant)
+            torch.cuda.synchronize()
+            assert got.data_ptr() == out.data_ptr()
+            assert torch.equal(got, ref)
+            if variant == 0:
+                assert torch.equal(got, w)
+
+
+def test_noalloc_entry_point_rejects_what_does_not_fit(cuda):
+    """8 MiB hold B * Hq * partials * 520 bytes: batch 64 x 64 query heads with a window (2 x 2 partials... ) fits, a
+    step with 64 sequences x 64 heads x 2 x 32 partials does not -- and says so instead of overrunning the array."""
+    lib = _lib.load()
+    B, Hq, Hkv, T, Tw = 64, 64, 8, 512, 4
+    q, ke, ve, kw, vw = _case(cuda, B, Hq, Hkv, T, Tw, seed=720)
+    plan = ops.AttnPlan(q, ke, ve, kw, vw, noalloc=True)     # 2 splits + 2 window pieces: 64 * 64 * 4 * 520 B = 8.1 MiB
+    with pytest.raises(ops.PackKVError) as e:
+        plan()
+    assert e.value.code == _lib.ERR_UNSUPPORTED and "static buffer" in str(e.value)
+    assert torch.equal(ops.attn_decode(q, ke, ve, kw, vw), ops.attn_decode(q, ke, ve, kw, vw))   # the allocating one takes it
