@@ -247,13 +247,15 @@ int pkv_attn_decode(const pkv_attn_args *args, float *ms_out, pkv_stream_t s);
 
 /* pkv_attn_decode_noalloc: pkv_attn_decode for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
- * arguments, kernels and results, but the per-split partial results ([B, Hq, partials, 130] fp32, which
- * pkv_attn_decode keeps in memory the library allocates and grows on demand) live in a fixed 8 MiB device array
- * inside the library; the call allocates and frees nothing and creates no events (hence no ms_out).  A step whose
- * partials do not fit 8 MiB is rejected with PKV_ERR_UNSUPPORTED and a message (B * Hq * partials * 520 bytes;
- * partials = splits, twice that with a tail window; splits ~ 1024 / (B * Hkv), at most T_c / 128).  All calls on
- * one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race; calls on one stream
- * are ordered.  Every partial a launch reads was written by that launch, so nothing needs clearing between calls. */
+ * arguments, kernels and results, but the per-split partial results ([B, Hq, partials, 130] fp32) and the tile
+ * counters, which pkv_attn_decode keeps in memory the library allocates per stream and grows on demand, live in a
+ * fixed 8 MiB device array inside the library (7.75 MiB of it for the partials); the call allocates and frees
+ * nothing and creates no events (hence no ms_out).  A step whose partials do not fit is rejected with
+ * PKV_ERR_UNSUPPORTED and a message (B * Hq * partials * 520 bytes; partials = splits, twice that with a tail
+ * window; splits ~ 1024 / (B * Hkv), at most T_c / 128).  All calls on one GPU share the one array: calls that
+ * overlap on a GPU (two streams, two threads) race; calls on one stream are ordered.  Every partial a launch reads
+ * was written by that launch and the counters are left at zero, so nothing needs clearing between calls.
+ * pkv_attn_decode itself uses the same array when its stream is capturing a graph and has no scratch of its own. */
 int pkv_attn_decode_noalloc(const pkv_attn_args *args, pkv_stream_t s);
 
 #ifdef __cplusplus

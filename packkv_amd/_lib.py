@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpackkv_hip.so")
+# PACKKV_HIP_LIB names another build of the same library (kernel development: A/B runs of two builds)
+LIB_PATH = os.environ.get("PACKKV_HIP_LIB") or os.path.join(_HERE, "libpackkv_hip.so")
 
 F16, BF16 = 0, 1
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_CAPACITY, ERR_INTERNAL = range(6)

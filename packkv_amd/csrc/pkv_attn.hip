@@ -15,6 +15,9 @@
 
 #include <mutex>
 
+#ifndef PKV_DYNAMIC_TILES
+#define PKV_DYNAMIC_TILES 1
+#endif
 #ifndef PKV_SPLIT_TARGET
 #define PKV_SPLIT_TARGET 1024
 #endif
@@ -60,6 +63,8 @@ struct AttnParams {
     uint32_t k_bytes, v_bytes;   // valid bytes of the streams
     int out_f32;          // `out` holds fp32 instead of the 16-bit storage type
     int direct_out;       // a single partial and a 16-bit result: the async-copy kernel writes `out` itself
+    int dynamic;          // async-copy kernel: the members of a (sequence, KV head) take tiles from a common counter
+    uint32_t *counters;   // [B Hkv] tile counters, then [B Hkv] counts of members that are done; zero between launches
 };
 
 // x rounded to the 16-bit storage type (nearest even), as fp32.
@@ -511,7 +516,7 @@ namespace pkv {
 template <int G, int KW, int VW>
 static int launch_dma(const AttnParams &p, hipStream_t s) {
     static_assert(dma_lds_bytes<G, KW, VW>() >= kWinPieceLds, "window pieces borrow the slots");
-    const dim3 grid((unsigned)p.nsplit, (unsigned)p.Hkv, (unsigned)p.B);
+    const dim3 grid((unsigned)p.nsplit * (unsigned)p.Hkv * (unsigned)p.B);
     if (p.dtype == PKV_BF16)
         attn_dma_kernel<G, KW, VW, true><<<grid, 256, 0, s>>>(p);
     else
@@ -520,8 +525,14 @@ static int launch_dma(const AttnParams &p, hipStream_t s) {
     return PKV_OK;
 }
 
+// PKV_ATTN_MINIMAL (kernel development only): instantiate the 4-bit kernels for groups of 4 and 1 alone; every other
+// shape is refused.  Cuts the compile of this file from minutes to seconds.
 template <int G>
 static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
+#ifdef PKV_ATTN_MINIMAL
+    if constexpr (G == 4 || G == 1) { if (p.k_bits == 4 && p.v_bits == 4) return launch_dma<G, 4, 4>(p, s); }
+    PKV_REQUIRE(false, PKV_ERR_UNSUPPORTED, "minimal build: 4-bit codes and groups of 4 only");
+#else
     switch (p.k_bits * 8 + p.v_bits) {
         case 2 * 8 + 2: return launch_dma<G, 2, 2>(p, s);
         case 2 * 8 + 3: return launch_dma<G, 2, 3>(p, s);
@@ -541,10 +552,14 @@ static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
         case 4 * 8 + 6: return launch_dma<G, 4, 6>(p, s);
         default: return launch_dma<G, 4, 4>(p, s);
     }
+#endif
 }
 
 template <int G>
 static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
+#ifdef PKV_ATTN_MINIMAL
+    PKV_REQUIRE(false, PKV_ERR_UNSUPPORTED, "minimal build: the asynchronous-copy kernel only");
+#else
     switch (p.k_bits * 8 + p.v_bits) {
         case 2 * 8 + 2: return launch_direct<G, 2, 2>(p, s);
         case 2 * 8 + 3: return launch_direct<G, 2, 3>(p, s);
@@ -556,6 +571,7 @@ static int launch_direct_bits(const AttnParams &p, hipStream_t s) {
         case 4 * 8 + 3: return launch_direct<G, 4, 3>(p, s);
         default: return launch_direct<G, 4, 4>(p, s);
     }
+#endif
 }
 
 template <int G>
@@ -606,6 +622,8 @@ static int launch_attn(const AttnParams &p, int variant, bool aligned16, bool re
 // below is only a handle for hipGetSymbolAddress: the device address it yields (per device) is what kernels get.
 #define PKV_ATTN_STATIC_SCRATCH_BYTES (8u << 20)
 static __device__ __align__(256) unsigned char scratch[PKV_ATTN_STATIC_SCRATCH_BYTES];
+// layout: partials, then the tile counters of the async-copy kernel (zero at load, left at zero by every launch)
+static constexpr size_t kStaticPartBytes = (size_t)PKV_ATTN_STATIC_SCRATCH_BYTES - (size_t)pkv::kAttnCounters * sizeof(uint32_t);
 
 namespace pkv {
 namespace {
@@ -720,23 +738,36 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     const uint32_t cap = p.k_cap > p.v_cap ? p.k_cap : p.v_cap;
     p.blk_stride = ((cap + 14u + 15u) & ~15u) + 32u;
     p.k_bytes = (uint32_t)a->k_bytes; p.v_bytes = (uint32_t)a->v_bytes;   // up to 14 bytes of phase in front, slack behind
-    void *part = nullptr;
-    const size_t part_bytes = (size_t)a->B * a->Hq * p.nparts * kPartStride * sizeof(float);
-    int rc;
-    if (static_partials) {
-        PKV_REQUIRE(part_bytes <= (size_t)PKV_ATTN_STATIC_SCRATCH_BYTES, PKV_ERR_UNSUPPORTED,
-                    "pkv_attn_decode_noalloc: %zu bytes of partials (batch %d x %d query heads x %d partials) exceed the "
-                    "%u-byte static buffer; use pkv_attn_decode", part_bytes, a->B, a->Hq, p.nparts,
-                    (unsigned)PKV_ATTN_STATIC_SCRATCH_BYTES);
-        rc = static_scratch_ptr(&part);
-    } else {
-        rc = scratch_get(part_bytes, &part);
-    }
-    if (rc) return rc;
-    p.part = (float *)part;
     p.out = (uint16_t *)a->out;
     p.out_f32 = (a->flags & PKV_ATTN_OUT_F32) ? 1 : 0;
     p.direct_out = p.nparts == 1 && !p.out_f32;
+    // The async-copy kernel balances the members of a head through two counters per head (with one member there is
+    // nothing to balance).
+    const bool dma_path = a->T_c > 0 && a->variant == 0 && aligned16 && (narrow || wide_fast);
+    p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && 2 * a->B * a->Hkv <= kAttnCounters;
+    p.counters = nullptr;
+    // Partials and counters: the stream's own scratch, or the static array -- for pkv_attn_decode_noalloc, and for a
+    // stream that is capturing a graph before it has scratch of its own.
+    void *part = nullptr, *static_part = nullptr;
+    const size_t part_bytes = (size_t)a->B * a->Hq * p.nparts * kPartStride * sizeof(float);
+    int rc = static_scratch_ptr(&static_part);     // looked up on the first call on a device, while nothing is capturing
+    if (rc) return rc;
+    bool use_static = static_partials;
+    if (!use_static) {
+        rc = scratch_get(part_bytes, s, &part);
+        if (rc == PKV_OK && p.dynamic) rc = attn_counters_get(s, &p.counters);
+        if (rc == PKV_ERR_CAPTURING && part_bytes <= kStaticPartBytes) use_static = true;
+        else if (rc) return rc == PKV_ERR_CAPTURING ? PKV_ERR_HIP : rc;
+    }
+    if (use_static) {
+        PKV_REQUIRE(part_bytes <= kStaticPartBytes, PKV_ERR_UNSUPPORTED,
+                    "pkv_attn_decode_noalloc: %zu bytes of partials (batch %d x %d query heads x %d partials) exceed the "
+                    "%zu bytes the static buffer has for them; use pkv_attn_decode", part_bytes, a->B, a->Hq, p.nparts,
+                    kStaticPartBytes);
+        part = static_part;
+        p.counters = reinterpret_cast<uint32_t *>(static_cast<unsigned char *>(part) + kStaticPartBytes);
+    }
+    p.part = (float *)part;
 
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;

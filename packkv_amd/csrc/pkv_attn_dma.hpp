@@ -41,6 +41,13 @@ template <int G> struct StagePrio<G, true> { static constexpr int K = 2, S = 1, 
 template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 0, V = 0; };
 #define PKV_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
+// PKV_ATTN_PROBE (measurement builds only, results are then meaningless): bit mask of pipeline stages to leave out
+// of the tile loop -- 1 the copies (the first two tiles are re-used), 2 the K stage, 4 the softmax, 8 the V stage,
+// 16 the parse.  30 = "loads only", 1 = "arithmetic only".
+#ifndef PKV_ATTN_PROBE
+#define PKV_ATTN_PROBE 0
+#endif
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // Raw buffer descriptor (base, stride 0, num_records = bytes, 32-bit raw format): reads past
@@ -53,12 +60,15 @@ __device__ __forceinline__ u32x4 dma_rsrc(const void *base, uint32_t bytes) {
 // One LDS-direct load: lane l's 16 (4) bytes at buffer offset voff (+ soff) land at LDS byte
 // lds_addr + 16 l (4 l).  lds_addr, rsrc and soff are wave-uniform.  M0 (the LDS base of the copy)
 // is written and consumed inside the one asm statement; nothing else in these kernels depends on M0.
+// The compiler does not see inside the statement, so it pads no hazards for it: the s_mov and the s_nop 3 are the
+// five wait states a memory instruction needs after a VALU instruction wrote one of its scalar operands (which is
+// what the compiler's restore of a spilled scalar register is).
 __device__ __forceinline__ void dma_b128(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 __device__ __forceinline__ void dma_b32(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
@@ -93,8 +103,8 @@ __device__ __forceinline__ int4v pair128(long a, long b) {
 
 // 64 bits at byte offset `off` (even) of an LDS array whose base is 4-byte aligned: the three
 // aligned dwords that cover it, funnel-shifted by bytes (a misaligned DS read stalls the LDS pipe).
-__device__ __forceinline__ uint64_t lds_word64(const uint8_t *base, uint32_t off) {
-    const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (off & ~3u));
+__device__ __forceinline__ uint64_t lds_word64(const uint8_t *base, uint32_t off) {   // base: a 4-byte aligned array; pass every
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (off & ~3u));      // variable part of the address in `off`
     const uint32_t d0 = q[0], d1 = q[1], d2 = q[2];
     const uint32_t lo = __builtin_amdgcn_alignbyte(d1, d0, off), hi = __builtin_amdgcn_alignbyte(d2, d1, off);
     return ((uint64_t)hi << 32) | lo;
@@ -211,16 +221,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     typedef typename UnitOf<KWIDE>::type KUnit;
     typedef typename UnitOf<VWIDE>::type VUnit;
     typedef StagePrio<G, WIDE> Prio;
-    constexpr int ROWS = 3 * G;
-    constexpr int NSETS = (ROWS + 15) / 16;
+    constexpr int ROWS = 4 * G;                   // MFMA row 4 g + digit (row 4 g + 3 stays zero): the three digits of a
+    constexpr int NSETS = (ROWS + 15) / 16;       // head come out in one lane
+    constexpr bool SCORE_INT = KW <= 4;           // 128 x 64 x 15 x 2^14 < 2^31: the digits combine in int32
     constexpr int NG4 = (G + 3) / 4;
     constexpr int GP = NG4 * 4;
     constexpr int GW = (G + 3) / 4;
     constexpr int KLB = len_field_bits(KW), VLB = len_field_bits(VW);
     constexpr uint32_t K_META = KW * 16 + KLB * 16, V_META = VW * 16 + VLB * 16;
     constexpr int kRoundBytes = 16 * kKtStride;
-    static_assert(16 * NSETS * 16 * 4 + 64 <= kRoundBytes, "score rows must fit the K-tile rows they reuse");
-    static_assert(NSETS * 4 * 16 * 32 <= 8 * kRoundBytes, "q digits borrow a slot");
+    static_assert(NSETS * 256 <= kRoundBytes, "score rows must fit the K-tile rows they reuse");
 
     constexpr int kPStride = kTile + 4;          // halves per head row of the weights: rows 8 bytes apart in bank space
     constexpr int kLdsBytes = dma_lds_bytes<G, KW, VW>();
@@ -233,9 +243,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     float *st_m = reinterpret_cast<float *>(p16lo + GP * 8);                 // 8 floats each
     float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8, *qsum = st_z + 8, *qs = qsum + 8;
     const uint32_t ring_lds = (uint32_t)reinterpret_cast<uintptr_t>(ring);   // LDS byte address of the slots
-    uint8_t *aq = ring;                                                      // q digits, prologue only
 
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // Workgroup L of the launch is member L / (B Hkv) of (sequence, KV head) L % (B Hkv): the members of one head are
+    // spread over the launch, so that each head has members among the workgroups a CU starts first and among those
+    // it starts last (the former run faster), and they even it out by taking tiles from a common counter.
+    const int n_heads = p.B * p.Hkv;
+    const int split = (int)blockIdx.x / n_heads, bh_ = (int)blockIdx.x % n_heads;
+    const int h = bh_ % p.Hkv, b = bh_ / p.Hkv;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int t = tid & 31, hw = tid >> 5;
@@ -247,12 +261,84 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     const uint16_t *par_arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
     const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.par_stride * 2));
 
-    // ---- prologue: split q into digits (through LDS, aliased onto the K tile) ----
+    // Tiles this member works on, by position in its own sequence.  Static split (p.dynamic == 0): the contiguous
+    // range [tile0, tile_end).  Dynamic: positions 0..4 are tiles split + k * nsplit (known at once, they fill the
+    // pipeline), every further position is 5 * nsplit + the next value of the head's counter, fetched five positions
+    // ahead; a faster member simply comes back for more.  Sequences are increasing, a tile number >= tile_end ends
+    // them, and attention does not depend on the order of the tokens.
+    const int n_tiles = p.T_c / kTile;
+    const int tile0 = split * p.tiles_per_split;
+    const int tile_end = p.dynamic ? n_tiles : min(n_tiles, tile0 + p.tiles_per_split);
+    auto first_tiles = [&](int k) -> int { return p.dynamic ? split + k * p.nsplit : tile0 + k; };
+    __shared__ int tau_lds[2];
+
+    // ---- block_info: wave-uniform scalar loads, fetched well before use ----
+    // this wave copies block `wave` of a tile and parses K block wave/2 and V block 2 + wave/2
+    // (read through the constant address space: block_info is read-only for the whole launch, and
+    // only loads known to be unclobbered are issued as scalar loads; a vector load here would make
+    // every later vmcnt wait drain the copies in flight)
+    typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
+    const int kj = wave >> 1;
+    const const_u32_ptr k_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.k_info));
+    const const_u32_ptr v_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.v_info));
+    const const_u32_ptr dma_info = wave < 2 ? k_info_c : v_info_c;
+    struct TileInfo { uint32_t dma_off, dma_size, k_off, v_off; };
+    auto load_info = [&](int tile) -> TileInfo {
+        const int tau = min(tile, n_tiles - 1);          // past the end: the last tile again, never used
+        const uint32_t ik0 = (uint32_t)((2 * tau) * n_hid_k + bh), iv0 = (uint32_t)(tau * n_hid_v + 2 * bh);
+        const uint32_t id = wave < 2 ? ik0 + (uint32_t)wave * (uint32_t)n_hid_k : iv0 + (uint32_t)(wave - 2);
+        TileInfo ti;
+        ti.dma_off = dma_info[2 * (size_t)id];
+        ti.dma_size = dma_info[2 * (size_t)id + 1];
+        ti.k_off = k_info_c[2 * (size_t)(ik0 + (uint32_t)kj * (uint32_t)n_hid_k)];
+        ti.v_off = v_info_c[2 * (size_t)(iv0 + (uint32_t)kj)];
+        return ti;
+    };
+
+    // ---- copy of one tile into slot `slot` ----
+    auto dma_issue = [&](int slot, int tile, const TileInfo &ti) {
+        const uint32_t phase = ti.dma_off & 15u;                  // the streams themselves are 16-byte aligned
+        const uint32_t src = ti.dma_off - phase;
+        uint32_t nq = (phase + ti.dma_size + 15u) >> 4;           // 16-byte quads to copy
+        nq = min(max(nq, 1u), (uint32_t)(Geo::kRegion / 16));     // corrupt block_info must not overrun the region
+        const uint32_t last = nq - 1u;
+        const uint32_t dst = ring_lds + (uint32_t)(slot * Geo::kSlot + wave * Geo::kRegion);
+#pragma unroll
+        for (int i = 0; i < Geo::kMaxInstr; i++) {
+            if ((uint32_t)(i * 64) < nq) {                        // wave-uniform
+                if (i * 1024 + 1024 <= Geo::kRegion || lane < (Geo::kRegion - i * 1024) / 16)
+                    dma_b128(blk_rsrc, dst + i * 1024, src + 16u * min((uint32_t)(i * 64 + lane), last));
+            }
+        }
+        // parameter array `wave` of the tile: 128 tokens x 2 bytes = 64 lanes x 4 bytes
+        const int tile_off = (b * p.par_stride + min(tile, n_tiles - 1) * kTile) * 2;
+        dma_b32(par_rsrc, ring_lds + (uint32_t)(slot * Geo::kSlot + Geo::kParOff + wave * 256), 4 * lane, (uint32_t)tile_off);
+    };
+
+    // tile 0 starts its way into slot 0 now, under the prologue's arithmetic
+    int t_cur = first_tiles(0), t1 = first_tiles(1), t2 = first_tiles(2), t3 = first_tiles(3);
+    TileInfo i0 = load_info(t_cur), i1 = load_info(t1), i2 = load_info(t2);
+    dma_issue(0, t_cur, i0);
+
+    auto cvt2 = [&](uint32_t w, float &lo, float &hi) {
+        if (!BF) {
+            lo = __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu)));
+            hi = __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+        } else {
+            lo = __uint_as_float(w << 16);
+            hi = __uint_as_float(w & 0xFFFF0000u);
+        }
+    };
+
+    // ---- prologue: LDS state; q split into signed 7-bit digits, staged through slot 1 (tile 0 is on its way into
+    // slot 0 meanwhile) ----
+    uint8_t *aq = ring + Geo::kSlot;
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
     for (int i = tid; i < GP * kPStride / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
     for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
     if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 1.f; }
-    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0xC07F);       // lgkmcnt(0): the zeroes are written; the copy in flight is not waited for
+    __builtin_amdgcn_s_barrier();
     for (int g = wave; g < G; g += 4) {
         const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
         const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
@@ -271,74 +357,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
             const int dig[3] = {d0, d1, d2};
 #pragma unroll
             for (int pp = 0; pp < 3; pp++) {
-                const int m = pp * G + g;
+                const int m = 4 * g + pp;
                 aq[(((m >> 4) * 4 + (d >> 5)) * 16 + (m & 15)) * 32 + (d & 31)] = (uint8_t)(int8_t)dig[pp];
             }
         }
     }
-    __syncthreads();
+    PKV_LDS_BARRIER();
     long aop[NSETS][4];
 #pragma unroll
     for (int s = 0; s < NSETS; s++)
 #pragma unroll
         for (int sl = 0; sl < 4; sl++)
             aop[s][sl] = *reinterpret_cast<const long *>(aq + ((s * 4 + sl) * 16 + (lane & 15)) * 32 + 8 * (lane >> 4));
-    float qs_r[GW], qsum_r[GW];
+    // score of a token in the log2 domain: (k_scale * c1) * (D + k_zero * c2), D = the integer dot product of the digits
+    float c1_r[GW], c2_r[GW];
 #pragma unroll
     for (int gi = 0; gi < GW; gi++) {
         const int g = min(wave + 4 * gi, G - 1);
-        qs_r[gi] = qs[g];
-        qsum_r[gi] = qsum[g];
+        c1_r[gi] = p.sm_scale * qs[g] * 1.44269504088896341f;
+        c2_r[gi] = qs[g] > 0.f ? qsum[g] / qs[g] : 0.f;
     }
-    __syncthreads();      // slot 0 is free from here on; the last workgroup fence of the kernel
-
-    const int n_tiles = p.T_c / kTile;
-    const int tile0 = split * p.tiles_per_split;
-    const int tile1 = min(n_tiles, tile0 + p.tiles_per_split);
-    const int ntl = tile1 - tile0;                 // tiles of this split (>= 1)
-
-    // ---- block_info: wave-uniform scalar loads, fetched well before use ----
-    // this wave copies block `wave` of a tile and parses K block wave/2 and V block 2 + wave/2
-    // (read through the constant address space: block_info is read-only for the whole launch, and
-    // only loads known to be unclobbered are issued as scalar loads; a vector load here would make
-    // every later vmcnt wait drain the copies in flight)
-    typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
-    const int kj = wave >> 1;
-    const const_u32_ptr k_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.k_info));
-    const const_u32_ptr v_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.v_info));
-    const const_u32_ptr dma_info = wave < 2 ? k_info_c : v_info_c;
-    struct TileInfo { uint32_t dma_off, dma_size, k_off, v_off; };
-    auto load_info = [&](int rel) -> TileInfo {
-        const int tau = tile0 + min(rel, ntl - 1);
-        const uint32_t ik0 = (uint32_t)((2 * tau) * n_hid_k + bh), iv0 = (uint32_t)(tau * n_hid_v + 2 * bh);
-        const uint32_t id = wave < 2 ? ik0 + (uint32_t)wave * (uint32_t)n_hid_k : iv0 + (uint32_t)(wave - 2);
-        TileInfo ti;
-        ti.dma_off = dma_info[2 * (size_t)id];
-        ti.dma_size = dma_info[2 * (size_t)id + 1];
-        ti.k_off = k_info_c[2 * (size_t)(ik0 + (uint32_t)kj * (uint32_t)n_hid_k)];
-        ti.v_off = v_info_c[2 * (size_t)(iv0 + (uint32_t)kj)];
-        return ti;
-    };
-
-    // ---- copy of one tile into slot `slot` ----
-    auto dma_issue = [&](int slot, int rel, const TileInfo &ti) {
-        const uint32_t phase = ti.dma_off & 15u;                  // the streams themselves are 16-byte aligned
-        const uint32_t src = ti.dma_off - phase;
-        uint32_t nq = (phase + ti.dma_size + 15u) >> 4;           // 16-byte quads to copy
-        nq = min(max(nq, 1u), (uint32_t)(Geo::kRegion / 16));     // corrupt block_info must not overrun the region
-        const uint32_t last = nq - 1u;
-        const uint32_t dst = ring_lds + (uint32_t)(slot * Geo::kSlot + wave * Geo::kRegion);
-#pragma unroll
-        for (int i = 0; i < Geo::kMaxInstr; i++) {
-            if ((uint32_t)(i * 64) < nq) {                        // wave-uniform
-                if (i * 1024 + 1024 <= Geo::kRegion || lane < (Geo::kRegion - i * 1024) / 16)
-                    dma_b128(blk_rsrc, dst + i * 1024, src + 16u * min((uint32_t)(i * 64 + lane), last));
-            }
-        }
-        // parameter array `wave` of the tile: 128 tokens x 2 bytes = 64 lanes x 4 bytes
-        const int tile_off = (b * p.par_stride + (tile0 + min(rel, ntl - 1)) * kTile) * 2;
-        dma_b32(par_rsrc, ring_lds + (uint32_t)(slot * Geo::kSlot + Geo::kParOff + wave * 256), 4 * lane, (uint32_t)tile_off);
-    };
+    // The softmax weights reach the matrix cores as fp16(p * v_scale * wscale), wscale = 2^(kWExp - emax), emax = the
+    // largest biased exponent of v_scale met so far: p * v_scale * wscale < 2^11 whatever the magnitude of V, at full
+    // fp16 precision, and the sum of a round's 16 weights (the pack-minimum term takes it as fp16) stays below 2^15.
+    // When a tile brings a larger exponent the accumulators are rescaled like for a new maximum.
+    constexpr int kWExp = BF ? 137 : 25;
+    uint32_t emax_pair = 0u;                      // emax in both 16-bit halves
+    float wscale = 0.f, wscale_inv = 0.f;
 
     // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
     const int ku = hw & 3;
@@ -364,30 +409,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         meta_pairs<VW>(v_mins, v_lens, vr);
         pack_offsets8(__builtin_amdgcn_perm(kr.len23, kr.len01, 0x06040200u), koff);
         pack_offsets8(__builtin_amdgcn_perm(vr.len23, vr.len01, 0x06040200u), voff);
+        // pack words are addressed from the start of LDS (the slots sit at its bottom), region base included, so that
+        // one shift-add and one mask make the aligned address
         const uint32_t kpay0 = k_unit + K_META, vpay0 = v_unit + V_META;
+        const uint32_t kabs = (uint32_t)(slot * Geo::kSlot + kj * Geo::kRegion) + kpay0;
+        const uint32_t vabs = (uint32_t)(slot * Geo::kSlot + (2 + kj) * Geo::kRegion) + vpay0;
         if constexpr (KWIDE) {
             wide_windows(kb, kpay0, koff, kr);
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) kr.word[i] = lds_word64(kb, kpay0 + 2u * koff[i]);
+            for (int i = 0; i < 4; i++) kr.word[i] = lds_word64(ring, kabs + 2u * koff[i]);
         }
         if constexpr (VWIDE) {
             wide_windows(vb, vpay0, voff, vr);
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) vr.word[i] = lds_word64(vb, vpay0 + 2u * voff[i]);
+            for (int i = 0; i < 4; i++) vr.word[i] = lds_word64(ring, vabs + 2u * voff[i]);
         }
     };
 
-    auto cvt2 = [&](uint32_t w, float &lo, float &hi) {
-        if (!BF) {
-            lo = __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu)));
-            hi = __half2float(__ushort_as_half((unsigned short)(w >> 16)));
-        } else {
-            lo = __uint_as_float(w << 16);
-            hi = __uint_as_float(w & 0xFFFF0000u);
-        }
-    };
 
     float4v acc[NG4];
 #pragma unroll
@@ -412,11 +452,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
             uint32_t *dst = reinterpret_cast<uint32_t *>(kt) + (hw * 16) * kKtDw + t;
 #pragma unroll
             for (int q = 0; q < NWIN; q++) {
+                uint32_t x01 = w01[q], x23 = w23[q];      // the window's last token first, one width further per token
 #pragma unroll
-                for (int pp = 0; pp < TPW; pp++) {
-                    const uint32_t x01 = pp == TPW - 1 ? w01[q] : pk_shr16(w01[q], len01 * (uint32_t)(TPW - 1 - pp));
-                    const uint32_t x23 = pp == TPW - 1 ? w23[q] : pk_shr16(w23[q], len23 * (uint32_t)(TPW - 1 - pp));
+                for (int pp = TPW - 1; pp >= 0; pp--) {
                     dst[(q * TPW + pp) * kKtDw] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + kr.mins;
+                    if (pp) { x01 = pk_shr16(x01, len01); x23 = pk_shr16(x23, len23); }
                 }
             }
         }
@@ -441,51 +481,73 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
 #pragma unroll
                 for (int sl = 0; sl < 4; sl += 2)
                     d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pair128(aop[s][sl], aop[s][sl + 1]), pair128(bop[sl], bop[sl + 1]), d, 0, 0, 0);
-                // row-major [m][token]; odd rounds sit 16 banks further so the softmax reads spread over all banks
-                // (the four rows one instruction writes, m = 4 (lane / 16) + jj, are stored as 4 jj + lane / 16:
-                // adjacent, so they alternate between the two halves of the banks)
-                int32_t *o = reinterpret_cast<int32_t *>(kt + R * kRoundBytes + (R & 1) * 64) +
-                             (s * 16 + (lane >> 4)) * 16 + (lane & 15);
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) o[jj * 64] = d[jj];
+                // lane group lg = lane / 16 holds rows 4 lg .. 4 lg + 3 = the three digits of head 4 s + lg for token
+                // lane % 16: one score per lane.  Row of 16 tokens per (round, head); the head rows of a round rotate
+                // with the round number so that the softmax reads (one head, all rounds) spread over the banks.
+                const int lg = lane >> 4;
+                const int lo = (d[1] << 7) + d[2];
+                uint32_t *o = reinterpret_cast<uint32_t *>(kt + R * kRoundBytes + 256 * s + 64 * ((lg + R) & 3)) + (lane & 15);
+                if constexpr (SCORE_INT)
+                    *o = (uint32_t)((d[0] << 14) + lo);
+                else
+                    *o = __float_as_uint(fmaf((float)d[0], 16384.f, (float)lo));
             }
         }
     };
 
     // ---- stage 2: online softmax; wave <-> query head, lane <-> tokens 2*lane, 2*lane+1 ----
-    auto score_row = [](int m) -> int { return (m & ~15) | ((m & 3) << 2) | ((m >> 2) & 3); };   // where row m of the scores is stored
+    // Biased exponents of the v_scale of this lane's two tokens against the largest met so far (every wave sees the
+    // same tokens, so all four take the same decision).  Runs ahead of the parse so that the rare branch does not
+    // split the block in which the compiler interleaves the parse with the softmax.
+    float grow = 1.f;
+    auto emax_check = [&](int slot) {
+        const uint32_t vs_raw = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff)[128 + lane];
+        const uint32_t ex = (vs_raw >> (BF ? 7 : 10)) & (BF ? 0x00FF00FFu : 0x001F001Fu);
+        const ushort2v mxp = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, ex), __builtin_bit_cast(ushort2v, emax_pair));
+        grow = 1.f;
+        if (__builtin_amdgcn_ballot_w64(__builtin_bit_cast(uint32_t, mxp) != emax_pair) != 0) {     // rare
+            const uint32_t mine = max(__builtin_bit_cast(uint32_t, mxp) & 0xFFFFu, __builtin_bit_cast(uint32_t, mxp) >> 16);
+            uint32_t e = (uint32_t)__builtin_bit_cast(int, wave_max(__builtin_bit_cast(float, mine)));   // small positive ints order like floats
+            e = max(e, BF ? 14u : 1u);
+            const uint32_t old = emax_pair & 0xFFFFu;
+            grow = __builtin_amdgcn_exp2f(-(float)(int)(e - old));       // 0 on the first tile (nothing accumulated yet)
+            emax_pair = e | (e << 16);
+            wscale = __uint_as_float((uint32_t)(kWExp - (int)e + 127) << 23);
+            wscale_inv = __uint_as_float((uint32_t)((int)e - kWExp + 127) << 23);
+        }
+    };
     auto softmax_stage = [&](int slot, const uint8_t *kt) {
         const uint32_t *par = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff) + lane;
+        const uint32_t vs_raw = par[128];
         float ks0, ks1, kz0, kz1, vs0, vs1, vz0, vz1;
-        cvt2(par[0], ks0, ks1); cvt2(par[64], kz0, kz1); cvt2(par[128], vs0, vs1); cvt2(par[192], vz0, vz1);
+        cvt2(par[0], ks0, ks1); cvt2(par[64], kz0, kz1); cvt2(vs_raw, vs0, vs1); cvt2(par[192], vz0, vz1);
 #pragma unroll
         for (int gi = 0; gi < GW; gi++) {
             const int g = wave + 4 * gi;
             if (g < G) {
-                const int32_t *r =
-                    reinterpret_cast<const int32_t *>(kt + (lane >> 3) * kRoundBytes + ((lane >> 3) & 1) * 64) + 2 * (lane & 7);
-                float sv[2];
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const float d0 = (float)r[score_row(g) * 16 + e], d1 = (float)r[score_row(G + g) * 16 + e],
-                                d2 = (float)r[score_row(2 * G + g) * 16 + e];
-                    const float dot = qs_r[gi] * (d0 * 16384.f + d1 * 128.f + d2);
-                    sv[e] = p.sm_scale * (e ? ks1 : ks0) * (dot + (e ? kz1 : kz0) * qsum_r[gi]);
-                }
-                const float mx = wave_max_fused(fmaxf(sv[0], sv[1]));
+                const int R = lane >> 3;
+                const uint2v raw = *reinterpret_cast<const uint2v *>(
+                    kt + R * kRoundBytes + 256 * (g >> 2) + 64 * (((g & 3) + R) & 3) + 8 * (lane & 7));
+                const float D0 = SCORE_INT ? (float)(int)raw[0] : __uint_as_float(raw[0]);
+                const float D1 = SCORE_INT ? (float)(int)raw[1] : __uint_as_float(raw[1]);
+                // log2-domain scores
+                const float sv0 = (ks0 * c1_r[gi]) * fmaf(kz0, c2_r[gi], D0);
+                const float sv1 = (ks1 * c1_r[gi]) * fmaf(kz1, c2_r[gi], D1);
+                const float mx = wave_max_fused(fmaxf(sv0, sv1));
                 const float m_new = fmaxf(m_run[gi], mx);
-                const float alpha = __expf(m_run[gi] - m_new);    // exp(-inf) = 0 on the first tile
+                const float alpha = __builtin_amdgcn_exp2f(m_run[gi] - m_new);    // exp2(-inf) = 0 on the first tile
                 m_run[gi] = m_new;
-                const float p0 = __expf(sv[0] - m_new), p1 = __expf(sv[1] - m_new);
-                const _Float16 h0 = (_Float16)(p0 * vs0 * kPScale), h1 = (_Float16)(p1 * vs1 * kPScale);
+                const float p0 = __builtin_amdgcn_exp2f(sv0 - m_new), p1 = __builtin_amdgcn_exp2f(sv1 - m_new);
+                const _Float16 h0 = (_Float16)(p0 * (vs0 * wscale)), h1 = (_Float16)(p1 * (vs1 * wscale));
                 const float f0 = (float)h0, f1 = (float)h1;
                 // V-side order: MFMA k of a segment contracts token k of its four rounds
                 const int tok0 = 2 * lane;
                 _Float16 *pb = pbuf + g * kPStride + (tok0 & 64) + ((tok0 & 15) << 2) + ((tok0 >> 4) & 3);
                 pb[0] = h0;
                 pb[4] = h1;      // token 2*lane+1: same round, next k
+                const float beta = alpha * grow;     // what the weighted sums so far are multiplied by
                 l_part[gi] = l_part[gi] * alpha + (p0 + p1);
-                z_part[gi] = z_part[gi] * alpha + (f0 * vz0 + f1 * vz1);
+                z_part[gi] = z_part[gi] * beta + (f0 * vz0 + f1 * vz1);
                 // per-round sums (16 tokens = 8 lanes) of the rounded weights, for the pack-minimum term
                 const float r16 = oct_sum_fused(f0 + f1);
                 if ((lane & 7) == 0) {
@@ -493,7 +555,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
                     p16hi[g * 8 + (lane >> 3)] = hi;
                     p16lo[g * 8 + (lane >> 3)] = (_Float16)(r16 - (float)hi);
                 }
-                if (lane == 0) st_a[g] = alpha;
+                if (lane == 0) st_a[g] = beta;
             }
         }
     };
@@ -562,12 +624,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
                     for (int i4 = 0; i4 < NG4; i4++)
                         a_w[pp][i4] = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kPStride + 64 * seg + 4 * (4 * q + pp));
             }
+            uint32_t x01 = 0, x23 = 0;
 #pragma unroll
-            for (int pp = 0; pp < 4; pp++) {
+            for (int pp = 3; pp >= 0; pp--) {
                 constexpr int SH_MAX = TPW - 1;
                 const int wi = (4 * q + pp) / TPW, ps = (4 * q + pp) % TPW;      // window and position of token 4q + pp
-                const uint32_t x01 = ps == SH_MAX ? w01[wi] : pk_shr16(w01[wi], len01 * (uint32_t)(SH_MAX - ps));
-                const uint32_t x23 = ps == SH_MAX ? w23[wi] : pk_shr16(w23[wi], len23 * (uint32_t)(SH_MAX - ps));
+                if (ps == SH_MAX) { x01 = w01[wi]; x23 = w23[wi]; }             // a window's last token first,
+                else { x01 = pk_shr16(x01, len01); x23 = pk_shr16(x23, len23); }  // then one width further per token
                 const half4v bop = __builtin_bit_cast(half4v, make_uint2(x01 & m01, x23 & m23));
 #pragma unroll
                 for (int i4 = 0; i4 < NG4; i4++)
@@ -577,44 +640,65 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     };
 
     // ---- pipeline ----
-    TileInfo i0 = load_info(0), i1 = load_info(1), i2 = load_info(2);
     KUnit kcur;
     VUnit vcur;
-    dma_issue(0, 0, i0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    PKV_LDS_BARRIER();
-    dma_issue(1, 1, i1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile 0 (issued before the prologue's arithmetic)
+    PKV_LDS_BARRIER();                                    // ... and every wave has its q operands out of slot 1
+    dma_issue(1, t1, i1);
     parse(0, i0, kcur, vcur);
     PKV_LDS_BARRIER();
 
-    // at step s: i1, i2 = block_info of tiles s+1, s+2
-    for (int s = 0; s < ntl; s++) {
+    // Step s works on position s of the sequence (tile t_cur); t1, t2, t3 = the tiles of positions s+1 .. s+3, i1, i2 =
+    // block_info of t1, t2.  Position s+4 becomes known in the middle of the step: wave 0 asked the head's counter
+    // for it during step s-1, receives it with the copies it waits for before barrier 1 and hands it on through LDS.
+    uint32_t fetched = 0u;      // wave 0, lane 0: counter value of the request in flight
+    // (the address travels in vector registers: a scalar base that the compiler had just restored with a VALU
+    // instruction would reach the memory instruction inside the asm statement without the wait states it needs)
+    const uint32_t one = 1u;
+    const uint64_t ctr_addr = reinterpret_cast<uint64_t>(p.counters + bh);
+    for (int s = 0; t_cur < tile_end; s++) {
         const int slot = s & 1;
         uint8_t *kt = ring + slot * Geo::kSlot;
-        const TileInfo i3 = load_info(s + 3);
+        const TileInfo i3 = load_info(t3);
         __builtin_amdgcn_s_setprio(Prio::K);
-        k_stage(kcur, kt);
+        if (!(PKV_ATTN_PROBE & 2)) k_stage(kcur, kt);
         __builtin_amdgcn_s_setprio(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile s+1 has landed
-        PKV_LDS_BARRIER();                                    // publishes the scores and tile s+1
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(fetched) :: "memory");     // this wave's part of tile t1 has landed
+        if (p.dynamic && wave == 0 && lane == 0) tau_lds[slot] = 5 * p.nsplit + (int)fetched;
+        PKV_LDS_BARRIER();                                    // publishes the scores, tile t1 and position s+4
+        int t4 = s == 0 || !p.dynamic ? (s == 0 ? first_tiles(4) : t3 + 1)
+                                      : __builtin_amdgcn_readfirstlane(tau_lds[slot]);
         KUnit knext;
         VUnit vnext;
         __builtin_amdgcn_s_setprio(Prio::S);
-        parse(slot ^ 1, i1, knext, vnext);
-        softmax_stage(slot, kt);
+        emax_check(slot);
+        if (!(PKV_ATTN_PROBE & 16)) parse(slot ^ 1, i1, knext, vnext); else { knext = kcur; vnext = vcur; }
+        if (!(PKV_ATTN_PROBE & 4)) softmax_stage(slot, kt);
         __builtin_amdgcn_s_setprio(0);
-        PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile s+1 is parsed
+        PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile t1 is parsed
         __builtin_amdgcn_s_setprio(Prio::D);
-        dma_issue(slot, s + 2, i2);
+        if (!(PKV_ATTN_PROBE & 1)) dma_issue(slot, t2, i2);
+        if (p.dynamic && wave == 0 && lane == 0)              // position s+5, collected at the wait above in step s+1
+            asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(fetched) : "v"(ctr_addr), "v"(one) : "memory");
         __builtin_amdgcn_s_setprio(Prio::V);
-        v_stage(vcur);
+        if (!(PKV_ATTN_PROBE & 8)) v_stage(vcur);
         __builtin_amdgcn_s_setprio(0);
         kcur = knext;
         vcur = vnext;
+        t_cur = t1; t1 = t2; t2 = t3; t3 = t4;
         i1 = i2; i2 = i3;
     }
     // drain: the copy issued in the last step must land before the workgroup's LDS is released
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(fetched) :: "memory");
+    // the last member of the head to get here (every request of the others has been answered) zeroes the head's two
+    // counters for the next launch
+    if (p.dynamic && tid == 0) {
+        uint32_t *done = p.counters + n_heads + bh;
+        if (atomicAdd(done, 1u) + 1u == (uint32_t)p.nsplit) {
+            p.counters[bh] = 0u;
+            *done = 0u;
+        }
+    }
 
     // ---- epilogue ----
 #pragma unroll
@@ -622,7 +706,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         const int g = wave + 4 * gi;
         if (g < G) {
             const float l = wave_sum(l_part[gi]), z = wave_sum(z_part[gi]);
-            if (lane == 0) { st_m[g] = m_run[gi]; st_l[g] = l; st_z[g] = z; }
+            if (lane == 0) { st_m[g] = m_run[gi] * 0.693147180559945309f; st_l[g] = l; st_z[g] = z; }   // natural-log domain for the merge
         }
     }
     PKV_LDS_BARRIER();
@@ -637,7 +721,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         for (int g = 0; g < G; g++) {
             const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
-            const float val = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
+            const float val = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * wscale_inv;
             if (p.direct_out) {                // one split and no window: this is the result, no merge launch follows
                 p.out[hq * kHeadDim + ch] = a_st16(val / st_l[g], p.dtype);
                 continue;

@@ -341,7 +341,7 @@ int finish_encode(ScanState *st, uint64_t *size_out, int bits, hipStream_t s) {
 int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s) {
     void *p = nullptr;
     const size_t bytes = sizeof(ScanState) + (size_t)nblocks * sizeof(uint64_t);
-    int rc = scratch_get(bytes, &p);
+    int rc = scratch_get(bytes, s, &p);
     if (rc) return rc;
     const size_t n64 = (bytes + 7) / 8;
     zero_state_kernel<<<(unsigned)((n64 + 255) / 256), 256, 0, s>>>((uint64_t *)p, n64);

@@ -266,7 +266,7 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
     PKV_REQUIRE(M <= 65535, PKV_ERR_UNSUPPORTED, "more than 65535 rows");
     const int nparts = (N + 4095) / 4096;
     void *scratch = nullptr;
-    if ((rc = scratch_get((size_t)M * nparts * sizeof(float), &scratch))) return rc;
+    if ((rc = scratch_get((size_t)M * nparts * sizeof(float), s, &scratch))) return rc;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     fused_wv_partial_kernel<<<dim3((unsigned)nparts, (unsigned)M), 256, 0, s>>>(

@@ -405,7 +405,7 @@ int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pac
                 "hidden_dim must be a multiple of 16 and the code matrix 16-byte aligned");
     PKV_REQUIRE(ctx_len % pack_len == 0, PKV_ERR_INVALID, "ctx_len must be divisible by the pack length");
     void *scratch = nullptr;
-    int rc = scratch_get(sizeof(PackSizeOut), &scratch);
+    int rc = scratch_get(sizeof(PackSizeOut), s, &scratch);
     if (rc) return rc;
     PackSizeOut *out = static_cast<PackSizeOut *>(scratch);
     LaunchTimer tm(s, ms_out != nullptr);
@@ -439,7 +439,7 @@ int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
     PKV_REQUIRE(block_size <= 1024 && ctx_len % block_size == 0, PKV_ERR_INVALID,
                 "ctx_len must be divisible by a block size of at most 1024 tokens");
     void *scratch = nullptr;
-    int rc = scratch_get((size_t)ctx_len, &scratch);
+    int rc = scratch_get((size_t)ctx_len, s, &scratch);
     if (rc) return rc;
     uint8_t *median = static_cast<uint8_t *>(scratch);
     LaunchTimer tm(s, ms_out != nullptr);

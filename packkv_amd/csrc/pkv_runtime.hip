@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
+#include <vector>
 
 namespace pkv {
 
@@ -17,30 +18,84 @@ void set_error(const char *fmt, ...) {
 }
 
 namespace {
-constexpr int kMaxDevices = 16;
-struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
-Scratch g_scratch[kMaxDevices];
-std::mutex g_scratch_mu;
-}  // namespace
+// One workspace per (device, stream): calls on different streams of one device never share scratch, so they may
+// overlap.  A buffer that has been handed out is never freed or moved while the process lives: a request for more
+// allocates a larger buffer beside it and retires the old one (a captured HIP graph may still hold its address), so
+// growth costs memory (at most twice the largest request, growth is geometric) but never a synchronisation.
+struct Workspace {
+    int dev;
+    hipStream_t stream;
+    void *ptr;
+    size_t bytes;
+    uint32_t *counters;     // kAttnCounters tile counters of the attention kernel, zero between launches
+};
+std::vector<Workspace> g_ws;
+std::vector<void *> g_retired;      // superseded buffers, kept until the process ends
+std::mutex g_ws_mu;
 
-int scratch_get(size_t bytes, void **out) {
+int workspace_for(hipStream_t s, Workspace **out) {     // caller holds g_ws_mu
     int dev = 0;
     PKV_HIP_CHECK(hipGetDevice(&dev));
-    PKV_REQUIRE(dev >= 0 && dev < kMaxDevices, PKV_ERR_INVALID, "device index %d out of range", dev);
-    std::lock_guard<std::mutex> lock(g_scratch_mu);
-    Scratch &sc = g_scratch[dev];
-    if (sc.bytes < bytes) {
-        if (sc.ptr) {
-            PKV_HIP_CHECK(hipDeviceSynchronize());
-            PKV_HIP_CHECK(hipFree(sc.ptr));
-            sc.ptr = nullptr;
-            sc.bytes = 0;
+    for (Workspace &w : g_ws)
+        if (w.dev == dev && w.stream == s) { *out = &w; return PKV_OK; }
+    g_ws.push_back(Workspace{dev, s, nullptr, 0, nullptr});
+    *out = &g_ws.back();
+    return PKV_OK;
+}
+}  // namespace
+
+size_t scratch_grown_size(size_t have, size_t want) {
+    if (want <= have) return have;
+    size_t n = have ? have : (size_t)(1 << 20);
+    while (n < want) n += n / 2 + (size_t)(1 << 20);
+    return n;
+}
+
+// True when `s` is recording a HIP graph: nothing may be allocated then.
+static bool capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+int scratch_get(size_t bytes, hipStream_t s, void **out) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    Workspace *w = nullptr;
+    int rc = workspace_for(s, &w);
+    if (rc) return rc;
+    if (w->bytes < bytes) {
+        if (capturing(s)) {
+            set_error("stream is capturing a graph and has no scratch buffer of %zu bytes yet: make one eager call "
+                      "of the same shape on this stream first", bytes);
+            return PKV_ERR_CAPTURING;
         }
-        size_t want = bytes < (size_t)(1 << 20) ? (size_t)(1 << 20) : bytes + bytes / 4;
-        PKV_HIP_CHECK(hipMalloc(&sc.ptr, want));
-        sc.bytes = want;
+        const size_t want = scratch_grown_size(w->bytes, bytes);
+        void *fresh = nullptr;
+        PKV_HIP_CHECK(hipMalloc(&fresh, want));
+        if (w->ptr) g_retired.push_back(w->ptr);
+        w->ptr = fresh;
+        w->bytes = want;
     }
-    *out = sc.ptr;
+    *out = w->ptr;
+    return PKV_OK;
+}
+
+int attn_counters_get(hipStream_t s, uint32_t **out) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    Workspace *w = nullptr;
+    int rc = workspace_for(s, &w);
+    if (rc) return rc;
+    if (!w->counters) {
+        if (capturing(s)) {
+            set_error("stream is capturing a graph and has no attention counters yet: make one eager call on this "
+                      "stream first");
+            return PKV_ERR_CAPTURING;
+        }
+        void *c = nullptr;
+        PKV_HIP_CHECK(hipMalloc(&c, (size_t)kAttnCounters * sizeof(uint32_t)));
+        PKV_HIP_CHECK(hipMemset(c, 0, (size_t)kAttnCounters * sizeof(uint32_t)));
+        w->counters = (uint32_t *)c;
+    }
+    *out = w->counters;
     return PKV_OK;
 }
 

@@ -5,9 +5,21 @@
 
 namespace pkv {
 
-// Returns a device buffer of at least `bytes` on the current device, grown on demand and
-// kept until the process ends.  Not safe for concurrent encodes on one device.
-int scratch_get(size_t bytes, void **out);
+// A device buffer of at least `bytes` that belongs to (current device, stream `s`): calls on different streams get
+// different buffers and may overlap; calls on one stream share it and are ordered by the stream.  Buffers grow on
+// demand; one that has been handed out is never freed or moved while the process lives (a larger one is allocated
+// beside it), so an address captured in a HIP graph stays valid and growing never synchronises.
+// While `s` is capturing a HIP graph nothing can be allocated: a request the stream's buffer cannot serve then
+// returns PKV_ERR_CAPTURING (library-internal; callers fall back or report it as PKV_ERR_HIP).
+constexpr int PKV_ERR_CAPTURING = 100;
+int scratch_get(size_t bytes, hipStream_t s, void **out);
+// Capacity after growing a buffer of `have` bytes to hold `want` (geometric, at least 1 MiB): host arithmetic only.
+size_t scratch_grown_size(size_t have, size_t want);
+
+// Tile counters of the attention kernel for (current device, stream `s`): kAttnCounters zeroed 32-bit words,
+// allocated on first use; the attention kernel leaves every counter it used at zero again.
+constexpr int kAttnCounters = 65536;
+int attn_counters_get(hipStream_t s, uint32_t **out);
 
 // Per-call timing: records start/stop events on `stream` around fn() and returns elapsed ms
 // after synchronising on the stop event (mirrors the reference launchers, which time every

@@ -165,9 +165,10 @@ def test_attn_decode_full_size_property(cuda):
 
 
 def test_attn_decode_replays_in_a_hip_graph(cuda):
-    """A decode step launches only kernels on the caller's stream (no allocation once the library's scratch exists,
-    no memset nodes), so a serving loop can capture it: four layers' worth of calls in one graph, replayed with new
-    queries and eager work in between, must reproduce the eager results every time."""
+    """A decode step launches only kernels on the caller's stream (no memset nodes), and while a stream is capturing it
+    allocates nothing: a capture stream that has no scratch of its own yet (torch captures on a side stream) keeps its
+    partials in the library's fixed device array, like pkv_attn_decode_noalloc.  Four layers' worth of calls in one
+    graph, replayed with new queries and eager work in between, must reproduce the eager results every time."""
     B, Hq, Hkv, T, Tw = 2, 16, 4, 1024, 150
     layers = []
     for i in range(4):
@@ -193,6 +194,34 @@ def test_attn_decode_replays_in_a_hip_graph(cuda):
         torch.cuda.synchronize()
         for o, w in zip(outs, want):
             assert torch.equal(o, w)
+
+
+def test_two_streams_do_not_share_scratch(cuda):
+    """The library keeps its scratch memory (attention partials and tile counters, the encoders' look-back state) per
+    stream: encodes on one stream and decode steps on another may overlap.  Forty rounds of both at once must give
+    the results of running them one after the other."""
+    B, Hq, Hkv, T = 4, 32, 8, 4096
+    k, v = synth.make_kv(B, Hkv, T, seed=300, device=cuda)
+    q = synth.make_q(B, Hq, seed=301, device=cuda)
+    ke, ve = ops.k_quant_encode(k, 0.1), ops.v_quant_encode(v, 0.1)
+    want_out = ops.attn_decode(q, ke, ve)
+    k2, _ = synth.make_kv(B, Hkv, T, seed=302, device=cuda)
+    want_enc = ops.k_quant_encode(k2, 0.1)
+    torch.cuda.synchronize()
+    s_enc, s_att = torch.cuda.Stream(), torch.cuda.Stream()
+    outs, encs = [], []
+    for _ in range(40):
+        with torch.cuda.stream(s_att):
+            outs.append(ops.attn_decode(q, ke, ve))
+        with torch.cuda.stream(s_enc):
+            encs.append(ops.k_quant_encode(k2, 0.1, want_size=False))      # no host synchronisation: the streams overlap
+    torch.cuda.synchronize()
+    n = want_enc["size"]
+    for o in outs:
+        assert torch.equal(o, want_out)
+    for e in encs:
+        assert torch.equal(e["stream"][:n], want_enc["stream"][:n])
+        assert torch.equal(e["info"].view(torch.int32), want_enc["info"].view(torch.int32))
 
 
 @pytest.mark.parametrize("rel,bits", [(0.05, 5), (0.03, 6)])
