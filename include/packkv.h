@@ -62,14 +62,21 @@ uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits);
  * pack word (src/k_encode_cpu.cpp:211); here the same layout rules run on with pack words of
  * up to 128 bits and a 4-bit length field at bits = 8.  A stream of such codes can be larger
  * than the code matrix: size the buffer with pkv_block_bound.
- * `capacity` = bytes available at `stream`; `size_out` (host, may be NULL) receives the
- * stream size and makes the call synchronous. */
+ * `capacity` = bytes available at `stream` (which must start at an even address); `size_out` (host, may be NULL)
+ * receives the stream size and makes the call synchronous.  With size_out = NULL nothing is reported by the call
+ * itself, not even a stream that did not fit: ask pkv_encode_status afterwards. */
 int pkv_k_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
                  int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
                  float *ms_out, pkv_stream_t s);
 int pkv_v_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
                  int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
                  float *ms_out, pkv_stream_t s);
+/* Outcome of the last encode launched on stream `s` (any of pkv_{k,v}_encode, pkv_{k,v}_quant_encode and their
+ * _append forms) -- for callers that passed size_out = NULL to keep the launch asynchronous: waits for the stream,
+ * then returns what the encoder itself would have returned with size_out (PKV_ERR_CAPACITY when the stream did not
+ * fit, PKV_ERR_INTERNAL, and with bits > 0 PKV_ERR_UNSUPPORTED when a code of a fused encode does not fit `bits`)
+ * and stores the stream size.  No counterpart in the reference, whose encoders are synchronous host code. */
+int pkv_encode_status(pkv_stream_t s, int bits, uint64_t *size_out);
 int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
 int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
@@ -195,10 +202,12 @@ int pkv_fused_wv(void *our_wv, const void *w, const void *v_zero, const void *v_
  *
  *   k_stream/k_info   K stream of the code matrix [T_c, B*Hkv*128], blocks 64 x 128
  *   v_stream/v_info   V stream of the same shape, blocks 128 x 64
- *   k_bytes, v_bytes  readable bytes of each stream BUFFER (below 4 GiB).  The kernels never read
- *                     past this, whatever block_info says; they fetch pack words as whole
- *                     8-byte words, so the buffer must extend at least 7 bytes past the encoded
- *                     size (size_out of the encoder) or the last block decodes wrongly
+ *   k_bytes, v_bytes  readable bytes of each stream BUFFER (below 4 GiB).  The kernels never read past
+ *                     this (rounded up to a whole dword), whatever block_info says.  The default
+ *                     kernel and variant 1 take a buffer that ends with its stream; variant 2 (and
+ *                     variant 0 on streams that are not 16-byte aligned, which runs it) fetches pack
+ *                     words as whole 8-byte words, so for it the buffer must extend at least 7 bytes
+ *                     past the encoded size (size_out of the encoder) or the last block decodes wrongly
  *   k_scale..v_zero   [B, T_c] `dtype`
  *   q, out            [B, Hq, 128] `dtype`
  *   k_win, v_win      optional uncompressed tail [B, Hkv, T_w, 128] `dtype`, k_win 16-byte aligned (the residual

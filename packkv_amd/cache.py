@@ -29,7 +29,8 @@ class PackKVCacheConfig:
     scripts/throughput_config_test.py:16-24 uses 64 / 192 / 0.1 / 0.1)."""
 
     def __init__(self, block_size=64, buffer_size=192, k_quant_scale_rel=0.1, v_quant_scale_rel=0.1,
-                 k_bits=None, v_bits=None):
+                 k_bits=None, v_bits=None, enable_quant=True):
+        self.enable_quant = enable_quant
         if block_size != 64:
             raise RuntimeError("not supported: block_size %d (the K block is 64 tokens)" % block_size)
         if buffer_size < block_size or buffer_size + 2 * block_size > 2048:
@@ -124,9 +125,11 @@ class PackKVCompressedCache:
         return self.layers[i]
 
     # -- reference contract --------------------------------------------------------------------------
-    def update(self, key_states, value_states, layer_idx, cache_kwargs=None, return_dense=False):
-        """Append key_states / value_states [B, H, n, 128].  Returns None, or with return_dense=True the dense
-        (K, V) [B, H, T, 128] the reference returns (packkv_quant.py:84-85)."""
+    def update(self, key_states, value_states, layer_idx, cache_kwargs=None, return_dense=True):
+        """Append key_states / value_states [B, H, n, 128].  Returns the dense (K, V) [B, H, T, 128] the reference's
+        update returns (packkv_quant.py:84-85), so that the caller's eager attention runs unchanged
+        (models/llama.py:261); a caller that attends through ``attend`` passes return_dense=False and gets None --
+        building the dense view decompresses the whole layer."""
         L = self._layer(layer_idx)
         cfg = self.config
         rotary = bool(cache_kwargs) and cache_kwargs.get("cos") is not None
@@ -247,3 +250,87 @@ class PackKVCompressedCache:
             es = L.k_win.element_size()
             total += 2 * self.batch_size * self.head_num * (L.win_len + L.pend) * 128 * es
         return total
+
+
+# ---- the reference's own class names ------------------------------------------------------------------
+
+class PackKVCacheConfigStatic:
+    """The process-wide configuration slot the reference's caches read (models/cache/packkv_quant.py:10-12):
+    ``PackKVCacheConfigStatic.config`` holds an object with block_size, buffer_size, k_quant_scale_rel,
+    v_quant_scale_rel (and optionally enable_quant) -- the reference's utils/config.py ``PackKVCacheConfig`` or this
+    module's ``PackKVCacheConfig``.  ``max_tokens`` sizes the per-layer tables of the compressed cache."""
+    config = None
+    max_tokens = 32768
+
+
+try:                                    # the reference's caches are transformers.Cache subclasses
+    from transformers import Cache as _HFCache
+except Exception:                       # pragma: no cover - transformers is an optional dependency of this class only
+    _HFCache = object
+
+
+class PackKVCache(_HFCache):
+    """Drop-in for the reference's ``PackKVCache`` (models/cache/packkv_cache.py:22-38; built by
+    models/llama.py:830-833 as ``PackKVCache(batch, heads, head_dim, layers)`` and called by its attention modules as
+    ``key_states, value_states = past_key_value.update(key_states, value_states, layer_idx, cache_kwargs)``,
+    models/llama.py:261): same constructor, same ``update`` return value (the dense K and V, the quantised prefix in
+    dequantised form followed by the 16-bit buffer), same ``get_seq_length``.  The quantised prefix is held as PackKV
+    streams on the device; ``attend`` / ``materialize`` / ``cache_bytes`` of the compressed cache are passed through
+    for callers that replace the eager attention of a decode step.  The compressed cache is created at the first
+    ``update`` (dtype and device of the tensors it is given; head_num is the number of KV heads those tensors have)."""
+
+    def __init__(self, batch_size, head_num, head_dim, layer_num, config=None, max_tokens=None):
+        if _HFCache is not object:
+            try:
+                super().__init__(layers=[])          # transformers 5: a Cache is a list of layers
+            except TypeError:
+                super().__init__()                   # transformers 4 (the reference pins 4.52)
+        # (transformers.Cache defines read-only properties of its own under some of the reference's attribute names)
+        self._shape = (batch_size, head_num, head_dim)
+        self._layer_num = layer_num
+        self._config, self._max_tokens = config, max_tokens
+        self.cache_instance = None
+        self._plain_k = [None] * layer_num           # enable_quant = False: everything stays in 16 bits
+        self._plain_v = [None] * layer_num
+
+    def _cfg(self):
+        cfg = self._config or PackKVCacheConfigStatic.config
+        if cfg is None:
+            raise ValueError("PackKVCacheConfigStatic.config is not set. Please set it before using PackKVCache.")
+        return cfg
+
+    def _instance(self, key_states):
+        if self.cache_instance is None:
+            cfg = self._cfg()
+            own = cfg if isinstance(cfg, PackKVCacheConfig) else PackKVCacheConfig(
+                cfg.block_size, cfg.buffer_size, cfg.k_quant_scale_rel, cfg.v_quant_scale_rel)
+            self.cache_instance = PackKVCompressedCache(
+                key_states.size(0), key_states.size(1), key_states.size(3), self._layer_num, own,
+                max_tokens=self._max_tokens or PackKVCacheConfigStatic.max_tokens, dtype=key_states.dtype,
+                device=key_states.device)
+        return self.cache_instance
+
+    def update(self, key_states, value_states, layer_idx, cache_kwargs=None, return_dense=True):
+        if getattr(self._cfg(), "enable_quant", True) is False:          # packkv_quant.py:87-99 (update_disable)
+            if cache_kwargs and cache_kwargs.get("cos") is not None:
+                key_states = apply_rotary_pos_emb_single(key_states, cache_kwargs["cos"], cache_kwargs["sin"])
+            k, v = self._plain_k[layer_idx], self._plain_v[layer_idx]
+            self._plain_k[layer_idx] = key_states if k is None else torch.cat([k, key_states], dim=2)
+            self._plain_v[layer_idx] = value_states if v is None else torch.cat([v, value_states], dim=2)
+            return self._plain_k[layer_idx], self._plain_v[layer_idx]
+        return self._instance(key_states).update(key_states, value_states, layer_idx, cache_kwargs, return_dense)
+
+    def get_seq_length(self, layer_idx=0):
+        if self.cache_instance is None:
+            k = self._plain_k[layer_idx or 0]
+            return 0 if k is None else k.shape[2]
+        return self.cache_instance.get_seq_length(layer_idx)
+
+    def attend(self, query_states, layer_idx, **kw):
+        return self.cache_instance.attend(query_states, layer_idx, **kw)
+
+    def materialize(self, layer_idx):
+        return self.cache_instance.materialize(layer_idx)
+
+    def cache_bytes(self, layer_idx=None):
+        return self.cache_instance.cache_bytes(layer_idx)

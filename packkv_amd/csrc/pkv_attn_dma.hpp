@@ -257,7 +257,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
 
     // the stream this wave copies from, range-checked: block_info is never trusted with an address
-    const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, wave < 2 ? p.k_bytes : p.v_bytes);
+    // (the size is rounded up to whole dwords: a copy is range-checked dword by dword, and the aligned dword that
+    // holds the buffer's last byte lies in the same page as that byte -- a buffer that ends with its stream loses
+    // nothing and nothing unmapped is touched)
+    const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, ((wave < 2 ? p.k_bytes : p.v_bytes) + 3u) & ~3u);
     const uint16_t *par_arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
     const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.par_stride * 2));
 

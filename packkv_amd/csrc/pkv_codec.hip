@@ -341,7 +341,7 @@ int finish_encode(ScanState *st, uint64_t *size_out, int bits, hipStream_t s) {
 int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s) {
     void *p = nullptr;
     const size_t bytes = sizeof(ScanState) + (size_t)nblocks * sizeof(uint64_t);
-    int rc = scratch_get(bytes, s, &p);
+    int rc = scratch_get(bytes, s, &p, kScratchEncoder);
     if (rc) return rc;
     const size_t n64 = (bytes + 7) / 8;
     zero_state_kernel<<<(unsigned)((n64 + 255) / 256), 256, 0, s>>>((uint64_t *)p, n64);
@@ -354,6 +354,8 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
                     int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
                     float *ms_out, hipStream_t s) {
     PKV_REQUIRE(stream && info && codes, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE((reinterpret_cast<uintptr_t>(stream) & 1u) == 0, PKV_ERR_INVALID,
+                "compressed_buffer must start at an even address (blocks are written in 2-byte units)");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
     // block_info holds 32-bit byte offsets: a stream past 4 GiB is reported as a full buffer, never wrapped
     if (capacity > (1ull << 32)) capacity = 1ull << 32;
@@ -425,6 +427,16 @@ int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *cod
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s) {
     return pkv::run_unpack(false, stream, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
                            ms_out, (hipStream_t)s);
+}
+
+int pkv_encode_status(pkv_stream_t s_, int bits, uint64_t *size_out) {
+    using namespace pkv;
+    hipStream_t s = (hipStream_t)s_;
+    PKV_REQUIRE(size_out != nullptr, PKV_ERR_INVALID, "null pointer argument");
+    void *st = nullptr;
+    int rc = encoder_state_peek(s, &st);
+    if (rc) return rc;
+    return finish_encode(static_cast<ScanState *>(st), size_out, bits, s);
 }
 
 uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits) {

@@ -1098,6 +1098,8 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     int rc = check_xshape(x, dtype, B, H, T);
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE((reinterpret_cast<uintptr_t>(stream) & 1u) == 0, PKV_ERR_INVALID,
+                "compressed_buffer must start at an even address (blocks are written in 2-byte units)");
     PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
     PKV_REQUIRE(bits >= 2 && bits <= 6, PKV_ERR_UNSUPPORTED,
                 "not supported: bits_len %d (the fused encoders take 2..6; wider codes go through pkv_quant_params, "

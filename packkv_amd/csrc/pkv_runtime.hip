@@ -25,9 +25,10 @@ namespace {
 struct Workspace {
     int dev;
     hipStream_t stream;
-    void *ptr;
-    size_t bytes;
+    void *ptr[2];           // kScratchGeneral, kScratchEncoder
+    size_t bytes[2];
     uint32_t *counters;     // kAttnCounters tile counters of the attention kernel, zero between launches
+    bool encoded;           // an encoder has run on this stream: ptr[kScratchEncoder] starts with its ScanState
 };
 std::vector<Workspace> g_ws;
 std::vector<void *> g_retired;      // superseded buffers, kept until the process ends
@@ -38,7 +39,7 @@ int workspace_for(hipStream_t s, Workspace **out) {     // caller holds g_ws_mu
     PKV_HIP_CHECK(hipGetDevice(&dev));
     for (Workspace &w : g_ws)
         if (w.dev == dev && w.stream == s) { *out = &w; return PKV_OK; }
-    g_ws.push_back(Workspace{dev, s, nullptr, 0, nullptr});
+    g_ws.push_back(Workspace{dev, s, {nullptr, nullptr}, {0, 0}, nullptr, false});
     *out = &g_ws.back();
     return PKV_OK;
 }
@@ -57,25 +58,36 @@ static bool capturing(hipStream_t s) {
     return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
 }
 
-int scratch_get(size_t bytes, hipStream_t s, void **out) {
+int scratch_get(size_t bytes, hipStream_t s, void **out, int kind) {
     std::lock_guard<std::mutex> lock(g_ws_mu);
     Workspace *w = nullptr;
     int rc = workspace_for(s, &w);
     if (rc) return rc;
-    if (w->bytes < bytes) {
+    if (kind == kScratchEncoder) w->encoded = true;
+    if (w->bytes[kind] < bytes) {
         if (capturing(s)) {
             set_error("stream is capturing a graph and has no scratch buffer of %zu bytes yet: make one eager call "
                       "of the same shape on this stream first", bytes);
             return PKV_ERR_CAPTURING;
         }
-        const size_t want = scratch_grown_size(w->bytes, bytes);
+        const size_t want = scratch_grown_size(w->bytes[kind], bytes);
         void *fresh = nullptr;
         PKV_HIP_CHECK(hipMalloc(&fresh, want));
-        if (w->ptr) g_retired.push_back(w->ptr);
-        w->ptr = fresh;
-        w->bytes = want;
+        if (w->ptr[kind]) g_retired.push_back(w->ptr[kind]);
+        w->ptr[kind] = fresh;
+        w->bytes[kind] = want;
     }
-    *out = w->ptr;
+    *out = w->ptr[kind];
+    return PKV_OK;
+}
+
+int encoder_state_peek(hipStream_t s, void **out) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    Workspace *w = nullptr;
+    int rc = workspace_for(s, &w);
+    if (rc) return rc;
+    PKV_REQUIRE(w->encoded && w->ptr[kScratchEncoder], PKV_ERR_INVALID, "no encode has been launched on this stream");
+    *out = w->ptr[kScratchEncoder];
     return PKV_OK;
 }
 

@@ -12,7 +12,12 @@ namespace pkv {
 // While `s` is capturing a HIP graph nothing can be allocated: a request the stream's buffer cannot serve then
 // returns PKV_ERR_CAPTURING (library-internal; callers fall back or report it as PKV_ERR_HIP).
 constexpr int PKV_ERR_CAPTURING = 100;
-int scratch_get(size_t bytes, hipStream_t s, void **out);
+// Two buffers per stream: the encoders' look-back state has one of its own, so that it (and the status it ends with)
+// survives whatever else runs on the stream until the next encode.
+constexpr int kScratchGeneral = 0, kScratchEncoder = 1;
+int scratch_get(size_t bytes, hipStream_t s, void **out, int kind = kScratchGeneral);
+// Start of the encoder-state buffer of stream `s` (the ScanState of the last encode launched on it).
+int encoder_state_peek(hipStream_t s, void **out);
 // Capacity after growing a buffer of `have` bytes to hold `want` (geometric, at least 1 MiB): host arithmetic only.
 size_t scratch_grown_size(size_t have, size_t want);
 

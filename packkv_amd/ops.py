@@ -20,7 +20,7 @@ __all__ = [
     "kq_mat_vec_mul", "wv_mat_vec_mul", "fused_kq", "fused_wv",
     "k_encode", "v_encode", "k_decode", "v_decode",
     "quant_params", "quantize", "dequantize", "k_quant_encode", "v_quant_encode",
-    "attn_decode", "AttnPlan", "block_bound", "bits_for_rel", "repack_quant_encode",
+    "attn_decode", "AttnPlan", "block_bound", "bits_for_rel", "repack_quant_encode", "encode_status",
 ]
 
 
@@ -93,6 +93,7 @@ def _check_codec_args(codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk
     _require(info.dtype == torch.uint32, "block_info_buffer must be a UInt32 tensor")
     _require(codes.is_contiguous() and stream.is_contiguous() and info.is_contiguous(),
              "tensors must be contiguous")
+    _require(not stream.is_cuda or stream.data_ptr() % 2 == 0, "compressed_buffer must start at an even address")
 
 
 def _encode(is_k, codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, want_size=True,
@@ -138,6 +139,17 @@ def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bi
     if on_host:
         codes.copy_(d_codes.cpu())
     return float(ms.value) if timed else None
+
+
+def encode_status(device=None, bits=0):
+    """Stream size of the last encode launched on the current stream of `device` with want_size=False; waits for the
+    stream and raises what the encode would have raised (a stream that did not fit, a code wider than `bits`)."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    size = ctypes.c_uint64(0)
+    with torch.cuda.device(dev):
+        rc = _lib.load().pkv_encode_status(_stream(dev), int(bits), ctypes.byref(size))
+    _lib.check(rc)
+    return int(size.value)
 
 
 def k_encode_cpu(quant_ints_tensor, compressed_buffer, block_info_buffer, ctx_len, hidden_dim,
@@ -553,11 +565,15 @@ def fused_kq(our_kq, q, k_quant_zero, k_quant_scale, t):
                     ("our_kq", our_kq)):
         if not x.is_cuda:
             raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not our_kq.is_contiguous(): raise RuntimeError("our_kq must be contiguous")
     ms = ctypes.c_float(0.0)
+    # contiguous copies of strided inputs must outlive the call: a temporary released between two .contiguous() calls
+    # can be handed the same memory again
+    q_c, z_c, s_c, t_c = q.contiguous(), k_quant_zero.contiguous(), k_quant_scale.contiguous(), t.contiguous()
     with torch.cuda.device(q.device):
-        rc = _lib.load().pkv_fused_kq(_ptr(our_kq), _ptr(q.contiguous()), _ptr(k_quant_zero.contiguous()),
-                                      _ptr(k_quant_scale.contiguous()), _ptr(t.contiguous()), M, K, N,
+        rc = _lib.load().pkv_fused_kq(_ptr(our_kq), _ptr(q_c), _ptr(z_c), _ptr(s_c), _ptr(t_c), M, K, N,
                                       _dtype_code(q), ctypes.byref(ms), _stream(q.device))
+    del q_c, z_c, s_c, t_c
     _lib.check(rc)
     return float(ms.value)
 
@@ -583,11 +599,13 @@ def fused_wv(our_wv, w, v_quant_zero, v_quant_scale, term1):
                     ("v_quant_scale", v_quant_scale), ("our_wv", our_wv)):
         if not x.is_cuda:
             raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not our_wv.is_contiguous(): raise RuntimeError("our_wv must be contiguous")
     ms = ctypes.c_float(0.0)
+    w_c, z_c, s_c, t_c = w.contiguous(), v_quant_zero.contiguous(), v_quant_scale.contiguous(), term1.contiguous()
     with torch.cuda.device(w.device):
-        rc = _lib.load().pkv_fused_wv(_ptr(our_wv), _ptr(w.contiguous()), _ptr(v_quant_zero.contiguous()),
-                                      _ptr(v_quant_scale.contiguous()), _ptr(term1.contiguous()), M, N, D,
+        rc = _lib.load().pkv_fused_wv(_ptr(our_wv), _ptr(w_c), _ptr(z_c), _ptr(s_c), _ptr(t_c), M, N, D,
                                       _dtype_code(w), ctypes.byref(ms), _stream(w.device))
+    del w_c, z_c, s_c, t_c
     _lib.check(rc)
     return float(ms.value)
 
@@ -623,11 +641,12 @@ class AttnPlan:
                      "block_info_buffer block num mismatch")
             a.k_stream, a.k_info = _ptr(k["stream"]), _ptr(k["info"])
             a.v_stream, a.v_info = _ptr(v["stream"]), _ptr(v["info"])
-            # readable bytes of each buffer: pack words are fetched as whole 8-byte words, so the last
-            # block needs 7 bytes of readable slack behind the encoded size
-            for d in (k, v):
-                _require(not d.get("size") or d["stream"].numel() >= int(d["size"]) + 7,
-                         "stream buffers need 7 readable bytes behind the encoded size")
+            # readable bytes of each buffer.  The default kernel copies whole dwords and needs no slack; the gather
+            # kernel (variant 2, and variant 0 on streams that are not 16-byte aligned) fetches pack words as whole
+            # 8-byte words and needs 7 readable bytes behind the encoded size: without them the plain kernel runs
+            gathers = int(variant) == 2 or (int(variant) == 0 and (k["stream"].data_ptr() | v["stream"].data_ptr()) % 16 != 0)
+            if gathers and any(d.get("size") and d["stream"].numel() < int(d["size"]) + 7 for d in (k, v)):
+                variant = 1
             a.k_bytes, a.v_bytes = k["stream"].numel(), v["stream"].numel()
             a.k_scale, a.k_zero = _ptr(k["scale"]), _ptr(k["zero"])
             a.v_scale, a.v_zero = _ptr(v["scale"]), _ptr(v["zero"])

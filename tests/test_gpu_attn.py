@@ -196,6 +196,21 @@ def test_attn_decode_replays_in_a_hip_graph(cuda):
             assert torch.equal(o, w)
 
 
+def test_attn_decode_takes_buffers_that_end_with_their_stream(cuda):
+    """Stream buffers without a byte of slack behind the encoded size (sizes that end in the middle of a dword and of
+    a 16-byte copy unit included) give the results of generously sized buffers, on every variant."""
+    for seed, (B, Hq, Hkv, T) in enumerate([(1, 8, 2, 128), (2, 16, 4, 512), (1, 32, 8, 1024), (1, 4, 1, 256), (3, 12, 3, 384)]):
+        k, v = synth.make_kv(B, Hkv, T, seed=900 + seed, device=cuda)
+        q = synth.make_q(B, Hq, seed=950 + seed, device=cuda)
+        ke, ve = ops.k_quant_encode(k, 0.1), ops.v_quant_encode(v, 0.1)
+        ke2, ve2 = dict(ke), dict(ve)
+        ke2["stream"], ve2["stream"] = ke["stream"][:ke["size"]].clone(), ve["stream"][:ve["size"]].clone()
+        _say("exact buffers: K size %% 16 = %d, V size %% 16 = %d" % (ke["size"] % 16, ve["size"] % 16))
+        for variant in (0, 1, 2):
+            want = ops.attn_decode(q, ke, ve, variant=1 if variant == 2 else variant)     # variant 2 falls back to 1
+            assert torch.equal(ops.attn_decode(q, ke2, ve2, variant=variant), want)
+
+
 def test_two_streams_do_not_share_scratch(cuda):
     """The library keeps its scratch memory (attention partials and tile counters, the encoders' look-back state) per
     stream: encodes on one stream and decode steps on another may overlap.  Forty rounds of both at once must give

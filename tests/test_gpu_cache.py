@@ -55,7 +55,7 @@ def test_cache_matches_restated_reference(cuda, dtype, rope):
             cos, sin = _rope_tables(B, pos, n, dtype)
         wk, wv = want.update(ks, vs, 0, cos, sin)
         kw = {"cos": cos.to(cuda), "sin": sin.to(cuda)} if rope else None
-        got.update(ks.to(cuda), vs.to(cuda), 0, kw)
+        got.update(ks.to(cuda), vs.to(cuda), 0, kw, return_dense=False)
         tok += n
         pos += n
         assert got.get_seq_length(0) == want.get_seq_length(0) == tok
@@ -115,10 +115,10 @@ def test_cache_bytes_and_prefill_only(cuda):
     B, H = 1, 8
     k, v = synth.make_kv(B, H, 1000, seed=97, device=cuda)
     c = PackKVCompressedCache(B, H, 128, 2, max_tokens=2048, device=cuda)
-    c.update(k[:, :, :191], v[:, :, :191], 0)
+    c.update(k[:, :, :191], v[:, :, :191], 0, return_dense=False)
     assert c.layers[0].k.tokens == 0 and c.layers[0].win_len == 191
     assert c.cache_bytes(0) == 2 * B * H * 191 * 128 * 2
-    c.update(k, v, 1)                     # 1000 tokens: 832 cut = 6 tiles + one pending cut of 64, 168 buffered
+    c.update(k, v, 1, return_dense=False)     # 1000 tokens: 832 cut = 6 tiles + one pending cut of 64, 168 buffered
     L = c.layers[1]
     assert L.k.tokens == 768 and L.pend == 64 and L.win_len == 64 + 168 and c.get_seq_length(1) == 1000
     fp16_bytes = 2 * B * H * 1000 * 128 * 2
@@ -190,7 +190,7 @@ def test_cache_with_five_bit_codes(cuda):
         n = T0 if step < 0 else 1
         ks, vs = k[:, :, tok:tok + n], v[:, :, tok:tok + n]
         wk, wv = want.update(ks, vs, 0, None, None)
-        got.update(ks.to(cuda), vs.to(cuda), 0, None)
+        got.update(ks.to(cuda), vs.to(cuda), 0, None, return_dense=False)
         tok += n
         if step in (-1, 0, 19, 20, 39):
             _say("5-bit cache case step", step, "tokens", tok, "compressed", got.layers[0].k.tokens)
@@ -201,3 +201,48 @@ def test_cache_with_five_bit_codes(cuda):
             ek, ev = want.exact(0)
             _attend_parity(got, 0, q, wk, wv, ek, ev, dtype, cuda, "5-bit step %d" % step)
     assert got.layers[0].k.tokens == 128 and got.layers[0].pend == 64      # 128 at the prefill, one more cut waiting for its partner
+
+
+def test_reference_cache_class_and_its_two_line_hook(cuda):
+    """The reference builds ``PackKVCache(batch, heads, head_dim, layers)`` (models/llama.py:830-833), configured
+    through ``PackKVCacheConfigStatic.config``, and its attention modules run (models/llama.py:260-261)
+
+        cache_kwargs = {"sin": sin, "cos": cos, "cache_position": cache_position}
+        key_states, value_states = past_key_value.update(key_states, value_states, self.layer_idx, cache_kwargs)
+
+    The drop-in class takes both lines as they stand: it is a transformers.Cache, and update returns the dense K and V
+    of the restated reference cache bit for bit -- prompt pass and decode steps across a cut, two layers."""
+    import transformers
+    from packkv_amd.cache import PackKVCache, PackKVCacheConfigStatic
+    dtype = torch.float16
+    B, H, T0, steps, layers = 2, 4, 300, 70, 2
+    k, v = synth.make_kv(B, H, T0 + steps, seed=610, dtype=dtype)
+    PackKVCacheConfigStatic.config = PackKVCacheConfig(64, 192, 0.1, 0.1)
+    PackKVCacheConfigStatic.max_tokens = 1024
+    try:
+        past_key_value = PackKVCache(B, H, 128, layers)
+        assert isinstance(past_key_value, transformers.Cache)
+        want = oc.SimulatedCache(layers, 64, 192, 0.1, 0.1)
+        pos = 0
+        for step in range(-1, steps):
+            n = T0 if step < 0 else 1
+            cos, sin = _rope_tables(B, pos, n, dtype)
+            cache_position = torch.arange(pos, pos + n)
+            for layer_idx in range(layers):
+                key_states = (k[:, :, pos:pos + n] * (1 + layer_idx)).to(cuda)
+                value_states = v[:, :, pos:pos + n].to(cuda)
+                wk, wv = want.update(key_states.cpu(), value_states.cpu(), layer_idx, cos, sin)
+                sin_d, cos_d = sin.to(cuda), cos.to(cuda)
+                # the reference's two lines, with sin / cos on the device
+                cache_kwargs = {"sin": sin_d, "cos": cos_d, "cache_position": cache_position}
+                key_states, value_states = past_key_value.update(key_states, value_states, layer_idx, cache_kwargs)
+                if step < 0 or step in (0, 18, 19, 20, 69):
+                    _say("reference hook: step", step, "layer", layer_idx, "K", tuple(key_states.shape))
+                    assert key_states.shape == wk.shape and value_states.shape == wv.shape
+                    assert torch.equal(key_states.cpu().view(torch.int16), wk.view(torch.int16))
+                    assert torch.equal(value_states.cpu().view(torch.int16), wv.view(torch.int16))
+            pos += n
+            assert past_key_value.get_seq_length(0) == past_key_value.get_seq_length(1) == pos
+    finally:
+        PackKVCacheConfigStatic.config = None
+        PackKVCacheConfigStatic.max_tokens = 32768

@@ -90,3 +90,25 @@ def test_unsupported_case_returns_zero(cuda, capsys):
     assert "Unsupported data type" in capsys.readouterr().out
     with pytest.raises(RuntimeError, match="2D"):
         packkv_cuda.fused_kq(t, q[0], t[0], t[0], t)
+
+
+def test_fused_fixups_take_strided_tensors(cuda):
+    """fused_kq / fused_wv on transposed and sliced views (every operand non-contiguous at once): the contiguous
+    copies the binding makes must all be alive during the call, so the results equal those of contiguous inputs."""
+    g = torch.Generator().manual_seed(77)
+    M, N = 8, 1024
+    q = torch.randn(128, M, generator=g).to(torch.float16).to(cuda).t()                 # [M, 128] view of [128, M]
+    t = torch.randn(N, M, generator=g).to(torch.float16).to(cuda).t()                   # [M, N] view
+    zero = torch.randn(2 * N, generator=g).round().to(torch.float16).to(cuda)[::2]      # stride 2
+    scale = (torch.rand(2 * N, generator=g) + 0.5).to(torch.float16).to(cuda)[::2]
+    assert not (q.is_contiguous() or t.is_contiguous() or zero.is_contiguous() or scale.is_contiguous())
+    got, want = torch.empty(M, N, dtype=torch.float16, device=cuda), torch.empty(M, N, dtype=torch.float16, device=cuda)
+    packkv_cuda.fused_kq(got, q, zero, scale, t)
+    packkv_cuda.fused_kq(want, q.contiguous(), zero.contiguous(), scale.contiguous(), t.contiguous())
+    assert torch.equal(got, want)
+    w = torch.rand(N, M, generator=g).to(torch.float16).to(cuda).t()
+    term1 = torch.randn(128, M, generator=g).to(torch.float16).to(cuda).t()
+    got, want = torch.empty(M, 128, dtype=torch.float16, device=cuda), torch.empty(M, 128, dtype=torch.float16, device=cuda)
+    packkv_cuda.fused_wv(got, w, zero, scale, term1)
+    packkv_cuda.fused_wv(want, w.contiguous(), zero.contiguous(), scale.contiguous(), term1.contiguous())
+    assert torch.equal(got, want)

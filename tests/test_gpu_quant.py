@@ -141,3 +141,34 @@ def test_fused_quant_encode_round_trip_full_size(cuda):
             ops.v_decode(r["stream"], r["info"], back, 128, 64, 4)
         assert torch.equal(back, codes)
         del r, codes, back
+
+
+def test_asynchronous_encode_reports_through_encode_status(cuda):
+    """want_size=False keeps the launch asynchronous and reports nothing by itself; ops.encode_status then gives the
+    size, or raises what the synchronous form raises: a stream that does not fit, a code wider than bits_len.  A
+    compressed buffer at an odd address is refused up front (blocks are written in 2-byte units)."""
+    B, H, T = 2, 4, 512
+    k, _ = synth.make_kv(B, H, T, seed=620, device=cuda)
+    sync = ops.k_quant_encode(k, 0.1)
+    a = ops.k_quant_encode(k, 0.1, want_size=False)
+    assert a["size"] == 0
+    q = synth.make_q(B, 4 * H, seed=621, device=cuda)
+    ops.attn_decode(q, sync, ops.v_quant_encode(k, 0.1))          # other work on the stream does not disturb the status
+    assert ops.encode_status(cuda, bits=4) == sync["size"]
+    assert torch.equal(a["stream"][:sync["size"]], sync["stream"][:sync["size"]])
+    small = torch.empty(1024, dtype=torch.uint8, device=cuda)
+    ops.k_quant_encode(k, 0.1, stream=small, want_size=False)     # does not fit: silent until asked
+    with pytest.raises(ops.PackKVError) as e:
+        ops.encode_status(cuda)
+    assert e.value.code == 4
+    ops.k_quant_encode(k, 0.1, bits=2, want_size=False)           # codes up to 11 do not fit 2 bits
+    with pytest.raises(ops.PackKVError) as e:
+        ops.encode_status(cuda, bits=2)
+    assert e.value.code == 1
+    odd = torch.empty(B * H * T * 128 + 1, dtype=torch.uint8, device=cuda)[1:]
+    with pytest.raises(ops.PackKVError) as e:
+        ops.k_quant_encode(k, 0.1, stream=odd)
+    assert e.value.code == 2 and "even address" in str(e.value)
+    codes = torch.zeros(64, 128, dtype=torch.uint8, device=cuda)
+    with pytest.raises(RuntimeError, match="even address"):
+        ops.k_encode(codes, odd, torch.zeros(1, 2, dtype=torch.uint32, device=cuda))
