@@ -28,6 +28,8 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
 DEFAULT_TRAFFIC_BYTES = int((208383 * (262144 / 131088) + 2176 * 1.0) * 1024)
+TRAFFIC_SOURCE = ("recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measurement of this workload "
+                  "(profiles/attn_dma_kernel_config1.md), not observed by this run")
 
 
 def parse():
@@ -80,11 +82,15 @@ def event_time_ms(torch, fn, iters):
     return s.elapsed_time(e) / iters
 
 
-def cpu_baseline(torch, args, k1, v1, q1):
+def cpu_baseline(torch, args, k1, v1, q1, threads=None, passes=5, warm=2):
     """Decompress-then-attend for a sample of the sequences in PyTorch CPU ops (the checker's restatement of
-    utils/compute.py:173-179 + models/llama.py:189-212), median of 5 after 2 warm-ups, scaled to the batch:
-    about ten seconds of host work at the default workload."""
+    utils/compute.py:173-179 + models/llama.py:189-212), median of `passes` after `warm` warm-ups, scaled to the
+    batch: about ten seconds of host work at the default workload.  threads: torch's thread count for the
+    measurement (None = all the cores torch uses by default)."""
     from oracle import quant as oq
+    all_threads = torch.get_num_threads()
+    if threads:
+        torch.set_num_threads(threads)
     ck, zk, sk = oq.quant_ints(k1, 64, args.rel)
     cv, zv, sv = oq.quant_ints(v1, 64, args.rel)
     qq = q1.unsqueeze(2)
@@ -93,21 +99,23 @@ def cpu_baseline(torch, args, k1, v1, q1):
         kd, vd = oq.dequant(ck, zk, sk), oq.dequant(cv, zv, sv)
         return oq.eager_attention(qq, kd, vd)
 
-    for _ in range(2):
+    for _ in range(warm):
         step()
     ts = []
-    for _ in range(5):
+    for _ in range(passes):
         t0 = time.perf_counter()
         step()
         ts.append(time.perf_counter() - t0)
     ts.sort()
     n = k1.shape[0]
     per_seq = ts[len(ts) // 2] / n
+    used = torch.get_num_threads()
+    torch.set_num_threads(all_threads)
     return {
-        "value": per_seq * args.batch * 1e6, "unit": "us/layer", "cores": torch.get_num_threads(),
+        "value": per_seq * args.batch * 1e6, "unit": "us/layer", "cores": used,
         "kind": "port",
-        "sample": "%d of %d sequences (dequantise + eager attention, %d tokens each), median of 5 passes, scaled x%g"
-                  % (n, args.batch, k1.shape[2], args.batch / n),
+        "sample": "%d of %d sequences (dequantise + eager attention, %d tokens each), median of %d passes, scaled x%g"
+                  % (n, args.batch, k1.shape[2], passes, args.batch / n),
     }
 
 
@@ -145,7 +153,7 @@ def decode_loop(torch, args, dev):
     torch.cuda.reset_peak_memory_stats()
     for layer in range(L):
         k, v = synth.make_kv(B, Hkv, T, seed=layer, device=dev)
-        cache.update(k, v, layer)
+        cache.update(k, v, layer, return_dense=False)
         del k, v
     torch.cuda.synchronize()
     q = synth.make_q(B, Hq, seed=1, device=dev)
@@ -154,7 +162,7 @@ def decode_loop(torch, args, dev):
 
     def token():
         for layer in range(L):
-            cache.update(kn, vn, layer)
+            cache.update(kn, vn, layer, return_dense=False)
             cache.attend(q, layer, out=outs[layer])
 
     def algo_bytes():
@@ -169,6 +177,7 @@ def decode_loop(torch, args, dev):
         token()
     torch.cuda.synchronize()
     bytes_step = algo_bytes()
+    comp0, win0, seq0 = cache.layers[0].k.tokens, cache.layers[0].win_len, cache.get_seq_length(0)   # at the start of timing
     t0 = time.perf_counter()
     for _ in range(args.steps):
         token()
@@ -181,8 +190,7 @@ def decode_loop(torch, args, dev):
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%d layers, batch %d, %d q / %d KV heads, head_dim 128, %d cached tokens per sequence "
                                "(%d compressed + %d in the 16-bit window at the start of timing), rel %.3g; a step appends "
-                               "one token to every layer and attends" % (L, B, Hq, Hkv, T, lay0.k.tokens,
-                                                                         T - lay0.k.tokens, args.rel)},
+                               "one token to every layer and attends" % (L, B, Hq, Hkv, seq0, comp0, win0, args.rel)},
         "tokens_per_s": B / (us_token * 1e-6),
         "roofline": {"bound": "hbm", "achieved": bytes_step / (us_token * 1e-6) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": bytes_step / (us_token * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
@@ -400,6 +408,18 @@ def main():
     def step():
         ops.attn_decode(q, ke, ve, kw, vw, out=out, variant=args.variant)
 
+    # Before anything is timed: the kernel under test against the library's plain kernel (variant 1: unpack to a code
+    # tile, fp32 arithmetic) on the whole batch -- both evaluate the same exact formula, so they may differ by the
+    # fast kernel's fp16 weights and one output rounding only.  A broken kernel is not timed.
+    step()
+    plain = ops.attn_decode(q, ke, ve, kw, vw, variant=1)
+    diff = (out.float() - plain.float()).abs()
+    bound = 1e-3 + 2.0 ** -9 * plain.float().abs()
+    sanity = {"max_abs_diff_vs_plain_kernel": float(diff.max()), "ok": bool((diff <= bound).all())}
+    if not sanity["ok"] or not bool(torch.isfinite(out.float()).all()):
+        raise SystemExit("bench: the attention kernel disagrees with the plain kernel: %r" % (sanity,))
+    del plain, diff, bound
+
     preheat_steps = 0
     t_end = time.perf_counter() + args.preheat_ms * 1e-3
     while time.perf_counter() < t_end:
@@ -436,7 +456,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": algo_bytes / (ms_kernel * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": algo_bytes / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": DEFAULT_TRAFFIC_BYTES if default_workload else None,
+                     "traffic_source": TRAFFIC_SOURCE if default_workload else None,
                      "kernel_ms": ms_kernel, "algorithmic_bytes": algo_bytes},
+        "sanity": sanity,
         "compression": {"k_bytes": ke["size"], "v_bytes": ve["size"], "fp16_bytes": fp16_bytes,
                         "ratio_k": fp16_bytes / 2 / ke["size"], "ratio_v": fp16_bytes / 2 / ve["size"]},
     }
@@ -525,6 +547,8 @@ def main():
         ns = min(B, 16)
         k1, v1, q1 = kc[:ns].cpu(), vc[:ns].cpu(), q[:ns].cpu()
         result["cpu_baseline"] = cpu_baseline(torch, args, k1, v1, q1)
+        # the same path on one host thread, on one sequence (a few seconds)
+        result["cpu_baseline_1thread"] = cpu_baseline(torch, args, k1[:1], v1[:1], q1[:1], threads=1, passes=3, warm=1)
         result["cpu_encode"] = cpu_encoder(torch, args, k1[:1])
     else:
         result["cpu_baseline"] = None

@@ -164,6 +164,54 @@ def test_attn_decode_full_size_property(cuda):
     assert err <= 1e-3 * want.abs().max().item() + 2 ** -11 * want.abs().max().item() + 2e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_long_context_layer_at_its_own_size(cuda, dtype):
+    """One layer of the long-context configuration at its own size -- batch 4, 32 query / 8 KV heads, 131072 cached
+    tokens per sequence, 1 GiB each of K and V -- where the oracle is far too slow; size-independent properties
+    instead: (i) the fused encoders' streams unpack to the codes of the stand-alone quantizer (which the small tests
+    hold bit-exact against the oracle), K and V; (ii) a query of zeros weighs all tokens alike, so the output is the
+    mean of the dequantised V; (iii) the last 128 tokens handed over as a 16-bit window holding their dequantised
+    values give the output of the all-compressed cache up to the contract; (iv) the stream sizes add up
+    (offsets = running sums of sizes, the last block ends the stream)."""
+    B, Hq, Hkv, T = 4, 32, 8, 131072
+    k, v = synth.make_kv(B, Hkv, T, seed=330, dtype=dtype, device=cuda)
+    hidden = B * Hkv * 128
+    ke, ve = ops.k_quant_encode(k, 0.1), ops.v_quant_encode(v, 0.1)
+    codes = torch.empty(T, hidden, dtype=torch.uint8, device=cuda)
+    deq = {}
+    for name, x, e, dec, cb, hb in (("K", k, ke, ops.k_decode, 64, 128), ("V", v, ve, ops.v_decode, 128, 64)):
+        _say("long context", dtype, name, "stream", e["size"], "bytes, ratio %.2f" % (x.numel() * 2 / e["size"]))
+        dec(e["stream"], e["info"], codes, cb, hb, e["bits"])
+        scale, zero = ops.quant_params(x, 0.1)
+        want_codes, _ = ops.quantize(x, scale, zero)
+        assert torch.equal(scale.view(torch.int16), e["scale"].view(torch.int16))
+        assert torch.equal(zero.view(torch.int16), e["zero"].view(torch.int16))
+        assert torch.equal(codes, want_codes)                                                       # (i)
+        del want_codes
+        info = e["info"].view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+        assert int(info[0, 0]) == 0 and bool((info[1:, 0] == info[:-1, 0] + info[:-1, 1]).all())    # (iv)
+        assert int(info[-1, 0] + info[-1, 1]) == e["size"]
+        deq[name] = ops.dequantize(codes, e["scale"], e["zero"], B, Hkv)
+    del k, v, codes
+    q0 = torch.zeros(B, Hq, 128, dtype=dtype, device=cuda)
+    got = ops.attn_decode(q0, ke, ve).float()
+    want = deq["V"].float().mean(dim=2).repeat_interleave(Hq // Hkv, dim=1)
+    half_ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    err = (got - want).abs()
+    _say("   zero-query mean-of-V: max err %.3e, max|ref| %.3e" % (err.max().item(), want.abs().max().item()))
+    assert bool((err <= 5e-4 + 1.05 * half_ulp * want.abs() + 2.0 ** -9 * want.abs().max()).all())      # (ii)
+    # (iii) all tokens compressed against [T - 128 compressed | the last 128 as a 16-bit window of their dequantised
+    # values]: the same numbers reach the kernel both ways, up to the 16-bit rounding of 128 tokens
+    q = synth.make_q(B, Hq, seed=331, dtype=dtype, device=cuda)
+    full = ops.attn_decode(q, ke, ve, out_f32=True)
+    kw, vw = deq["K"][:, :, T - 128:].contiguous(), deq["V"][:, :, T - 128:].contiguous()
+    ke_c, ve_c = dict(ke, tokens=T - 128, heads=Hkv), dict(ve, tokens=T - 128, heads=Hkv)
+    part = ops.attn_decode(q, ke_c, ve_c, kw, vw, out_f32=True)
+    err = (part - full).abs()
+    _say("   compressed + window vs all compressed: max err %.3e, max|ref| %.3e" % (err.max().item(), full.abs().max().item()))
+    assert bool((err <= 2e-3 + 1e-3 * full.abs()).all())
+
+
 def test_attn_decode_replays_in_a_hip_graph(cuda):
     """A decode step launches only kernels on the caller's stream (no memset nodes), and while a stream is capturing it
     allocates nothing: a capture stream that has no scratch of its own yet (torch captures on a side stream) keeps its
