@@ -250,6 +250,28 @@ __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01,
     }
 }
 
+// The usual case of quant4 for fp16 (sub2 != 0) on its own, for rounds whose 16 tokens all take it (one test per
+// round instead of one branch per token).  The first product x * r reads the fp16 x directly (v_fma_mix_f32 with
+// -0 as the addend: x * r + (-0) is the product, sign of zero included), which saves the conversion of x.
+__device__ __forceinline__ void quant4_f16_fast(uint2 xw, const TokPar tp, uint32_t &c01, uint32_t &c23) {
+    const uint32_t negzero = 0x80000000u;
+    float q0[4];
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(q0[0]) : "v"(xw.x), "v"(tp.r), "s"(negzero));
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(q0[1]) : "v"(xw.x), "v"(tp.r), "s"(negzero));
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(q0[2]) : "v"(xw.y), "v"(tp.r), "s"(negzero));
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(q0[3]) : "v"(xw.y), "v"(tp.r), "s"(negzero));
+    const f16x2 x01 = __builtin_bit_cast(f16x2, xw.x), x23 = __builtin_bit_cast(f16x2, xw.y);
+    const float f[4] = {(float)x01[0], (float)x01[1], (float)x23[0], (float)x23[1]};
+    _Float16 h[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) h[i] = (_Float16)__fmaf_rn(__fmaf_rn(-tp.s, q0[i], f[i]), tp.r, q0[i]);
+    const f16x2 h01 = {h[0], h[1]}, h23 = {h[2], h[3]};
+    const f16x2 add = __builtin_bit_cast(f16x2, tp.add2);
+    const u16x2 sub = as_u16x2(tp.sub2);
+    c01 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h01 + add)) - sub));
+    c23 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h23 + add)) - sub));
+}
+
 // bit_length of both 16-bit halves, clamped to 4 (values above 15 mean the codes overflow the
 // format; the launch reports that through max_code)
 __device__ __forceinline__ uint32_t pk_bitlen4(uint32_t d) {
@@ -316,6 +338,88 @@ __device__ __forceinline__ void minmax8(const uint4 v, float &mn, float &mx) {
     }
 }
 
+struct TokPar;
+template <int DT> __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits);
+
+// min and max over the 16 lanes of a row of the wavefront (every lane gets the results): the exchanges are DPP
+// operands of the min / max instructions themselves (quad permutes, then the half-row and row mirrors).
+__device__ __forceinline__ void row16_minmax(float &mn, float &mx) {
+    // (written out: the compiler keeps the exchanges as separate moves; a VGPR written by a VALU instruction must be
+    // two instructions old before a DPP operand reads it, which the interleaving and the s_nop provide)
+    asm("s_nop 1\n\t"
+        "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_min_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_min_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf"
+        : "+v"(mn), "+v"(mx));
+}
+// packed fp16 min / max as the instructions themselves (the builtins first quieten every operand with an extra
+// instruction; the instructions ignore quiet NaNs as the builtins do)
+__device__ __forceinline__ f16x2 pk_min_h(f16x2 a, f16x2 b) {
+    f16x2 r;
+    asm("v_pk_min_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ f16x2 pk_max_h(f16x2 a, f16x2 b) {
+    f16x2 r;
+    asm("v_pk_max_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
+// Token parameters of one round of the round-major encoders.  256 threads per 16 tokens: thread (tt = token, l16)
+// reads 8 channels of every head (heads beyond H - 1 repeat the last: a repeated row changes no min / max); lane
+// l16 == 0 writes the token's scale and zero and its constants for quant4.  `rows` is x at (sequence, head 0, the
+// round's first token) and uniform, so the eight loads are one 32-bit lane offset on eight scalar bases.
+template <int DT>
+__device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
+                                                   uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
+    const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;          // bytes
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)min(i, H - 1) * head_stride) + lane_off);
+    float mn, mx;
+    if (DT == PKV_F16) {               // packed fp16 comparisons all the way down to one word each
+        f16x2 lo[8], hi[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const f16x2 a = __builtin_bit_cast(f16x2, v[i].x), b = __builtin_bit_cast(f16x2, v[i].y),
+                        c = __builtin_bit_cast(f16x2, v[i].z), d = __builtin_bit_cast(f16x2, v[i].w);
+            lo[i] = pk_min_h(pk_min_h(a, b), pk_min_h(c, d));
+            hi[i] = pk_max_h(pk_max_h(a, b), pk_max_h(c, d));
+        }
+#pragma unroll
+        for (int w = 4; w >= 1; w >>= 1)
+#pragma unroll
+            for (int i = 0; i < w; i++) {
+                lo[i] = pk_min_h(lo[i], lo[i + w]);
+                hi[i] = pk_max_h(hi[i], hi[i + w]);
+            }
+        mn = fminf((float)lo[0][0], (float)lo[0][1]);
+        mx = fmaxf((float)hi[0][0], (float)hi[0][1]);
+    } else {
+        mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+    }
+    row16_minmax(mn, mx);
+    if (l16 == 0) {
+        const float range = round_t<DT>(mx - mn);
+        const float sc = round_t<DT>(range * rel);
+        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+        *scale_out = (uint16_t)T16<DT>::to_bits(sc);
+        *zero_out = (uint16_t)zb;
+        *par_out = token_par<DT>(sc, zb);
+    }
+}
+
 __device__ __forceinline__ void cell_load(const uint16_t *xc, uint2 xr[16]) {
 #pragma unroll
     for (int k = 0; k < 16; k++) xr[k] = *reinterpret_cast<const uint2 *>(xc + (size_t)k * kHeadDim);
@@ -350,12 +454,23 @@ __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
     return tp;
 }
 
+// True (uniformly) when all 16 tokens of the round at `par` (LDS) take the usual case of quant4.
+__device__ __forceinline__ bool round_all_fast(const TokPar *par) {
+    const uint32_t sub2 = par[threadIdx.x & 15].sub2;
+    return !__any(sub2 == 0u);
+}
+
 // The four packs of a loaded cell (rows xr, the 16 tokens' constants at par): words, minima, widths.
 template <int DT>
 __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par, UnitPacks &u, uint32_t &cmax) {
     uint32_t c01[16], c23[16];
+    if (DT == PKV_F16 && round_all_fast(par)) {
 #pragma unroll
-    for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+        for (int k = 0; k < 16; k++) quant4_f16_fast(xr[k], par[k], c01[k], c23[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+    }
     uint32_t mn01, mn23, len01, len23, mx01, mx23;
     build_pair(c01, mn01, len01, mx01, u.word[0], u.word[1]);
     build_pair(c23, mn23, len23, mx23, u.word[2], u.word[3]);
@@ -418,8 +533,13 @@ __device__ __forceinline__ void build_pair_wide(const uint32_t c[16], uint32_t &
 template <int DT>
 __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par, UnitPacksW &u, uint32_t &cmax) {
     uint32_t c01[16], c23[16];
+    if (DT == PKV_F16 && round_all_fast(par)) {
 #pragma unroll
-    for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+        for (int k = 0; k < 16; k++) quant4_f16_fast(xr[k], par[k], c01[k], c23[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+    }
     uint32_t mn01, mn23, len01, len23, mx01, mx23;
     build_pair_wide(c01, mn01, len01, mx01, u.lo[0], u.hi[0], u.lo[1], u.hi[1]);
     build_pair_wide(c23, mn23, len23, mx23, u.lo[2], u.hi[2], u.lo[3], u.hi[3]);
@@ -771,27 +891,9 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
-            float mn = INFINITY, mx = -INFINITY;
-            uint4 v[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                v[i] = *reinterpret_cast<const uint4 *>(
-                    x + (((size_t)b * H + min(i, H - 1)) * T + tok0 + 16 * r + tt) * kHeadDim + l16 * 8);
-#pragma unroll
-            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
-#pragma unroll
-            for (int d = 8; d >= 1; d >>= 1) {
-                mn = fminf(mn, __shfl_xor(mn, d, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, d, 16));
-            }
-            if (l16 == 0) {
-                const float range = round_t<DT>(mx - mn);
-                const float sc = round_t<DT>(range * rel);
-                const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-                scale[(size_t)b * par_stride + tok0 + 16 * r + tt] = (uint16_t)T16<DT>::to_bits(sc);
-                zero[(size_t)b * par_stride + tok0 + 16 * r + tt] = (uint16_t)zb;
-                s_par[tt] = token_par<DT>(sc, zb);
-            }
+            const size_t tok = (size_t)b * par_stride + tok0 + 16 * r + tt;
+            round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
+                                   scale + tok, zero + tok, s_par + tt);
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
         uint2 xr[16];
@@ -967,27 +1069,9 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
-            float mn = INFINITY, mx = -INFINITY;
-            uint4 v[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                v[i] = *reinterpret_cast<const uint4 *>(
-                    x + (((size_t)b * H + min(i, H - 1)) * T + tok0 + 32 * it + tt) * kHeadDim + l16 * 8);
-#pragma unroll
-            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
-#pragma unroll
-            for (int d = 8; d >= 1; d >>= 1) {
-                mn = fminf(mn, __shfl_xor(mn, d, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, d, 16));
-            }
-            if (l16 == 0) {
-                const float range = round_t<DT>(mx - mn);
-                const float sc = round_t<DT>(range * rel);
-                const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-                scale[(size_t)b * par_stride + tok0 + 32 * it + tt] = (uint16_t)T16<DT>::to_bits(sc);
-                zero[(size_t)b * par_stride + tok0 + 32 * it + tt] = (uint16_t)zb;
-                s_par[tt] = token_par<DT>(sc, zb);
-            }
+            const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + tt;
+            round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
+                                   scale + tok, zero + tok, s_par + tt);
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
         uint2 xr[16];
