@@ -269,7 +269,7 @@ def pack_sweep(torch, H, T, dev, rels=SWEEP_RELS, packs=SWEEP_PACKS, time_codec=
     [0.1, 10], V ~ N(0, 1).  For every error bound (one per code width) the tensors are quantised once; every
     (pack size, repacking method) is then priced with the reference's size model (`repack_and_encode`,
     utils/compute.py:329-357: integers, so the ratios are the reference's wherever its token order is defined),
-    and the real block codec (16-token packs) is timed on the same codes."""
+    and the real block codec is run and timed on the same codes at every pack length."""
     from packkv_amd import ops, synth
     hid = H * 128
     k, v = kv if kv is not None else synth.make_kv(1, H, T, seed=2, device=dev, k_mode="channel_scale")
@@ -291,28 +291,33 @@ def pack_sweep(torch, H, T, dev, rels=SWEEP_RELS, packs=SWEEP_PACKS, time_codec=
                 rows.append({"rel": rel, "bits": bits, "pack": pack, "method": method, "block": bs,
                              "k_bytes": k_aft, "v_bytes": v_aft, "k_cr": fp16 / k_aft, "v_cr": fp16 / v_aft})
         if time_codec:
-            stream = torch.empty(2 * T * hid + 4096, dtype=torch.uint8, device=dev)
-            ik = torch.empty((T // 64) * H, 2, dtype=torch.uint32, device=dev)
-            iv = torch.empty((T // 128) * H * 2, 2, dtype=torch.uint32, device=dev)
+            # the real block codec at every pack length (16 = the reference's format; longer packs = this build's
+            # extension of it): stream bytes - 8 per block equal the size model's bytes of the "none" rows above
             back = torch.empty_like(kc)
-            k_size = ops.k_encode(kc, stream, ik, 64, 128, bits)
-            ke = event_time_ms(torch, lambda: ops.k_encode(kc, stream, ik, 64, 128, bits, want_size=False), 10)
-            kd = event_time_ms(torch, lambda: ops.k_decode(stream, ik, back, 64, 128, bits), 10)
-            assert torch.equal(back, kc)
-            v_size = ops.v_encode(vc, stream, iv, 128, 64, bits)
-            ve = event_time_ms(torch, lambda: ops.v_encode(vc, stream, iv, 128, 64, bits, want_size=False), 10)
-            vd = event_time_ms(torch, lambda: ops.v_decode(stream, iv, back, 128, 64, bits), 10)
-            assert torch.equal(back, vc)
             gbs = lambda ms: T * hid / (ms * 1e-3) / 1e9
-            codec.append({"rel": rel, "bits": bits, "k_stream_bytes": k_size, "v_stream_bytes": v_size,
-                          "k_cr": fp16 / k_size, "v_cr": fp16 / v_size,
-                          "k_encode_gbs_codes": gbs(ke), "v_encode_gbs_codes": gbs(ve),
-                          "k_decode_gbs_codes": gbs(kd), "v_decode_gbs_codes": gbs(vd)})
+            for pack in packs:
+                if T % (8 * pack):
+                    continue
+                row = {"rel": rel, "bits": bits, "pack": pack}
+                for name, is_k, mat in (("k", True, kc), ("v", False, vc)):
+                    ctx_blk, hid_blk = ops.long_block_shape(is_k, pack)
+                    nblk = (T // ctx_blk) * (hid // hid_blk)
+                    stream = torch.empty(nblk * ops.block_bound_p(pack, bits), dtype=torch.uint8, device=dev)
+                    info = torch.empty(nblk, 2, dtype=torch.uint32, device=dev)
+                    size = ops.encode_p(is_k, mat, stream, info, pack, bits)
+                    enc = event_time_ms(torch, lambda: ops.encode_p(is_k, mat, stream, info, pack, bits, want_size=False), 10)
+                    dec = event_time_ms(torch, lambda: ops.decode_p(is_k, stream, info, back, pack, bits), 10)
+                    assert torch.equal(back, mat)
+                    model = [r for r in rows if r["rel"] == rel and r["pack"] == pack and r["method"] == "none"][0]
+                    assert size - 8 * nblk == model[name + "_bytes"], (rel, pack, name)
+                    row.update({name + "_stream_bytes": size, name + "_cr": fp16 / size,
+                                name + "_encode_gbs_codes": gbs(enc), name + "_decode_gbs_codes": gbs(dec)})
+                codec.append(row)
     return {"metric": "repack + bit-pack sweep", "n_gpus": 1, "data": "synthetic", "dtype": "u8",
             "config": {"workload": "configs[2]: %d KV heads x 128 x %d tokens, K per-channel scale log-uniform in "
                                    "[0.1, 10], V ~ N(0, 1); sizes by the reference's size model (payload + pack "
                                    "metadata, no quantiser parameters), ratios against fp16" % (H, T)},
-            "rows": rows, "codec_16_token_packs": codec}
+            "rows": rows, "codec": codec}
 
 
 def gemv_surface(torch, ops, synth, dev):

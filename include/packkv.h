@@ -82,6 +82,29 @@ int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *cod
 int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
 
+/* ---- packs longer than 16 tokens ------------------------------------------------------
+ * The block codec for pack_len in {32, 64, 128, 256} tokens: an extension of the stream format.  No counterpart in the
+ * reference's codec, which fixes PACK_ELE_NUM = 16 (packkv_cuda_ext/include/static_def.h:6); they realise what the
+ * reference only prices, bit_pack(tensor, pack_len) (utils/compute.py:272-297): the stream holds 8 bytes per block
+ * plus exactly that model's bytes.  A pack is pack_len consecutive tokens of one channel, its word
+ * sum_k (code_k - min) << ((pack_len - 1 - k) * len) stored as pack_len * len / 8 little-endian bytes; K blocks are
+ * 4 pack_len tokens x 128 channels, V blocks 8 pack_len tokens x 64 channels (ctx_len / hidden_dim must be
+ * multiples), units, metadata arrays and payload order as in the 16-token format; the four u16 cumulative unit sizes
+ * of a block header count 4-byte words.  codes: uint8 [ctx_len, hidden_dim] (4-byte aligned for K); block_info:
+ * uint32 [n_blocks, 2]; bits 2..8; the stream starts at an even address.  pack_len 16 forwards to the functions
+ * above with the reference's block shapes (64 x 128, 128 x 64).  The decoders take the stream's size and skip blocks
+ * whose block_info row or header points outside it. */
+int pkv_k_encode_p(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, uint64_t *size_out, float *ms_out, pkv_stream_t s);
+int pkv_v_encode_p(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, uint64_t *size_out, float *ms_out, pkv_stream_t s);
+int pkv_k_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s);
+int pkv_v_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s);
+/* Worst-case bytes of one block with packs of pack_len tokens (K and V blocks both hold 512 packs). */
+uint64_t pkv_block_bound_p(int pack_len, int bits);
+
 /* ---- per-token affine quantizer ------------------------------------------------------
  * Device counterpart of quant_ints(..., QuantMode.TokenQuant) and of the dequantisation
  * (code + zero) * scale (utils/compute.py:84-112, :173-179): x is [B, H, T, 128] in

@@ -99,3 +99,43 @@ def ref():
 
 def block_bound(is_k, ctx_blk, hid_blk, W):
     return int(oracle().lib.pkv_oracle_block_bound(int(is_k), ctx_blk, hid_blk, W))
+
+
+# ---- packs longer than 16 tokens (this build's extension of the format; see packkv_oracle.c) ----
+
+def long_block_bound(pack_len, W):
+    lib = oracle().lib
+    lib.pkv_oracle_long_block_bound.restype = ctypes.c_uint64
+    lib.pkv_oracle_long_block_bound.argtypes = [ctypes.c_int] * 2
+    return int(lib.pkv_oracle_long_block_bound(pack_len, W))
+
+
+def long_encode(is_k, codes, pack_len, W):
+    """codes uint8 [ctx_len, hidden] -> (stream, block_info [n_blocks, 2], size) with packs of `pack_len` tokens:
+    K blocks of 4 pack_len x 128, V blocks of 8 pack_len x 64."""
+    lib = oracle().lib
+    lib.pkv_oracle_long_encode.restype = ctypes.c_uint64
+    lib.pkv_oracle_long_encode.argtypes = [ctypes.c_int, _u8p, _u8p, ctypes.c_uint64, _u32p] + [ctypes.c_int] * 4
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    ctx_len, hidden = codes.shape
+    nblk = (ctx_len // ((4 if is_k else 8) * pack_len)) * (hidden // (128 if is_k else 64))
+    stream = np.zeros(nblk * long_block_bound(pack_len, W), dtype=np.uint8)
+    info = np.zeros((nblk, 2), dtype=np.uint32)
+    size = lib.pkv_oracle_long_encode(int(is_k), codes.ctypes.data_as(_u8p), stream.ctypes.data_as(_u8p), stream.size,
+                                      info.ctypes.data_as(_u32p), ctx_len, hidden, pack_len, W)
+    if size == 2 ** 64 - 1:
+        raise RuntimeError("not supported")
+    return stream, info, int(size)
+
+
+def long_decode(is_k, stream, info, ctx_len, hidden, pack_len, W):
+    lib = oracle().lib
+    lib.pkv_oracle_long_decode.restype = ctypes.c_int
+    lib.pkv_oracle_long_decode.argtypes = [ctypes.c_int, _u8p, _u32p, _u8p] + [ctypes.c_int] * 4
+    stream = np.ascontiguousarray(stream, dtype=np.uint8)
+    info = np.ascontiguousarray(info, dtype=np.uint32)
+    out = np.zeros((ctx_len, hidden), dtype=np.uint8)
+    if lib.pkv_oracle_long_decode(int(is_k), stream.ctypes.data_as(_u8p), info.ctypes.data_as(_u32p),
+                                  out.ctypes.data_as(_u8p), ctx_len, hidden, pack_len, W) != 0:
+        raise RuntimeError("not supported")
+    return out

@@ -293,6 +293,159 @@ int pkv_oracle_decode(int is_k, const uint8_t *stream, const uint32_t *block_inf
     return 0;
 }
 
+/* ------------------------------------------------- packs longer than 16 tokens --
+ *
+ * FORMAT EXTENSION of this build (the reference fixes PACK_ELE_NUM = 16, include/static_def.h:6, and only its
+ * analytic size model, utils/compute.py:272-297, knows other pack lengths).  No reference exists for it -- parity
+ * unpinned; it is pinned by the definition below restated with big integers in the tests, by the closed-form size
+ * (stream bytes - 8 per block == the size model's bytes), by round trips, and by P = 16 reproducing the format above.
+ *
+ * A pack is P consecutive tokens of one channel, P in {16, 32, 64, 128, 256}; min and len as before over the P
+ * tokens; word = sum_k (code_k - min) << ((P-1-k) * len), P * len bits, stored as its low P * len / 8 bytes,
+ * little-endian (so the last 16 tokens of the pack come first in the stream).  Everything else scales with it: a
+ * K block is 4 rounds of P tokens x 128 channels, a V block 2 warps x 2 segments of 4 slots of P tokens (8 P
+ * tokens x 64 channels); metadata arrays and payload order as above.  The header keeps four u16 cumulative unit
+ * sizes; for P >= 32 they count 4-byte words (every unit size is then a multiple of 4), since a unit can exceed
+ * 65535 / 4 bytes.
+ */
+static void long_stats(const uint8_t *codes, size_t row_stride, size_t tok0, size_t ch, int P,
+                       unsigned *mn_out, int *len_out) {
+    unsigned mn = 255, mx = 0;
+    for (int k = 0; k < P; k++) {
+        unsigned c = codes[(tok0 + k) * row_stride + ch];
+        if (c < mn) mn = c;
+        if (c > mx) mx = c;
+    }
+    *mn_out = mn;
+    *len_out = bit_length(mx - mn);
+}
+
+/* payload bytes of one pack at dst (zeroed by the caller); returns their count */
+static size_t long_put(uint8_t *dst, const uint8_t *codes, size_t row_stride, size_t tok0, size_t ch, int P,
+                       unsigned mn, int len) {
+    for (int k = 0; k < P; k++)
+        put_bits(dst, (size_t)(P - 1 - k) * len, len, codes[(tok0 + k) * row_stride + ch] - mn);
+    return (size_t)P * len / 8;
+}
+
+static size_t long_get(const uint8_t *src, uint8_t *codes, size_t row_stride, size_t tok0, size_t ch, int P,
+                       unsigned mn, int len) {
+    for (int k = 0; k < P; k++)
+        codes[(tok0 + k) * row_stride + ch] = (uint8_t)(get_bits(src, (size_t)(P - 1 - k) * len, len) + mn);
+    return (size_t)P * len / 8;
+}
+
+static void put_cum(uint8_t *hdr, int idx, size_t cum, int P) {
+    unsigned v = (unsigned)(P == 16 ? cum : cum / 4);
+    hdr[2 * idx] = (uint8_t)(v & 0xFF);
+    hdr[2 * idx + 1] = (uint8_t)((v >> 8) & 0xFF);
+}
+
+/* Unit u of a block (K: round u; V: warp u / 2, segment u % 2): pack (lane t, slot i) -> first token, channel. */
+static void long_pack_at(int is_k, int u, int t, int i, int P, size_t *tok0, size_t *ch) {
+    if (is_k) { *tok0 = (size_t)u * P; *ch = (size_t)(t * 4 + i); }
+    else { *tok0 = (size_t)((u % V_SEGS) * V_SLOTS + i) * P; *ch = (size_t)((u / V_SEGS) * LANES + t); }
+}
+
+size_t pkv_oracle_long_block_encode(int is_k, const uint8_t *codes, size_t row_stride, int P, int W, uint8_t *out,
+                                    size_t out_cap) {
+    const int LB = len_field_bits(W);
+    const size_t mins_bytes = (size_t)W * 128 / 8, lens_bytes = (size_t)LB * 128 / 8;
+    size_t off = 8, cum = 0;
+    for (int u = 0; u < 4; u++) {
+        uint8_t *mins = out + off, *lens = mins + mins_bytes, *payload = lens + lens_bytes;
+        memset(mins, 0, mins_bytes + lens_bytes);
+        size_t pay = 0;
+        for (int i = 0; i < 4; i++) {           /* payload order: slot-major, lane-minor */
+            for (int t = 0; t < LANES; t++) {
+                size_t tok0, ch; unsigned mn; int len;
+                long_pack_at(is_k, u, t, i, P, &tok0, &ch);
+                long_stats(codes, row_stride, tok0, ch, P, &mn, &len);
+                put_bits(mins, (size_t)(t * 4 + i) * W, W, mn);
+                put_bits(lens, (size_t)(t * 4 + i) * LB, LB, (unsigned)len);
+                if ((size_t)(payload - out) + pay + (size_t)P * len / 8 > out_cap) return 0;
+                memset(payload + pay, 0, (size_t)P * len / 8);
+                pay += long_put(payload + pay, codes, row_stride, tok0, ch, P, mn, len);
+            }
+        }
+        cum += mins_bytes + lens_bytes + pay;
+        put_cum(out, u, cum, P);
+        off += mins_bytes + lens_bytes + pay;
+    }
+    return off;
+}
+
+void pkv_oracle_long_block_decode(int is_k, const uint8_t *in, int P, int W, uint8_t *codes, size_t row_stride) {
+    const int LB = len_field_bits(W);
+    const size_t mins_bytes = (size_t)W * 128 / 8, lens_bytes = (size_t)LB * 128 / 8;
+    size_t off = 8;
+    for (int u = 0; u < 4; u++) {
+        const uint8_t *mins = in + off, *lens = mins + mins_bytes, *payload = lens + lens_bytes;
+        size_t pay = 0;
+        for (int i = 0; i < 4; i++) {
+            for (int t = 0; t < LANES; t++) {
+                size_t tok0, ch;
+                long_pack_at(is_k, u, t, i, P, &tok0, &ch);
+                unsigned mn = get_bits(mins, (size_t)(t * 4 + i) * W, W);
+                int len = (int)get_bits(lens, (size_t)(t * 4 + i) * LB, LB);
+                pay += long_get(payload + pay, codes, row_stride, tok0, ch, P, mn, len);
+            }
+        }
+        off += mins_bytes + lens_bytes + pay;
+    }
+}
+
+static int check_long(int is_k, int ctx_len, int hidden_dim, int P, int W) {
+    if (W < 2 || W > 8) return -1;
+    if (P != 16 && P != 32 && P != 64 && P != 128 && P != 256) return -1;
+    if (ctx_len <= 0 || hidden_dim <= 0) return -1;
+    if (ctx_len % ((is_k ? 4 : 8) * P) || hidden_dim % (is_k ? 128 : 64)) return -1;
+    return 0;
+}
+
+/* Whole tensor with packs of P tokens: K blocks of 4 P x 128, V blocks of 8 P x 64, in (context block, hidden block)
+ * order.  Returns the stream size in bytes, or (uint64_t)-1 for an unsupported shape or a stream buffer too small. */
+uint64_t pkv_oracle_long_encode(int is_k, const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
+                                int ctx_len, int hidden_dim, int P, int W) {
+    if (check_long(is_k, ctx_len, hidden_dim, P, W)) return (uint64_t)-1;
+    const int ctx_blk = (is_k ? 4 : 8) * P, hid_blk = is_k ? 128 : 64;
+    const int n_ctx = ctx_len / ctx_blk, n_hid = hidden_dim / hid_blk;
+    uint64_t total = 0;
+    for (int cb = 0; cb < n_ctx; cb++) {
+        for (int hb = 0; hb < n_hid; hb++) {
+            const uint8_t *tile = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+            size_t sz = pkv_oracle_long_block_encode(is_k, tile, (size_t)hidden_dim, P, W, stream + total,
+                                                     (size_t)(capacity - total));
+            if (!sz) return (uint64_t)-1;
+            size_t idx = (size_t)cb * n_hid + hb;
+            block_info[2 * idx] = (uint32_t)total;
+            block_info[2 * idx + 1] = (uint32_t)sz;
+            total += sz;
+        }
+    }
+    return total;
+}
+
+int pkv_oracle_long_decode(int is_k, const uint8_t *stream, const uint32_t *block_info, uint8_t *codes,
+                           int ctx_len, int hidden_dim, int P, int W) {
+    if (check_long(is_k, ctx_len, hidden_dim, P, W)) return -1;
+    const int ctx_blk = (is_k ? 4 : 8) * P, hid_blk = is_k ? 128 : 64;
+    const int n_ctx = ctx_len / ctx_blk, n_hid = hidden_dim / hid_blk;
+    for (int cb = 0; cb < n_ctx; cb++)
+        for (int hb = 0; hb < n_hid; hb++) {
+            size_t idx = (size_t)cb * n_hid + hb;
+            pkv_oracle_long_block_decode(is_k, stream + block_info[2 * idx], P, W,
+                                         codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk,
+                                         (size_t)hidden_dim);
+        }
+    return 0;
+}
+
+/* Worst case of one block with packs of P tokens: header, metadata of 512 packs, every pack at full width. */
+uint64_t pkv_oracle_long_block_bound(int P, int W) {
+    return 8ull + 4ull * (uint64_t)(W + len_field_bits(W)) * 128 / 8 + 512ull * (uint64_t)P * W / 8;
+}
+
 /* Worst-case bytes one block can take (every pack at full width W). */
 uint64_t pkv_oracle_block_bound(int is_k, int ctx_blk, int hid_blk, int W) {
     const int LB = len_field_bits(W);

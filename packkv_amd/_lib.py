@@ -43,6 +43,11 @@ SIGNATURES = {
     "pkv_k_encode": (_i, [_vp, _vp, _u64, _vp, _i, _i, _i, _i, _i, _u64p, _fp, _vp]),
     "pkv_v_encode": (_i, [_vp, _vp, _u64, _vp, _i, _i, _i, _i, _i, _u64p, _fp, _vp]),
     "pkv_encode_status": (_i, [_vp, _i, _u64p]),
+    "pkv_k_encode_p": (_i, [_vp, _vp, _u64, _vp, _i, _i, _i, _i, _u64p, _fp, _vp]),
+    "pkv_v_encode_p": (_i, [_vp, _vp, _u64, _vp, _i, _i, _i, _i, _u64p, _fp, _vp]),
+    "pkv_k_decode_p": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_v_decode_p": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_block_bound_p": (_u64, [_i, _i]),
     "pkv_k_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_v_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_quant_params": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _vp, _fp, _vp]),

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libpackkv_hip.so")
-SOURCES = ["pkv_runtime.hip", "pkv_codec.hip", "pkv_quant.hip", "pkv_legacy.hip", "pkv_attn.hip", "pkv_repack.hip", "pkv_cache.hip"]
+SOURCES = ["pkv_runtime.hip", "pkv_codec.hip", "pkv_codec_long.hip", "pkv_quant.hip", "pkv_legacy.hip", "pkv_attn.hip", "pkv_repack.hip", "pkv_cache.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # keep the compiler from forming packed-fp32 VALU ops

@@ -1,0 +1,374 @@
+// Block codec for packs LONGER than 16 tokens (32, 64, 128, 256): an extension of the stream format with no
+// counterpart in the reference, whose codec fixes PACK_ELE_NUM = 16 (packkv_cuda_ext/include/static_def.h:6) while
+// its analytic size model prices any pack length (utils/compute.py:272-297).  These kernels make that model's
+// numbers real: stream bytes - 8 per block equal the model's bytes for the same codes, pack length and width.
+//
+// The format scales the reference's with the pack length P:
+//   pack     P consecutive tokens of one channel; min, len = bit_length(max - min) over the P tokens;
+//            word = sum_k (code_k - min) << ((P - 1 - k) * len), stored as its low P * len / 8 bytes, little-endian
+//            -- i.e. P / 16 sub-words of the reference's shape, the LAST 16 tokens first;
+//   K block  4 P tokens x 128 channels: four units (rounds of P tokens); V block 8 P tokens x 64 channels: four
+//            units (warp, segment) of 4 slots of P tokens x 32 channels; unit = mins | lens | payload with the
+//            metadata bit arrays and the slot-major, lane-minor payload order of the reference's format;
+//   header   four u16 cumulative unit sizes, counted in 4-byte words for P >= 32 (every unit size is then a
+//            multiple of 4; in bytes a unit of 256-token packs would not fit 16 bits).
+// One workgroup of 128 threads per block, one 32-lane half-wavefront per unit, lane t <-> 4 packs.  The encoder
+// reads the block's codes twice (minima / widths, then the words; the second time from L2), obtains the block's
+// offset by the same ticket + look-back as the 16-token codec and writes the words straight into the stream.
+#include "pkv_block.hpp"
+#include "pkv_runtime.hpp"
+
+namespace pkv {
+
+// (first token, channel) of pack (unit u, lane t, slot i) relative to the block's first token and channel
+template <bool IS_K>
+__device__ __forceinline__ void long_pack_at(int u, int t, int i, int P, int &tok0, int &ch) {
+    if (IS_K) { tok0 = u * P; ch = 4 * t + i; }
+    else { tok0 = ((u & 1) * 4 + i) * P; ch = (u >> 1) * kLanes + t; }
+}
+
+// the 2 * len bytes of one 16-token sub-word: codes c[0..15] (min already subtracted)
+__device__ __forceinline__ void long_put_sub(uint16_t *dst, const uint32_t c[16], uint32_t len) {
+    uint64_t hi = 0, lo = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        hi = (hi << len) | c[k];
+        lo = (lo << len) | c[8 + k];
+    }
+    unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
+    for (uint32_t q = 0; q < len; q++) {
+        dst[q] = (uint16_t)wd;
+        wd >>= 16;
+    }
+}
+
+__device__ __forceinline__ void long_get_sub(const uint16_t *src, uint32_t c[16], uint32_t len) {
+    unsigned __int128 wd = 0;
+    for (uint32_t q = 0; q < len; q++) wd |= (unsigned __int128)src[q] << (16u * q);
+    const uint64_t lo = (uint64_t)(wd & (((unsigned __int128)1 << (8u * len)) - 1));
+    const uint64_t hi = (uint64_t)(wd >> (8u * len));
+    const uint32_t mask = (1u << len) - 1u;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        c[k] = (uint32_t)(hi >> ((7 - k) * len)) & mask;
+        c[8 + k] = (uint32_t)(lo >> ((7 - k) * len)) & mask;
+    }
+}
+
+// OR lane t's 4 * nbits-bit metadata word into the LSB-first bit array `arr` (dword-aligned LDS, zeroed)
+__device__ __forceinline__ void long_put_meta(uint32_t *arr, int t, int nbits, uint32_t w) {
+    const uint32_t bit = (uint32_t)t * 4u * (uint32_t)nbits;
+    const uint32_t sh = bit & 31u;
+    atomicOr(arr + (bit >> 5), w << sh);
+    if (sh + 4u * (uint32_t)nbits > 32u) atomicOr(arr + (bit >> 5) + 1, w >> (32u - sh));
+}
+
+constexpr int kLongMetaWords = 52;      // 16 * (8 + 4) bytes of metadata at most, and a dword of slack for reads
+
+template <bool IS_K>
+__global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                                                        uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                                                        int hidden_dim, int P, int W, uint32_t nblocks) {
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t s_unit[4];
+    __shared__ uint32_t s_meta[4][kLongMetaWords];
+    const int tid = threadIdx.x, u = tid >> 5, t = tid & 31;
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t b = s_idx;
+    if (b >= nblocks) return;
+    const int hid_blk = IS_K ? 128 : 64, ctx_blk = (IS_K ? 4 : 8) * P;
+    const int n_hid = hidden_dim / hid_blk;
+    const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+    const uint8_t *tile = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+
+    // ---- minima and widths of the lane's four packs ----
+    uint32_t mn[4], len[4];
+    if (IS_K) {     // one dword per token row holds the four channels
+        const uint8_t *col = tile + (size_t)(u * P) * hidden_dim + 4 * t;
+        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+        u16x2 amn2 = {255, 255}, amx2 = {0, 0}, bmn2 = {255, 255}, bmx2 = {0, 0};   // channels (0, 2) and (1, 3) as 16-bit pairs
+        for (int k = 0; k < P; k += 8) {
+            uint32_t d[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) d[q] = *reinterpret_cast<const uint32_t *>(col + (size_t)(k + q) * hidden_dim);
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const u16x2 a = __builtin_bit_cast(u16x2, d[q] & 0x00FF00FFu), c = __builtin_bit_cast(u16x2, (d[q] >> 8) & 0x00FF00FFu);
+                amn2 = __builtin_elementwise_min(amn2, a);
+                amx2 = __builtin_elementwise_max(amx2, a);
+                bmn2 = __builtin_elementwise_min(bmn2, c);
+                bmx2 = __builtin_elementwise_max(bmx2, c);
+            }
+        }
+        const uint32_t amn = __builtin_bit_cast(uint32_t, amn2), amx = __builtin_bit_cast(uint32_t, amx2),
+                       bmn = __builtin_bit_cast(uint32_t, bmn2), bmx = __builtin_bit_cast(uint32_t, bmx2);
+        mn[0] = amn & 0xFFFFu; mn[2] = amn >> 16; mn[1] = bmn & 0xFFFFu; mn[3] = bmn >> 16;
+        len[0] = (uint32_t)bit_length_u32((amx & 0xFFFFu) - mn[0]);
+        len[2] = (uint32_t)bit_length_u32((amx >> 16) - mn[2]);
+        len[1] = (uint32_t)bit_length_u32((bmx & 0xFFFFu) - mn[1]);
+        len[3] = (uint32_t)bit_length_u32((bmx >> 16) - mn[3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int tok0, ch;
+            long_pack_at<false>(u, t, i, P, tok0, ch);
+            const uint8_t *col = tile + (size_t)tok0 * hidden_dim + ch;
+            uint32_t lo = 255u, hi = 0u;
+            for (int k = 0; k < P; k += 8) {
+                uint32_t c[8];
+#pragma unroll
+                for (int q = 0; q < 8; q++) c[q] = col[(size_t)(k + q) * hidden_dim];
+#pragma unroll
+                for (int q = 0; q < 8; q++) { lo = min(lo, c[q]); hi = max(hi, c[q]); }
+            }
+            mn[i] = lo;
+            len[i] = (uint32_t)bit_length_u32(hi - lo);
+        }
+    }
+    // byte offsets of the packs inside the unit's payload: those of 16-token packs times P / 16
+    uint32_t off[4], payload;
+    pack_offsets(len, off, payload);
+    const uint32_t nsub = (uint32_t)P / 16u;
+    payload *= nsub;
+    if (t == 0) s_unit[u] = meta + payload;
+    // metadata bit arrays, assembled in LDS (each half-wavefront its own area)
+    uint32_t *area = s_meta[u];
+    area[t] = 0u;
+    if (t < kLongMetaWords - 32) area[32 + t] = 0u;
+    {
+        uint32_t minsw = 0, lensw = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            minsw |= (mn[i] & ((1u << W) - 1u)) << (i * W);
+            lensw |= len[i] << (i * g.LB);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        long_put_meta(area, t, W, minsw);
+        long_put_meta(area + g.mins_bytes / 4, t, g.LB, lensw);
+    }
+    __syncthreads();
+    const uint32_t bytes = 8u + s_unit[0] + s_unit[1] + s_unit[2] + s_unit[3];
+    if (tid == 0) lookback_publish(st, b, bytes);
+    if (tid < 64) {
+        const uint64_t o = lookback_offset(st, b, bytes, true);
+        if (tid == 0) {
+            s_off = o;
+            info[2 * (size_t)b] = (uint32_t)o;
+            info[2 * (size_t)b + 1] = bytes;
+            if (b == nblocks - 1) st->total = o + bytes;
+            if (o + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t o = s_off;
+    if (o + bytes > capacity) return;
+    uint8_t *dst_blk = stream + o;
+    if (tid < 4) {
+        uint32_t cum = 0;
+        for (int q = 0; q <= tid; q++) cum += s_unit[q];
+        reinterpret_cast<uint16_t *>(dst_blk)[tid] = (uint16_t)(P == 16 ? cum : cum >> 2);
+    }
+    uint32_t ustart = 8u;
+    for (int q = 0; q < u; q++) ustart += s_unit[q];
+    uint8_t *dst_u = dst_blk + ustart;
+    for (uint32_t q = (uint32_t)t; q < meta / 2u; q += 32u)
+        reinterpret_cast<uint16_t *>(dst_u)[q] = reinterpret_cast<const uint16_t *>(area)[q];
+    // ---- the words: sub-word s of a pack holds its tokens P - 16 (s + 1) .. P - 16 s - 1 ----
+    uint8_t *pay = dst_u + meta;
+    if (IS_K) {
+        for (uint32_t s = 0; s < nsub; s++) {
+            const uint8_t *row = tile + (size_t)(u * P + P - 16 * (int)(s + 1)) * hidden_dim + 4 * t;
+            uint32_t d[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) d[k] = *reinterpret_cast<const uint32_t *>(row + (size_t)k * hidden_dim);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t c[16];
+#pragma unroll
+                for (int k = 0; k < 16; k++) c[k] = ((d[k] >> (8 * i)) & 0xFFu) - mn[i];
+                long_put_sub(reinterpret_cast<uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int tok0, ch;
+            long_pack_at<false>(u, t, i, P, tok0, ch);
+            for (uint32_t s = 0; s < nsub; s++) {
+                const uint8_t *col = tile + (size_t)(tok0 + P - 16 * (int)(s + 1)) * hidden_dim + ch;
+                uint32_t c[16];
+#pragma unroll
+                for (int k = 0; k < 16; k++) c[k] = (uint32_t)col[(size_t)k * hidden_dim] - mn[i];
+                long_put_sub(reinterpret_cast<uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+            }
+        }
+    }
+}
+
+template <bool IS_K>
+__global__ void __launch_bounds__(128) unpack_long_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+                                                          uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
+                                                          uint64_t stream_bytes) {
+    __shared__ uint32_t s_meta[4][kLongMetaWords];
+    const int tid = threadIdx.x, u = tid >> 5, t = tid & 31;
+    const uint32_t b = blockIdx.x;
+    const int hid_blk = IS_K ? 128 : 64, ctx_blk = (IS_K ? 4 : 8) * P;
+    const int n_hid = hidden_dim / hid_blk;
+    const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+    uint8_t *tile = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const uint64_t boff = info[2 * (size_t)b];
+    const uint32_t bsize = info[2 * (size_t)b + 1];
+    // a block_info row that points outside the stream decodes nothing (the codes of the block stay as they are)
+    if (boff + bsize > stream_bytes || bsize < 8u + 4u * meta) return;
+    const uint16_t *hdr = reinterpret_cast<const uint16_t *>(stream + boff);
+    const uint32_t gran = P == 16 ? 1u : 4u;
+    const uint32_t ustart = 8u + (u ? (uint32_t)hdr[u - 1] * gran : 0u);
+    const uint32_t uend = 8u + (uint32_t)hdr[u] * gran;
+    const bool sane = ustart + meta <= uend && uend <= bsize;      // uniform per half-wavefront
+    uint32_t *area = s_meta[u];
+    const uint8_t *src_u = stream + boff + ustart;
+    if (sane)
+        for (uint32_t q = (uint32_t)t; q < meta / 2u; q += 32u)
+            reinterpret_cast<uint16_t *>(area)[q] = reinterpret_cast<const uint16_t *>(src_u)[q];
+    __syncthreads();
+    if (!sane) return;
+    const uint32_t minsw = lds_meta_word(reinterpret_cast<const uint8_t *>(area), t, W);
+    const uint32_t lensw = lds_meta_word(reinterpret_cast<const uint8_t *>(area) + g.mins_bytes, t, g.LB);
+    uint32_t mn[4], len[4], off[4], payload;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        mn[i] = (minsw >> (i * W)) & ((1u << W) - 1u);
+        len[i] = min((lensw >> (i * g.LB)) & ((1u << g.LB) - 1u), (uint32_t)kMaxBits);
+    }
+    pack_offsets(len, off, payload);
+    const uint32_t nsub = (uint32_t)P / 16u;
+    if (ustart + meta + payload * nsub > uend) return;             // (uniform) widths that overrun the unit
+    const uint8_t *pay = src_u + meta;
+    if (IS_K) {
+        for (uint32_t s = 0; s < nsub; s++) {
+            uint32_t d[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) d[k] = 0u;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t c[16];
+                long_get_sub(reinterpret_cast<const uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+#pragma unroll
+                for (int k = 0; k < 16; k++) d[k] |= ((c[k] + mn[i]) & 0xFFu) << (8 * i);
+            }
+            uint8_t *row = tile + (size_t)(u * P + P - 16 * (int)(s + 1)) * hidden_dim + 4 * t;
+#pragma unroll
+            for (int k = 0; k < 16; k++) *reinterpret_cast<uint32_t *>(row + (size_t)k * hidden_dim) = d[k];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int tok0, ch;
+            long_pack_at<false>(u, t, i, P, tok0, ch);
+            for (uint32_t s = 0; s < nsub; s++) {
+                uint32_t c[16];
+                long_get_sub(reinterpret_cast<const uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+                uint8_t *col = tile + (size_t)(tok0 + P - 16 * (int)(s + 1)) * hidden_dim + ch;
+#pragma unroll
+                for (int k = 0; k < 16; k++) col[(size_t)k * hidden_dim] = (uint8_t)(c[k] + mn[i]);
+            }
+        }
+    }
+}
+
+static int check_long(bool is_k, const void *codes, const void *stream, const void *info, int ctx_len, int hidden_dim,
+                      int P, int bits) {
+    PKV_REQUIRE(codes && stream && info, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(P == 32 || P == 64 || P == 128 || P == 256, PKV_ERR_UNSUPPORTED,
+                "not supported: pack_len %d (16, 32, 64, 128 or 256 tokens)", P);
+    PKV_REQUIRE(bits >= 2 && bits <= kMaxBits, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (2..8)", bits);
+    PKV_REQUIRE(ctx_len > 0 && hidden_dim > 0, PKV_ERR_INVALID, "sizes must be positive");
+    PKV_REQUIRE(ctx_len % ((is_k ? 4 : 8) * P) == 0, PKV_ERR_INVALID,
+                "ctx_len must be divisible by the block's tokens (%d packs of pack_len)", is_k ? 4 : 8);
+    PKV_REQUIRE(hidden_dim % (is_k ? 128 : 64) == 0, PKV_ERR_INVALID, "hidden_dim must be divisible by %d", is_k ? 128 : 64);
+    PKV_REQUIRE((reinterpret_cast<uintptr_t>(stream) & 1u) == 0, PKV_ERR_INVALID,
+                "compressed_buffer must start at an even address (blocks are written in 2-byte units)");
+    PKV_REQUIRE(!is_k || (reinterpret_cast<uintptr_t>(codes) & 3u) == 0, PKV_ERR_INVALID,
+                "the code matrix must start at a 4-byte boundary");
+    return PKV_OK;
+}
+
+static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *info, int ctx_len,
+                         int hidden_dim, int P, int bits, uint64_t *size_out, float *ms_out, hipStream_t s) {
+    int rc = check_long(is_k, codes, stream, info, ctx_len, hidden_dim, P, bits);
+    if (rc) return rc;
+    PKV_REQUIRE(capacity > 0, PKV_ERR_INVALID, "compressed_buffer must be a non-empty tensor");
+    if (capacity > (1ull << 32)) capacity = 1ull << 32;          // block_info offsets are 32 bits: never wrapped
+    const uint32_t nblocks = (uint32_t)(ctx_len / ((is_k ? 4 : 8) * P)) * (uint32_t)(hidden_dim / (is_k ? 128 : 64));
+    ScanState *st = nullptr;
+    if ((rc = prepare_scan_state(nblocks, &st, s))) return rc;
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    if (is_k) pack_long_kernel<true><<<nblocks, 128, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    else pack_long_kernel<false><<<nblocks, 128, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    PKV_HIP_CHECK(hipGetLastError());
+    if ((rc = tm.end(ms_out))) return rc;
+    return finish_encode(st, size_out, 0, s);
+}
+
+static int run_unpack_long(bool is_k, const uint8_t *stream, uint64_t stream_bytes, const uint32_t *info, uint8_t *codes,
+                           int ctx_len, int hidden_dim, int P, int bits, float *ms_out, hipStream_t s) {
+    int rc = check_long(is_k, codes, stream, info, ctx_len, hidden_dim, P, bits);
+    if (rc) return rc;
+    const uint32_t nblocks = (uint32_t)(ctx_len / ((is_k ? 4 : 8) * P)) * (uint32_t)(hidden_dim / (is_k ? 128 : 64));
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    if (is_k) unpack_long_kernel<true><<<nblocks, 128, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    else unpack_long_kernel<false><<<nblocks, 128, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    PKV_HIP_CHECK(hipGetLastError());
+    return tm.end(ms_out);
+}
+
+}  // namespace pkv
+
+extern "C" {
+
+int pkv_k_encode_p(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, uint64_t *size_out, float *ms_out, pkv_stream_t s) {
+    if (pack_len == 16)
+        return pkv_k_encode(codes, stream, capacity, block_info, ctx_len, hidden_dim, 64, 128, bits, size_out, ms_out, s);
+    return pkv::run_pack_long(true, codes, stream, capacity, block_info, ctx_len, hidden_dim, pack_len, bits, size_out,
+                              ms_out, (hipStream_t)s);
+}
+
+int pkv_v_encode_p(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, uint64_t *size_out, float *ms_out, pkv_stream_t s) {
+    if (pack_len == 16)
+        return pkv_v_encode(codes, stream, capacity, block_info, ctx_len, hidden_dim, 128, 64, bits, size_out, ms_out, s);
+    return pkv::run_pack_long(false, codes, stream, capacity, block_info, ctx_len, hidden_dim, pack_len, bits, size_out,
+                              ms_out, (hipStream_t)s);
+}
+
+int pkv_k_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s) {
+    if (pack_len == 16)
+        return pkv_k_decode(stream, block_info, codes, ctx_len, hidden_dim, 64, 128, bits, ms_out, s);
+    return pkv::run_unpack_long(true, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, pack_len, bits, ms_out,
+                                (hipStream_t)s);
+}
+
+int pkv_v_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+                   int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s) {
+    if (pack_len == 16)
+        return pkv_v_decode(stream, block_info, codes, ctx_len, hidden_dim, 128, 64, bits, ms_out, s);
+    return pkv::run_unpack_long(false, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, pack_len, bits, ms_out,
+                                (hipStream_t)s);
+}
+
+uint64_t pkv_block_bound_p(int pack_len, int bits) {
+    if (pack_len < 16 || bits < 2 || bits > pkv::kMaxBits) return 0;
+    return 8ull + 4ull * (uint64_t)(bits + pkv::len_field_bits(bits)) * 16ull + 512ull * (uint64_t)pack_len * (uint64_t)bits / 8ull;
+}
+
+}  // extern "C"

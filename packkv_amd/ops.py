@@ -204,6 +204,62 @@ def v_decode(stream, info, codes, ctx_blk=128, hid_blk=64, bits=4, timed=False):
     return _decode(False, stream, info, codes, codes.size(0), codes.size(1), ctx_blk, hid_blk, bits, timed, MAX_BITS)
 
 
+# ---- packs longer than 16 tokens (an extension of the format: the reference only prices them, utils/compute.py:272-297) ----
+
+PACK_LENS = (16, 32, 64, 128, 256)
+
+
+def long_block_shape(is_k, pack_len):
+    """(tokens, channels) of a block with packs of `pack_len` tokens: the reference's 64 x 128 / 128 x 64 scaled."""
+    return ((4 * pack_len, 128) if is_k else (8 * pack_len, 64))
+
+
+def block_bound_p(pack_len, bits):
+    return int(_lib.load().pkv_block_bound_p(pack_len, bits))
+
+
+def _check_long(is_k, codes, stream, info, pack_len, bits):
+    _require(pack_len in PACK_LENS, "not supported: pack_len %d (16, 32, 64, 128 or 256)" % pack_len)
+    ctx_blk, hid_blk = long_block_shape(is_k, pack_len)
+    _require(codes.dim() == 2 and codes.dtype == torch.uint8, "quant_ints_tensor must be a 2-D UInt8 tensor")
+    _require(codes.size(0) % ctx_blk == 0, "ctx_len must be divisible by %d (the block's tokens at this pack_len)" % ctx_blk)
+    _require(codes.size(1) % hid_blk == 0, "hidden_dim must be divisible by hidden_dim_block_size")
+    nblk = (codes.size(0) // ctx_blk) * (codes.size(1) // hid_blk)
+    _require(info.dim() == 2 and info.size(0) == nblk and info.size(1) == 2, "block_info_buffer block num mismatch")
+    _require(stream.dtype == torch.uint8 and stream.numel() > 0, "compressed_buffer must be a non-empty UInt8 tensor")
+    _require(info.dtype == torch.uint32, "block_info_buffer must be a UInt32 tensor")
+    _require(2 <= bits <= MAX_BITS, "bits_len must be 2..%d" % MAX_BITS)
+    _require(codes.is_cuda and stream.is_cuda and info.is_cuda, "tensors must be on the GPU")
+    _require(codes.is_contiguous() and stream.is_contiguous() and info.is_contiguous(), "tensors must be contiguous")
+    _require(stream.data_ptr() % 2 == 0, "compressed_buffer must start at an even address")
+
+
+def encode_p(is_k, codes, stream, info, pack_len, bits, want_size=True, timed=False):
+    """Encode a uint8 code matrix [ctx_len, hidden] with packs of `pack_len` tokens (16 = the reference's format with
+    its block shapes).  Returns the stream size (and ms)."""
+    _check_long(is_k, codes, stream, info, pack_len, bits)
+    dev = _device_of(codes, stream, info)
+    size, ms = ctypes.c_uint64(0), ctypes.c_float(0.0)
+    fn = _lib.load().pkv_k_encode_p if is_k else _lib.load().pkv_v_encode_p
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(codes), _ptr(stream), stream.numel(), _ptr(info), codes.size(0), codes.size(1), pack_len, bits,
+                ctypes.byref(size) if want_size else None, ctypes.byref(ms) if timed else None, _stream(dev))
+    _lib.check(rc)
+    return (int(size.value), float(ms.value)) if timed else int(size.value)
+
+
+def decode_p(is_k, stream, info, codes, pack_len, bits, timed=False):
+    _check_long(is_k, codes, stream, info, pack_len, bits)
+    dev = _device_of(codes, stream, info)
+    ms = ctypes.c_float(0.0)
+    fn = _lib.load().pkv_k_decode_p if is_k else _lib.load().pkv_v_decode_p
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(stream), stream.numel(), _ptr(info), _ptr(codes), codes.size(0), codes.size(1), pack_len, bits,
+                ctypes.byref(ms) if timed else None, _stream(dev))
+    _lib.check(rc)
+    return float(ms.value) if timed else None
+
+
 # --------------------------------------------------------------- quantizer -----------
 
 def _check_x(x):

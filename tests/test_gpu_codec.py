@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import codec
+from oracle import quant as oq
 from packkv_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -217,3 +218,93 @@ def test_wide_codes_stream_matches_restatement(cuda, oracle_codec, W):
         back = torch.zeros_like(d)
         (ops.k_decode if is_k else ops.v_decode)(stream, info, back, cb, hb, W)
         assert torch.equal(back, d)
+
+
+# ---- packs longer than 16 tokens (this build's extension of the format; the oracle's restatement of it is pinned
+# on the CPU by tests/test_oracle_codec.py) ---------------------------------------------------------------------
+
+def _gpu_encode_p(cuda, is_k, c, P, W):
+    ctx_blk, hid_blk = ops.long_block_shape(is_k, P)
+    nblk = (c.shape[0] // ctx_blk) * (c.shape[1] // hid_blk)
+    d_codes = torch.from_numpy(c).to(cuda)
+    d_stream = torch.zeros(nblk * ops.block_bound_p(P, W), dtype=torch.uint8, device=cuda)
+    d_info = torch.zeros(nblk, 2, dtype=torch.uint32, device=cuda)
+    size = ops.encode_p(is_k, d_codes, d_stream, d_info, P, W)
+    return d_codes, d_stream, d_info, size
+
+
+@pytest.mark.parametrize("is_k", [1, 0])
+@pytest.mark.parametrize("P", [32, 64, 128, 256])
+def test_long_packs_bit_exact_vs_oracle(cuda, oracle_codec, is_k, P):
+    rng = np.random.default_rng(500 + 10 * is_k + P)
+    ctx_blk, hid_blk = ops.long_block_shape(is_k, P)
+    for W in (2, 3, 4, 5, 6, 7, 8):
+        for kind in ("uniform", "const", "narrow", "gauss"):
+            T, H = ctx_blk * (3 if P <= 64 else 2), hid_blk * 5
+            _say("long-pack case", "K" if is_k else "V", "pack", P, "bits", W, kind, (T, H))
+            c = _rand_codes(rng, T, H, W, kind)
+            so, io, zo = codec.long_encode(is_k, c, P, W)
+            d_codes, d_stream, d_info, size = _gpu_encode_p(cuda, is_k, c, P, W)
+            assert size == zo
+            assert np.array_equal(d_info.cpu().numpy(), io)
+            assert np.array_equal(d_stream[:size].cpu().numpy(), so[:zo])
+            assert size - 8 * len(io) == oq.bit_pack_bytes(c, P, W)
+            back = torch.full_like(d_codes, 0xEE)
+            ops.decode_p(is_k, d_stream, d_info, back, P, W)
+            assert torch.equal(back, d_codes)
+            # the oracle's stream decodes on the GPU too
+            back.fill_(0xEE)
+            ops.decode_p(is_k, torch.from_numpy(so).to(cuda), torch.from_numpy(io).to(cuda), back, P, W)
+            assert torch.equal(back, d_codes)
+
+
+def test_long_packs_of_16_tokens_forward_to_the_reference_format(cuda, oracle_codec):
+    rng = np.random.default_rng(77)
+    for is_k, (cb, hb) in ((1, (64, 128)), (0, (128, 64))):
+        c = _rand_codes(rng, 256, 512, 4, "gauss")
+        so, io, zo = oracle_codec.encode(is_k, c, cb, hb, 4)
+        d_codes, d_stream, d_info, size = _gpu_encode_p(cuda, is_k, c, 16, 4)
+        assert size == zo and np.array_equal(d_info.cpu().numpy(), io)
+        assert np.array_equal(d_stream[:size].cpu().numpy(), so[:zo])
+        back = torch.zeros_like(d_codes)
+        ops.decode_p(is_k, d_stream, d_info, back, 16, 4)
+        assert torch.equal(back, d_codes)
+
+
+def test_long_packs_sweep_layer_round_trip_and_size_model(cuda):
+    """The sweep's layer (8 KV heads x 128 x 16384 tokens) at every pack length: round trip, and stream bytes - 8 per
+    block equal to the size model with the pack widths counted on the GPU (ops.code_stats, itself checked against the
+    oracle in tests/test_gpu_repack.py)."""
+    g = torch.Generator().manual_seed(3)
+    for W in (3, 4, 6):
+        c = torch.clamp(torch.round(torch.randn(16384, 1024, generator=g) * 1.5 + (1 << (W - 1))), 0, (1 << W) - 1).to(torch.uint8).to(cuda)
+        for P in (32, 64, 128, 256):
+            for is_k in (1, 0):
+                ctx_blk, hid_blk = ops.long_block_shape(is_k, P)
+                nblk = (16384 // ctx_blk) * (1024 // hid_blk)
+                stream = torch.empty(nblk * ops.block_bound_p(P, W), dtype=torch.uint8, device=cuda)
+                info = torch.empty(nblk, 2, dtype=torch.uint32, device=cuda)
+                size = ops.encode_p(is_k, c, stream, info, P, W)
+                len_sum, _ = ops.code_stats(c, P)                 # sum of the packs' widths, counted on the GPU
+                lb = max(1, int(W).bit_length())
+                assert size - 8 * nblk == (len_sum * P + (16384 // P) * 1024 * (W + lb)) // 8, (W, P, is_k)
+                back = torch.zeros_like(c)
+                ops.decode_p(is_k, stream, info, back, P, W)
+                assert torch.equal(back, c), (W, P, is_k)
+
+
+def test_long_pack_argument_checks(cuda):
+    c = torch.zeros(1024, 128, dtype=torch.uint8, device=cuda)
+    stream = torch.zeros(1 << 20, dtype=torch.uint8, device=cuda)
+    with pytest.raises(Exception):
+        ops.encode_p(1, c, stream, torch.zeros(2, 2, dtype=torch.uint32, device=cuda), 48, 4)      # pack length
+    with pytest.raises(Exception):
+        ops.encode_p(1, c[:1000], stream, torch.zeros(1, 2, dtype=torch.uint32, device=cuda), 256, 4)   # tokens
+    with pytest.raises(Exception):
+        ops.encode_p(1, c, stream[:64], torch.zeros(1, 2, dtype=torch.uint32, device=cuda), 256, 4)   # capacity
+    # a block_info row that points outside the stream decodes nothing and faults nothing
+    info = torch.tensor([[1 << 30, 4096]], dtype=torch.int64).to(torch.uint32).to(cuda)
+    out = torch.full_like(c, 7)
+    ops.decode_p(1, stream, info, out, 256, 4)
+    torch.cuda.synchronize()
+    assert int(out.min()) == 7 and int(out.max()) == 7

@@ -220,18 +220,18 @@ def test_repacked_cache_attends_like_the_original(cuda):
 
 def test_pack_sweep_rows_match_restatement(cuda):
     """The sweep mode of bench.py (pack sizes x code widths x repacking methods on one layer) on a small layer:
-    every row's sizes equal the restated size model on the restated quantiser's codes, and the real codec's stream
-    of 16-token packs is the analytic payload plus its own metadata and block headers."""
+    every row's sizes equal the restated size model on the restated quantiser's codes, and the real codec's stream at
+    every pack length (bench.py asserts it while it runs) is that model's bytes plus 8 per block."""
     import importlib.util
     import os
     spec = importlib.util.spec_from_file_location("bench_mod", os.path.join(os.path.dirname(__file__), "..", "bench.py"))
     bench = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(bench)
-    H, T = 2, 512
+    H, T = 2, 2048
     k, v = synth.make_kv(1, H, T, seed=2, k_mode="channel_scale")
     rels, packs = (0.2, 0.05, 0.0125), (16, 64, 256)
     res = bench.pack_sweep(torch, H, T, cuda, rels=rels, packs=packs, kv=(k.to(cuda), v.to(cuda)))
-    assert len(res["rows"]) == len(rels) * len(packs) * 3 and len(res["codec_16_token_packs"]) == len(rels)
+    assert len(res["rows"]) == len(rels) * len(packs) * 3 and len(res["codec"]) == len(rels) * len(packs)
     mats = {}
     for rel in rels:
         ck, _, _ = oq.quant_ints(k, 64, rel)
@@ -243,5 +243,8 @@ def test_pack_sweep_rows_match_restatement(cuda):
         want = orp.repack_and_encode(kc, vc, row["pack"], row["method"], row["block"])
         assert (row["k_bytes"], row["v_bytes"]) == (want[2], want[3])
         assert row["bits"] >= int(max(kc.max(), vc.max())).bit_length()
-    for c in res["codec_16_token_packs"]:
+    for c in res["codec"]:
+        none = [r for r in res["rows"] if (r["rel"], r["pack"], r["method"]) == (c["rel"], c["pack"], "none")][0]
+        nk, nv = (T // (4 * c["pack"])) * H, (T // (8 * c["pack"])) * 2 * H
+        assert (c["k_stream_bytes"] - 8 * nk, c["v_stream_bytes"] - 8 * nv) == (none["k_bytes"], none["v_bytes"])
         assert c["k_cr"] > 1.0 and c["v_cr"] > 1.0 and c["k_decode_gbs_codes"] > 0
