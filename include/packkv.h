@@ -176,6 +176,25 @@ int pkv_window_append(const void *k_new, const void *v_new, const void *cos, con
  *   of the token's V codes over all hidden_dim channels.  Equal medians keep their original order
  *   (the reference leaves that order to torch.sort's backend).  perm[blk * block_size + r] is
  *   the index inside the block of the token that moves to position r. */
+/* Median repacking inside the fused encode (north-star "quantize, token repack, bit-pack" as one encode; reference
+ * order utils/compute.py:329-357: quantise, repack, bit-pack): no code matrix is formed.
+ * pkv_median_order: the permutation pkv_median_repack would produce for V [B, H, T, 128] quantised at `rel` -- the
+ *   medians are counted straight from V (every value quantised in registers).  H <= 8, bits 2..6.  scale_out /
+ *   zero_out (both or neither; [B, T] of V's type) receive V's per-token parameters as pkv_quant_params writes them.
+ * pkv_{k,v}_quant_encode_perm: pkv_{k,v}_quant_encode on the tokens in that order: position p of the stream, of
+ *   block_info's blocks and of scale / zero holds token (p / perm_block) * perm_block + perm[p] of x (perm_block a
+ *   multiple of 64 that divides T).  The stream equals pkv_quant_params + pkv_quantize + pkv_median_repack +
+ *   pkv_{k,v}_encode.  H <= 8.  The V form takes the parameters pkv_median_order wrote (scale_in / zero_in, [B, T]
+ *   in the order of x; both NULL: computed again) and then reads V once instead of going over every row twice.
+ *   No counterpart in the reference, which repacks only to price the packs. */
+int pkv_median_order(const void *v, int dtype, int B, int H, int T, float rel, int bits, int block_size, uint32_t *perm,
+                     void *scale_out, void *zero_out, float *ms_out, pkv_stream_t s);
+int pkv_k_quant_encode_perm(const void *x, int dtype, int B, int H, int T, float rel, int bits, const uint32_t *perm,
+                            int perm_block, uint8_t *stream, uint64_t capacity, uint32_t *block_info, void *scale,
+                            void *zero, uint64_t *size_out, float *ms_out, pkv_stream_t s);
+int pkv_v_quant_encode_perm(const void *x, int dtype, int B, int H, int T, float rel, int bits, const uint32_t *perm,
+                            int perm_block, const void *scale_in, const void *zero_in, uint8_t *stream, uint64_t capacity,
+                            uint32_t *block_info, void *scale, void *zero, uint64_t *size_out, float *ms_out, pkv_stream_t s);
 int pkv_bit_pack_size(const uint8_t *codes, int ctx_len, int hidden_dim, int pack_len, uint64_t *len_sum_out,
                       uint32_t *n_unique_out, float *ms_out, pkv_stream_t s);
 int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,

@@ -53,6 +53,9 @@ SIGNATURES = {
     "pkv_quant_params": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _vp, _fp, _vp]),
     "pkv_quantize": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _fp, _vp]),
     "pkv_dequantize": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _fp, _vp]),
+    "pkv_median_order": (_i, [_vp, _i, _i, _i, _i, _f, _i, _i, _vp, _vp, _vp, _fp, _vp]),
+    "pkv_k_quant_encode_perm": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
+    "pkv_v_quant_encode_perm": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _i, _vp, _vp, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
     "pkv_k_quant_encode": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
     "pkv_v_quant_encode": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _vp, _vp, _vp, _u64p, _fp, _vp]),
     "pkv_k_quant_encode_append": (_i, [_vp, _i, _i, _i, _i, _f, _i, _vp, _u64, _u64, _vp, _vp, _vp, _i, _u64p, _fp, _vp]),

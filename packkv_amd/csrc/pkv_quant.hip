@@ -339,7 +339,7 @@ __device__ __forceinline__ void minmax8(const uint4 v, float &mn, float &mx) {
 }
 
 struct TokPar;
-template <int DT> __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits);
+template <int DT> __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits, bool general_form = false);
 
 // min and max over the 16 lanes of a row of the wavefront (every lane gets the results): the exchanges are DPP
 // operands of the min / max instructions themselves (quad permutes, then the half-row and row mirrors).
@@ -416,7 +416,7 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
         const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
         *scale_out = (uint16_t)T16<DT>::to_bits(sc);
         *zero_out = (uint16_t)zb;
-        *par_out = token_par<DT>(sc, zb);
+        *par_out = token_par<DT>(sc, zb, false);
     }
 }
 
@@ -425,8 +425,18 @@ __device__ __forceinline__ void cell_load(const uint16_t *xc, uint2 xr[16]) {
     for (int k = 0; k < 16; k++) xr[k] = *reinterpret_cast<const uint2 *>(xc + (size_t)k * kHeadDim);
 }
 
+// The same cell from permuted rows: row k is token rows[k] (uniform: the indices come from scalar loads) of the
+// tokens that start at `seq`, which is uniform too; `lane_off` is the lane's byte offset inside a token's rows.
+__device__ __forceinline__ void cell_load_rows(const uint16_t *seq, const uint32_t *rows, uint32_t lane_off, uint2 xr[16]) {
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+        xr[k] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(seq + (size_t)rows[k] * kHeadDim) + lane_off);
+}
+
+// (general_form: the constants of the general sequence whatever the zero point -- for callers whose wavefronts hold
+// several tokens and must take one path for all of them)
 template <int DT>
-__device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
+__device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits, bool general_form) {
     float r = __builtin_amdgcn_rcpf(sc);
     r = __fmaf_rn(__fmaf_rn(-sc, r, 1.f), r, r);
     TokPar tp;
@@ -435,7 +445,7 @@ __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
     tp.sub2 = 0;
     if (DT == PKV_F16) {
         const float z = T16<DT>::from_bits(zero_bits);        // an integer (or inf / nan for degenerate tokens)
-        if (z >= -500.f && z <= 3000.f) {
+        if (!general_form && z >= -500.f && z <= 3000.f) {
             const int zi = (int)z, odd = zi & 1;
             tp.add2 = (uint32_t)__half_as_ushort(__float2half_rn((float)(1536 + odd - zi))) * 0x00010001u;   // exact: |c| < 2048
             tp.sub2 = (uint32_t)(0x6600 + odd) * 0x00010001u;
@@ -444,7 +454,7 @@ __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits) {
         }
     } else {
         const float z = T16<DT>::from_bits(zero_bits);        // an integer (or inf / nan for degenerate tokens)
-        if (fabsf(z) <= 1048576.f) {       // 2^23 - zero and the sums below stay exact
+        if (!general_form && fabsf(z) <= 1048576.f) {       // 2^23 - zero and the sums below stay exact
             tp.add2 = __float_as_uint(8388608.f - z);
             tp.sub2 = 1u;
         } else {
@@ -862,11 +872,15 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
 // workgroup), then at once re-read them as cells -- the lines are still in L2 -- quantize, and emit
 // unit `round` of every block behind the units already there.  x therefore crosses HBM once.
 // Blocks sit in worst-case slots in LDS and are compacted by the final copy.
-template <int DT, bool WIDE>
+// PERM: the tokens are encoded in the order of a repacking -- position p of the output holds token
+// (p / perm_block) * perm_block + perm[p] of x (perm_block a multiple of 64) -- so a round's rows are gathered; scale
+// and zero are written in the output order.
+template <int DT, bool WIDE, bool PERM>
 __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride) {
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
+    const uint32_t *__restrict__ perm, int perm_block) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -875,7 +889,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const int tid = threadIdx.x;
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    const uint32_t gidx = s_idx;
+    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);   // uniform: the rows' addresses become scalar
     if (gidx >= ngroups) return;
     const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 64;
@@ -886,18 +900,36 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     uint8_t *blk = gbuf + (size_t)j * bound;
     uint32_t my_off = 8u;                                 // bytes of this block so far (uniform per half-wavefront)
     uint32_t cmax_all = 0;
+    uint32_t src_tok[4] = {0u, 0u, 0u, 0u};               // PERM: the thread's token of every round's parameter pass
+    if (PERM)
+#pragma unroll
+        for (int r = 0; r < 4; r++) src_tok[r] = perm[tok0 + 16 * r + (tid >> 4)];
+#pragma unroll 1
     for (int r = 0; r < 4; r++) {
         // token parameters of the round: 16 lanes x 8 channels per token, all heads
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
             const size_t tok = (size_t)b * par_stride + tok0 + 16 * r + tt;
-            round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
-                                   scale + tok, zero + tok, s_par + tt);
+            if (PERM) {
+                const size_t pb = (tok0 / (size_t)perm_block) * (size_t)perm_block;      // first token of the repacking block
+                const uint32_t src = r == 0 ? src_tok[0] : r == 1 ? src_tok[1] : r == 2 ? src_tok[2] : src_tok[3];
+                round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
+                                       (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
+            } else {
+                round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
+                                       scale + tok, zero + tok, s_par + tt);
+            }
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
         uint2 xr[16];
-        cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
+        if (PERM) {
+            const size_t pb = (tok0 / (size_t)perm_block) * (size_t)perm_block;
+            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 16 * r,
+                           (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
+        } else {
+            cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
+        }
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         typename PacksOf<WIDE>::type u;
@@ -1034,11 +1066,13 @@ __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, con
 // unit (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight
 // threads of a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed
 // in with LDS atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.
-template <int DT, bool WIDE>
+template <int DT, bool WIDE, bool PERM>
 __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride) {
+    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
+    const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
+    const uint16_t *__restrict__ zero_in) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1049,7 +1083,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const int tid = threadIdx.x;
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    const uint32_t gidx = s_idx;
+    const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
     if (gidx >= ngroups) return;
     const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
@@ -1064,18 +1098,46 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
     uint32_t run_off = 0;                                  // payload bytes of the thread's current unit so far
     uint32_t cmax_all = 0;
+    uint32_t src_tok[4] = {0u, 0u, 0u, 0u};                // PERM: the thread's token of every iteration's parameter pass
+    if (PERM)
+#pragma unroll
+        for (int it = 0; it < 4; it++) src_tok[it] = perm[tok0 + 32 * it + (tid >> 4)];
+#pragma unroll 1
     for (int it = 0; it < 4; it++) {
         // token parameters of the 32 tokens: 16 lanes x 8 channels per token, all heads
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
             const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + tt;
-            round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
-                                   scale + tok, zero + tok, s_par + tt);
+            if (PERM) {     // (the 32 tokens of an iteration lie in one repacking block: perm_block is a multiple of 64)
+                const size_t pb = ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block;
+                const uint32_t src = it == 0 ? src_tok[0] : it == 1 ? src_tok[1] : it == 2 ? src_tok[2] : src_tok[3];
+                if (scale_in) {       // (uniform) the tokens' parameters are known, in the order of x: no pass over the rows
+                    if (l16 == 0) {
+                        const uint32_t sb = scale_in[(size_t)b * T + pb + src], zb = zero_in[(size_t)b * T + pb + src];
+                        scale[tok] = (uint16_t)sb;
+                        zero[tok] = (uint16_t)zb;
+                        s_par[tt] = token_par<DT>(T16<DT>::from_bits(sb), zb, false);
+                    }
+                } else {
+                    round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
+                                           (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
+                }
+            } else {
+                round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
+                                       scale + tok, zero + tok, s_par + tt);
+            }
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
         uint2 xr[16];
-        cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
+        if (PERM) {
+            const size_t pb = ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block;
+            const int rps = __builtin_amdgcn_readfirstlane(rp);          // uniform per wavefront
+            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 32 * it + 16 * rps,
+                           (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
+        } else {
+            cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
+        }
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         typename PacksOf<WIDE>::type u;
@@ -1167,6 +1229,144 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     }
 }
 
+// ---- per-token median of the V codes, straight from V -----------------------------------------------------------
+// `median_repacking` (utils/compute.py:262-270) orders the tokens of a block by the lower median of each token's
+// V codes over ALL channels of all sequences and heads.  This kernel gets those medians without a code matrix: a
+// workgroup of 256 threads owns 16 tokens and walks the sequences; thread (token tt, l16) reads 8 channels of every
+// head (the parameter pass of the round-major encoders), every lane of a token's row computes the token's scale and
+// zero for itself, quantises its 64 values and counts them into a histogram column of its own in LDS
+// (hist[level][thread]: one LDS add per value, no two threads on one word).  At the end the columns of a token are
+// summed per level and the level that reaches rank (n - 1) / 2 is the median.  H <= 8, code width <= 6 bits.
+template <int DT>
+__global__ void __launch_bounds__(256) token_median_from_x_kernel(const uint16_t *__restrict__ x, int B, int H, int T, float rel,
+                                                                  int W, uint8_t *__restrict__ median,
+                                                                  uint16_t *__restrict__ scale_out, uint16_t *__restrict__ zero_out) {
+    extern __shared__ uint32_t hist[];                     // [1 << W][256]
+    const int tid = threadIdx.x, tt = tid >> 4, l16 = tid & 15;
+    const int levels = 1 << W;
+    const size_t tok0 = (size_t)blockIdx.x * 16;
+    for (int l = 0; l < levels; l++) hist[l * 256 + tid] = 0u;       // the thread's own column: no barrier needed
+    const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;
+    // the rows of sequence b + 1 are requested head by head as soon as the head's values of sequence b have been
+    // quantised (into the registers they leave), so the next round trip to memory runs under this sequence's work
+    auto load_row = [&](int b, int i) {
+        const uint16_t *rows = x + (((size_t)b * H) * T + tok0) * kHeadDim;
+        return *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)min(i, H - 1) * T * kHeadDim) + lane_off);
+    };
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = load_row(0, i);
+    for (int b = 0; b < B; b++) {
+        const int bn = min(b + 1, B - 1);                  // (the last sequence is requested once more and not used)
+        float mn, mx;
+        if (DT == PKV_F16) {
+            f16x2 lo[8], hi[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const f16x2 a = __builtin_bit_cast(f16x2, v[i].x), b2 = __builtin_bit_cast(f16x2, v[i].y),
+                            c = __builtin_bit_cast(f16x2, v[i].z), d = __builtin_bit_cast(f16x2, v[i].w);
+                lo[i] = pk_min_h(pk_min_h(a, b2), pk_min_h(c, d));
+                hi[i] = pk_max_h(pk_max_h(a, b2), pk_max_h(c, d));
+            }
+#pragma unroll
+            for (int w = 4; w >= 1; w >>= 1)
+#pragma unroll
+                for (int i = 0; i < w; i++) {
+                    lo[i] = pk_min_h(lo[i], lo[i + w]);
+                    hi[i] = pk_max_h(hi[i], hi[i + w]);
+                }
+            mn = fminf((float)lo[0][0], (float)lo[0][1]);
+            mx = fmaxf((float)hi[0][0], (float)hi[0][1]);
+        } else {
+            mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+        }
+        row16_minmax(mn, mx);
+        const float range = round_t<DT>(mx - mn);
+        const float sc = round_t<DT>(range * rel);
+        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+        // a wavefront holds four tokens: it takes the usual quantisation sequence when all four can, else the general
+        // one for all (quant4 branches on the first lane's constants)
+        if (scale_out && l16 == 0) {                       // the parameters pkv_quant_params would write, for the encoder
+            scale_out[(size_t)b * T + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
+            zero_out[(size_t)b * T + tok0 + tt] = (uint16_t)zb;
+        }
+        TokPar tp = token_par<DT>(sc, zb, false);
+        const bool wave_usual = !__any(tp.sub2 == 0u);
+        if (!wave_usual) tp = token_par<DT>(sc, zb, true);
+        // count one head's eight codes (four 16-bit pairs): both halves clamped to the top level and turned into byte
+        // offsets of the level's row with packed 16-bit operations, then one add per code selects the half (SDWA)
+        auto count = [&](const uint32_t c[4], int i) {
+            const uint32_t one = i < H ? 1u : 0u;          // heads beyond H - 1 repeat the last one: counted as nothing
+            const u16x2 top = {(unsigned short)(levels - 1), (unsigned short)(levels - 1)};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // (a code that does not fit W bits is counted at the top level; the encoders report it)
+                const uint32_t rows2 = pk_u16((u16x2)(__builtin_elementwise_min(as_u16x2(c[q]), top) << (unsigned short)10));
+                atomicAdd(reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(hist) + ((rows2 & 0xFFFFu) + 4u * (uint32_t)tid)), one);
+                atomicAdd(reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(hist) + ((rows2 >> 16) + 4u * (uint32_t)tid)), one);
+            }
+        };
+        if (DT == PKV_F16 && wave_usual) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                uint32_t c[4];
+                quant4_f16_fast(make_uint2(v[i].x, v[i].y), tp, c[0], c[1]);
+                quant4_f16_fast(make_uint2(v[i].z, v[i].w), tp, c[2], c[3]);
+                v[i] = load_row(bn, i);
+                count(c, i);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                uint32_t c[4];
+                quant4<DT>(make_uint2(v[i].x, v[i].y), tp, c[0], c[1]);
+                quant4<DT>(make_uint2(v[i].z, v[i].w), tp, c[2], c[3]);
+                v[i] = load_row(bn, i);
+                count(c, i);
+            }
+        }
+    }
+    __syncthreads();
+    // thread (tt, l16) sums the columns of token tt for its levels l16 * nper .. (a level per lane up to 16 levels)
+    const int nper = levels > 16 ? levels / 16 : 1;
+    uint32_t cnt[4] = {0u, 0u, 0u, 0u}, tot = 0;
+    for (int sl = 0; sl < nper; sl++) {
+        const int l = l16 * nper + sl;
+        if (l < levels)
+            for (int q = 0; q < 16; q++) cnt[sl] += hist[l * 256 + tt * 16 + ((q + l16) & 15)];
+        tot += cnt[sl];
+    }
+    uint32_t incl = tot;                                   // inclusive scan over the 16 lanes of the token's row
+    incl += __builtin_amdgcn_update_dpp(0u, incl, 0x111, 0xF, 0xF, true);
+    incl += __builtin_amdgcn_update_dpp(0u, incl, 0x112, 0xF, 0xF, true);
+    incl += __builtin_amdgcn_update_dpp(0u, incl, 0x114, 0xF, 0xF, true);
+    incl += __builtin_amdgcn_update_dpp(0u, incl, 0x118, 0xF, 0xF, true);
+    const uint32_t need = (uint32_t)((size_t)B * H * kHeadDim - 1) / 2u + 1u;      // values at or below the lower median
+    uint32_t run = incl - tot;
+    int found = -1;
+    for (int sl = 0; sl < nper; sl++) {
+        run += cnt[sl];
+        if (found < 0 && run >= need) found = l16 * nper + sl;
+    }
+    const uint64_t has = __ballot(found >= 0);
+    const uint32_t mine = (uint32_t)(has >> (16 * (tt & 3))) & 0xFFFFu;            // the token's row of the wavefront
+    if (found >= 0 && (mine & ((1u << l16) - 1u)) == 0u) median[tok0 + tt] = (uint8_t)found;
+}
+
+// medians of the V codes of every token (device array of T bytes) from V itself
+static int launch_token_median_from_x(const void *x, int dtype, int B, int H, int T, float rel, int bits, uint8_t *median,
+                                      void *scale_out, void *zero_out, hipStream_t s) {
+    const size_t lds = (size_t)(1 << bits) * 256 * sizeof(uint32_t);
+    auto kern = dtype == PKV_F16 ? token_median_from_x_kernel<PKV_F16> : token_median_from_x_kernel<PKV_BF16>;
+    if (lds > 48 * 1024)
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    kern<<<(unsigned)(T / 16), 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, bits, median, (uint16_t *)scale_out, (uint16_t *)zero_out);
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
 static int check_xshape(const void *x, int dtype, int B, int H, int T) {
     PKV_REQUIRE(x != nullptr, PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(dtype == PKV_F16 || dtype == PKV_BF16, PKV_ERR_UNSUPPORTED, "Unsupported data type");
@@ -1178,7 +1378,9 @@ static int check_xshape(const void *x, int dtype, int B, int H, int T) {
 template <bool IS_K>
 static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float rel, int bits,
                             uint8_t *stream, uint64_t capacity, uint64_t base, uint32_t *info, void *scale,
-                            void *zero, int par_stride, uint64_t *size_out, float *ms_out, hipStream_t s) {
+                            void *zero, int par_stride, uint64_t *size_out, float *ms_out, hipStream_t s,
+                            const uint32_t *perm = nullptr, int perm_block = 0, const void *scale_in = nullptr,
+                            const void *zero_in = nullptr) {
     int rc = check_xshape(x, dtype, B, H, T);
     if (rc) return rc;
     PKV_REQUIRE(stream && info && scale && zero, PKV_ERR_INVALID, "null pointer argument");
@@ -1192,6 +1394,13 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     const int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     PKV_REQUIRE(T % ctx_blk == 0, PKV_ERR_INVALID, "ctx_len must be divisible by ctx_len_block_size");
     PKV_REQUIRE(par_stride >= T, PKV_ERR_INVALID, "parameter row stride shorter than the token count");
+    if (perm) {
+        PKV_REQUIRE(H <= kSubBlocks, PKV_ERR_UNSUPPORTED, "not supported: a token order with more than 8 KV heads");
+        PKV_REQUIRE(perm_block >= 64 && perm_block % 64 == 0 && T % perm_block == 0, PKV_ERR_INVALID,
+                    "the repacking block must be a multiple of 64 tokens that divides ctx_len");
+        PKV_REQUIRE((uint64_t)H * (uint64_t)T * 256ull < (1ull << 32), PKV_ERR_UNSUPPORTED,
+                    "not supported: a token order on more than 4 GiB of rows per sequence");
+    }
     PKV_REQUIRE(base <= capacity, PKV_ERR_INVALID, "stream offset beyond the buffer");
     // block_info holds 32-bit byte offsets (uint32 in the reference too, evaluation/evaluation.py:420-426): a stream
     // that would grow past 4 GiB is reported as a full buffer instead of wrapping its offsets
@@ -1213,23 +1422,32 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
             const uint32_t lds = 64u * unit_slot + 64u;
             const uint32_t ngroups = (uint32_t)(T / ctx_blk) * (uint32_t)B;
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true>)
-                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false>);
+            auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, true>
+                                                             : v_quant_encode_rounds_kernel<PKV_BF16, true, true>)
+                                         : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, true>
+                                                             : v_quant_encode_rounds_kernel<PKV_BF16, false, true>))
+                             : (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false>
+                                                             : v_quant_encode_rounds_kernel<PKV_BF16, true, false>)
+                                         : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false>
+                                                             : v_quant_encode_rounds_kernel<PKV_BF16, false, false>));
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
-                                           stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride);
+                                           stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
+                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in);
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
             const uint32_t lds = (uint32_t)H * slot + 32u;
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true>)
-                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false>);
+            auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, true>
+                                                             : k_quant_encode_rounds_kernel<PKV_BF16, true, true>)
+                                         : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, true>
+                                                             : k_quant_encode_rounds_kernel<PKV_BF16, false, true>))
+                             : (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false>
+                                                             : k_quant_encode_rounds_kernel<PKV_BF16, true, false>)
+                                         : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
+                                                             : k_quant_encode_rounds_kernel<PKV_BF16, false, false>));
             kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                        capacity, info, st, bits, nsub, slot, base, par_stride);
+                                        capacity, info, st, bits, nsub, slot, base, par_stride, perm, perm_block);
         } else {
             auto kern = bits > 4 ? (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, true>
                                                       : quant_encode_group_kernel<IS_K, PKV_BF16, true>)
@@ -1247,6 +1465,48 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
 }  // namespace pkv
 
 extern "C" {
+
+int pkv_median_order(const void *v, int dtype, int B, int H, int T, float rel, int bits, int block_size, uint32_t *perm,
+                     void *scale_out, void *zero_out, float *ms_out, pkv_stream_t s_) {
+    using namespace pkv;
+    hipStream_t s = (hipStream_t)s_;
+    int rc = check_xshape(v, dtype, B, H, T);
+    if (rc) return rc;
+    PKV_REQUIRE(perm != nullptr, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE((scale_out == nullptr) == (zero_out == nullptr), PKV_ERR_INVALID, "scale_out and zero_out go together");
+    PKV_REQUIRE(rel > 0.f, PKV_ERR_INVALID, "quant_scale_rel must be positive");
+    PKV_REQUIRE(H <= kSubBlocks, PKV_ERR_UNSUPPORTED, "not supported: more than 8 KV heads (order the code matrix with pkv_median_repack)");
+    PKV_REQUIRE(bits >= 2 && bits <= 6, PKV_ERR_UNSUPPORTED, "not supported: bits_len %d (2..6)", bits);
+    PKV_REQUIRE(block_size > 0 && block_size <= 1024 && T % block_size == 0 && T % 16 == 0, PKV_ERR_INVALID,
+                "ctx_len must be divisible by 16 and by a block size of at most 1024 tokens");
+    void *scratch = nullptr;
+    if ((rc = scratch_get((size_t)T, s, &scratch))) return rc;
+    uint8_t *median = static_cast<uint8_t *>(scratch);
+    LaunchTimer tm(s, ms_out != nullptr);
+    if ((rc = tm.begin())) return rc;
+    if ((rc = launch_token_median_from_x(v, dtype, B, H, T, rel, bits, median, scale_out, zero_out, s))) return rc;
+    if ((rc = launch_block_order(median, T, block_size, perm, s))) return rc;
+    return tm.end(ms_out);
+}
+
+int pkv_k_quant_encode_perm(const void *x, int dtype, int B, int H, int T, float rel, int bits, const uint32_t *perm,
+                            int perm_block, uint8_t *stream, uint64_t capacity, uint32_t *block_info, void *scale,
+                            void *zero, uint64_t *size_out, float *ms_out, pkv_stream_t s) {
+    PKV_REQUIRE(perm != nullptr, PKV_ERR_INVALID, "null pointer argument");
+    return pkv::run_quant_encode<true>(x, dtype, B, H, T, rel, bits, stream, capacity, 0, block_info, scale, zero, T,
+                                       size_out, ms_out, (hipStream_t)s, perm, perm_block);
+}
+
+int pkv_v_quant_encode_perm(const void *x, int dtype, int B, int H, int T, float rel, int bits, const uint32_t *perm,
+                            int perm_block, const void *scale_in, const void *zero_in, uint8_t *stream, uint64_t capacity,
+                            uint32_t *block_info, void *scale, void *zero, uint64_t *size_out, float *ms_out, pkv_stream_t s) {
+    PKV_REQUIRE(perm != nullptr, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE((scale_in == nullptr) == (zero_in == nullptr), PKV_ERR_INVALID, "scale_in and zero_in go together");
+    PKV_REQUIRE(scale_in == nullptr || (scale_in != scale && zero_in != zero), PKV_ERR_INVALID,
+                "the known parameters (order of x) and the written ones (order of the stream) are different arrays");
+    return pkv::run_quant_encode<false>(x, dtype, B, H, T, rel, bits, stream, capacity, 0, block_info, scale, zero, T,
+                                        size_out, ms_out, (hipStream_t)s, perm, perm_block, scale_in, zero_in);
+}
 
 int pkv_quant_params(const void *x, int dtype, int B, int H, int T, float rel, void *scale, void *zero,
                      float *ms_out, pkv_stream_t s_) {

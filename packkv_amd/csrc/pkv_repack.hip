@@ -116,6 +116,13 @@ __global__ void block_order_kernel(const uint8_t *__restrict__ median, int block
     perm[base + rank] = (uint32_t)i;
 }
 
+int launch_block_order(const uint8_t *median, int ctx_len, int block_size, uint32_t *perm, hipStream_t s) {
+    const int threads = (block_size + 63) / 64 * 64;
+    block_order_kernel<<<(unsigned)(ctx_len / block_size), threads, (size_t)block_size, s>>>(median, block_size, perm);
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
 // ---- greedy order of the tokens of every block: one workgroup of 1024 threads per block ----
 // `greedy_repacking` (utils/compute.py:210-260): a block's N tokens are rows of D2 = 2 * hidden codes (K half, then
 // V half).  Every pack starts from the remaining token with the largest cosine to the rounded mean of the remaining

@@ -39,6 +39,10 @@ struct LaunchTimer {
     ~LaunchTimer();
 };
 
+// perm[blk * block_size + r] = index inside block blk of the token that moves to position r: descending median, equal
+// medians in their original order (pkv_repack.hip).
+int launch_block_order(const uint8_t *median, int ctx_len, int block_size, uint32_t *perm, hipStream_t s);
+
 struct ScanState;
 // Zeroed look-back state for `nblocks` blocks, from the per-device scratch.
 int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s);

@@ -305,8 +305,9 @@ def dequantize(codes, scale, zero, B, H):
     return x
 
 
-def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed):
+def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed, perm=None, perm_block=0, params=None):
     B, H, T = _check_x(x)
+    _require(perm is None or (bits <= 6 and H <= 8), "a token order is taken by the fused encoders only (bits <= 6, H <= 8)")
     hidden = B * H * 128
     ctx_blk, hid_blk = (64, 128) if is_k else (128, 64)
     nblk = (T // ctx_blk) * (hidden // hid_blk)
@@ -331,11 +332,22 @@ def _quant_encode(is_k, x, rel, bits, stream, info, want_size, timed):
     zero = torch.empty(B, T, dtype=x.dtype, device=x.device)
     size = ctypes.c_uint64(0)
     ms = ctypes.c_float(0.0)
-    fn = _lib.load().pkv_k_quant_encode if is_k else _lib.load().pkv_v_quant_encode
     with torch.cuda.device(x.device):
-        rc = fn(_ptr(x), _dtype_code(x), B, H, T, float(rel), bits, _ptr(stream), stream.numel(), _ptr(info),
-                _ptr(scale), _ptr(zero), ctypes.byref(size) if want_size else None,
+        tail = (_ptr(stream), stream.numel(), _ptr(info), _ptr(scale), _ptr(zero), ctypes.byref(size) if want_size else None,
                 ctypes.byref(ms) if timed else None, _stream(x.device))
+        if perm is None:
+            fn = _lib.load().pkv_k_quant_encode if is_k else _lib.load().pkv_v_quant_encode
+            rc = fn(_ptr(x), _dtype_code(x), B, H, T, float(rel), bits, *tail)
+        else:
+            _require(perm.is_cuda and perm.dtype in (torch.uint32, torch.int32) and perm.numel() == T and perm.is_contiguous(),
+                     "perm must hold one 32-bit index per token")
+            if is_k:
+                rc = _lib.load().pkv_k_quant_encode_perm(_ptr(x), _dtype_code(x), B, H, T, float(rel), bits, _ptr(perm),
+                                                         int(perm_block), *tail)
+            else:       # params: V's (scale, zero) [B, T] in the order of x, as median_order writes them
+                sp, zp = (None, None) if params is None else (_ptr(params[0]), _ptr(params[1]))
+                rc = _lib.load().pkv_v_quant_encode_perm(_ptr(x), _dtype_code(x), B, H, T, float(rel), bits, _ptr(perm),
+                                                         int(perm_block), sp, zp, *tail)
     _lib.check(rc)
     return {"stream": stream, "info": info, "scale": scale, "zero": zero, "size": int(size.value),
             "ms": float(ms.value), "bits": bits}
@@ -503,16 +515,48 @@ def repack_and_encode(k_codes, v_codes, pack_size, repack_method="none", block_s
     return k_pre, v_pre, k_aft, v_aft
 
 
-def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=64, k_bits=None, v_bits=None):
+def median_order(v, rel, bits=None, block_size=64, timed=False, want_params=False):
+    """perm [T] int32 of `median_repacking` (utils/compute.py:262-270) for V [B, H, T, 128] quantised at `rel`,
+    counted straight from V: perm[blk * block_size + r] = index inside the block of the token that moves to r."""
+    B, H, T = _check_x(v)
+    bits = bits or bits_for_rel(rel)
+    perm = torch.empty(T, dtype=torch.int32, device=v.device)
+    scale = torch.empty(B, T, dtype=v.dtype, device=v.device) if want_params else None
+    zero = torch.empty(B, T, dtype=v.dtype, device=v.device) if want_params else None
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(v.device):
+        rc = _lib.load().pkv_median_order(_ptr(v), _dtype_code(v), B, H, T, float(rel), bits, int(block_size), _ptr(perm),
+                                          _ptr(scale) if want_params else None, _ptr(zero) if want_params else None,
+                                          ctypes.byref(ms) if timed else None, _stream(v.device))
+    _lib.check(rc)
+    out = (perm, scale, zero) if want_params else perm          # want_params: V's (scale, zero) in the order of v
+    return (out, float(ms.value)) if timed else out
+
+
+def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=64, k_bits=None, v_bits=None, fused=None):
     """Quantize K and V [B, H, T, 128], reorder the tokens of every quantisation block (jointly for K and V, as the
     reference's repacking does before it prices the packs, utils/compute.py:329-357) and encode.  Returns (k, v,
     perm): dicts like k_quant_encode / v_quant_encode -- stream, info, scale, zero in the REPACKED token order, so
     attn_decode takes them as they are (attention does not depend on the order of the cached tokens) -- and the
-    permutation [T] int32 (perm[blk * block_size + r] = position inside the block the token at r came from)."""
+    permutation [T] int32 (perm[blk * block_size + r] = position inside the block the token at r came from).
+    `fused` (default: whenever it applies -- median method, H <= 8, codes of at most 6 bits) takes the order from V
+    itself (median_order) and runs the fused encoders on the permuted tokens; fused=False goes through the code
+    matrices (quantize, repack, block codec), which gives the same streams."""
     B, H, T = _check_x(k)
     _require(v.shape == k.shape and v.dtype == k.dtype and v.is_cuda and v.is_contiguous(), "K and V must have one shape")
     _require(T % 128 == 0 and T % block_size == 0, "the token count must be a multiple of 128 and of block_size")
     k_bits, v_bits = k_bits or bits_for_rel(k_rel), v_bits or bits_for_rel(v_rel)
+    can_fuse = repack_method == "median" and H <= 8 and max(k_bits, v_bits) <= 6 and block_size % 64 == 0 and block_size <= 1024
+    if fused is None:
+        fused = can_fuse
+    if fused:
+        # the order from V itself, then the fused encoders on the tokens in that order: no code matrix in HBM
+        _require(can_fuse, "the fused path takes the median method, at most 8 KV heads, codes of at most 6 bits and blocks "
+                           "of a multiple of 64 tokens")
+        perm, vs, vz = median_order(v, v_rel, v_bits, block_size, want_params=True)
+        ke = _quant_encode(True, k, k_rel, k_bits, None, None, True, False, perm, block_size)
+        ve = _quant_encode(False, v, v_rel, v_bits, None, None, True, False, perm, block_size, (vs, vz))
+        return ke, ve, perm
     ks, kz = quant_params(k, k_rel)
     vs, vz = quant_params(v, v_rel)
     kc, kmx = quantize(k, ks, kz)

@@ -248,3 +248,79 @@ def test_pack_sweep_rows_match_restatement(cuda):
         nk, nv = (T // (4 * c["pack"])) * H, (T // (8 * c["pack"])) * 2 * H
         assert (c["k_stream_bytes"] - 8 * nk, c["v_stream_bytes"] - 8 * nv) == (none["k_bytes"], none["v_bytes"])
         assert c["k_cr"] > 1.0 and c["v_cr"] > 1.0 and c["k_decode_gbs_codes"] > 0
+
+
+def _same_encoding(a, b, label):
+    assert a["size"] == b["size"], label
+    assert torch.equal(a["info"], b["info"]), label
+    assert torch.equal(a["stream"][:a["size"]], b["stream"][:b["size"]]), label
+    assert torch.equal(a["scale"].view(torch.int16), b["scale"].view(torch.int16)), label
+    assert torch.equal(a["zero"].view(torch.int16), b["zero"].view(torch.int16)), label
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_median_repack_inside_the_fused_encode_equals_the_code_matrix_path(cuda, dtype):
+    """repack_quant_encode("median") with the order counted straight from V and the fused encoders gathering the
+    permuted rows (no code matrix) against the path through the code matrices (quantize, median repack, block codec):
+    the same permutation, streams, block_info and parameters.  The permutation is also checked against the NumPy
+    restatement on the restated quantiser's codes."""
+    cases = [(2, 4, 512, 0.1, 0.1, 64), (3, 8, 256, 0.2, 0.05, 64), (1, 2, 1024, 0.1, 0.2, 128), (2, 8, 512, 0.05, 0.1, 256),
+             (1, 1, 256, 0.5, 0.1, 64)]
+    for n, (B, H, T, k_rel, v_rel, bs) in enumerate(cases):
+        _say("fused median case", dtype, B, H, T, k_rel, v_rel, bs)
+        k, v = synth.make_kv(B, H, T, seed=300 + n)
+        g = torch.Generator().manual_seed(400 + n)
+        v = v.float() * 0.4 + torch.randn(1, 1, T, 1, generator=g) * 1.5       # token-wise level shifts: medians differ
+        if n == 0 and dtype == torch.float16:
+            # every third token far from zero with a small range: its zero point (about 100 / (range * rel)) leaves
+            # the span of the usual quantisation sequence, so wavefronts hold tokens of both kinds
+            v[:, :, ::3] = 100.0 + 0.1 * torch.randn(B, H, (T + 2) // 3, 128, generator=g)
+            k[:, :, 1::3] = -60.0 + 0.05 * torch.randn(B, H, (T + 1) // 3, 128, generator=g)
+        k, v = k.to(dtype), v.to(dtype)
+        kd, vd = k.to(cuda), v.to(cuda)
+        kf, vf, pf = ops.repack_quant_encode(kd, vd, k_rel, v_rel, "median", bs, fused=True)
+        km, vm, pm = ops.repack_quant_encode(kd, vd, k_rel, v_rel, "median", bs, fused=False)
+        assert torch.equal(pf.view(torch.int32), pm.view(torch.int32))
+        assert not torch.equal(pf.view(-1, bs), torch.arange(bs, dtype=torch.int32, device=cuda).expand(T // bs, bs))
+        _same_encoding(kf, km, "K")
+        _same_encoding(vf, vm, "V")
+        cv, _, _ = oq.quant_ints(v, 64, v_rel)
+        ck, _, _ = oq.quant_ints(k, 64, k_rel)
+        blocks = orp.blocks_from_code_matrices(oq.code_matrix(ck).numpy(), oq.code_matrix(cv).numpy(), bs)
+        _, order = orp.median_repacking(blocks)
+        assert np.array_equal(pf.cpu().numpy().reshape(-1, bs), order)
+    # the default takes the fused path where it applies and the code matrices elsewhere (here: 7-bit codes)
+    k, v = synth.make_kv(1, 2, 256, seed=9)
+    a = ops.repack_quant_encode(k.to(cuda), v.to(cuda), 0.1, 0.0125, "median")
+    b = ops.repack_quant_encode(k.to(cuda), v.to(cuda), 0.1, 0.0125, "median", fused=False)
+    _same_encoding(a[0], b[0], "K 7-bit V")
+    _same_encoding(a[1], b[1], "V 7-bit")
+    with pytest.raises(Exception):
+        ops.repack_quant_encode(k.to(cuda), v.to(cuda), 0.1, 0.0125, "median", fused=True)
+
+
+def test_fused_median_repack_at_the_benchmark_shape(cuda):
+    """16 sequences x 8 KV heads x 32768 tokens: the fused path's streams decode (unpack kernels) to codes whose
+    every 64-token block is the natural-order block permuted by perm, and the medians along the new order descend."""
+    B, H, T = 16, 8, 32768
+    k, v = synth.make_kv(B, H, T, seed=0, device=cuda)
+    kf, vf, perm = ops.repack_quant_encode(k, v, 0.1, 0.1, "median")
+    kn, vn = ops.k_quant_encode(k, 0.1), ops.v_quant_encode(v, 0.1)
+    del k, v
+    hidden = B * H * 128
+    src = (torch.arange(T, device=cuda) // 64) * 64 + perm.to(torch.int64)
+    assert torch.equal(torch.sort(perm.view(-1, 64).to(torch.int64), dim=1).values,
+                       torch.arange(64, device=cuda).expand(T // 64, 64))
+    for (f, n, dec) in ((kf, kn, ops.k_decode), (vf, vn, ops.v_decode)):
+        cf = torch.empty(T, hidden, dtype=torch.uint8, device=cuda)
+        cn = torch.empty(T, hidden, dtype=torch.uint8, device=cuda)
+        dec(f["stream"], f["info"], cf, bits=f["bits"])
+        dec(n["stream"], n["info"], cn, bits=n["bits"])
+        for lo in range(0, T, 8192):
+            assert torch.equal(cf[lo:lo + 8192], cn[src[lo:lo + 8192]])
+        assert torch.equal(f["scale"], n["scale"][:, src]) and torch.equal(f["zero"].view(torch.int16), n["zero"][:, src].view(torch.int16))
+        med = torch.sort(cf[:4096].to(torch.int16), dim=1).values[:, (hidden - 1) // 2] if dec is ops.v_decode else None
+        if med is not None:
+            m = med.view(-1, 64)
+            assert bool((m[:, 1:] <= m[:, :-1]).all())
+        del cf, cn
