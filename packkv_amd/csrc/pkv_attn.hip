@@ -274,7 +274,6 @@ typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
 
 constexpr int kKtStride = 136;         // bytes per token row of the int8 K tile (128 + 8 pad)
 constexpr int kKtDw = kKtStride / 4;
-constexpr float kPScale = 256.f;       // softmax weights are stored as fp16(p * v_scale * 256)
 
 __device__ __forceinline__ uint32_t pk_shr16(uint32_t v, uint32_t sh) {
     ushort2v a = __builtin_bit_cast(ushort2v, v), b = __builtin_bit_cast(ushort2v, sh);

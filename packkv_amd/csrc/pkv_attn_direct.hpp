@@ -303,6 +303,12 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     float m_run[GW], l_part[GW], z_part[GW];
 #pragma unroll
     for (int i = 0; i < GW; i++) { m_run[i] = -INFINITY; l_part[i] = 0.f; z_part[i] = 0.f; }
+    // The softmax weights reach the matrix cores as fp16(p * v_scale * wscale), wscale = 2^(kWExp - emax), emax = the
+    // largest biased exponent of v_scale among the tokens met so far: weights stay below 2^11 and a round's 16-weight
+    // sum below 2^15 whatever the magnitude of V; when emax grows the running sums are rescaled (factor `grow`).
+    constexpr int kWExp = BF ? 137 : 25;
+    uint32_t emax = 0u;
+    float wscale = 0.f, wscale_inv = 0.f;
 
     // ---- one tile: consume (K unit, V unit, parameters) that are already in registers ----
     auto process = [&](const UnitRegs &ku_r, const UnitRegs &vu_r, const QPar &qp) {
@@ -356,6 +362,19 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
         // online softmax: wave <-> query head, lane <-> tokens 2*lane, 2*lane+1 (round lane / 8)
         float ks0, ks1, kz0, kz1, vs0, vs1, vz0, vz1;
         cvt2(qp.ks, ks0, ks1); cvt2(qp.kz, kz0, kz1); cvt2(qp.vs, vs0, vs1); cvt2(qp.vz, vz0, vz1);
+        float grow = 1.f;
+        {   // every wavefront sees the same 128 tokens, so all four take the same decision
+            const uint32_t ex = (qp.vs >> (BF ? 7 : 10)) & (BF ? 0x00FF00FFu : 0x001F001Fu);
+            const uint32_t mine = max(ex & 0xFFFFu, ex >> 16);
+            uint32_t e = (uint32_t)__builtin_bit_cast(int, wave_max_fused(__builtin_bit_cast(float, mine)));   // small positive ints order like floats
+            e = max(e, BF ? 14u : 1u);
+            if (e > emax) {
+                grow = emax ? __builtin_amdgcn_exp2f(-(float)(int)(e - emax)) : 1.f;    // nothing accumulated before the first tile
+                emax = e;
+                wscale = __uint_as_float((uint32_t)(kWExp - (int)e + 127) << 23);
+                wscale_inv = __uint_as_float((uint32_t)((int)e - kWExp + 127) << 23);
+            }
+        }
 #pragma unroll
         for (int gi = 0; gi < GW; gi++) {
             const int g = wave + 4 * gi;
@@ -374,7 +393,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
                 const float alpha = __expf(m_run[gi] - m_new);    // exp(-inf) = 0 on the first tile
                 m_run[gi] = m_new;
                 const float p0 = __expf(sv[0] - m_new), p1 = __expf(sv[1] - m_new);
-                const _Float16 h0 = (_Float16)(p0 * vs0 * kPScale), h1 = (_Float16)(p1 * vs1 * kPScale);
+                const _Float16 h0 = (_Float16)(p0 * vs0 * wscale), h1 = (_Float16)(p1 * vs1 * wscale);
                 const float f0 = (float)h0, f1 = (float)h1;
                 // V-side order: MFMA k of a segment contracts token k of its four rounds
                 const int tok0 = 2 * lane;
@@ -382,7 +401,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
                 pb[0] = h0;
                 pb[4] = h1;      // token 2*lane+1: same round, next k
                 l_part[gi] = l_part[gi] * alpha + (p0 + p1);
-                z_part[gi] = z_part[gi] * alpha + (f0 * vz0 + f1 * vz1);
+                z_part[gi] = z_part[gi] * (alpha * grow) + (f0 * vz0 + f1 * vz1);
                 // per-round sums (16 tokens = 8 lanes) of the rounded weights, for the pack-minimum term
                 const float r16 = oct_sum_fused(f0 + f1);
                 if ((lane & 7) == 0) {
@@ -390,7 +409,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
                     p16hi[g * 8 + (lane >> 3)] = hi;
                     p16lo[g * 8 + (lane >> 3)] = (_Float16)(r16 - (float)hi);
                 }
-                if (lane == 0) st_a[g] = alpha;
+                if (lane == 0) st_a[g] = alpha * grow;
             }
         }
         __syncthreads();
@@ -495,7 +514,7 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
             const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
             float *dst = p.part + (hq * p.nparts + split) * kPartStride;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
-            dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * (1.f / kPScale);
+            dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * wscale_inv;
             if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
         }
     }

@@ -345,3 +345,37 @@ def test_attn_decode_mixed_widths(cuda, rel_k, rel_v, bits):
     outs = _parity(cuda, q, ke, ve, want, exact, torch.float16, [0, 1], label="K %d / V %d bits" % bits)
     # the two kernels differ by their own rounding only: twice the allowance of the faster one + an output rounding
     assert (outs[0] - outs[1]).abs().max().item() <= 2 * 5e-4 + 2 ** -10 * outs[1].abs().max().item()
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attn_decode_with_values_of_large_and_mixed_magnitude(cuda, dtype, variant):
+    """V of large magnitude (v_scale in the thousands: a fixed weight scale overflowed fp16 there) and V whose
+    magnitude jumps by 2^17 inside one split (the running exponent of the weight scale grows mid-stream).
+    Attention is linear in V and powers of two commute with the quantiser (same codes, scaled parameters), so the
+    outputs are held to the usual bounds after division by the power of two that sets the outputs' magnitude."""
+    B, Hq, Hkv, T = 2, 16, 4, 1024
+    k, v = synth.make_kv(B, Hkv, T, seed=700, dtype=dtype)
+    q = synth.make_q(B, Hq, seed=701, dtype=dtype)
+    big = 2048.0 if dtype == torch.float16 else 4096.0
+    cases = {"large": v.float() * big}
+    mixed = v.float().clone()
+    mixed[:, :, :192] *= 2.0 ** -6          # the first tile and a half: small values, then 2^11 times larger ones
+    mixed[:, :, 192:] *= 2.0 ** 11
+    cases["mixed"] = mixed
+    ke = ops.k_quant_encode(k.to(cuda), 0.1)
+    for name, vv in cases.items():
+        vv = vv.to(dtype)
+        c = big if name == "large" else 2.0 ** 11
+        _say("large-V case", name, dtype, "variant", variant, "max |v| %.0f" % float(vv.abs().max()))
+        want = _reference(q, k, vv, 0.1, 0.1).double() / c
+        exact = _exact(q, k, vv, 0.1, 0.1) / c
+        ve = ops.v_quant_encode(vv.to(cuda), 0.1)
+        assert float(ve["scale"].float().max()) > 250.0
+        qd = q.to(cuda)
+        chk = ops.attn_decode(qd, ke, ve, variant=1, ref_rounding=True, out_f32=True)
+        assert bool(torch.isfinite(chk).all())
+        check_reference_mode(chk.double().cpu() / c, want, name)
+        got = ops.attn_decode(qd, ke, ve, variant=variant)
+        assert bool(torch.isfinite(got).all()), (name, variant)
+        check_fast(got.double().cpu() / c, want, exact, dtype, variant, label="%s variant %d" % (name, variant))
