@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 # for a plain 256 MiB device copy in the same run (131088 -> factor 1.99976; 262144 -> factor 1.0);
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
-DEFAULT_TRAFFIC_BYTES = int((208383 * (262144 / 131088) + 2176 * 1.0) * 1024)
+DEFAULT_TRAFFIC_BYTES = int((208311 * (262144 / 131088) + 3141 * 1.0) * 1024)
 TRAFFIC_SOURCE = ("recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measurement of this workload "
                   "(profiles/attn_dma_kernel_config1.md), not observed by this run")
 
@@ -50,6 +50,9 @@ def parse():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip encode / unpack timing")
+    ap.add_argument("--no-sanity", action="store_true",
+                    help="do not stop when the kernel disagrees with the plain kernel (development builds that switch "
+                         "parts of the kernel off, -DPKV_ATTN_PROBE: their results are wrong by design)")
     ap.add_argument("--layers", type=int, default=0,
                     help="instead of the single-layer step: a decode loop over this many layers through the growing "
                          "compressed cache (configs[4] is --layers 32 --batch 4 --ctx 131072); prints its own JSON line")
@@ -421,7 +424,7 @@ def main():
     diff = (out.float() - plain.float()).abs()
     bound = 1e-3 + 2.0 ** -9 * plain.float().abs()
     sanity = {"max_abs_diff_vs_plain_kernel": float(diff.max()), "ok": bool((diff <= bound).all())}
-    if not sanity["ok"] or not bool(torch.isfinite(out.float()).all()):
+    if not args.no_sanity and (not sanity["ok"] or not bool(torch.isfinite(out.float()).all())):
         raise SystemExit("bench: the attention kernel disagrees with the plain kernel: %r" % (sanity,))
     del plain, diff, bound
 

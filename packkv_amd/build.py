@@ -2,6 +2,9 @@
 
     python -m packkv_amd.build          # compile every kernel source and link
     python -m packkv_amd.build --changed   # recompile only what is older than its sources
+    python -m packkv_amd.build --define PKV_ATTN_PROBE=30 --out /tmp/libpackkv_probe.so
+                                        # a development build with extra -D flags under another name (objects in a
+                                        # directory of their own); PACKKV_HIP_LIB=/tmp/libpackkv_probe.so loads it
 
 The library has no PyTorch dependency: it is a plain C-ABI shared object (include/packkv.h)
 that takes raw device pointers and a hipStream_t.
@@ -41,11 +44,11 @@ def _stale(src, obj):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def _compile(src, only_stale=False):
-    obj = os.path.join(OBJ, src.replace(".hip", ".o"))
+def _compile(src, only_stale=False, defines=(), obj_dir=OBJ):
+    obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
     if only_stale and not _stale(src, obj):
         return obj
-    cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc()] + FLAGS + ["-D" + d for d in defines] + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines()
                     if "packed-fp32-ops" not in l and "warning generated" not in l and l.strip())
@@ -56,20 +59,28 @@ def _compile(src, only_stale=False):
     return obj
 
 
-def build(verbose=True, only_stale=False):
+def build(verbose=True, only_stale=False, defines=(), out=None):
     """Compile and link.  only_stale=True (``--changed`` on the command line) recompiles only the sources whose
-    object file is older than the source or a header."""
-    os.makedirs(OBJ, exist_ok=True)
+    object file is older than the source or a header.  `defines` / `out`: a development build with extra -D flags,
+    linked under another name."""
+    lib = out or LIB
+    obj_dir = OBJ if not defines else OBJ + "_" + "_".join(d.replace("=", "-") for d in defines)
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        objs = list(ex.map(lambda src: _compile(src, only_stale), SOURCES))
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+        objs = list(ex.map(lambda src: _compile(src, only_stale, defines, obj_dir), SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
-        print("built", LIB)
-    return LIB
+        print("built", lib)
+    return lib
 
 
 if __name__ == "__main__":
-    build(only_stale="--changed" in sys.argv[1:])
+    argv = sys.argv[1:]
+    defs = [argv[i + 1] for i, a in enumerate(argv) if a == "--define" and i + 1 < len(argv)]
+    outs = [argv[i + 1] for i, a in enumerate(argv) if a == "--out" and i + 1 < len(argv)]
+    if defs and not outs:
+        raise SystemExit("--define needs --out: a build with extra flags does not replace the library")
+    build(only_stale="--changed" in argv, defines=tuple(defs), out=outs[0] if outs else None)

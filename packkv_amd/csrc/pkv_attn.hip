@@ -743,7 +743,10 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     // The async-copy kernel balances the members of a head through two counters per head (with one member there is
     // nothing to balance).
     const bool dma_path = a->T_c > 0 && a->variant == 0 && aligned16 && (narrow || wide_fast);
-    p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && 2 * a->B * a->Hkv <= kAttnCounters;
+    // Tiles by counter pay when a member has many tiles (the first five are its own anyway): short launches -- a few
+    // tiles per member, the small-batch decode steps -- only get the counters' atomic round trips on top (batch 1,
+    // 32768 tokens: 46 us against 19 us with fixed shares).
+    p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && tps >= 12 && 2 * a->B * a->Hkv <= kAttnCounters;
     p.counters = nullptr;
     // Partials and counters: the stream's own scratch, or the static array -- for pkv_attn_decode_noalloc, and for a
     // stream that is capturing a graph before it has scratch of its own.
