@@ -427,10 +427,10 @@ __device__ __forceinline__ void cell_load(const uint16_t *xc, uint2 xr[16]) {
 
 // The same cell from permuted rows: row k is token rows[k] (uniform: the indices come from scalar loads) of the
 // tokens that start at `seq`, which is uniform too; `lane_off` is the lane's byte offset inside a token's rows.
-__device__ __forceinline__ void cell_load_rows(const uint16_t *seq, const uint32_t *rows, uint32_t lane_off, uint2 xr[16]) {
+__device__ __forceinline__ void cell_load_rows(const uint16_t *seq, const uint32_t *rows, uint32_t last_row, uint32_t lane_off, uint2 xr[16]) {
 #pragma unroll
-    for (int k = 0; k < 16; k++)
-        xr[k] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(seq + (size_t)rows[k] * kHeadDim) + lane_off);
+    for (int k = 0; k < 16; k++)                          // (row indices clamped: a damaged order cannot read outside the block)
+        xr[k] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(seq + (size_t)min(rows[k], last_row) * kHeadDim) + lane_off);
 }
 
 // (general_form: the constants of the general sequence whatever the zero point -- for callers whose wavefronts hold
@@ -903,7 +903,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     uint32_t src_tok[4] = {0u, 0u, 0u, 0u};               // PERM: the thread's token of every round's parameter pass
     if (PERM)
 #pragma unroll
-        for (int r = 0; r < 4; r++) src_tok[r] = perm[tok0 + 16 * r + (tid >> 4)];
+        for (int r = 0; r < 4; r++) src_tok[r] = min(perm[tok0 + 16 * r + (tid >> 4)], (uint32_t)perm_block - 1u);
 #pragma unroll 1
     for (int r = 0; r < 4; r++) {
         // token parameters of the round: 16 lanes x 8 channels per token, all heads
@@ -925,7 +925,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         uint2 xr[16];
         if (PERM) {
             const size_t pb = (tok0 / (size_t)perm_block) * (size_t)perm_block;
-            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 16 * r,
+            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 16 * r, (uint32_t)perm_block - 1u,
                            (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
         } else {
             cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
@@ -1101,7 +1101,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     uint32_t src_tok[4] = {0u, 0u, 0u, 0u};                // PERM: the thread's token of every iteration's parameter pass
     if (PERM)
 #pragma unroll
-        for (int it = 0; it < 4; it++) src_tok[it] = perm[tok0 + 32 * it + (tid >> 4)];
+        for (int it = 0; it < 4; it++) src_tok[it] = min(perm[tok0 + 32 * it + (tid >> 4)], (uint32_t)perm_block - 1u);
 #pragma unroll 1
     for (int it = 0; it < 4; it++) {
         // token parameters of the 32 tokens: 16 lanes x 8 channels per token, all heads
@@ -1133,7 +1133,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         if (PERM) {
             const size_t pb = ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block;
             const int rps = __builtin_amdgcn_readfirstlane(rp);          // uniform per wavefront
-            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 32 * it + 16 * rps,
+            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 32 * it + 16 * rps, (uint32_t)perm_block - 1u,
                            (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
         } else {
             cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
