@@ -268,6 +268,13 @@ def _check_x(x):
     return x.size(0), x.size(1), x.size(2)
 
 
+def _check_params(scale, zero, B, T, dtype, device):
+    for name, t in (("scale", scale), ("zero", zero)):
+        _require(t.is_cuda and t.device == device and t.dtype == dtype and t.dtype in (torch.float16, torch.bfloat16) and
+                 t.numel() == B * T and t.is_contiguous(),
+                 name + " must be a contiguous device tensor of B*T values in the tensor's 16-bit dtype")
+
+
 def quant_params(x, rel, timed=False):
     """Per-(batch, token) scale and zero of quant_ints(TokenQuant) (utils/compute.py:84-112);
     returns (scale, zero) as [B, T] tensors of x.dtype."""
@@ -285,6 +292,7 @@ def quant_params(x, rel, timed=False):
 def quantize(x, scale, zero):
     """uint8 code matrix [T, B*H*128] (layout of evaluation/evaluation.py:406) and the largest code."""
     B, H, T = _check_x(x)
+    _check_params(scale, zero, B, T, x.dtype, x.device)
     codes = torch.empty(T, B * H * 128, dtype=torch.uint8, device=x.device)
     mx = torch.zeros(1, dtype=torch.int32, device=x.device)
     with torch.cuda.device(x.device):
@@ -296,7 +304,10 @@ def quantize(x, scale, zero):
 
 def dequantize(codes, scale, zero, B, H):
     """(code + zero) * scale in the storage dtype -> [B, H, T, 128] (utils/compute.py:173-179)."""
+    _require(codes.is_cuda and codes.dtype == torch.uint8 and codes.dim() == 2 and codes.is_contiguous() and
+             codes.size(1) == B * H * 128, "codes must be a contiguous uint8 device tensor [T, B*H*128]")
     T = codes.size(0)
+    _check_params(scale, zero, B, T, scale.dtype, codes.device)
     x = torch.empty(B, H, T, 128, dtype=scale.dtype, device=codes.device)
     with torch.cuda.device(codes.device):
         rc = _lib.load().pkv_dequantize(_ptr(codes), _dtype_code(scale), B, H, T, _ptr(scale), _ptr(zero),
