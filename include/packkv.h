@@ -64,7 +64,10 @@ uint64_t pkv_block_bound(int is_k, int ctx_blk, int hid_blk, int bits);
  * than the code matrix: size the buffer with pkv_block_bound.
  * `capacity` = bytes available at `stream` (which must start at an even address); `size_out` (host, may be NULL)
  * receives the stream size and makes the call synchronous.  With size_out = NULL nothing is reported by the call
- * itself, not even a stream that did not fit: ask pkv_encode_status afterwards. */
+ * itself, not even a stream that did not fit: ask pkv_encode_status afterwards.
+ * The decoders (and the kq / wv products further down) take `stream_bytes`, the size of the buffer at `stream` --
+ * what the reference's binding knows as compressed_buffer.numel(): a block whose block_info entry points outside
+ * the buffer decodes to arbitrary codes, it is never read from there. */
 int pkv_k_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint32_t *block_info,
                  int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, uint64_t *size_out,
                  float *ms_out, pkv_stream_t s);
@@ -77,9 +80,9 @@ int pkv_v_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint3
  * fit, PKV_ERR_INTERNAL, and with bits > 0 PKV_ERR_UNSUPPORTED when a code of a fused encode does not fit `bits`)
  * and stores the stream size.  No counterpart in the reference, whose encoders are synchronous host code. */
 int pkv_encode_status(pkv_stream_t s, int bits, uint64_t *size_out);
-int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+int pkv_k_decode(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
-int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+int pkv_v_decode(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s);
 
 /* ---- packs longer than 16 tokens ------------------------------------------------------
@@ -223,10 +226,10 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
  *     our_wv[m, d] = sum_n w[m, n] * zero[n] * scale[n] + term1[m, d]
  * Any head count M and any hidden_dim multiple of 128 are accepted (the reference
  * instantiates hidden_dim in {5120, 1024}, M in {40, 8} only). */
-int pkv_kq_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *q, void *kq_out,
+int pkv_kq_mat_vec_mul(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, const void *q, void *kq_out,
                        int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
                        int q_interleaved, float *ms_out, pkv_stream_t s);
-int pkv_wv_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *w, float *wv_out,
+int pkv_wv_mat_vec_mul(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, const void *w, float *wv_out,
                        int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
                        float *ms_out, pkv_stream_t s);
 int pkv_fused_kq(void *our_kq, const void *q, const void *k_zero, const void *k_scale, const void *t, int M,

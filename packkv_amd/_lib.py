@@ -48,8 +48,8 @@ SIGNATURES = {
     "pkv_k_decode_p": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_v_decode_p": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_block_bound_p": (_u64, [_i, _i]),
-    "pkv_k_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
-    "pkv_v_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_k_decode": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_v_decode": (_i, [_vp, _u64, _vp, _vp, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_quant_params": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _vp, _fp, _vp]),
     "pkv_quantize": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _fp, _vp]),
     "pkv_dequantize": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _fp, _vp]),
@@ -65,8 +65,8 @@ SIGNATURES = {
     "pkv_bit_pack_size": (_i, [_vp, _i, _i, _i, _u64p, ctypes.POINTER(ctypes.c_uint32), _fp, _vp]),
     "pkv_median_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _fp, _vp]),
     "pkv_greedy_repack": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
-    "pkv_kq_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _fp, _vp]),
-    "pkv_wv_mat_vec_mul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_kq_mat_vec_mul": (_i, [_vp, _u64, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _fp, _vp]),
+    "pkv_wv_mat_vec_mul": (_i, [_vp, _u64, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _fp, _vp]),
     "pkv_fused_kq": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_fused_wv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_attn_decode": (_i, [ctypes.POINTER(AttnArgs), _fp, _vp]),

@@ -124,10 +124,8 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
                                        : (uint32_t)(tau * n_hid_v + 2 * bh + (j - 2));
             const uint32_t *info = is_k ? p.k_info : p.v_info;
             const uint8_t *stream = is_k ? p.k_stream : p.v_stream;
-            const uint32_t off = info[2 * bidx];
-            uint32_t size = info[2 * bidx + 1];
-            const uint32_t cap = is_k ? p.k_cap : p.v_cap;
-            if (size > cap) size = cap;
+            uint32_t off, size;
+            block_span(info, bidx, is_k ? p.k_cap : p.v_cap, is_k ? p.k_bytes : p.v_bytes, off, size);
             const uint32_t ph = stage_to_lds(stream + off, size, blkbuf + j * p.blk_stride, tid, 256);
             if (tid == 0) s_phase[j] = ph;
         }

@@ -14,7 +14,7 @@ namespace pkv {
 __host__ __device__ inline uint32_t round_up16(uint32_t v) { return (v + 15u) & ~15u; }
 
 template <bool IS_K>
-__global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+__global__ void unpack_kernel(const uint8_t *__restrict__ stream, uint64_t stream_bytes, const uint32_t *__restrict__ info,
                               uint8_t *__restrict__ codes, int hidden_dim, int ctx_blk, int hid_blk,
                               int nunits, int W, uint32_t blk_cap) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -23,9 +23,8 @@ __global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t
     const int n_hid = hidden_dim / hid_blk;
     const uint32_t b = blockIdx.x;
     const uint32_t cb = b / n_hid, hb = b % n_hid;
-    const uint32_t off = info[2 * b];
-    uint32_t size = info[2 * b + 1];
-    if (size > blk_cap) size = blk_cap;   // corrupt block_info must not overrun LDS
+    uint32_t off, size;
+    block_span(info, b, blk_cap, stream_bytes, off, size);
     const uint32_t phase = stage_to_lds(stream + off, size, blk, threadIdx.x, blockDim.x);
     __syncthreads();
     block_decode<IS_K>(blk, phase, nunits, W, tile, hid_blk);
@@ -55,7 +54,7 @@ __global__ void unpack_kernel(const uint8_t *__restrict__ stream, const uint32_t
 // V blocks of 64 channels, two adjacent ones (the two halves of a head) per workgroup of 256 threads: the pair
 // decodes into one tile of 128 tokens x 128 channels, so the write-back stores whole 128-byte lines.  In tile
 // addressing the pair is a V block of 128 channels whose units 4 j + u are the units u of block j.
-__global__ void __launch_bounds__(256) unpack_v_pair_kernel(const uint8_t *__restrict__ stream,
+__global__ void __launch_bounds__(256) unpack_v_pair_kernel(const uint8_t *__restrict__ stream, uint64_t stream_bytes,
                                                             const uint32_t *__restrict__ info,
                                                             uint8_t *__restrict__ codes, int hidden_dim, int W,
                                                             uint32_t blk_cap) {
@@ -69,9 +68,8 @@ __global__ void __launch_bounds__(256) unpack_v_pair_kernel(const uint8_t *__res
     const int tid = threadIdx.x;
     const int j = tid >> 7;                                   // which block of the pair this half of the workgroup serves
     uint8_t *blk = lds + kCtx * kPairHid + j * blk_stride;
-    const uint32_t off = info[2 * (b0 + j)];
-    uint32_t size = info[2 * (b0 + j) + 1];
-    if (size > blk_cap) size = blk_cap;   // corrupt block_info must not overrun LDS
+    uint32_t off, size;
+    block_span(info, b0 + j, blk_cap, stream_bytes, off, size);
     const uint32_t phase = stage_to_lds(stream + off, size, blk, tid & 127, 128);
     __syncthreads();
     {
@@ -294,10 +292,11 @@ static int codec_shape(bool is_k, int ctx_len, int hidden_dim, int ctx_blk, int 
     return PKV_OK;
 }
 
-static int run_unpack(bool is_k, const uint8_t *stream, const uint32_t *info, uint8_t *codes,
+static int run_unpack(bool is_k, const uint8_t *stream, uint64_t stream_bytes, const uint32_t *info, uint8_t *codes,
                       int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out,
                       hipStream_t s) {
     PKV_REQUIRE(stream && info && codes, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(stream_bytes > 0 && stream_bytes < (1ull << 32), PKV_ERR_INVALID, "stream size must be in 1 .. 4 GiB - 1");
     CodecShape cs;
     int rc = codec_shape(is_k, ctx_len, hidden_dim, ctx_blk, hid_blk, bits, &cs);
     if (rc) return rc;
@@ -305,13 +304,13 @@ static int run_unpack(bool is_k, const uint8_t *stream, const uint32_t *info, ui
     if ((rc = tm.begin())) return rc;
     if (is_k)
         unpack_kernel<true><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
-            stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
+            stream, stream_bytes, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
     else if (hid_blk == 64 && hidden_dim % 128 == 0 && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0)
         unpack_v_pair_kernel<<<cs.nblocks / 2, 256, 128 * 128 + 2 * (round_up16(cs.blk_cap) + 32u), s>>>(
-            stream, info, codes, hidden_dim, bits, cs.blk_cap);
+            stream, stream_bytes, info, codes, hidden_dim, bits, cs.blk_cap);
     else
         unpack_kernel<false><<<cs.nblocks, cs.threads, cs.lds_bytes, s>>>(
-            stream, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
+            stream, stream_bytes, info, codes, hidden_dim, ctx_blk, hid_blk, cs.nunits, bits, cs.blk_cap);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
@@ -417,15 +416,15 @@ int pkv_v_encode(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uint3
                          bits, size_out, ms_out, (hipStream_t)s);
 }
 
-int pkv_k_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+int pkv_k_decode(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s) {
-    return pkv::run_unpack(true, stream, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+    return pkv::run_unpack(true, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
                            ms_out, (hipStream_t)s);
 }
 
-int pkv_v_decode(const uint8_t *stream, const uint32_t *block_info, uint8_t *codes, int ctx_len,
+int pkv_v_decode(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                  int hidden_dim, int ctx_blk, int hid_blk, int bits, float *ms_out, pkv_stream_t s) {
-    return pkv::run_unpack(false, stream, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+    return pkv::run_unpack(false, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
                            ms_out, (hipStream_t)s);
 }
 

@@ -353,7 +353,7 @@ int pkv_v_encode_p(const uint8_t *codes, uint8_t *stream, uint64_t capacity, uin
 int pkv_k_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                    int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s) {
     if (pack_len == 16)
-        return pkv_k_decode(stream, block_info, codes, ctx_len, hidden_dim, 64, 128, bits, ms_out, s);
+        return pkv_k_decode(stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, 64, 128, bits, ms_out, s);
     return pkv::run_unpack_long(true, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, pack_len, bits, ms_out,
                                 (hipStream_t)s);
 }
@@ -361,7 +361,7 @@ int pkv_k_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t 
 int pkv_v_decode_p(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, uint8_t *codes, int ctx_len,
                    int hidden_dim, int pack_len, int bits, float *ms_out, pkv_stream_t s) {
     if (pack_len == 16)
-        return pkv_v_decode(stream, block_info, codes, ctx_len, hidden_dim, 128, 64, bits, ms_out, s);
+        return pkv_v_decode(stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, 128, 64, bits, ms_out, s);
     return pkv::run_unpack_long(false, stream, stream_bytes, block_info, codes, ctx_len, hidden_dim, pack_len, bits, ms_out,
                                 (hipStream_t)s);
 }

@@ -127,6 +127,17 @@ __device__ __forceinline__ uint32_t lds_meta_word(const uint8_t *arr, int t, int
     return nbits >= 8 ? v : v & ((1u << (4 * nbits)) - 1u);
 }
 
+// Where block b of a stream of `stream_bytes` bytes lies according to block_info, made safe to read: never more
+// than `cap` bytes, never outside the stream.  (block_info is device data the library does not own: a damaged entry
+// yields garbage codes, not an access outside the buffer.)
+__device__ __forceinline__ void block_span(const uint32_t *__restrict__ info, uint32_t b, uint32_t cap, uint64_t stream_bytes,
+                                           uint32_t &off, uint32_t &size) {
+    off = info[2 * (size_t)b];
+    size = min(info[2 * (size_t)b + 1], cap);
+    if ((uint64_t)off > stream_bytes) off = (uint32_t)stream_bytes;       // (streams are below 4 GiB)
+    size = (uint32_t)min((uint64_t)size, stream_bytes - (uint64_t)off);
+}
+
 // Copy `nbytes` from global `src` (any alignment) into LDS `dst` (16-byte aligned, room for nbytes + 30) so that
 // dst[(src & 15) + i] == src[i]; touches only the aligned 16-byte chunks that overlap the range (a chunk never
 // straddles a page, so the bytes around the range that come along are always mapped).  Returns the phase (src & 15).

@@ -26,7 +26,7 @@ __device__ __forceinline__ uint16_t st16(float x, int dtype) {
 // grid = number of K blocks, threads = 2 * ctx_blk (one half-wavefront per round).  (Padding the tile rows so
 // that the dot product's reads spread over the LDS banks changes nothing measurable: the kernel's time is the
 // latency chain stage -> decode -> dot of many small workgroups.)
-__global__ void kq_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+__global__ void kq_kernel(const uint8_t *__restrict__ stream, uint64_t stream_bytes, const uint32_t *__restrict__ info,
                           const uint16_t *__restrict__ q, uint16_t *__restrict__ kq_out, int ctx_len,
                           int hidden_dim, int ctx_blk, int nunits, int W, uint32_t blk_cap, int dtype,
                           int q_interleaved) {
@@ -37,9 +37,8 @@ __global__ void kq_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
     const int n_hid = hidden_dim / kHeadDim;
     const uint32_t b = blockIdx.x;
     const uint32_t cb = b / n_hid, hb = b % n_hid;
-    const uint32_t off = info[2 * b];
-    uint32_t size = info[2 * b + 1];
-    if (size > blk_cap) size = blk_cap;
+    uint32_t off, size;
+    block_span(info, b, blk_cap, stream_bytes, off, size);
     const uint32_t phase = stage_to_lds(stream + off, size, blk, threadIdx.x, blockDim.x);
     for (int c = threadIdx.x; c < kHeadDim; c += blockDim.x) {
         int src = c;
@@ -70,7 +69,7 @@ __global__ void kq_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
 }
 
 // grid = number of V blocks, threads = 2 * hid_blk (one half-wavefront per segment; 8 * hid_blk / 4 in the dot product).
-__global__ void wv_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+__global__ void wv_kernel(const uint8_t *__restrict__ stream, uint64_t stream_bytes, const uint32_t *__restrict__ info,
                           const uint16_t *__restrict__ w, float *__restrict__ wv_out, int ctx_len,
                           int hidden_dim, int hid_blk, int nunits, int W, uint32_t blk_cap, int dtype) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -81,9 +80,8 @@ __global__ void wv_kernel(const uint8_t *__restrict__ stream, const uint32_t *__
     const uint32_t b = blockIdx.x;
     const uint32_t cb = b / n_hid, hb = b % n_hid;
     const uint32_t head = (hb * (uint32_t)hid_blk) / kHeadDim;
-    const uint32_t off = info[2 * b];
-    uint32_t size = info[2 * b + 1];
-    if (size > blk_cap) size = blk_cap;
+    uint32_t off, size;
+    block_span(info, b, blk_cap, stream_bytes, off, size);
     const uint32_t phase = stage_to_lds(stream + off, size, blk, threadIdx.x, blockDim.x);
     for (int t = threadIdx.x; t < 128; t += blockDim.x)
         ws[t] = ld16(w, (size_t)head * ctx_len + (size_t)cb * 128 + t, dtype);
@@ -188,7 +186,7 @@ static int check_dtype(int dtype) {
 
 extern "C" {
 
-int pkv_kq_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *q, void *kq_out,
+int pkv_kq_mat_vec_mul(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, const void *q, void *kq_out,
                        int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
                        int q_interleaved, float *ms_out, pkv_stream_t s_) {
     using namespace pkv;
@@ -196,6 +194,7 @@ int pkv_kq_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const 
     int rc = check_dtype(dtype);
     if (rc) return rc;
     PKV_REQUIRE(stream && block_info && q && kq_out, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(stream_bytes > 0 && stream_bytes < (1ull << 32), PKV_ERR_INVALID, "stream size must be in 1 .. 4 GiB - 1");
     PKV_REQUIRE(bits >= 2 && bits <= 4 && hid_blk == kHeadDim && ctx_blk > 0 && ctx_blk % kPackTok == 0 &&
                     ctx_blk <= 256 && ctx_len > 0 && ctx_len % ctx_blk == 0 && hidden_dim > 0 &&
                     hidden_dim % hid_blk == 0,
@@ -207,14 +206,14 @@ int pkv_kq_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const 
     const int threads = ((2 * ctx_blk + 63) / 64) * 64;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    kq_kernel<<<nblocks, threads, lds_bytes, s>>>(stream, block_info, (const uint16_t *)q, (uint16_t *)kq_out,
+    kq_kernel<<<nblocks, threads, lds_bytes, s>>>(stream, stream_bytes, block_info, (const uint16_t *)q, (uint16_t *)kq_out,
                                                    ctx_len, hidden_dim, ctx_blk, nunits, bits, cap, dtype,
                                                    q_interleaved);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
 
-int pkv_wv_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const void *w, float *wv_out,
+int pkv_wv_mat_vec_mul(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *block_info, const void *w, float *wv_out,
                        int ctx_len, int hidden_dim, int ctx_blk, int hid_blk, int bits, int dtype,
                        float *ms_out, pkv_stream_t s_) {
     using namespace pkv;
@@ -222,6 +221,7 @@ int pkv_wv_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const 
     int rc = check_dtype(dtype);
     if (rc) return rc;
     PKV_REQUIRE(stream && block_info && w && wv_out, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(stream_bytes > 0 && stream_bytes < (1ull << 32), PKV_ERR_INVALID, "stream size must be in 1 .. 4 GiB - 1");
     PKV_REQUIRE(bits >= 2 && bits <= 4 && ctx_blk == 128 && (hid_blk == 32 || hid_blk == 64 || hid_blk == 128) &&
                     ctx_len > 0 && ctx_len % ctx_blk == 0 && hidden_dim > 0 && hidden_dim % kHeadDim == 0,
                 PKV_ERR_UNSUPPORTED, "no such case");
@@ -231,7 +231,7 @@ int pkv_wv_mat_vec_mul(const uint8_t *stream, const uint32_t *block_info, const 
     const uint32_t lds_bytes = (uint32_t)(128 * hid_blk) + ((cap + 15u) & ~15u) + 32u;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    wv_kernel<<<nblocks, 2 * hid_blk, lds_bytes, s>>>(stream, block_info, (const uint16_t *)w, wv_out, ctx_len,
+    wv_kernel<<<nblocks, 2 * hid_blk, lds_bytes, s>>>(stream, stream_bytes, block_info, (const uint16_t *)w, wv_out, ctx_len,
                                                       hidden_dim, hid_blk, nunits, bits, cap, dtype);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);

@@ -110,7 +110,7 @@ def _encode(is_k, codes, stream, info, ctx_len, hidden_dim, ctx_blk, hid_blk, bi
     ms = ctypes.c_float(0.0)
     fn = lib.pkv_k_encode if is_k else lib.pkv_v_encode
     with torch.cuda.device(dev):
-        rc = fn(_ptr(d_codes), _ptr(d_stream), d_stream.numel(), _ptr(d_info), ctx_len, hidden_dim,
+        rc = fn(_ptr(d_codes), _ptr(d_stream), d_stream.numel() * d_stream.element_size(), _ptr(d_info), ctx_len, hidden_dim,
                 ctx_blk, hid_blk, bits, ctypes.byref(size) if (want_size or on_host) else None,
                 ctypes.byref(ms) if timed else None, _stream(dev))
     _lib.check(rc)
@@ -133,7 +133,7 @@ def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bi
     ms = ctypes.c_float(0.0)
     fn = lib.pkv_k_decode if is_k else lib.pkv_v_decode
     with torch.cuda.device(dev):
-        rc = fn(_ptr(d_stream), _ptr(d_info), _ptr(d_codes), ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
+        rc = fn(_ptr(d_stream), d_stream.numel() * d_stream.element_size(), _ptr(d_info), _ptr(d_codes), ctx_len, hidden_dim, ctx_blk, hid_blk, bits,
                 ctypes.byref(ms) if timed else None, _stream(dev))
     _lib.check(rc)
     if on_host:
@@ -621,7 +621,7 @@ def kq_mat_vec_mul(compressed_buffer, block_info_buffer, q, kq_out, ctx_len, hid
         return 0.0
     ms = ctypes.c_float(0.0)
     with torch.cuda.device(q.device):
-        rc = _lib.load().pkv_kq_mat_vec_mul(_ptr(compressed_buffer), _ptr(block_info_buffer), _ptr(q),
+        rc = _lib.load().pkv_kq_mat_vec_mul(_ptr(compressed_buffer), compressed_buffer.numel() * compressed_buffer.element_size(), _ptr(block_info_buffer), _ptr(q),
                                             _ptr(kq_out), ctx_len, hidden_dim, ctx_len_block_size,
                                             hidden_dim_block_size, bits_len, _dtype_code(q),
                                             int(bool(q_interleaved)), ctypes.byref(ms), _stream(q.device))
@@ -644,7 +644,7 @@ def wv_mat_vec_mul(compressed_buffer, block_info_buffer, w, wv_out, ctx_len, hid
         raise RuntimeError("wv_out must be a float32 tensor")
     ms = ctypes.c_float(0.0)
     with torch.cuda.device(w.device):
-        rc = _lib.load().pkv_wv_mat_vec_mul(_ptr(compressed_buffer), _ptr(block_info_buffer), _ptr(w),
+        rc = _lib.load().pkv_wv_mat_vec_mul(_ptr(compressed_buffer), compressed_buffer.numel() * compressed_buffer.element_size(), _ptr(block_info_buffer), _ptr(w),
                                             _ptr(wv_out), ctx_len, hidden_dim, ctx_len_block_size,
                                             hidden_dim_block_size, bits_len, _dtype_code(w),
                                             ctypes.byref(ms), _stream(w.device))

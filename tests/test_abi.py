@@ -31,7 +31,7 @@ def test_version_bounds_and_error_text():
     assert lib.pkv_block_bound(1, 64, 128, 4) == 4552      # 8 + 4*112 + 512*8
     assert lib.pkv_block_bound(0, 128, 64, 3) == 3400      # 8 + 4*80 + 512*6
     # argument validation happens before any GPU call: a bad width is reported, not crashed on
-    rc = lib.pkv_k_decode(None, None, None, 64, 128, 64, 128, 4, None, None)
+    rc = lib.pkv_k_decode(None, 0, None, None, 64, 128, 64, 128, 4, None, None)
     assert rc == _lib.ERR_INVALID
     assert b"null" in lib.pkv_last_error()
     one = ctypes.c_void_p(16)

@@ -379,3 +379,30 @@ def test_attn_decode_with_values_of_large_and_mixed_magnitude(cuda, dtype, varia
         got = ops.attn_decode(qd, ke, ve, variant=variant)
         assert bool(torch.isfinite(got).all()), (name, variant)
         check_fast(got.double().cpu() / c, want, exact, dtype, variant, label="%s variant %d" % (name, variant))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_attn_decode_survives_damaged_block_info(cuda, variant):
+    """block_info entries that point outside the streams or claim absurd sizes: the step returns (with arbitrary
+    numbers for the heads concerned); no kernel reads outside the buffers it was given."""
+    dtype = torch.float16
+    B, Hq, Hkv, T = 2, 16, 4, 1024
+    k, v = synth.make_kv(B, Hkv, T, seed=77, dtype=dtype)
+    q = synth.make_q(B, Hq, seed=78, dtype=dtype).to(cuda)
+    ke = ops.k_quant_encode(k.to(cuda), 0.1)
+    ve = ops.v_quant_encode(v.to(cuda), 0.1)
+    good = ops.attn_decode(q, ke, ve, variant=variant).float().cpu()
+    for side in (ke, ve):
+        info = side["info"].cpu().numpy().astype(np.int64)
+        info[1] = (side["stream"].numel() + 4096, 3000)
+        info[10] = (0xFFFFFFF0, 0xFFFFFFFF)
+        info[17] = (side["size"] - 5, 0xFFFF)
+        side["info"] = torch.from_numpy(info.astype(np.uint32)).to(cuda)
+    got = ops.attn_decode(q, ke, ve, variant=variant)
+    torch.cuda.synchronize()
+    assert got.shape == good.shape
+    # blocks 1, 10, 17 belong to (sequence, KV head) (0, 1), (0, 2), (0, 1) in K's block_info [8 blocks per 64 tokens]
+    # and to (0, 0), (1, 1), (0, 0) in V's [16 per 128 tokens]: KV heads 0 and 3 of sequence 1 are untouched
+    G = Hq // Hkv
+    for h in (0, 3):
+        assert torch.equal(got.float().cpu()[1, h * G:(h + 1) * G], good[1, h * G:(h + 1) * G])

@@ -308,3 +308,32 @@ def test_long_pack_argument_checks(cuda):
     ops.decode_p(1, stream, info, out, 256, 4)
     torch.cuda.synchronize()
     assert int(out.min()) == 7 and int(out.max()) == 7
+
+
+@pytest.mark.parametrize("is_k", [1, 0])
+def test_damaged_block_info_is_survived(cuda, is_k):
+    """block_info is device data the decoders do not own: entries that point outside the stream, or claim absurd
+    sizes, yield arbitrary codes for their own blocks and nothing else -- the other blocks decode as before."""
+    rng = np.random.default_rng(5)
+    cb, hb = (64, 128) if is_k else (128, 64)
+    T, H, W = 2 * cb, 4 * hb, 4
+    c = _rand_codes(rng, T, H, W, "normal")
+    d_stream, d_info, size = _gpu_encode(cuda, is_k, c, cb, hb, W)
+    stream = d_stream[:size].clone()                      # a buffer that ends with the stream
+    info = d_info.cpu().numpy().astype(np.int64)
+    bad = info.copy()
+    bad[1] = (size + 12345, 4000)                         # behind the buffer
+    bad[2] = (0xFFFFFFF0, 0xFFFFFFFF)                     # far outside, absurd size
+    bad[5] = (size - 3, 0xFFFF)                           # starts inside, runs out
+    bad[6] = (size, 16)                                   # exactly at the end
+    d_bad = torch.from_numpy(bad.astype(np.uint32)).to(cuda)
+    out = torch.zeros(T, H, dtype=torch.uint8, device=cuda)
+    (ops.k_decode if is_k else ops.v_decode)(stream, d_bad, out, cb, hb, W)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    n_hid = H // hb
+    for b in range(info.shape[0]):
+        if b in (1, 2, 5, 6):
+            continue
+        r, h = b // n_hid, b % n_hid
+        assert np.array_equal(got[r * cb:(r + 1) * cb, h * hb:(h + 1) * hb], c[r * cb:(r + 1) * cb, h * hb:(h + 1) * hb]), b

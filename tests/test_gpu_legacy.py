@@ -112,3 +112,34 @@ def test_fused_fixups_take_strided_tensors(cuda):
     packkv_cuda.fused_wv(got, w, zero, scale, term1)
     packkv_cuda.fused_wv(want, w.contiguous(), zero.contiguous(), scale.contiguous(), term1.contiguous())
     assert torch.equal(got, want)
+
+
+def test_damaged_block_info_is_survived(cuda):
+    """Entries of block_info that point outside the compressed buffer give arbitrary products for their blocks;
+    nothing outside the buffer is read and the other blocks' results stand."""
+    H, T = 8, 512
+    cm, zero, scale, comp, info, W, cb, hb = _setup(cuda, H, T, 0.1, True, torch.float16, 43)
+    torch.manual_seed(1)
+    q = torch.randn(H, 128).to(torch.float16).to(cuda)
+    good = torch.zeros(H, T, dtype=torch.float16, device=cuda)
+    ops.kq_mat_vec_mul(comp, info, q, good, T, H * 128, cb, hb, W, q_interleaved=False)
+    bad_info = info.cpu().numpy().astype(np.int64)
+    bad_info[3] = (comp.numel() + 999, 3000)
+    bad_info[9] = (0xFFFFFFF0, 0xFFFFFFFF)
+    t = torch.zeros(H, T, dtype=torch.float16, device=cuda)
+    ops.kq_mat_vec_mul(comp, torch.from_numpy(bad_info.astype(np.uint32)).to(cuda), q, t, T, H * 128, cb, hb, W,
+                       q_interleaved=False)
+    torch.cuda.synchronize()
+    keep = torch.ones(H, T, dtype=torch.bool)
+    for b in (3, 9):                                      # block b = (context block b // H, head b % H)
+        keep[b % H, (b // H) * cb:(b // H + 1) * cb] = False
+    assert torch.equal(t.cpu()[keep], good.cpu()[keep])
+    cm, zero, scale, comp, info, W, cb, hb = _setup(cuda, H, T, 0.1, False, torch.float16, 44)
+    w = torch.rand(H, T).to(torch.float16).to(cuda)
+    bad_info = info.cpu().numpy().astype(np.int64)
+    bad_info[0] = (comp.numel(), 1 << 20)
+    bad_info[7] = (comp.numel() - 1, 77)
+    out = torch.zeros(H, 128, dtype=torch.float32, device=cuda)
+    ops.wv_mat_vec_mul(comp, torch.from_numpy(bad_info.astype(np.uint32)).to(cuda), w, out, T, H * 128, cb, hb, W)
+    torch.cuda.synchronize()
+    assert out.shape == (H, 128)
