@@ -144,13 +144,14 @@ template <bool IS_K, bool WIDE>
 __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                          uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
                                                          int hidden_dim, int ctx_blk, int hid_blk, int W, uint32_t nblocks,
-                                                         uint32_t ngroups) {
+                                                         uint32_t ngroups, const Stagger stagger) {
     extern __shared__ __align__(16) uint8_t lds[];         // two code tiles | the group's bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
     __shared__ uint32_t unit_bytes[2][4];
     __shared__ uint32_t blk_off[kPackGroup + 1];
     const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
     if (tid == 0) { s_idx = atomicAdd(&st->ticket, 1u); blk_off[0] = 0u; }
     __syncthreads();
     const uint32_t gidx = s_idx;
@@ -374,10 +375,12 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
                              : (is_k ? pack_group_kernel<true, false> : pack_group_kernel<false, false>);
         if (lds > 48u * 1024u)
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        Stagger sg;
+        if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, ngroups, &sg))) return rc;
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
         kern<<<ngroups, 256, lds, s>>>(codes, stream, capacity, info, st, hidden_dim, ctx_blk, hid_blk, bits,
-                                       (uint32_t)cs.nblocks, ngroups);
+                                       (uint32_t)cs.nblocks, ngroups, sg);
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
         return finish_encode(st, size_out, 0, s);

@@ -8,11 +8,6 @@
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
 
-#include <map>
-#include <mutex>
-#include <tuple>
-#include <utility>
-
 namespace pkv {
 
 template <int DT> struct T16;
@@ -868,54 +863,6 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
     const uint32_t done = head + 16u * nq;
     for (uint32_t i = tid; i < ((bytes - done) >> 1); i += 256)
         reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(gbuf + done)[i];
-}
-
-// ---- first generation of a large launch, out of phase -----------------------------------------------------------
-// The workgroups that are resident first all start within a few microseconds of each other and go through their
-// phases together: the memory system sees every parameter pass at once, the vector ALUs every pack phase at once,
-// and the whole generation reaches its look-back together and retires in a convoy -- a pattern that repeats, damped,
-// for two or three generations (measured per workgroup: three quarters of the resident workgroups waiting in the
-// look-back at the same time).  So the workgroups that fill the second, third, ... residency slot of the CUs wait
-// kStaggerTicks each per slot before they take their ticket; tickets are handed out in the order of arrival, so the
-// stream order follows the new start order and the generations after the first inherit the spread.  Worth 4 % on the
-// K and 6 % on the V encoder for 1 GiB of input; launches of fewer than four generations start as they are.
-constexpr uint32_t kStaggerTicks = 400;                    // of the 100 MHz wall clock: 4 us per residency slot
-struct Stagger {
-    uint32_t cus;       // workgroups that make up one residency slot over the whole device (0: no stagger)
-    uint32_t slots;     // resident workgroups per CU
-};
-__device__ __forceinline__ void stagger_first_generation(const Stagger sg) {
-    if (sg.cus != 0u && blockIdx.x < sg.cus * sg.slots) {
-        const uint64_t wait = (uint64_t)(blockIdx.x / sg.cus) * kStaggerTicks;
-        const uint64_t t0 = wall_clock64();
-        while (wall_clock64() - t0 < wait) __builtin_amdgcn_s_sleep(32);
-    }
-}
-// Host side: the figures for `kernel` launched with `threads` and `lds` bytes over `nwg` workgroups.
-static int stagger_for(const void *kernel, int threads, uint32_t lds, uint32_t nwg, Stagger *out) {
-    out->cus = out->slots = 0u;
-    if (nwg < 1024u) return PKV_OK;                         // the appends of a growing cache: a handful of workgroups
-    int dev = 0, cus = 0, per_cu = 0;
-    PKV_HIP_CHECK(hipGetDevice(&dev));
-    {   // the two figures are looked up once per (device, kernel, LDS size)
-        static std::mutex mu;
-        static std::map<std::tuple<int, const void *, uint32_t>, std::pair<int, int>> known;
-        std::lock_guard<std::mutex> lock(mu);
-        const auto key = std::make_tuple(dev, kernel, lds);
-        auto it = known.find(key);
-        if (it == known.end()) {
-            PKV_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-            PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, (size_t)lds));
-            it = known.emplace(key, std::make_pair(cus, per_cu)).first;
-        }
-        cus = it->second.first;
-        per_cu = it->second.second;
-    }
-    if (cus > 0 && per_cu > 1 && (uint64_t)nwg >= 4ull * (uint64_t)cus * (uint64_t)per_cu) {
-        out->cus = (uint32_t)cus;
-        out->slots = (uint32_t)per_cu;
-    }
-    return PKV_OK;
 }
 
 // ---- K, all heads in one workgroup: round-major single trip over x --------------------------

@@ -1,5 +1,9 @@
 // Host-side runtime for the C-ABI library: last-error text, scratch, launch timing.
+#include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
+#include <utility>
+#include <tuple>
+#include <map>
 
 #include <cstdarg>
 #include <cstdio>
@@ -132,6 +136,32 @@ int LaunchTimer::end(float *ms_out) {
 LaunchTimer::~LaunchTimer() {
     if (start) (void)hipEventDestroy(start);
     if (stop) (void)hipEventDestroy(stop);
+}
+
+int stagger_for(const void *kernel, int threads, uint32_t lds, uint32_t nwg, Stagger *out) {
+    out->cus = out->slots = 0u;
+    if (nwg < 1024u) return PKV_OK;                         // the appends of a growing cache: a handful of workgroups
+    int dev = 0, cus = 0, per_cu = 0;
+    PKV_HIP_CHECK(hipGetDevice(&dev));
+    {   // the two figures are looked up once per (device, kernel, LDS size)
+        static std::mutex mu;
+        static std::map<std::tuple<int, const void *, uint32_t>, std::pair<int, int>> known;
+        std::lock_guard<std::mutex> lock(mu);
+        const auto key = std::make_tuple(dev, kernel, lds);
+        auto it = known.find(key);
+        if (it == known.end()) {
+            PKV_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+            PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, (size_t)lds));
+            it = known.emplace(key, std::make_pair(cus, per_cu)).first;
+        }
+        cus = it->second.first;
+        per_cu = it->second.second;
+    }
+    if (cus > 0 && per_cu > 1 && (uint64_t)nwg >= 4ull * (uint64_t)cus * (uint64_t)per_cu) {
+        out->cus = (uint32_t)cus;
+        out->slots = (uint32_t)per_cu;
+    }
+    return PKV_OK;
 }
 
 }  // namespace pkv

@@ -44,7 +44,13 @@ struct LaunchTimer {
 int launch_block_order(const uint8_t *median, int ctx_len, int block_size, uint32_t *perm, hipStream_t s);
 
 struct ScanState;
+struct Stagger;
 // Zeroed look-back state for `nblocks` blocks, from the per-device scratch.
+// The stagger of the first resident generation (stagger_first_generation, pkv_block.hpp) for `kernel` launched with
+// `threads` threads and `lds` bytes of dynamic LDS over `nwg` workgroups: CU count and workgroups per CU from the
+// occupancy query (looked up once per device, kernel and LDS size); zeros -- no stagger -- for launches of fewer
+// than four generations.
+int stagger_for(const void *kernel, int threads, uint32_t lds, uint32_t nwg, Stagger *out);
 int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s);
 // Reads back {error, total, max_code}; when `size_out` is NULL returns at once (no sync).
 // `bits` > 0 additionally rejects a launch whose largest code does not fit `bits` bits.
