@@ -12,9 +12,12 @@
 //            metadata bit arrays and the slot-major, lane-minor payload order of the reference's format;
 //   header   four u16 cumulative unit sizes, counted in 4-byte words for P >= 32 (every unit size is then a
 //            multiple of 4; in bytes a unit of 256-token packs would not fit 16 bits).
-// One workgroup of 128 threads per block, one 32-lane half-wavefront per unit, lane t <-> 4 packs.  The encoder
-// reads the block's codes twice (minima / widths, then the words; the second time from L2), obtains the block's
-// offset by the same ticket + look-back as the 16-token codec and writes the words straight into the stream.
+// One workgroup per block: 128 threads -- one 32-lane half-wavefront per unit, lane t <-> 4 packs -- times the number
+// of CHUNKS a pack is cut into (P / 16 of them, at most 8: 256 .. 1024 threads), since a long pack is a row of
+// independent 16-token sub-words and blocks of long packs are few.  A thread handles its chunk's sub-words of its
+// four packs; minima and widths are combined over the chunks through LDS.  The encoder reads the block's codes twice
+// (minima / widths, then the words; the second time from L2), obtains the block's offset by the same ticket +
+// look-back as the 16-token codec and writes the words straight into the stream.
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
 
@@ -65,15 +68,23 @@ __device__ __forceinline__ void long_put_meta(uint32_t *arr, int t, int nbits, u
 
 constexpr int kLongMetaWords = 52;      // 16 * (8 + 4) bytes of metadata at most, and a dword of slack for reads
 
+constexpr int kLongMaxChunks = 8;
+__host__ __device__ inline int long_chunks(int P) { return P / 16 < kLongMaxChunks ? P / 16 : kLongMaxChunks; }
+
 template <bool IS_K>
-__global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+__global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                         uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
                                                         int hidden_dim, int P, int W, uint32_t nblocks) {
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
     __shared__ uint32_t s_unit[4];
     __shared__ uint32_t s_meta[4][kLongMetaWords];
-    const int tid = threadIdx.x, u = tid >> 5, t = tid & 31;
+    __shared__ uint4 s_mm[kLongMaxChunks][128];            // minima and maxima of a thread's four packs over its chunk
+    const int tid = threadIdx.x, u = (tid >> 5) & 3, t = tid & 31;
+    const int chunk = tid >> 7, nch = (int)blockDim.x >> 7;       // this thread's chunk of every pack; chunks per pack
+    const uint32_t nsub = (uint32_t)P / 16u;
+    const uint32_t s0 = nsub * (uint32_t)chunk / (uint32_t)nch, s1 = nsub * (uint32_t)(chunk + 1) / (uint32_t)nch;   // its sub-words
+    const int k0 = P - 16 * (int)s1, k1 = P - 16 * (int)s0;      // ... hold tokens k0 .. k1 - 1 of the pack
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
     const uint32_t b = s_idx;
@@ -91,7 +102,7 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
         const uint8_t *col = tile + (size_t)(u * P) * hidden_dim + 4 * t;
         typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
         u16x2 amn2 = {255, 255}, amx2 = {0, 0}, bmn2 = {255, 255}, bmx2 = {0, 0};   // channels (0, 2) and (1, 3) as 16-bit pairs
-        for (int k = 0; k < P; k += 8) {
+        for (int k = k0; k < k1; k += 8) {
             uint32_t d[8];
 #pragma unroll
             for (int q = 0; q < 8; q++) d[q] = *reinterpret_cast<const uint32_t *>(col + (size_t)(k + q) * hidden_dim);
@@ -104,6 +115,16 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
                 bmx2 = __builtin_elementwise_max(bmx2, c);
             }
         }
+        s_mm[chunk][tid & 127] = make_uint4(__builtin_bit_cast(uint32_t, amn2), __builtin_bit_cast(uint32_t, amx2),
+                                            __builtin_bit_cast(uint32_t, bmn2), __builtin_bit_cast(uint32_t, bmx2));
+        __syncthreads();
+        for (int c = 0; c < nch; c++) {
+            const uint4 o = s_mm[c][tid & 127];
+            amn2 = __builtin_elementwise_min(amn2, __builtin_bit_cast(u16x2, o.x));
+            amx2 = __builtin_elementwise_max(amx2, __builtin_bit_cast(u16x2, o.y));
+            bmn2 = __builtin_elementwise_min(bmn2, __builtin_bit_cast(u16x2, o.z));
+            bmx2 = __builtin_elementwise_max(bmx2, __builtin_bit_cast(u16x2, o.w));
+        }
         const uint32_t amn = __builtin_bit_cast(uint32_t, amn2), amx = __builtin_bit_cast(uint32_t, amx2),
                        bmn = __builtin_bit_cast(uint32_t, bmn2), bmx = __builtin_bit_cast(uint32_t, bmx2);
         mn[0] = amn & 0xFFFFu; mn[2] = amn >> 16; mn[1] = bmn & 0xFFFFu; mn[3] = bmn >> 16;
@@ -112,34 +133,45 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
         len[1] = (uint32_t)bit_length_u32((bmx & 0xFFFFu) - mn[1]);
         len[3] = (uint32_t)bit_length_u32((bmx >> 16) - mn[3]);
     } else {
+        uint32_t lohi[4];                                  // minimum | maximum << 16 of each pack over the chunk
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             int tok0, ch;
             long_pack_at<false>(u, t, i, P, tok0, ch);
             const uint8_t *col = tile + (size_t)tok0 * hidden_dim + ch;
             uint32_t lo = 255u, hi = 0u;
-            for (int k = 0; k < P; k += 8) {
+            for (int k = k0; k < k1; k += 8) {
                 uint32_t c[8];
 #pragma unroll
                 for (int q = 0; q < 8; q++) c[q] = col[(size_t)(k + q) * hidden_dim];
 #pragma unroll
                 for (int q = 0; q < 8; q++) { lo = min(lo, c[q]); hi = max(hi, c[q]); }
             }
-            mn[i] = lo;
-            len[i] = (uint32_t)bit_length_u32(hi - lo);
+            lohi[i] = lo | (hi << 16);
         }
+        s_mm[chunk][tid & 127] = make_uint4(lohi[0], lohi[1], lohi[2], lohi[3]);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; i++) { mn[i] = 255u; len[i] = 0u; }    // (len holds the maximum for the moment)
+        for (int c = 0; c < nch; c++) {
+            const uint4 o = s_mm[c][tid & 127];
+            const uint32_t w[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) { mn[i] = min(mn[i], w[i] & 0xFFFFu); len[i] = max(len[i], w[i] >> 16); }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) len[i] = (uint32_t)bit_length_u32(len[i] - mn[i]);
     }
     // byte offsets of the packs inside the unit's payload: those of 16-token packs times P / 16
     uint32_t off[4], payload;
     pack_offsets(len, off, payload);
-    const uint32_t nsub = (uint32_t)P / 16u;
     payload *= nsub;
-    if (t == 0) s_unit[u] = meta + payload;
-    // metadata bit arrays, assembled in LDS (each half-wavefront its own area)
+    if (t == 0 && chunk == 0) s_unit[u] = meta + payload;
+    // metadata bit arrays, assembled in LDS (each half-wavefront of chunk 0 its own area)
     uint32_t *area = s_meta[u];
-    area[t] = 0u;
-    if (t < kLongMetaWords - 32) area[32 + t] = 0u;
-    {
+    if (chunk == 0) {
+        area[t] = 0u;
+        if (t < kLongMetaWords - 32) area[32 + t] = 0u;
         uint32_t minsw = 0, lensw = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -175,12 +207,13 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
     uint32_t ustart = 8u;
     for (int q = 0; q < u; q++) ustart += s_unit[q];
     uint8_t *dst_u = dst_blk + ustart;
-    for (uint32_t q = (uint32_t)t; q < meta / 2u; q += 32u)
-        reinterpret_cast<uint16_t *>(dst_u)[q] = reinterpret_cast<const uint16_t *>(area)[q];
+    if (chunk == 0)
+        for (uint32_t q = (uint32_t)t; q < meta / 2u; q += 32u)
+            reinterpret_cast<uint16_t *>(dst_u)[q] = reinterpret_cast<const uint16_t *>(area)[q];
     // ---- the words: sub-word s of a pack holds its tokens P - 16 (s + 1) .. P - 16 s - 1 ----
     uint8_t *pay = dst_u + meta;
     if (IS_K) {
-        for (uint32_t s = 0; s < nsub; s++) {
+        for (uint32_t s = s0; s < s1; s++) {
             const uint8_t *row = tile + (size_t)(u * P + P - 16 * (int)(s + 1)) * hidden_dim + 4 * t;
             uint32_t d[16];
 #pragma unroll
@@ -198,7 +231,7 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
         for (int i = 0; i < 4; i++) {
             int tok0, ch;
             long_pack_at<false>(u, t, i, P, tok0, ch);
-            for (uint32_t s = 0; s < nsub; s++) {
+            for (uint32_t s = s0; s < s1; s++) {
                 const uint8_t *col = tile + (size_t)(tok0 + P - 16 * (int)(s + 1)) * hidden_dim + ch;
                 uint32_t c[16];
 #pragma unroll
@@ -210,11 +243,12 @@ __global__ void __launch_bounds__(128) pack_long_kernel(const uint8_t *__restric
 }
 
 template <bool IS_K>
-__global__ void __launch_bounds__(128) unpack_long_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+__global__ void __launch_bounds__(1024) unpack_long_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
                                                           uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
                                                           uint64_t stream_bytes) {
     __shared__ uint32_t s_meta[4][kLongMetaWords];
-    const int tid = threadIdx.x, u = tid >> 5, t = tid & 31;
+    const int tid = threadIdx.x, u = (tid >> 5) & 3, t = tid & 31;
+    const int chunk = tid >> 7, nch = (int)blockDim.x >> 7;       // as in the encoder
     const uint32_t b = blockIdx.x;
     const int hid_blk = IS_K ? 128 : 64, ctx_blk = (IS_K ? 4 : 8) * P;
     const int n_hid = hidden_dim / hid_blk;
@@ -233,7 +267,7 @@ __global__ void __launch_bounds__(128) unpack_long_kernel(const uint8_t *__restr
     const bool sane = ustart + meta <= uend && uend <= bsize;      // uniform per half-wavefront
     uint32_t *area = s_meta[u];
     const uint8_t *src_u = stream + boff + ustart;
-    if (sane)
+    if (sane && chunk == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 2u; q += 32u)
             reinterpret_cast<uint16_t *>(area)[q] = reinterpret_cast<const uint16_t *>(src_u)[q];
     __syncthreads();
@@ -249,9 +283,10 @@ __global__ void __launch_bounds__(128) unpack_long_kernel(const uint8_t *__restr
     pack_offsets(len, off, payload);
     const uint32_t nsub = (uint32_t)P / 16u;
     if (ustart + meta + payload * nsub > uend) return;             // (uniform) widths that overrun the unit
+    const uint32_t s0 = nsub * (uint32_t)chunk / (uint32_t)nch, s1 = nsub * (uint32_t)(chunk + 1) / (uint32_t)nch;
     const uint8_t *pay = src_u + meta;
     if (IS_K) {
-        for (uint32_t s = 0; s < nsub; s++) {
+        for (uint32_t s = s0; s < s1; s++) {
             uint32_t d[16];
 #pragma unroll
             for (int k = 0; k < 16; k++) d[k] = 0u;
@@ -271,7 +306,7 @@ __global__ void __launch_bounds__(128) unpack_long_kernel(const uint8_t *__restr
         for (int i = 0; i < 4; i++) {
             int tok0, ch;
             long_pack_at<false>(u, t, i, P, tok0, ch);
-            for (uint32_t s = 0; s < nsub; s++) {
+            for (uint32_t s = s0; s < s1; s++) {
                 uint32_t c[16];
                 long_get_sub(reinterpret_cast<const uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
                 uint8_t *col = tile + (size_t)(tok0 + P - 16 * (int)(s + 1)) * hidden_dim + ch;
@@ -310,8 +345,9 @@ static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint6
     if ((rc = prepare_scan_state(nblocks, &st, s))) return rc;
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    if (is_k) pack_long_kernel<true><<<nblocks, 128, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
-    else pack_long_kernel<false><<<nblocks, 128, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    const int threads = 128 * long_chunks(P);
+    if (is_k) pack_long_kernel<true><<<nblocks, threads, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    else pack_long_kernel<false><<<nblocks, threads, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
     PKV_HIP_CHECK(hipGetLastError());
     if ((rc = tm.end(ms_out))) return rc;
     return finish_encode(st, size_out, 0, s);
@@ -324,8 +360,9 @@ static int run_unpack_long(bool is_k, const uint8_t *stream, uint64_t stream_byt
     const uint32_t nblocks = (uint32_t)(ctx_len / ((is_k ? 4 : 8) * P)) * (uint32_t)(hidden_dim / (is_k ? 128 : 64));
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    if (is_k) unpack_long_kernel<true><<<nblocks, 128, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
-    else unpack_long_kernel<false><<<nblocks, 128, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    const int threads = 128 * long_chunks(P);
+    if (is_k) unpack_long_kernel<true><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    else unpack_long_kernel<false><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
