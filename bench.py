@@ -564,6 +564,25 @@ def main():
                 "ratio_k": fp16_bytes / 2 / ke2["size"], "ratio_v": fp16_bytes / 2 / ve2["size"]}
             del ke2, ve2, codes2
         result["other_error_bounds"] = other
+        # the same bytes as fewer, longer sequences (one layer of configs[4] is 4 x 131072 tokens): the tensors read as
+        # [B / f, Hkv, f * Tc, 128], encoded and attended at that shape -- more members share a KV head there
+        longer = {}
+        for f in (4, 16):
+            if B % f or f * Tc % 128:
+                continue
+            k4, v4 = kc.view(B // f, Hkv, f * Tc, 128), vc.view(B // f, Hkv, f * Tc, 128)
+            ke4, ve4 = ops.k_quant_encode(k4, args.rel, bits), ops.v_quant_encode(v4, args.rel, bits)
+            q4 = q[:B // f].contiguous()
+            out4 = torch.empty_like(q4)
+            f4 = lambda: ops.attn_decode(q4, ke4, ve4, out=out4)
+            for _ in range(100):
+                f4()
+            a_ms = event_time_ms(torch, f4, 300)
+            bytes4 = ke4["size"] + ve4["size"] + 8 * (nblk_k + nblk_v) + 8 * B * Tc + 2 * 2 * (B // f) * Hq * 128
+            longer["batch %d x %d tokens" % (B // f, f * Tc)] = {
+                "attn_us": a_ms * 1e3, "attn_roofline_frac": bytes4 / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            del ke4, ve4
+        result["longer_sequences"] = longer
 
     if not args.no_extras and default_workload:
         result["gemv_surface"] = gemv_surface(torch, ops, synth, dev)

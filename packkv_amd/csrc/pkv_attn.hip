@@ -743,8 +743,11 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     const bool dma_path = a->T_c > 0 && a->variant == 0 && aligned16 && (narrow || wide_fast);
     // Tiles by counter pay when a member has many tiles (the first five are its own anyway): short launches -- a few
     // tiles per member, the small-batch decode steps -- only get the counters' atomic round trips on top (batch 1,
-    // 32768 tokens: 46 us against 19 us with fixed shares).
-    p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && tps >= 12 && 2 * a->B * a->Hkv <= kAttnCounters;
+    // 32768 tokens: 46 us against 19 us with fixed shares).  And only up to eight members per head: every member asks
+    // its head's counter once per tile, and atomics on one address retire one after the other -- with 16 members a
+    // step of batch 8 x 65536 tokens takes 172 us against 126 us with fixed shares, with 64 (batch 2 x 131072) 206
+    // against 67 us; at 4 and 8 members the counters are worth 1-2 %.
+    p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && nsplit <= 8 && tps >= 12 && 2 * a->B * a->Hkv <= kAttnCounters;
     p.counters = nullptr;
     // Partials and counters: the stream's own scratch, or the static array -- for pkv_attn_decode_noalloc, and for a
     // stream that is capturing a graph before it has scratch of its own.
