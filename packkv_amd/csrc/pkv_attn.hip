@@ -706,13 +706,22 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     const int n_tiles = a->T_c / kTile;
     int nsplit = 0, tps = 0;
     if (n_tiles > 0) {
+        // Members per (sequence, KV head): about PKV_SPLIT_TARGET workgroups in all -- four resident on each of 256
+        // CUs.  When the heads do not divide that number, rounding the members up leaves a few workgroups over that
+        // only start once others have finished, each with a full share of tiles (12 sequences x 8 heads: 11 members,
+        // 1056 workgroups, 115 us per step against 99 us with 10 members); so both roundings are priced as
+        // generations x tiles per member and the cheaper one is taken, the finer cut on a tie.
         const int pairs = a->B * a->Hkv;
-        const int target = PKV_SPLIT_TARGET;       // four resident workgroups on each of 256 CUs
-        int want = (target + pairs - 1) / pairs;   // aim for ~8 workgroups per CU
-        if (want < 1) want = 1;
-        if (want > n_tiles) want = n_tiles;
-        tps = (n_tiles + want - 1) / want;
-        nsplit = (n_tiles + tps - 1) / tps;
+        const int target = PKV_SPLIT_TARGET;
+        long best_cost = -1;
+        for (int up = 1; up >= 0; up--) {
+            int want = up ? (target + pairs - 1) / pairs : target / pairs;
+            if (want < 1) want = 1;
+            if (want > n_tiles) want = n_tiles;
+            const int t = (n_tiles + want - 1) / want, n = (n_tiles + t - 1) / t;
+            const long cost = (((long)pairs * n + target - 1) / target) * (long)t;
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; tps = t; nsplit = n; }
+        }
     }
     p.tiles_per_split = tps; p.nsplit = nsplit;
     // The async-copy kernel spreads the tail window over its splits (each takes win_piece tokens after its
