@@ -374,7 +374,7 @@ __device__ __forceinline__ f16x2 pk_max_h(f16x2 a, f16x2 b) {
 }
 
 // Token parameters of one round of the round-major encoders.  256 threads per 16 tokens: thread (tt = token, l16)
-// reads 8 channels of every head (heads beyond H - 1 repeat the last: a repeated row changes no min / max); lane
+// reads 8 channels of every head (slots beyond H - 1 repeat the first row: a repeated row changes no min / max); lane
 // l16 == 0 writes the token's scale and zero and its constants for quant4.  `rows` is x at (sequence, head 0, the
 // round's first token) and uniform, so the eight loads are one 32-bit lane offset on eight scalar bases.
 template <int DT>
@@ -382,9 +382,12 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
                                                    uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
     const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;          // bytes
     uint4 v[8];
+    v[0] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows) + lane_off);
 #pragma unroll
-    for (int i = 0; i < 8; i++)
-        v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)min(i, H - 1) * head_stride) + lane_off);
+    for (int i = 1; i < 8; i++) {                          // (H is uniform: a row that does not exist is not fetched)
+        if (i < H) v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)i * head_stride) + lane_off);
+        else v[i] = v[0];
+    }
     float mn, mx;
     if (DT == PKV_F16) {               // packed fp16 comparisons all the way down to one word each
         f16x2 lo[8], hi[8];
@@ -408,6 +411,49 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
         mn = INFINITY, mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
+    }
+    row16_minmax(mn, mx);
+    if (l16 == 0) {
+        const float range = round_t<DT>(mx - mn);
+        const float sc = round_t<DT>(range * rel);
+        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+        *scale_out = (uint16_t)T16<DT>::to_bits(sc);
+        *zero_out = (uint16_t)zb;
+        *par_out = token_par<DT>(sc, zb, false);
+    }
+}
+
+// The same for groups of up to four heads (several of which share a workgroup): only the rows that exist are
+// fetched and compared.
+template <int DT>
+__device__ __forceinline__ void round_token_params_few(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
+                                                       uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
+    const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;          // bytes
+    uint4 v[4];
+    v[0] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows) + lane_off);
+#pragma unroll
+    for (int i = 1; i < 4; i++)
+        if (i < H) v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)i * head_stride) + lane_off);
+    float mn, mx;
+    if (DT == PKV_F16) {
+        f16x2 lo, hi;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (i < H) {
+                const f16x2 a = __builtin_bit_cast(f16x2, v[i].x), b = __builtin_bit_cast(f16x2, v[i].y),
+                            c = __builtin_bit_cast(f16x2, v[i].z), d = __builtin_bit_cast(f16x2, v[i].w);
+                const f16x2 l = pk_min_h(pk_min_h(a, b), pk_min_h(c, d)), h = pk_max_h(pk_max_h(a, b), pk_max_h(c, d));
+                lo = i ? pk_min_h(lo, l) : l;
+                hi = i ? pk_max_h(hi, h) : h;
+            }
+        }
+        mn = fminf((float)lo[0], (float)lo[1]);
+        mx = fmaxf((float)hi[0], (float)hi[1]);
+    } else {
+        mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < H) minmax8<DT>(v[i], mn, mx);
     }
     row16_minmax(mn, mx);
     if (l16 == 0) {
@@ -880,24 +926,35 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
-    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger) {
+    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger, int gpw, uint32_t ngroups_total) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
     __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the group's bytes
-    __shared__ __attribute__((aligned(16))) TokPar s_par[16];
+    __shared__ __attribute__((aligned(16))) TokPar s_par[kSubBlocks * 16];      // [group of the workgroup][token of the round]
     const int tid = threadIdx.x;
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
     const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);   // uniform: the rows' addresses become scalar
     if (gidx >= ngroups) return;
-    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    // Fewer than five heads: a workgroup takes gpw = 8 / H (rounded down) consecutive groups -- consecutive in the
+    // stream too -- so that its eight half-wavefronts all have a block; `ngroups` then counts workgroups and
+    // `ngroups_all` groups.  Half-wavefront j serves head j % H of group gidx * gpw + j / H; everything below that is
+    // written for "the group" uses this half-wavefront's group (with gpw == 1 the one group, uniformly).
+    const uint32_t ngroups_all = ngroups_total;
+    const int j = tid >> 5, t = tid & 31;                 // block and lane of the unit
+    const int jg = gpw > 1 ? j / H : 0, jh = gpw > 1 ? j % H : j;
+    const uint32_t grp_first = gidx * (uint32_t)gpw;
+    const int ng = (int)min((uint32_t)gpw, ngroups_all - grp_first);          // groups of this workgroup
+    const int nblk = gpw > 1 ? ng * H : H;                // blocks of this workgroup
+    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : gidx;
+    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 64;
     const UnitGeom g = unit_geom(W);
-    const int j = tid >> 5, t = tid & 31;                 // block (= head) and lane of the unit
-    const bool active = j < H;
-    const int jc = min(j, H - 1);
+    const bool active = gpw > 1 ? (jg < ng && j < gpw * H) : j < H;
+    const int jc = gpw > 1 ? jh : min(j, H - 1);
+    const TokPar *my_par = s_par + 16 * (gpw > 1 ? min(jg, ng - 1) : 0);
     uint8_t *blk = gbuf + (size_t)j * bound;
     uint32_t my_off = 8u;                                 // bytes of this block so far (uniform per half-wavefront)
     uint32_t cmax_all = 0;
@@ -917,9 +974,17 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
                 const uint32_t src = r == 0 ? src_tok[0] : r == 1 ? src_tok[1] : r == 2 ? src_tok[2] : src_tok[3];
                 round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
                                        (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
-            } else {
+            } else if (gpw == 1) {
                 round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
                                        scale + tok, zero + tok, s_par + tt);
+            } else {
+                for (int q = 0; q < ng; q++) {              // one group after the other: H rows each
+                    const uint32_t gq = grp_first + (uint32_t)q;
+                    const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
+                    const size_t tq = (size_t)bq * par_stride + (size_t)cq * 64 + 16 * r + tt;
+                    round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 64 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H,
+                                               tt, l16, rel, scale + tq, zero + tq, s_par + 16 * q + tt);
+                }
             }
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
@@ -935,7 +1000,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         typename PacksOf<WIDE>::type u;
         uint32_t cmax;
-        cell_packs<DT>(xr, s_par, u, cmax);
+        cell_packs<DT>(xr, my_par, u, cmax);
         __syncthreads();                                  // s_par is rewritten by the next round
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
@@ -947,8 +1012,8 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
             if (tid == 0) blk_off[0] = 0;
             __syncthreads();
             if (tid == 0) {                                               // ... then their running sum
-                for (int q = 1; q <= H; q++) blk_off[q] += blk_off[q - 1];
-                lookback_publish(st, gidx, blk_off[H]);
+                for (int q = 1; q <= nblk; q++) blk_off[q] += blk_off[q - 1];
+                lookback_publish(st, gidx, blk_off[nblk]);
             }
         }
         if (active) {
@@ -964,7 +1029,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
         if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
     }
     __syncthreads();
-    const uint32_t bytes = blk_off[H];
+    const uint32_t bytes = blk_off[nblk];
     if (tid < 64) {
         const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
         if (tid == 0) {
@@ -976,8 +1041,8 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     __syncthreads();
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
-    if (tid < H) {
-        const uint32_t first = cb * (uint32_t)(B * H) + b * (uint32_t)H;
+    if (tid < nblk) {
+        const uint32_t first = (gpw > 1 ? grp_first : gidx) * (uint32_t)H;      // block index = group * H + head
         info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
         info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
@@ -1073,27 +1138,35 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
     const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
-    const uint16_t *__restrict__ zero_in, const Stagger stagger) {
+    const uint16_t *__restrict__ zero_in, const Stagger stagger, int gpw, uint32_t ngroups_total) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
     __shared__ uint32_t blk_off[17];                       // byte offset of each block inside the group's bytes
     __shared__ uint32_t s_tot[2][8][4];                    // payload bytes the two rounds of an iteration append per unit
     __shared__ uint16_t s_usz[16][4];                      // bytes of every unit (block, unit index 2 w + sg)
-    __shared__ __attribute__((aligned(16))) TokPar s_par[32];
+    __shared__ __attribute__((aligned(16))) TokPar s_par[kSubBlocks * 32];      // [group of the workgroup][token of the iteration]
     const int tid = threadIdx.x;
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
     const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
     if (gidx >= ngroups) return;
-    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    // Fewer than five heads: gpw = 8 / H (rounded down) consecutive groups to a workgroup, as in the K kernel --
+    // `ngroups` counts workgroups, `ngroups_total` groups; head slot j serves head j % H of group gidx * gpw + j / H.
+    const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31;
+    const int jg = gpw > 1 ? j / H : 0, jh = gpw > 1 ? j % H : j;
+    const uint32_t grp_first = gidx * (uint32_t)gpw;
+    const int ng = (int)min((uint32_t)gpw, ngroups_total - grp_first);        // groups of this workgroup
+    const int nheads = gpw > 1 ? ng * H : H;              // head slots in use
+    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : gidx;
+    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
-    const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31;
-    const bool active = j < H;
-    const int jc = min(j, H - 1);
+    const bool active = gpw > 1 ? jg < ng : j < H;
+    const int jc = gpw > 1 ? jh : min(j, H - 1);
+    const TokPar *my_par = s_par + 32 * (gpw > 1 ? min(jg, ng - 1) : 0) + 16 * rp;
     const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
     // metadata areas start as zeros (fields are OR-ed in)
     for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)
@@ -1125,9 +1198,17 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
                     round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
                                            (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
                 }
-            } else {
+            } else if (gpw == 1) {
                 round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
                                        scale + tok, zero + tok, s_par + tt);
+            } else {
+                for (int q = 0; q < ng; q++) {              // one group after the other: H rows each
+                    const uint32_t gq = grp_first + (uint32_t)q;
+                    const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
+                    const size_t tq = (size_t)bq * par_stride + (size_t)cq * 128 + 32 * it + tt;
+                    round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 128 + 32 * it) * kHeadDim, (size_t)T * kHeadDim,
+                                               H, tt, l16, rel, scale + tq, zero + tq, s_par + 32 * q + tt);
+                }
             }
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
@@ -1144,7 +1225,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         typename PacksOf<WIDE>::type u;
         uint32_t cmax;
-        cell_packs<DT>(xr, s_par + 16 * rp, u, cmax);
+        cell_packs<DT>(xr, my_par, u, cmax);
         // bytes of the thread's four packs, their offsets inside the (unit, slot) and the slot's total
         const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
         uint32_t inc = pb;
@@ -1165,11 +1246,11 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
             __syncthreads();
             if (tid == 0) {
                 uint32_t run = 0;
-                for (int q = 0; q < 2 * H; q++) {
+                for (int q = 0; q < 2 * nheads; q++) {
                     blk_off[q] = run;
                     run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
                 }
-                blk_off[2 * H] = run;
+                blk_off[2 * nheads] = run;
                 lookback_publish(st, gidx, run);
             }
         }
@@ -1198,7 +1279,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
     }
     __syncthreads();
-    const int nblk = 2 * H;
+    const int nblk = 2 * nheads;
     const uint32_t bytes = blk_off[nblk];
     if (tid < 64) {
         const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
@@ -1212,7 +1293,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < nblk) {
-        const uint32_t first = cb * (uint32_t)(B * nblk) + b * (uint32_t)nblk;
+        const uint32_t first = grp_first * (uint32_t)(2 * H);                 // block index = group * 2 H + 2 head + half
         info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
         info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
@@ -1423,7 +1504,10 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
         if (!IS_K && H <= 8) {               // one workgroup per group of 2 H blocks
             const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
             const uint32_t lds = 64u * unit_slot + 64u;
-            const uint32_t ngroups = (uint32_t)(T / ctx_blk) * (uint32_t)B;
+            const uint32_t ngroups_all = (uint32_t)(T / ctx_blk) * (uint32_t)B;
+            // up to four heads: 8 / H groups to a workgroup, so that all eight head slots have blocks
+            const int gpw = (H <= 4 && !perm) ? kSubBlocks / H : 1;
+            const uint32_t ngroups = (ngroups_all + (uint32_t)gpw - 1u) / (uint32_t)gpw;
             auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, true>
                                                              : v_quant_encode_rounds_kernel<PKV_BF16, true, true>)
                                          : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, true>
@@ -1438,10 +1522,13 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
             kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
                                            stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
-                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg);
+                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all);
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
-            const uint32_t lds = (uint32_t)H * slot + 32u;
+            // up to four heads: 8 / H groups to a workgroup, so that all eight half-wavefronts have a block
+            const int gpw = (H <= 4 && !perm) ? kSubBlocks / H : 1;
+            const uint32_t nwg = (nsub + (uint32_t)gpw - 1u) / (uint32_t)gpw;
+            const uint32_t lds = (uint32_t)(gpw * H) * slot + 32u;
             auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, true>
                                                              : k_quant_encode_rounds_kernel<PKV_BF16, true, true>)
                                          : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, true>
@@ -1451,9 +1538,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
                                          : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
                                                              : k_quant_encode_rounds_kernel<PKV_BF16, false, false>));
             Stagger sg;
-            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nsub, &sg))) return rc;
-            kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                        capacity, info, st, bits, nsub, slot, base, par_stride, perm, perm_block, sg);
+            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
+            kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                       capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub);
         } else {
             auto kern = bits > 4 ? (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, true>
                                                       : quant_encode_group_kernel<IS_K, PKV_BF16, true>)

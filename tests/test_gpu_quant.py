@@ -39,6 +39,8 @@ def test_quantizer_bit_exact(cuda, dtype, rel):
 def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
     for (B, H, T, rel) in ((1, 2, 128, 0.1), (2, 8, 256, 0.1), (1, 32, 128, 0.1), (2, 4, 256, 0.2), (1, 8, 128, 0.34),
                            (1, 3, 128, 0.1), (2, 5, 256, 0.14), (3, 1, 128, 0.1),
+                           # few heads: several groups to a workgroup, the last workgroup partly filled
+                           (3, 2, 384, 0.1), (5, 1, 256, 0.1), (3, 3, 384, 0.2), (3, 4, 128, 0.1),
                            # widths 5 and 6 (format extension): round-major kernels up to eight heads, group kernel beyond
                            (2, 8, 256, 0.05), (1, 4, 384, 0.03), (1, 3, 128, 0.05), (1, 16, 128, 0.05), (2, 12, 256, 0.03)):
         k, v = synth.make_kv(B, H, T, seed=31 + H, dtype=dtype)
