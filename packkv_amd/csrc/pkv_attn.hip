@@ -64,6 +64,7 @@ struct AttnParams {
     int out_f32;          // `out` holds fp32 instead of the 16-bit storage type
     int direct_out;       // a single partial and a 16-bit result: the async-copy kernel writes `out` itself
     int dynamic;          // async-copy kernel: the members of a (sequence, KV head) take tiles from a common counter
+    int batch_shift;      // ... in batches of (tiles left >> batch_shift), at least 1 and at most 4
     uint32_t *counters;   // [B Hkv] tile counters, then [B Hkv] counts of members that are done; zero between launches
 };
 
@@ -757,6 +758,8 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     // step of batch 8 x 65536 tokens takes 172 us against 126 us with fixed shares, with 64 (batch 2 x 131072) 206
     // against 67 us; at 4 and 8 members the counters are worth 1-2 %.
     p.dynamic = PKV_DYNAMIC_TILES && dma_path && nsplit > 1 && nsplit <= 8 && tps >= 12 && 2 * a->B * a->Hkv <= kAttnCounters;
+    p.batch_shift = 1;                     // a member asks for 1 / (2 nsplit) of what is left: ceil(log2(2 nsplit))
+    while ((1 << p.batch_shift) < 2 * nsplit) p.batch_shift++;
     p.counters = nullptr;
     // Partials and counters: the stream's own scratch, or the static array -- for pkv_attn_decode_noalloc, and for a
     // stream that is capturing a graph before it has scratch of its own.

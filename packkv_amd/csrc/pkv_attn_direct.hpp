@@ -92,17 +92,15 @@ __device__ __forceinline__ float oct_sum_fused(float x) {   // every lane gets t
 __device__ __forceinline__ void pack_offsets8(uint32_t lens_b, uint32_t off2[4]) {
     const uint32_t incl = half_incl_scan(lens_b);
     const uint32_t excl = incl - lens_b;
-    const uint32_t ta = __builtin_amdgcn_readlane(incl, 31), tb = __builtin_amdgcn_readlane(incl, 63);
-    // slot bases = running sums of the slot totals; uniform per half, so this is scalar work
-    const uint32_t a0 = ta & 0xFFu, a01 = a0 + ((ta >> 8) & 0xFFu), a012 = a01 + ((ta >> 16) & 0xFFu);
-    const uint32_t b0 = tb & 0xFFu, b01 = b0 + ((tb >> 8) & 0xFFu), b012 = b01 + ((tb >> 16) & 0xFFu);
-    const bool upper = (threadIdx.x & 32) != 0;
-    const uint32_t base12 = upper ? (b0 | (b01 << 16)) : (a0 | (a01 << 16));
-    const uint32_t base3 = upper ? b012 : a012;
+    // the four slot totals of this lane's half = the running sums of its lane 31: one cross-lane read on the LDS
+    // crossbar (bit-mask swizzle within 32 lanes: lane | 31), no memory access, no scalar round trip, and the slot
+    // bases are byte-select additions
+    const uint32_t tot = (uint32_t)__builtin_amdgcn_ds_swizzle((int)incl, 0x03E0);
+    const uint32_t a0 = tot & 0xFFu, a01 = a0 + ((tot >> 8) & 0xFFu), a012 = a01 + ((tot >> 16) & 0xFFu);
     off2[0] = excl & 0xFFu;
-    off2[1] = ((excl >> 8) & 0xFFu) + (base12 & 0xFFFFu);
-    off2[2] = ((excl >> 16) & 0xFFu) + (base12 >> 16);
-    off2[3] = (excl >> 24) + base3;
+    off2[1] = ((excl >> 8) & 0xFFu) + a0;
+    off2[2] = ((excl >> 16) & 0xFFu) + a01;
+    off2[3] = (excl >> 24) + a012;
 }
 
 template <int G, int KW, int VW, bool BF>

@@ -40,6 +40,10 @@ template <int G, bool WIDE> struct StagePrio {                       // 4 workgr
 template <int G> struct StagePrio<G, true> { static constexpr int K = 2, S = 1, D = 0, V = 0; };
 template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 0, V = 0; };
 #define PKV_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+// A wave-uniform value the compiler may not look through: keeps scalar min / max chains on the scalar unit (it forms
+// three-operand vector instructions plus a v_readfirstlane out of them otherwise) and keeps cheap address arithmetic
+// inside the loop instead of in scalar registers that live across it.
+#define PKV_SCALAR(x) asm volatile("" : "+s"(x))
 
 // PKV_ATTN_PROBE (measurement builds only, results are then meaningless): bit mask of pipeline stages to leave out
 // of the tile loop -- 1 the copies (the first two tiles are re-used), 2 the K stage, 4 the softmax, 8 the V stage,
@@ -71,6 +75,16 @@ __device__ __forceinline__ void dma_b32(u32x4 rsrc, uint32_t lds_addr, uint32_t 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
+
+// The same descriptor moved `add` bytes forward and cut to `bytes`: scalar arithmetic only.  A copy whose lanes address
+// `16 lane` through such a descriptor needs no per-lane address arithmetic and no per-lane clamp: lanes past the end
+// get zeroes (and touch no memory).
+__device__ __forceinline__ u32x4 dma_rsrc_at(u32x4 r, uint32_t add, uint32_t bytes) {
+    const uint64_t a = (((uint64_t)r[1] << 32) | r[0]) + add;
+    return (u32x4){(uint32_t)a, (uint32_t)(a >> 32), bytes, r[3]};
+}
+
+template <int N> struct IntC { static constexpr int value = N; };
 
 template <int KW, int VW>
 struct DmaGeom {
@@ -110,16 +124,19 @@ __device__ __forceinline__ uint64_t lds_word64(const uint8_t *base, uint32_t off
     return ((uint64_t)hi << 32) | lo;
 }
 
-// Lane t's 4*NB-bit metadata word of the LSB-first bit array at byte offset `off` (even) of `base`.
+// Lane t's 4*NB-bit metadata word of an LSB-first bit array in LDS.  `base` is 4-byte aligned and holds everything the
+// compiler knows of the address (it becomes the instruction's offset field); `a` = byte offset of the array (even)
+// + meta_lane_byte<NB>(t), everything that varies; the word starts meta_lane_bit<NB>(t) bits into that byte.
+template <int NB> __device__ __forceinline__ uint32_t meta_lane_byte(int t) { return (uint32_t)(t * 4 * NB) >> 3; }
+template <int NB> __device__ __forceinline__ uint32_t meta_lane_bit(int t) { return (uint32_t)(t * 4 * NB) & 7u; }
 template <int NB>
-__device__ __forceinline__ uint32_t lds_meta(const uint8_t *base, uint32_t off, int t) {
-    if (NB == 4) return *reinterpret_cast<const uint16_t *>(base + off + 2 * t);
-    if (NB == 2) return base[off + t];
-    // 4 NB bits at bit 4 NB t: byte (4 NB t) / 8, then 0 or 4 bits further (4 NB + 4 <= 32 for NB <= 7)
-    const uint32_t bit = (uint32_t)(t * 4 * NB), a = off + (bit >> 3);
+__device__ __forceinline__ uint32_t lds_meta(const uint8_t *base, uint32_t a, uint32_t lane_bit) {
+    if (NB == 4) return *reinterpret_cast<const uint16_t *>(base + a);
+    if (NB == 2) return base[a];
+    // 4 NB bits, then 0 or 4 bits further (4 NB + 4 <= 32 for NB <= 7)
     const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (a & ~3u));
     const uint32_t v = __builtin_amdgcn_alignbyte(q[1], q[0], a);
-    return (v >> (bit & 7u)) & ((1u << (4 * NB)) - 1u);
+    return (v >> lane_bit) & ((1u << (4 * NB)) - 1u);
 }
 
 template <int W, typename U>
@@ -139,11 +156,15 @@ __device__ __forceinline__ void meta_pairs(uint32_t minsw, uint32_t lensw, U &u)
 // win01[q] = tokens 4q..4q+3 of packs 0 and 1 in the low / high 16 bits (token 4q on top), win23
 // likewise; bits above 4*len in a half are other tokens' fields, every consumer masks.
 __device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[4], uint32_t win23[4]) {
-    const uint32_t len[4] = {u.len01 & 0xFFFFu, u.len01 >> 16, u.len23 & 0xFFFFu, u.len23 >> 16};
+    // shift amounts, two to a register like the widths: 8 len (the upper eight tokens) and 4 len (the upper four of
+    // eight).  A shift takes the low six (five) bits of its amount, and 8 len <= 32 leaves the bits above untouched,
+    // so the low half of a pair serves as it stands and the high half is one byte-select away.
+    const uint32_t s8[2] = {u.len01 << 3, u.len23 << 3}, s4[2] = {u.len01 << 2, u.len23 << 2};
     uint32_t hlf[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        hlf[i][0] = (uint32_t)(u.word[i] >> (8u * len[i]));   // tokens 0..7
+        const uint32_t a8 = (i & 1) ? s8[i >> 1] >> 16 : s8[i >> 1];
+        hlf[i][0] = (uint32_t)(u.word[i] >> (a8 & 63u));    // tokens 0..7
         hlf[i][1] = (uint32_t)u.word[i];                      // tokens 8..15
     }
 #pragma unroll
@@ -152,7 +173,8 @@ __device__ __forceinline__ void pair_windows(const UnitPairs &u, uint32_t win01[
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t src = hlf[i][q >> 1];
-            qd[i] = (q & 1) ? src : (src >> (4u * len[i]));
+            const uint32_t a4 = (i & 1) ? s4[i >> 1] >> 16 : s4[i >> 1];
+            qd[i] = (q & 1) ? src : (src >> (a4 & 31u));
         }
         win01[q] = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);
         win23[q] = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
@@ -207,7 +229,7 @@ template <> struct UnitOf<true> { typedef UnitWide type; };
 template <int G, int KW, int VW>
 constexpr int dma_lds_bytes() {          // static LDS of attn_dma_kernel: two slots, weights, round sums, state
     constexpr int GP = (G + 3) / 4 * 4;
-    return 2 * DmaGeom<KW, VW>::kSlot + GP * (kTile + 4) * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4;
+    return 2 * DmaGeom<KW, VW>::kSlot + GP * (kTile + 4) * 2 + 2 * GP * 8 * 2 + 8 * 8 * 4;
 }
 
 template <int G, int KW, int VW, bool BF>
@@ -234,14 +256,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
 
     constexpr int kPStride = kTile + 4;          // halves per head row of the weights: rows 8 bytes apart in bank space
     constexpr int kLdsBytes = dma_lds_bytes<G, KW, VW>();
-    static_assert(kLdsBytes == 2 * Geo::kSlot + GP * kPStride * 2 + 2 * GP * 8 * 2 + 6 * 8 * 4, "LDS layout");
+    static_assert(kLdsBytes == 2 * Geo::kSlot + GP * kPStride * 2 + 2 * GP * 8 * 2 + 8 * 8 * 4, "LDS layout");
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLdsBytes];
     uint8_t *ring = smem;                                                    // [2 slots][4 block regions | parameters]
     _Float16 *pbuf = reinterpret_cast<_Float16 *>(smem + 2 * Geo::kSlot);    // [GP][128 + 4]
     _Float16 *p16hi = pbuf + GP * kPStride;                                     // [GP][8]
     _Float16 *p16lo = p16hi + GP * 8;
     float *st_m = reinterpret_cast<float *>(p16lo + GP * 8);                 // 8 floats each
-    float *st_l = st_m + 8, *st_a = st_l + 8, *st_z = st_a + 8, *qsum = st_z + 8, *qs = qsum + 8;
+    float *st_l = st_m + 8, *st_z = st_l + 8, *qsum = st_z + 8, *qs = qsum + 8;
+    float *st_a = qs + 8;                                                    // [2 slot parities][8]: accumulator factors of a step
+    uint32_t *resc = reinterpret_cast<uint32_t *>(st_a + 16);                // [2]: some head's factor of that step is not 1
     const uint32_t ring_lds = (uint32_t)reinterpret_cast<uintptr_t>(ring);   // LDS byte address of the slots
 
     // Workgroup L of the launch is member L / (B Hkv) of (sequence, KV head) L % (B Hkv): the members of one head are
@@ -257,23 +281,29 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     const int h = bh_ % p.Hkv, b = bh_ / p.Hkv;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    __builtin_assume(wave >= 0 && wave < 4);
     const int t = tid & 31, hw = tid >> 5;
     const int bh = b * p.Hkv + h;
-    const int n_hid_k = p.B * p.Hkv, n_hid_v = 2 * p.B * p.Hkv;
+    const int n_hid_k = p.B * p.Hkv;
 
     // the stream this wave copies from, range-checked: block_info is never trusted with an address
     // (the size is rounded up to whole dwords: a copy is range-checked dword by dword, and the aligned dword that
     // holds the buffer's last byte lies in the same page as that byte -- a buffer that ends with its stream loses
     // nothing and nothing unmapped is touched)
-    const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, ((wave < 2 ? p.k_bytes : p.v_bytes) + 3u) & ~3u);
+    const uint32_t blk_bytes4 = ((wave < 2 ? p.k_bytes : p.v_bytes) + 3u) & ~3u;
+    const u32x4 blk_rsrc = dma_rsrc(wave < 2 ? p.k_stream : p.v_stream, blk_bytes4);
     const uint16_t *par_arr = wave == 0 ? p.k_scale : wave == 1 ? p.k_zero : wave == 2 ? p.v_scale : p.v_zero;
     const u32x4 par_rsrc = dma_rsrc(par_arr, (uint32_t)(p.B * p.par_stride * 2));
+    const uint32_t par_row = (uint32_t)(b * p.par_stride * 2);        // byte offset of this sequence's parameter rows
 
     // Tiles this member works on, by position in its own sequence.  Static split (p.dynamic == 0): the contiguous
     // range [tile0, tile_end).  Dynamic: positions 0..4 are tiles split + k * nsplit (known at once, they fill the
-    // pipeline), every further position is 5 * nsplit + the next value of the head's counter, fetched five positions
-    // ahead; a faster member simply comes back for more.  Sequences are increasing, a tile number >= tile_end ends
-    // them, and attention does not depend on the order of the tokens.
+    // pipeline); every further position comes out of the head's counter, which counts the tiles handed out so far:
+    // a member adds the size of the batch it wants (up to four tiles while many are left, single tiles towards the
+    // end, so that the members finish together) and owns tiles 5 nsplit + [old value, old value + size); a faster
+    // member simply comes back sooner.  The request for the next batch goes out when the current one is first drawn
+    // on, so its round trip lies at least a whole step before the value is needed.  Sequences are increasing, a
+    // tile number >= tile_end ends them, and attention does not depend on the order of the tokens.
     const int n_tiles = p.T_c / kTile;
     const int tile0 = split * p.tiles_per_split;
     const int tile_end = p.dynamic ? n_tiles : min(n_tiles, tile0 + p.tiles_per_split);
@@ -289,44 +319,70 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     const int kj = wave >> 1;
     const const_u32_ptr k_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.k_info));
     const const_u32_ptr v_info_c = reinterpret_cast<const_u32_ptr>(reinterpret_cast<uintptr_t>(p.v_info));
-    const const_u32_ptr dma_info = wave < 2 ? k_info_c : v_info_c;
-    struct TileInfo { uint32_t dma_off, dma_size, k_off, v_off; };
-    auto load_info = [&](int tile) -> TileInfo {
-        const int tau = min(tile, n_tiles - 1);          // past the end: the last tile again, never used
-        const uint32_t ik0 = (uint32_t)((2 * tau) * n_hid_k + bh), iv0 = (uint32_t)(tau * n_hid_v + 2 * bh);
-        const uint32_t id = wave < 2 ? ik0 + (uint32_t)wave * (uint32_t)n_hid_k : iv0 + (uint32_t)(wave - 2);
-        TileInfo ti;
-        ti.dma_off = dma_info[2 * (size_t)id];
-        ti.dma_size = dma_info[2 * (size_t)id + 1];
-        ti.k_off = k_info_c[2 * (size_t)(ik0 + (uint32_t)kj * (uint32_t)n_hid_k)];
-        ti.v_off = v_info_c[2 * (size_t)(iv0 + (uint32_t)kj)];
-        return ti;
+    // entry of this wave's blocks for tile 0; a tile further on is 2 K rows = 1 V row = 4 B Hkv words further
+    const const_u32_ptr dma_info0 = wave < 2 ? k_info_c + 2 * (size_t)(bh + wave * n_hid_k) : v_info_c + 2 * (size_t)(2 * bh + wave - 2);
+    const const_u32_ptr k_info0 = k_info_c + 2 * (size_t)(bh + kj * n_hid_k), v_info0 = v_info_c + 2 * (size_t)(2 * bh + kj);
+    const uint32_t info_stride = 4u * (uint32_t)n_hid_k;
+    const uint32_t last_tile = (uint32_t)(n_tiles - 1);
+    struct RawInfo { uint32_t dma_off, dma_size, k_off, v_off; };          // as loaded
+    struct TileInfo { uint32_t dma_off, dma_size, ph; };                    // ph: k_off % 16 | v_off % 16 << 4
+    auto load_info = [&](int tile) -> RawInfo {
+        const size_t o = (size_t)min((uint32_t)tile, last_tile) * info_stride;   // past the end (or a damaged counter): the last tile again, never used
+        RawInfo ri;
+        ri.dma_off = dma_info0[o];
+        ri.dma_size = dma_info0[o + 1];
+        ri.k_off = k_info0[o];
+        ri.v_off = v_info0[o];
+        return ri;
+    };
+    auto pack_info = [&](const RawInfo &ri) -> TileInfo {
+        return TileInfo{ri.dma_off, ri.dma_size, (ri.k_off & 15u) | ((ri.v_off & 15u) << 4)};
     };
 
     // ---- copy of one tile into slot `slot` ----
-    auto dma_issue = [&](int slot, int tile, const TileInfo &ti) {
+    // Every copy instruction gets a descriptor of its own (scalar arithmetic): base = the 16-byte boundary below the
+    // block + 1 KiB per instruction, length = what that KiB holds of the block and of the stream.  All instructions
+    // then share one per-lane offset, 16 lane, and lanes past the end of the block fetch nothing and store zeroes.
+    const uint32_t lane16 = 16u * (uint32_t)lane;
+    const uint32_t dst_wave = ring_lds + (uint32_t)wave * (uint32_t)Geo::kRegion;
+    auto dma_issue = [&](auto slot_c, int tile, const TileInfo &ti) {
+        constexpr int slot = decltype(slot_c)::value;
         const uint32_t phase = ti.dma_off & 15u;                  // the streams themselves are 16-byte aligned
         const uint32_t src = ti.dma_off - phase;
-        uint32_t nq = (phase + ti.dma_size + 15u) >> 4;           // 16-byte quads to copy
-        nq = min(max(nq, 1u), (uint32_t)(Geo::kRegion / 16));     // corrupt block_info must not overrun the region
-        const uint32_t last = nq - 1u;
-        const uint32_t dst = ring_lds + (uint32_t)(slot * Geo::kSlot + wave * Geo::kRegion);
+        uint32_t nb = (phase + ti.dma_size + 15u) & ~15u;         // bytes to copy: whole 16-byte quads
+        nb = max(nb, 16u);
+        PKV_SCALAR(nb);
+        nb = min(nb, (uint32_t)Geo::kRegion);                     // corrupt block_info must not overrun the region
+        PKV_SCALAR(nb);
+        uint32_t have = src < blk_bytes4 ? min(nb, blk_bytes4 - src) : 0u;   // ... nor the stream
+        PKV_SCALAR(have);
+        uint32_t dst = dst_wave;                                  // (kept out of the loop-invariant code: ten LDS
+        PKV_SCALAR(dst);                                          // addresses held in scalar registers were spilled)
+        dst += (uint32_t)(slot * Geo::kSlot);
 #pragma unroll
         for (int i = 0; i < Geo::kMaxInstr; i++) {
-            if ((uint32_t)(i * 64) < nq) {                        // wave-uniform
-                if (i * 1024 + 1024 <= Geo::kRegion || lane < (Geo::kRegion - i * 1024) / 16)
-                    dma_b128(blk_rsrc, dst + i * 1024, src + 16u * min((uint32_t)(i * 64 + lane), last));
+            if ((uint32_t)(i * 1024) < nb) {                      // wave-uniform
+                const uint32_t len = have > (uint32_t)(i * 1024) ? min(have - (uint32_t)(i * 1024), 1024u) : 0u;
+                // (the lane test of a partial last instruction is made here, from a value the compiler cannot trace
+                // back to the lane number: as loop-invariant code it would hold a register pair for its mask)
+                uint32_t l16 = lane16;
+                if (i * 1024 + 1024 > Geo::kRegion) asm volatile("" : "+v"(l16));
+                if (i * 1024 + 1024 <= Geo::kRegion || l16 < (uint32_t)(Geo::kRegion - i * 1024))
+                    dma_b128(dma_rsrc_at(blk_rsrc, src + (uint32_t)(i * 1024), len), dst + i * 1024, lane16);
             }
         }
-        // parameter array `wave` of the tile: 128 tokens x 2 bytes = 64 lanes x 4 bytes
-        const int tile_off = (b * p.par_stride + min(tile, n_tiles - 1) * kTile) * 2;
-        dma_b32(par_rsrc, ring_lds + (uint32_t)(slot * Geo::kSlot + Geo::kParOff + wave * 256), 4 * lane, (uint32_t)tile_off);
+        // parameter array `wave` of the tile: 128 tokens x 2 bytes = 16 lanes x 16 bytes
+        const uint32_t tile_off = par_row + min((uint32_t)tile, last_tile) * (uint32_t)(kTile * 2);
+        uint32_t l16p = lane16;
+        asm volatile("" : "+v"(l16p));
+        if (l16p < 256u)
+            dma_b128(dma_rsrc_at(par_rsrc, tile_off, 256u), dst + (uint32_t)Geo::kParOff - (uint32_t)wave * (uint32_t)(Geo::kRegion - 256), lane16);
     };
 
     // tile 0 starts its way into slot 0 now, under the prologue's arithmetic
     int t_cur = first_tiles(0), t1 = first_tiles(1), t2 = first_tiles(2), t3 = first_tiles(3);
-    TileInfo i0 = load_info(t_cur), i1 = load_info(t1), i2 = load_info(t2);
-    dma_issue(0, t_cur, i0);
+    TileInfo i0 = pack_info(load_info(t_cur)), i1 = pack_info(load_info(t1)), i2 = pack_info(load_info(t2));
+    dma_issue(IntC<0>{}, t_cur, i0);
 
     auto cvt2 = [&](uint32_t w, float &lo, float &hi) {
         if (!BF) {
@@ -344,7 +400,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     for (int i = tid; i < NSETS * 4 * 16 * 32 / 4; i += 256) reinterpret_cast<uint32_t *>(aq)[i] = 0u;
     for (int i = tid; i < GP * kPStride / 2; i += 256) reinterpret_cast<uint32_t *>(pbuf)[i] = 0u;
     for (int i = tid; i < GP * 8; i += 256) reinterpret_cast<uint32_t *>(p16hi)[i] = 0u;   // hi and lo
-    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 1.f; }
+    if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 1.f; st_a[8 + tid] = 1.f; resc[tid] = 0u; }
     __builtin_amdgcn_s_waitcnt(0xC07F);       // lgkmcnt(0): the zeroes are written; the copy in flight is not waited for
     __builtin_amdgcn_s_barrier();
     for (int g = wave; g < G; g += 4) {
@@ -395,14 +451,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
 
     // ---- parse of this half-wave's K unit and V unit out of a landed slot ----
     const int ku = hw & 3;
-    auto parse = [&](int slot, const TileInfo &ti, KUnit &kr, VUnit &vr) {
-        const uint8_t *kb = ring + slot * Geo::kSlot + kj * Geo::kRegion;
-        const uint8_t *vb = ring + slot * Geo::kSlot + (2 + kj) * Geo::kRegion;
-        const uint32_t kph = ti.k_off & 15u, vph = ti.v_off & 15u;
+    // what a lane adds to a unit's offset inside its block region to reach its own metadata (the region of K block
+    // kj included; V block 2 + kj lies two regions further, a constant)
+    const uint32_t kj_region = (uint32_t)(kj * Geo::kRegion);
+    const uint32_t hdr_c = kj_region + 2u * (uint32_t)max(ku - 1, 0);
+    const uint32_t kmin_c = kj_region + meta_lane_byte<KW>(t), klen_c = kj_region + meta_lane_byte<KLB>(t);
+    const uint32_t vmin_c = VW == KW ? kmin_c : kj_region + meta_lane_byte<VW>(t);
+    const uint32_t vlen_c = VLB == KLB ? klen_c : kj_region + meta_lane_byte<VLB>(t);
+    const uint32_t kmin_b = meta_lane_bit<KW>(t), klen_b = meta_lane_bit<KLB>(t), vmin_b = meta_lane_bit<VW>(t), vlen_b = meta_lane_bit<VLB>(t);
+    auto parse = [&](auto slot_c, const TileInfo &ti, KUnit &kr, VUnit &vr) {
+        constexpr int slot = decltype(slot_c)::value;
+        const uint8_t *kb0 = ring + slot * Geo::kSlot, *vb0 = kb0 + 2 * Geo::kRegion;   // region of K block 0 / V block 0
+        const uint8_t *kb = kb0 + kj * Geo::kRegion;
+        const uint8_t *vb = vb0 + kj * Geo::kRegion;
+        const uint32_t kph = ti.ph & 15u, vph = ti.ph >> 4;
         // header: four cumulative u16 unit sizes; unit u starts at 8 + cum[u - 1] (read unconditionally, then selected)
-        const uint32_t hsel = 2u * (uint32_t)max(ku - 1, 0);
-        uint32_t kc = *reinterpret_cast<const uint16_t *>(kb + kph + hsel);
-        uint32_t vc = *reinterpret_cast<const uint16_t *>(vb + vph + hsel);
+        uint32_t kc = *reinterpret_cast<const uint16_t *>(kb0 + (kph + hdr_c));
+        uint32_t vc = *reinterpret_cast<const uint16_t *>(vb0 + (vph + hdr_c));
         kc = ku ? kc : 0u;
         vc = ku ? vc : 0u;
         // A corrupt header must not send the metadata reads out of the block's region.  The pack
@@ -410,8 +475,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         // workgroup's LDS (2.3 KiB follow the last region); garbage in, garbage out, no fault.
         const uint32_t k_unit = min(kph + 8u + kc, (uint32_t)(Geo::kRegion - K_META - 16));
         const uint32_t v_unit = min(vph + 8u + vc, (uint32_t)(Geo::kRegion - V_META - 16));
-        const uint32_t k_mins = lds_meta<KW>(kb, k_unit, t), k_lens = lds_meta<KLB>(kb, k_unit + KW * 16, t);
-        const uint32_t v_mins = lds_meta<VW>(vb, v_unit, t), v_lens = lds_meta<VLB>(vb, v_unit + VW * 16, t);
+        const uint32_t k_mins = lds_meta<KW>(kb0, k_unit + kmin_c, kmin_b), k_lens = lds_meta<KLB>(kb0 + KW * 16, k_unit + klen_c, klen_b);
+        const uint32_t v_mins = lds_meta<VW>(vb0, v_unit + vmin_c, vmin_b), v_lens = lds_meta<VLB>(vb0 + VW * 16, v_unit + vlen_c, vlen_b);
         uint32_t koff[4], voff[4];
         meta_pairs<KW>(k_mins, k_lens, kr);
         meta_pairs<VW>(v_mins, v_lens, vr);
@@ -504,58 +569,94 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     };
 
     // ---- stage 2: online softmax; wave <-> query head, lane <-> tokens 2*lane, 2*lane+1 ----
-    // Biased exponents of the v_scale of this lane's two tokens against the largest met so far (every wave sees the
-    // same tokens, so all four take the same decision).  Runs ahead of the parse so that the rare branch does not
-    // split the block in which the compiler interleaves the parse with the softmax.
-    float grow = 1.f;
-    auto emax_check = [&](int slot) {
-        const uint32_t vs_raw = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff)[128 + lane];
-        const uint32_t ex = (vs_raw >> (BF ? 7 : 10)) & (BF ? 0x00FF00FFu : 0x001F001Fu);
-        const ushort2v mxp = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, ex), __builtin_bit_cast(ushort2v, emax_pair));
-        grow = 1.f;
-        if (__builtin_amdgcn_ballot_w64(__builtin_bit_cast(uint32_t, mxp) != emax_pair) != 0) {     // rare
-            const uint32_t mine = max(__builtin_bit_cast(uint32_t, mxp) & 0xFFFFu, __builtin_bit_cast(uint32_t, mxp) >> 16);
-            uint32_t e = (uint32_t)__builtin_bit_cast(int, wave_max(__builtin_bit_cast(float, mine)));   // small positive ints order like floats
-            e = max(e, BF ? 14u : 1u);
-            const uint32_t old = emax_pair & 0xFFFFu;
-            grow = __builtin_amdgcn_exp2f(-(float)(int)(e - old));       // 0 on the first tile (nothing accumulated yet)
-            emax_pair = e | (e << 16);
-            wscale = __uint_as_float((uint32_t)(kWExp - (int)e + 127) << 23);
-            wscale_inv = __uint_as_float((uint32_t)((int)e - kWExp + 127) << 23);
-        }
-    };
-    auto softmax_stage = [&](int slot, const uint8_t *kt) {
+    // The usual tile changes neither the running maximum of its head nor the largest exponent of v_scale: then no
+    // cross-lane maximum is formed, nothing is rescaled and the V stage is told nothing.  A tile in which some lane
+    // sees a larger score or a larger exponent takes the full update instead (about 1 / n of the tiles at position n
+    // of a member's sequence).  Both tests are per lane and meet in one branch.
+    // ethr_pair: in both halves the largest raw 16-bit pattern whose exponent does not exceed emax (a negative
+    // v_scale, which no quantiser produces, compares above it and merely takes the full update every time).
+    constexpr int kMant = BF ? 7 : 10;
+    uint32_t ethr_pair = 0u;
+    int stale_factors = 0;           // this wave published factors != 1 in the previous step: put them back to 1
+    auto softmax_stage = [&](auto slot_c, const uint8_t *kt) {
+        constexpr int slot = decltype(slot_c)::value;
         const uint32_t *par = reinterpret_cast<const uint32_t *>(ring + slot * Geo::kSlot + Geo::kParOff) + lane;
         const uint32_t vs_raw = par[128];
         float ks0, ks1, kz0, kz1, vs0, vs1, vz0, vz1;
         cvt2(par[0], ks0, ks1); cvt2(par[64], kz0, kz1); cvt2(vs_raw, vs0, vs1); cvt2(par[192], vz0, vz1);
+        if (stale_factors) {         // rare; the V stage that read them lies before this step's first barrier
+            if (lane == 0) {
+#pragma unroll
+                for (int gi = 0; gi < GW; gi++)
+                    if (wave + 4 * gi < G) st_a[(slot ^ 1) * 8 + wave + 4 * gi] = 1.f;
+                resc[slot ^ 1] = 0u;
+            }
+            stale_factors = 0;
+        }
+        float sv0[GW], sv1[GW];
+        const ushort2v cap = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, vs_raw), __builtin_bit_cast(ushort2v, ethr_pair));
+        bool up = __builtin_bit_cast(uint32_t, cap) != ethr_pair;
+#pragma unroll
+        for (int gi = 0; gi < GW; gi++) {
+            const int g = min(wave + 4 * gi, G - 1);
+            const int R = lane >> 3;
+            const uint2v raw = *reinterpret_cast<const uint2v *>(
+                kt + R * kRoundBytes + 256 * (g >> 2) + 64 * (((g & 3) + R) & 3) + 8 * (lane & 7));
+            const float D0 = SCORE_INT ? (float)(int)raw[0] : __uint_as_float(raw[0]);
+            const float D1 = SCORE_INT ? (float)(int)raw[1] : __uint_as_float(raw[1]);
+            // log2-domain scores
+            sv0[gi] = fmaf(ks0, c1_r[gi], 0.f) * fmaf(kz0, c2_r[gi], D0);     // (a fused multiply-add takes the 16-bit
+            sv1[gi] = fmaf(ks1, c1_r[gi], 0.f) * fmaf(kz1, c2_r[gi], D1);     // operand as it is: no conversion first)
+            if (wave + 4 * gi < G) up = up || fmaxf(sv0[gi], sv1[gi]) > m_run[gi];
+        }
+        const bool full = __builtin_amdgcn_ballot_w64(up) != 0;
+        float grow = 1.f;
+        if (full) {
+            // biased exponents of the v_scale of this lane's two tokens against the largest met so far (every wave
+            // sees the same tokens, so all four take the same decision)
+            const uint32_t ex = (vs_raw >> kMant) & (BF ? 0x00FF00FFu : 0x001F001Fu);
+            const ushort2v mxp = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, ex), __builtin_bit_cast(ushort2v, emax_pair));
+            if (__builtin_amdgcn_ballot_w64(__builtin_bit_cast(uint32_t, mxp) != emax_pair) != 0) {
+                const uint32_t mine = max(__builtin_bit_cast(uint32_t, mxp) & 0xFFFFu, __builtin_bit_cast(uint32_t, mxp) >> 16);
+                uint32_t e = (uint32_t)__builtin_bit_cast(int, wave_max(__builtin_bit_cast(float, mine)));   // small positive ints order like floats
+                e = max(e, BF ? 14u : 1u);
+                const uint32_t old = emax_pair & 0xFFFFu;
+                grow = __builtin_amdgcn_exp2f(-(float)(int)(e - old));       // 0 on the first tile (nothing accumulated yet)
+                emax_pair = e | (e << 16);
+                wscale = __uint_as_float((uint32_t)(kWExp - (int)e + 127) << 23);
+                wscale_inv = __uint_as_float((uint32_t)((int)e - kWExp + 127) << 23);
+                const uint32_t thr = ((e + 1u) << kMant) - 1u;
+                ethr_pair = thr | (thr << 16);
+            }
+        }
 #pragma unroll
         for (int gi = 0; gi < GW; gi++) {
             const int g = wave + 4 * gi;
             if (g < G) {
-                const int R = lane >> 3;
-                const uint2v raw = *reinterpret_cast<const uint2v *>(
-                    kt + R * kRoundBytes + 256 * (g >> 2) + 64 * (((g & 3) + R) & 3) + 8 * (lane & 7));
-                const float D0 = SCORE_INT ? (float)(int)raw[0] : __uint_as_float(raw[0]);
-                const float D1 = SCORE_INT ? (float)(int)raw[1] : __uint_as_float(raw[1]);
-                // log2-domain scores
-                const float sv0 = (ks0 * c1_r[gi]) * fmaf(kz0, c2_r[gi], D0);
-                const float sv1 = (ks1 * c1_r[gi]) * fmaf(kz1, c2_r[gi], D1);
-                const float mx = wave_max_fused(fmaxf(sv0, sv1));
-                const float m_new = fmaxf(m_run[gi], mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run[gi] - m_new);    // exp2(-inf) = 0 on the first tile
-                m_run[gi] = m_new;
-                const float p0 = __builtin_amdgcn_exp2f(sv0 - m_new), p1 = __builtin_amdgcn_exp2f(sv1 - m_new);
-                const _Float16 h0 = (_Float16)(p0 * (vs0 * wscale)), h1 = (_Float16)(p1 * (vs1 * wscale));
+                float alpha = 1.f, beta = 1.f;
+                if (full) {
+                    const float mx = wave_max_fused(fmaxf(sv0[gi], sv1[gi]));
+                    const float m_new = fmaxf(m_run[gi], mx);
+                    alpha = __builtin_amdgcn_exp2f(m_run[gi] - m_new);    // exp2(-inf) = 0 on the first tile
+                    m_run[gi] = m_new;
+                    beta = alpha * grow;     // what the weighted sums so far are multiplied by
+                }
+                const float p0 = __builtin_amdgcn_exp2f(sv0[gi] - m_run[gi]), p1 = __builtin_amdgcn_exp2f(sv1[gi] - m_run[gi]);
+                const _Float16 h0 = (_Float16)(p0 * fmaf(vs0, wscale, 0.f)), h1 = (_Float16)(p1 * fmaf(vs1, wscale, 0.f));
                 const float f0 = (float)h0, f1 = (float)h1;
                 // V-side order: MFMA k of a segment contracts token k of its four rounds
                 const int tok0 = 2 * lane;
                 _Float16 *pb = pbuf + g * kPStride + (tok0 & 64) + ((tok0 & 15) << 2) + ((tok0 >> 4) & 3);
                 pb[0] = h0;
                 pb[4] = h1;      // token 2*lane+1: same round, next k
-                const float beta = alpha * grow;     // what the weighted sums so far are multiplied by
-                l_part[gi] = l_part[gi] * alpha + (p0 + p1);
-                z_part[gi] = z_part[gi] * beta + (f0 * vz0 + f1 * vz1);
+                if (full) {
+                    l_part[gi] = l_part[gi] * alpha + (p0 + p1);
+                    z_part[gi] = z_part[gi] * beta + (f0 * vz0 + f1 * vz1);
+                    if (lane == 0) { st_a[slot * 8 + g] = beta; resc[slot] = 1u; }
+                } else {
+                    l_part[gi] += p0 + p1;
+                    z_part[gi] += f0 * vz0 + f1 * vz1;
+                }
                 // per-round sums (16 tokens = 8 lanes) of the rounded weights, for the pack-minimum term
                 const float r16 = oct_sum_fused(f0 + f1);
                 if ((lane & 7) == 0) {
@@ -563,9 +664,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
                     p16hi[g * 8 + (lane >> 3)] = hi;
                     p16lo[g * 8 + (lane >> 3)] = (_Float16)(r16 - (float)hi);
                 }
-                if (lane == 0) st_a[g] = beta;
             }
         }
+        if (full) stale_factors = 1;
     };
 
     // ---- stage 3: V segment hw; lane = channel, MFMA k contracts token k of the lane's four packs ----
@@ -581,7 +682,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         for (int pp = 0; pp < 4; pp++) a_w[pp][i4] = (half4v){0, 0, 0, 0};
     }
     const bool a_loader = (lane & 31) < 4;
-    auto v_stage = [&](const VUnit &vr) {
+    // LDS address of this lane's weights (head lane % 4, segment half hw % 2), handed to the compiler as a value it
+    // cannot split: it would otherwise keep the per-lane part and add the array's base again at every read
+    typedef const __attribute__((address_space(3))) half4v *lds_half4_ptr;
+    uint32_t aw_addr = (uint32_t)reinterpret_cast<uintptr_t>(pbuf + (lane & 3) * kPStride + 64 * (hw & 1));
+    asm volatile("" : "+v"(aw_addr));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wint-to-pointer-cast"      // the host pass sees a 64-bit pointer here; LDS pointers are 32 bits wide
+    const lds_half4_ptr aw_ptr = (lds_half4_ptr)aw_addr;
+#pragma clang diagnostic pop
+    auto v_stage = [&](auto slot_c, const VUnit &vr) {
+        constexpr int slot = decltype(slot_c)::value;
         constexpr int TPW = VTPW, NWIN = VNWIN;
         const int seg = hw & 1;
         uint32_t w01[NWIN], w23[NWIN];
@@ -593,18 +704,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         }
         const uint32_t len01 = vr.len01, len23 = vr.len23;
         const uint32_t m01 = pk_mask16(len01), m23 = pk_mask16(len23);
-        // rescale the accumulators only when some head's running maximum moved (alpha <= 1, so the
-        // product is 1 exactly when every alpha is)
-        {
-            float prod = 1.f;
+        // rescale the accumulators only when the softmax of this step said that some head's factor is not 1
+        if (__builtin_amdgcn_readfirstlane(resc[slot]) != 0u) {
 #pragma unroll
-            for (int g = 0; g < GP; g++) prod *= st_a[g];
-            if (__builtin_amdgcn_readfirstlane(__float_as_uint(prod)) != 0x3F800000u) {
-#pragma unroll
-                for (int i4 = 0; i4 < NG4; i4++) {
-                    const float4v al = *reinterpret_cast<const float4v *>(st_a + 4 * i4);
-                    acc[i4] *= al;
-                }
+            for (int i4 = 0; i4 < NG4; i4++) {
+                const float4v al = *reinterpret_cast<const float4v *>(st_a + slot * 8 + 4 * i4);
+                acc[i4] *= al;
             }
         }
         const int gl = lane & 3;
@@ -630,7 +735,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
                 for (int pp = 0; pp < 4; pp++)
 #pragma unroll
                     for (int i4 = 0; i4 < NG4; i4++)
-                        a_w[pp][i4] = *reinterpret_cast<const half4v *>(pbuf + (4 * i4 + gl) * kPStride + 64 * seg + 4 * (4 * q + pp));
+                        a_w[pp][i4] = aw_ptr[i4 * kPStride + 4 * q + pp];     // head 4 i4 + lane % 4, tokens 4 (4 q + pp) ..+3 of the segment half
             }
             uint32_t x01 = 0, x23 = 0;
 #pragma unroll
@@ -648,56 +753,84 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     };
 
     // ---- pipeline ----
-    KUnit kcur;
-    VUnit vcur;
+    KUnit k_a, k_b;               // the units of the tile a step works on and of the one it parses alternate between
+    VUnit v_a, v_b;               // the two sets; the loop below is written out twice so that nothing is copied
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile 0 (issued before the prologue's arithmetic)
     PKV_LDS_BARRIER();                                    // ... and every wave has its q operands out of slot 1
-    dma_issue(1, t1, i1);
-    parse(0, i0, kcur, vcur);
+    dma_issue(IntC<1>{}, t1, i1);
+    parse(IntC<0>{}, i0, k_a, v_a);
+    // the head's counter: tiles 5 nsplit + [old value, old value + size) belong to whoever added `size`
+    const int n_dyn = n_tiles - 5 * p.nsplit;                   // tiles that are handed out by counter
+    uint32_t fetched = 0u;        // wave 0, lane 0: old counter value of the request in flight
+    int pend_n = 0, cur_base = 0, cur_left = 0;                 // size of that request; the batch being drawn on
+    // (the index goes through a vector register the compiler cannot see into: with an address it knows to be the
+    // same in every lane it rewrites the atomic as a reduction over the active lanes whose epilogue waits for the
+    // answer on the spot -- and with it for the copies just issued)
+    uint32_t ctr_idx = (uint32_t)bh;
+    asm volatile("" : "+v"(ctr_idx));
+    auto batch_of = [&](int handed) -> int {
+        int n = (n_dyn - handed) >> p.batch_shift;
+        n = max(n, 1);
+        PKV_SCALAR(n);
+        return min(n, 4);
+    };
+    auto request = [&](int n) {
+        if (wave == 0 && lane == 0)
+            fetched = __hip_atomic_fetch_add(p.counters + ctr_idx, (uint32_t)n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        pend_n = n;
+    };
+    if (p.dynamic) request(batch_of(0));
     PKV_LDS_BARRIER();
 
     // Step s works on position s of the sequence (tile t_cur); t1, t2, t3 = the tiles of positions s+1 .. s+3, i1, i2 =
-    // block_info of t1, t2.  Position s+4 becomes known in the middle of the step: wave 0 asked the head's counter
-    // for it during step s-1, receives it with the copies it waits for before barrier 1 and hands it on through LDS.
-    uint32_t fetched = 0u;      // wave 0, lane 0: counter value of the request in flight
-    // (the address travels in vector registers: a scalar base that the compiler had just restored with a VALU
-    // instruction would reach the memory instruction inside the asm statement without the wait states it needs)
-    const uint32_t one = 1u;
-    const uint64_t ctr_addr = reinterpret_cast<uint64_t>(p.counters + bh);
-    for (int s = 0; t_cur < tile_end; s++) {
-        const int slot = s & 1;
+    // block_info of t1, t2.  Position s+4 becomes known in the middle of the step: from the batch being drawn on, or,
+    // when that is used up, from the request wave 0 sent at least a step ago -- its answer has arrived with the
+    // copies the wave waits for before barrier 1 and is handed to the other waves through LDS.
+    int s = 0;
+    auto step = [&](auto slot_c, KUnit &kcur, VUnit &vcur, KUnit &knext, VUnit &vnext) {
+        constexpr int slot = decltype(slot_c)::value;
         uint8_t *kt = ring + slot * Geo::kSlot;
-        const TileInfo i3 = load_info(t3);
+        const RawInfo i3 = load_info(t3);
+        const bool take = p.dynamic && s > 0 && cur_left == 0;       // this step starts on the next batch
         __builtin_amdgcn_s_setprio(Prio::K);
         if (!(PKV_ATTN_PROBE & 2)) k_stage(kcur, kt);
         __builtin_amdgcn_s_setprio(0);
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(fetched) :: "memory");     // this wave's part of tile t1 has landed
-        if (p.dynamic && wave == 0 && lane == 0) tau_lds[slot] = 5 * p.nsplit + (int)fetched;
-        PKV_LDS_BARRIER();                                    // publishes the scores, tile t1 and position s+4
-        int t4 = s == 0 || !p.dynamic ? (s == 0 ? first_tiles(4) : t3 + 1)
-                                      : __builtin_amdgcn_readfirstlane(tau_lds[slot]);
-        KUnit knext;
-        VUnit vnext;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile t1 has landed
+        if (take && wave == 0 && lane == 0) tau_lds[slot] = (int)fetched;
+        PKV_LDS_BARRIER();                                    // publishes the scores, tile t1 and the new batch
+        int t4;
+        if (!p.dynamic) {
+            t4 = t3 + 1;
+        } else if (s == 0) {
+            t4 = first_tiles(4);
+        } else {
+            if (take) { cur_base = __builtin_amdgcn_readfirstlane(tau_lds[slot]); cur_left = pend_n; }
+            t4 = 5 * p.nsplit + cur_base;
+            cur_base++;
+            cur_left--;
+        }
         __builtin_amdgcn_s_setprio(Prio::S);
-        emax_check(slot);
-        if (!(PKV_ATTN_PROBE & 16)) parse(slot ^ 1, i1, knext, vnext); else { knext = kcur; vnext = vcur; }
-        if (!(PKV_ATTN_PROBE & 4)) softmax_stage(slot, kt);
+        if (!(PKV_ATTN_PROBE & 16)) parse(IntC<slot ^ 1>{}, i1, knext, vnext); else { knext = kcur; vnext = vcur; }
+        if (!(PKV_ATTN_PROBE & 4)) softmax_stage(slot_c, kt);
         __builtin_amdgcn_s_setprio(0);
         PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile t1 is parsed
         __builtin_amdgcn_s_setprio(Prio::D);
-        if (!(PKV_ATTN_PROBE & 1)) dma_issue(slot, t2, i2);
-        if (p.dynamic && wave == 0 && lane == 0)              // position s+5, collected at the wait above in step s+1
-            asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(fetched) : "v"(ctr_addr), "v"(one) : "memory");
+        if (!(PKV_ATTN_PROBE & 1)) dma_issue(slot_c, t2, i2);
+        if (take) request(batch_of(cur_base));                // collected at the wait above, a step or more from now
         __builtin_amdgcn_s_setprio(Prio::V);
-        if (!(PKV_ATTN_PROBE & 8)) v_stage(vcur);
+        if (!(PKV_ATTN_PROBE & 8)) v_stage(slot_c, vcur);
         __builtin_amdgcn_s_setprio(0);
-        kcur = knext;
-        vcur = vnext;
         t_cur = t1; t1 = t2; t2 = t3; t3 = t4;
-        i1 = i2; i2 = i3;
+        i1 = i2; i2 = pack_info(i3);
+        s++;
+    };
+    while ((uint32_t)t_cur < (uint32_t)tile_end) {
+        step(IntC<0>{}, k_a, v_a, k_b, v_b);
+        if (!((uint32_t)t_cur < (uint32_t)tile_end)) break;
+        step(IntC<1>{}, k_b, v_b, k_a, v_a);
     }
     // drain: the copy issued in the last step must land before the workgroup's LDS is released
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(fetched) :: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // the last member of the head to get here (every request of the others has been answered) zeroes the head's two
     // counters for the next launch
     if (p.dynamic && tid == 0) {

@@ -164,6 +164,29 @@ def test_attn_decode_full_size_property(cuda):
     assert err <= 1e-3 * want.abs().max().item() + 2 ** -11 * want.abs().max().item() + 2e-5
 
 
+@pytest.mark.parametrize("dtype,hq,rel", [(torch.float16, 32, 0.1), (torch.bfloat16, 32, 0.1), (torch.float16, 8, 0.1),
+                                          (torch.float16, 16, 0.1), (torch.bfloat16, 64, 0.1), (torch.float16, 32, 0.05),
+                                          (torch.bfloat16, 32, 0.03), (torch.float16, 32, 0.2)])
+def test_attn_decode_tiles_handed_out_by_counter(cuda, dtype, hq, rel):
+    """Shapes at which the members of a (sequence, KV head) take their tiles from the head's counter (eight members
+    with twelve tiles each and more): random queries, every group size, both dtypes, the reference's widths and the
+    extension widths, against the plain kernel, whose workgroups own fixed tile ranges.  The two kernels differ by
+    their own rounding only.  Three steps in a row: the counters must come back to zero after each."""
+    B, Hkv, T = 16, 8, 12288
+    k, v = synth.make_kv(B, Hkv, T, seed=410, dtype=dtype, device=cuda)
+    ke, ve = ops.k_quant_encode(k, rel), ops.v_quant_encode(v, rel)
+    del k, v
+    half_ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    for rep in range(3):
+        q = synth.make_q(B, hq, seed=411 + rep, dtype=dtype, device=cuda)
+        fast = ops.attn_decode(q, ke, ve, variant=0).float()
+        plain = ops.attn_decode(q, ke, ve, variant=1).float()
+        err = (fast - plain).abs()
+        _say("tiles by counter", dtype, "group of", hq // Hkv, "rel", rel, "step", rep, "max diff %.3e" % err.max().item())
+        assert bool(torch.isfinite(fast).all())
+        assert bool((err <= 2 * 5e-4 + 2.1 * half_ulp * plain.abs()).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_long_context_layer_at_its_own_size(cuda, dtype):
     """One layer of the long-context configuration at its own size -- batch 4, 32 query / 8 KV heads, 131072 cached
