@@ -35,7 +35,11 @@ namespace pkv {
 // to fewer resident workgroups: with three (groups of 8) equal priorities are best (197 us against 218), with two
 // (widths 5 and 6) the K stage first (211 us against 218).
 template <int G, bool WIDE> struct StagePrio {                       // 4 workgroups per CU
+#ifdef PKV_PRIO_K
+    static constexpr int K = PKV_PRIO_K, S = PKV_PRIO_S, D = PKV_PRIO_D, V = PKV_PRIO_V;
+#else
     static constexpr int K = 1, S = 2, D = 0, V = 3;                 // K stage, parse + softmax, copy issue and waits, V stage
+#endif
 };
 template <int G> struct StagePrio<G, true> { static constexpr int K = 2, S = 1, D = 0, V = 0; };
 template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 0, V = 0; };
@@ -47,7 +51,7 @@ template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 
 
 // PKV_ATTN_PROBE (measurement builds only, results are then meaningless): bit mask of pipeline stages to leave out
 // of the tile loop -- 1 the copies (the first two tiles are re-used), 2 the K stage, 4 the softmax, 8 the V stage,
-// 16 the parse.  30 = "loads only", 1 = "arithmetic only".
+// 16 the parse, 32 the wait for the copies.  30 = "loads only", 1 = "arithmetic only".
 #ifndef PKV_ATTN_PROBE
 #define PKV_ATTN_PROBE 0
 #endif
@@ -70,6 +74,14 @@ __device__ __forceinline__ u32x4 dma_rsrc(const void *base, uint32_t bytes) {
 __device__ __forceinline__ void dma_b128(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+// The same with an immediate offset, which the hardware adds on both sides: to the buffer offset (and its range
+// check) and to the LDS address (measured: data of `offset:1024` lands 1 KiB behind M0's address).
+template <int IMM>
+__device__ __forceinline__ void dma_b128_imm(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
+    static_assert(IMM >= 0 && IMM < 4096, "12-bit immediate");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen offset:%3 lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "n"(IMM) : "memory");
 }
 __device__ __forceinline__ void dma_b32(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
@@ -340,9 +352,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     };
 
     // ---- copy of one tile into slot `slot` ----
-    // Every copy instruction gets a descriptor of its own (scalar arithmetic): base = the 16-byte boundary below the
-    // block + 1 KiB per instruction, length = what that KiB holds of the block and of the stream.  All instructions
-    // then share one per-lane offset, 16 lane, and lanes past the end of the block fetch nothing and store zeroes.
+    // The block gets a descriptor of its own (scalar arithmetic): base = the 16-byte boundary below the block, length
+    // = what the block and the stream hold from there.  Every copy instruction then uses the same per-lane offset,
+    // 16 lane, plus 1 KiB per instruction as an immediate; lanes past the end fetch nothing and store zeroes.
     const uint32_t lane16 = 16u * (uint32_t)lane;
     const uint32_t dst_wave = ring_lds + (uint32_t)wave * (uint32_t)Geo::kRegion;
     auto dma_issue = [&](auto slot_c, int tile, const TileInfo &ti) {
@@ -359,24 +371,34 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         uint32_t dst = dst_wave;                                  // (kept out of the loop-invariant code: ten LDS
         PKV_SCALAR(dst);                                          // addresses held in scalar registers were spilled)
         dst += (uint32_t)(slot * Geo::kSlot);
+        const u32x4 rs = dma_rsrc_at(blk_rsrc, src, have);
+        dma_b128_imm<0>(rs, dst, lane16);
+        if (nb > 1024u) dma_b128_imm<1024>(rs, dst, lane16);      // wave-uniform
+        if (Geo::kRegion > 2048 && nb > 2048u) dma_b128_imm<2048>(rs, dst, lane16);
+        if (Geo::kRegion > 3072 && nb > 3072u) dma_b128_imm<3072>(rs, dst, lane16);
 #pragma unroll
-        for (int i = 0; i < Geo::kMaxInstr; i++) {
-            if ((uint32_t)(i * 1024) < nb) {                      // wave-uniform
-                const uint32_t len = have > (uint32_t)(i * 1024) ? min(have - (uint32_t)(i * 1024), 1024u) : 0u;
+        for (int i = 4; i < Geo::kMaxInstr; i++) {                // beyond the immediate's reach: rare, large blocks
+            if ((uint32_t)(i * 1024) < nb) {
+                uint32_t len = max(have, (uint32_t)(i * 1024));        // (a conditional difference becomes a saturating
+                PKV_SCALAR(len);                                       // subtraction, which only the vector unit has)
+                len -= (uint32_t)(i * 1024);
                 // (the lane test of a partial last instruction is made here, from a value the compiler cannot trace
                 // back to the lane number: as loop-invariant code it would hold a register pair for its mask)
                 uint32_t l16 = lane16;
                 if (i * 1024 + 1024 > Geo::kRegion) asm volatile("" : "+v"(l16));
+                const u32x4 rs_i = dma_rsrc_at(blk_rsrc, src + (uint32_t)(i * 1024), len);     // scalar: before the lane test
+                const uint32_t dst_i = dst + (uint32_t)(i * 1024);
                 if (i * 1024 + 1024 <= Geo::kRegion || l16 < (uint32_t)(Geo::kRegion - i * 1024))
-                    dma_b128(dma_rsrc_at(blk_rsrc, src + (uint32_t)(i * 1024), len), dst + i * 1024, lane16);
+                    dma_b128(rs_i, dst_i, lane16);
             }
         }
         // parameter array `wave` of the tile: 128 tokens x 2 bytes = 16 lanes x 16 bytes
         const uint32_t tile_off = par_row + min((uint32_t)tile, last_tile) * (uint32_t)(kTile * 2);
+        const u32x4 rs_p = dma_rsrc_at(par_rsrc, tile_off, 256u);
+        const uint32_t dst_p = dst + (uint32_t)Geo::kParOff - (uint32_t)wave * (uint32_t)(Geo::kRegion - 256);
         uint32_t l16p = lane16;
         asm volatile("" : "+v"(l16p));
-        if (l16p < 256u)
-            dma_b128(dma_rsrc_at(par_rsrc, tile_off, 256u), dst + (uint32_t)Geo::kParOff - (uint32_t)wave * (uint32_t)(Geo::kRegion - 256), lane16);
+        if (l16p < 256u) dma_b128(rs_p, dst_p, lane16);
     };
 
     // tile 0 starts its way into slot 0 now, under the prologue's arithmetic
@@ -538,32 +560,40 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // both rounds' operands first, then the products of the two rounds in turn: a round's second product waits
+        // for its first, the other round's fills the gap
+        long bop[2][4];
 #pragma unroll
         for (int rr = 0; rr < 2; rr++) {
-            const int R = 2 * wave + rr;
-            const uint8_t *row = kt + (R * 16 + (lane & 15)) * kKtStride + 8 * (lane >> 4);
-            long bop[4];
+            const uint8_t *row = kt + ((2 * wave + rr) * 16 + (lane & 15)) * kKtStride + 8 * (lane >> 4);
 #pragma unroll
-            for (int sl = 0; sl < 4; sl++) bop[sl] = *reinterpret_cast<const long *>(row + 32 * sl);
+            for (int sl = 0; sl < 4; sl++) bop[rr][sl] = *reinterpret_cast<const long *>(row + 32 * sl);
+        }
 #pragma unroll
-            for (int s = 0; s < NSETS; s++) {
-                int4v d = {0, 0, 0, 0};
-                // two K = 64 products: which 64 channels an instruction contracts does not matter as long
-                // as A and B pair up the same ones, and both operands were loaded in the same pattern
-                // (the 8 channels at 32 sl + 8 (lane / 16)), so slices (0, 1) and (2, 3) simply concatenate
+        for (int s = 0; s < NSETS; s++) {
+            int4v d[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+            // two K = 64 products per round: which 64 channels an instruction contracts does not matter as long
+            // as A and B pair up the same ones, and both operands were loaded in the same pattern
+            // (the 8 channels at 32 sl + 8 (lane / 16)), so slices (0, 1) and (2, 3) simply concatenate
 #pragma unroll
-                for (int sl = 0; sl < 4; sl += 2)
-                    d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pair128(aop[s][sl], aop[s][sl + 1]), pair128(bop[sl], bop[sl + 1]), d, 0, 0, 0);
+            for (int sl = 0; sl < 4; sl += 2)
+#pragma unroll
+                for (int rr = 0; rr < 2; rr++)
+                    d[rr] = __builtin_amdgcn_mfma_i32_16x16x64_i8(pair128(aop[s][sl], aop[s][sl + 1]), pair128(bop[rr][sl], bop[rr][sl + 1]), d[rr], 0, 0, 0);
+#pragma unroll
+            for (int rr = 0; rr < 2; rr++) {
+                const int R = 2 * wave + rr;
                 // lane group lg = lane / 16 holds rows 4 lg .. 4 lg + 3 = the three digits of head 4 s + lg for token
                 // lane % 16: one score per lane.  Row of 16 tokens per (round, head); the head rows of a round rotate
                 // with the round number so that the softmax reads (one head, all rounds) spread over the banks.
                 const int lg = lane >> 4;
-                const int lo = (d[1] << 7) + d[2];
+                int lo = (d[rr][1] << 7) + d[rr][2];
+                asm volatile("" : "+v"(lo));         // two shift-adds; the compiler makes two shifts and a three-operand add of them
                 uint32_t *o = reinterpret_cast<uint32_t *>(kt + R * kRoundBytes + 256 * s + 64 * ((lg + R) & 3)) + (lane & 15);
                 if constexpr (SCORE_INT)
-                    *o = (uint32_t)((d[0] << 14) + lo);
+                    *o = (uint32_t)((d[rr][0] << 14) + lo);
                 else
-                    *o = __float_as_uint(fmaf((float)d[0], 16384.f, (float)lo));
+                    *o = __float_as_uint(fmaf((float)d[rr][0], 16384.f, (float)lo));
             }
         }
     };
@@ -795,7 +825,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         __builtin_amdgcn_s_setprio(Prio::K);
         if (!(PKV_ATTN_PROBE & 2)) k_stage(kcur, kt);
         __builtin_amdgcn_s_setprio(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile t1 has landed
+        if (!(PKV_ATTN_PROBE & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's part of tile t1 has landed
         if (take && wave == 0 && lane == 0) tau_lds[slot] = (int)fetched;
         PKV_LDS_BARRIER();                                    // publishes the scores, tile t1 and the new batch
         int t4;
@@ -812,6 +842,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         __builtin_amdgcn_s_setprio(Prio::S);
         if (!(PKV_ATTN_PROBE & 16)) parse(IntC<slot ^ 1>{}, i1, knext, vnext); else { knext = kcur; vnext = vcur; }
         if (!(PKV_ATTN_PROBE & 4)) softmax_stage(slot_c, kt);
+        // the pack words of tile t1 are put together here, not wherever the compiler finds room before their first
+        // use: it kept the three raw dwords of every word alive through the V stage (24 registers instead of 16)
+        if constexpr (!KWIDE) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) asm volatile("" : "+v"(knext.word[i]));
+        }
+        if constexpr (!VWIDE) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) asm volatile("" : "+v"(vnext.word[i]));
+        }
         __builtin_amdgcn_s_setprio(0);
         PKV_LDS_BARRIER();                                    // publishes the weights; slot s is free, tile t1 is parsed
         __builtin_amdgcn_s_setprio(Prio::D);
@@ -819,7 +859,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         if (take) request(batch_of(cur_base));                // collected at the wait above, a step or more from now
         __builtin_amdgcn_s_setprio(Prio::V);
         if (!(PKV_ATTN_PROBE & 8)) v_stage(slot_c, vcur);
+#ifdef PKV_PRIO_TOP
+        __builtin_amdgcn_s_setprio(PKV_PRIO_TOP);
+#else
         __builtin_amdgcn_s_setprio(0);
+#endif
         t_cur = t1; t1 = t2; t2 = t3; t3 = t4;
         i1 = i2; i2 = pack_info(i3);
         s++;
