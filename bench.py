@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the decode kernel on the default workload, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 208383 and WRITE_SIZE 2176 per dispatch), each scaled by what the same counter read
+# (FETCH_SIZE 208311 and WRITE_SIZE 3141 KiB per dispatch), each scaled by what the same counter read
 # for a plain 256 MiB device copy in the same run (131088 -> factor 1.99976; 262144 -> factor 1.0);
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
@@ -53,6 +53,8 @@ def parse():
     ap.add_argument("--no-sanity", action="store_true",
                     help="do not stop when the kernel disagrees with the plain kernel (development builds that switch "
                          "parts of the kernel off, -DPKV_ATTN_PROBE: their results are wrong by design)")
+    ap.add_argument("--no-config-legs", action="store_true",
+                    help="skip the configs[4] loop and the configs[3] decoder legs of the default run")
     ap.add_argument("--layers", type=int, default=0,
                     help="instead of the single-layer step: a decode loop over this many layers through the growing "
                          "compressed cache (configs[4] is --layers 32 --batch 4 --ctx 131072); prints its own JSON line")
@@ -202,7 +204,7 @@ def decode_loop(torch, args, dev):
         "peak_device_bytes": torch.cuda.max_memory_allocated(),
         "cpu_baseline": None,
     }
-    print(json.dumps(result))
+    return result
 
 
 def e2e_decode(torch, args, dev):
@@ -260,7 +262,7 @@ def e2e_decode(torch, args, dev):
         "peak_device_bytes": torch.cuda.max_memory_allocated(),
         "roofline": None, "cpu_baseline": None,
     }
-    print(json.dumps(result))
+    return result
 
 
 SWEEP_RELS = (0.5, 0.2, 0.1, 0.05, 0.025, 0.0125, 0.00625)      # code widths 2, 3, 4, 5, 6, 7, 8 bits
@@ -377,10 +379,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.layers > 0:
-        decode_loop(torch, args, dev)
+        print(json.dumps(decode_loop(torch, args, dev)))
         return
     if args.e2e:
-        e2e_decode(torch, args, dev)
+        print(json.dumps(e2e_decode(torch, args, dev)))
         return
     if args.sweep:
         print(json.dumps(pack_sweep(torch, args.hkv, args.ctx, dev)))
@@ -596,6 +598,40 @@ def main():
         result["cpu_encode"] = cpu_encoder(torch, args, k1[:1])
     else:
         result["cpu_baseline"] = None
+
+    if not args.no_extras and not args.no_config_legs and default_workload:
+        # the two configurations that run more than one layer, at their own sizes and in this same run: configs[4]'s
+        # loop over 32 layers of the growing cache and configs[3]'s greedy decode through the decoder (both have flags
+        # of their own for longer runs: --layers / --e2e).  A leg that fails reports its error instead of a figure.
+        del k, v, kc, vc, ke, ve, q, out
+        import copy
+        import gc
+        for name, fn, over in (
+                ("configs4_loop", decode_loop, dict(layers=32, batch=4, ctx=131072, steps=70, warmup=5)),
+                ("configs3_e2e", e2e_decode, dict(batch=32, ctx=8192, steps=64, warmup=4, e2e_dense_steps=2))):
+            a2 = copy.copy(args)
+            for key, val in over.items():
+                setattr(a2, key, val)
+            gc.collect()
+            torch.cuda.empty_cache()
+            t0 = time.perf_counter()
+            try:
+                r = fn(torch, a2, dev)
+            except Exception as e:      # noqa: BLE001 -- the headline line must still be printed
+                result[name] = {"error": "%s: %s" % (type(e).__name__, e)}
+                continue
+            if name == "configs4_loop":
+                result[name] = {"us_per_token": r["value"], "us_per_layer": r["value"] / a2.layers,
+                                "roofline_frac": r["roofline"]["frac"], "algorithmic_bytes": r["roofline"]["algorithmic_bytes"],
+                                "tokens_per_s": r["tokens_per_s"], "kv_bytes": r["kv_bytes"], "fp16_kv_bytes": r["fp16_kv_bytes"],
+                                "peak_device_bytes": r["peak_device_bytes"], "steps": r["steps"], "workload": r["config"]["workload"]}
+            else:
+                result[name] = {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "kv_bytes": r["kv_bytes"],
+                                "fp16_kv_bytes": r["fp16_kv_bytes"], "prefill_tokens_per_s": r["prefill_tokens_per_s"],
+                                "decompress_then_attend_ms_per_step": r["decompress_then_attend_ms_per_step"],
+                                "peak_device_bytes": r["peak_device_bytes"], "steps": r["steps"], "dtype": r["dtype"],
+                                "workload": r["config"]["workload"]}
+            result[name]["leg_seconds"] = time.perf_counter() - t0
     print(json.dumps(result))
 
 

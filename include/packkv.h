@@ -312,6 +312,16 @@ int pkv_attn_decode(const pkv_attn_args *args, float *ms_out, pkv_stream_t s);
  * pkv_attn_decode itself uses the same array when its stream is capturing a graph and has no scratch of its own. */
 int pkv_attn_decode_noalloc(const pkv_attn_args *args, pkv_stream_t s);
 
+/* pkv_stream_release: gives back the device memory the library keeps for stream `s` of the current device -- its
+ * scratch buffers (attention partials, the encoders' look-back state), its tile counters and every buffer it has
+ * outgrown (kept until now because a captured HIP graph might still hold its address).  It has no counterpart in the
+ * reference (whose extension allocates per call through torch).  Call it before destroying a stream the library has
+ * been used on -- a server that creates and destroys streams would otherwise accumulate one workspace per stream
+ * handle -- and only when no graph captured on `s` will be replayed again.  Waits for the stream's work; a stream the
+ * library has never seen is not an error.  The stream can be used with the library again afterwards (its scratch is
+ * allocated afresh). */
+int pkv_stream_release(pkv_stream_t s);
+
 #ifdef __cplusplus
 }
 #endif

@@ -71,6 +71,7 @@ SIGNATURES = {
     "pkv_fused_wv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _fp, _vp]),
     "pkv_attn_decode": (_i, [ctypes.POINTER(AttnArgs), _fp, _vp]),
     "pkv_attn_decode_noalloc": (_i, [ctypes.POINTER(AttnArgs), _vp]),
+    "pkv_stream_release": (_i, [_vp]),
 }
 
 _lib = None

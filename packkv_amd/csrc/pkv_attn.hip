@@ -52,6 +52,7 @@ struct AttnParams {
     float *part;          // [B, Hq, nparts, kPartStride]
     uint16_t *out;        // [B, Hq, 128]: written directly by the attention kernel when there is a single partial
     int B, Hq, Hkv, T_c, T_w;
+    int Gq;               // query heads per KV head; the kernels are built for the next of 1, 2, 4, 8 and leave the rest idle
     int par_stride;       // tokens per sequence row of the scale / zero arrays (>= T_c)
     int win_stride;       // tokens per (sequence, KV head) row of k_win / v_win (>= T_w)
     int k_bits, v_bits, dtype;
@@ -102,7 +103,7 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
     const UnitGeom gk = unit_geom(p.k_bits), gv = unit_geom(p.v_bits);
 
     for (int i = tid; i < G * kHeadDim; i += 256)
-        qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
+        qf[i] = i < p.Gq * kHeadDim ? a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * p.Gq) * kHeadDim + i, p.dtype) : 0.f;
     if (tid < G) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; }
     __syncthreads();
     if (tid < G) {
@@ -241,8 +242,8 @@ __global__ void __launch_bounds__(256) attn_tiles_kernel(const AttnParams p) {
             for (int g = 0; g < G; g++) red[g * kTile + ch] = acc[g];
         __syncthreads();
         if (half == 0) {
-            for (int g = 0; g < G; g++) {
-                const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            for (int g = 0; g < p.Gq; g++) {
+                const size_t hq = (size_t)b * p.Hq + (size_t)h * p.Gq + g;
                 float *dst = p.part + (hq * p.nparts + split) * kPartStride;
                 dst[2 + ch] = acc[g] + red[g * kTile + ch] + st_z[g];
                 if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
@@ -327,7 +328,7 @@ __device__ __forceinline__ void window_body(const AttnParams &p, uint8_t *lds, i
     const int tid = threadIdx.x;
     const int Tw = t1 > t0 ? t1 - t0 : 0;
     for (int i = tid; i < G * kHeadDim; i += 256)
-        qf[i] = a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * G) * kHeadDim + i, p.dtype);
+        qf[i] = i < p.Gq * kHeadDim ? a_ld16(p.q, ((size_t)b * p.Hq + (size_t)h * p.Gq) * kHeadDim + i, p.dtype) : 0.f;
     __syncthreads();
     const uint16_t *kbase = p.k_win + (((size_t)b * p.Hkv + h) * p.win_stride + t0) * kHeadDim;
     const uint16_t *vbase = p.v_win + (((size_t)b * p.Hkv + h) * p.win_stride + t0) * kHeadDim;
@@ -409,7 +410,8 @@ __device__ __forceinline__ void window_body(const AttnParams &p, uint8_t *lds, i
         if (!half) {
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+                if (g >= p.Gq) break;
+                const size_t hq = (size_t)b * p.Hq + (size_t)h * p.Gq + g;
                 float *dst = p.part + (hq * p.nparts + part_idx) * kPartStride;
                 dst[2 + ch] = acc[g] + qf[g * kHeadDim + ch];
                 if (ch == 0) { dst[0] = st_m[g]; dst[1] = st_l[g]; }
@@ -691,9 +693,9 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
         PKV_REQUIRE((reinterpret_cast<uintptr_t>(a->k_win) & 15u) == 0, PKV_ERR_INVALID,
                     "k_win must be 16-byte aligned");
     }
-    const int G = a->Hq / a->Hkv;
-    PKV_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, PKV_ERR_UNSUPPORTED,
-                "not supported: query heads per KV head must be 1, 2, 4 or 8");
+    const int Gq = a->Hq / a->Hkv;
+    PKV_REQUIRE(Gq <= 8, PKV_ERR_UNSUPPORTED, "not supported: more than 8 query heads per KV head");
+    const int G = Gq <= 2 ? Gq : Gq <= 4 ? 4 : 8;      // groups of 3 and of 5..7 run the kernels of 4 and 8 with idle head slots
 
     AttnParams p;
     p.k_stream = a->k_stream; p.k_info = a->k_info; p.v_stream = a->v_stream; p.v_info = a->v_info;
@@ -702,6 +704,7 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     p.q = (const uint16_t *)a->q;
     p.k_win = (const uint16_t *)a->k_win; p.v_win = (const uint16_t *)a->v_win;
     p.B = a->B; p.Hq = a->Hq; p.Hkv = a->Hkv; p.T_c = a->T_c; p.T_w = a->T_w;
+    p.Gq = Gq;
     p.par_stride = par_stride; p.win_stride = win_stride;
     p.k_bits = a->k_bits; p.v_bits = a->v_bits; p.dtype = a->dtype; p.sm_scale = a->sm_scale;
     const int n_tiles = a->T_c / kTile;

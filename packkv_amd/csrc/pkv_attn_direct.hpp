@@ -152,7 +152,11 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
     if (tid < 8) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_z[tid] = 0.f; st_a[tid] = 0.f; }
     __syncthreads();
     for (int g = wave; g < G; g += 4) {
-        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
+        if (g >= p.Gq) {                       // an idle head slot: a query of zeros
+            if (lane == 0) { qsum[g] = 0.f; qs[g] = 0.f; }
+            continue;
+        }
+        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * p.Gq + g) * kHeadDim;
         const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
         const float mx = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
         const float sm = wave_sum(q0 + q1);
@@ -509,7 +513,8 @@ __global__ void __launch_bounds__(256) attn_direct_kernel(const AttnParams p) {
         const int ch = 64 * j + 32 * w + t;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            if (g >= p.Gq) break;
+            const size_t hq = (size_t)b * p.Hq + (size_t)h * p.Gq + g;
             float *dst = p.part + (hq * p.nparts + split) * kPartStride;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
             dst[2 + ch] = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * wscale_inv;

@@ -71,9 +71,14 @@ __device__ __forceinline__ u32x4 dma_rsrc(const void *base, uint32_t bytes) {
 // The compiler does not see inside the statement, so it pads no hazards for it: the s_mov and the s_nop 3 are the
 // five wait states a memory instruction needs after a VALU instruction wrote one of its scalar operands (which is
 // what the compiler's restore of a spilled scalar register is).
+// M0 is on the clobber list: the compiler reserves the register for its own short-lived uses (lane-indexed writes, LDS
+// parameters) and may merge or hoist the initialisations it emits for them; told about the write, it keeps none of them
+// alive across these statements.  (It warns that a reserved register is named; that is the point.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma_b128(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
 }
 // The same with an immediate offset, which the hardware adds on both sides: to the buffer offset (and its range
 // check) and to the LDS address (measured: data of `offset:1024` lands 1 KiB behind M0's address).
@@ -81,12 +86,13 @@ template <int IMM>
 __device__ __forceinline__ void dma_b128_imm(u32x4 rsrc, uint32_t lds_addr, uint32_t voff) {
     static_assert(IMM >= 0 && IMM < 4096, "12-bit immediate");
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen offset:%3 lds"
-                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "n"(IMM) : "memory");
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "n"(IMM) : "memory", "m0");
 }
 __device__ __forceinline__ void dma_b32(u32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
-                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // The same descriptor moved `add` bytes forward and cut to `bytes`: scalar arithmetic only.  A copy whose lanes address
 // `16 lane` through such a descriptor needs no per-lane address arithmetic and no per-lane clamp: lanes past the end
@@ -426,7 +432,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     __builtin_amdgcn_s_waitcnt(0xC07F);       // lgkmcnt(0): the zeroes are written; the copy in flight is not waited for
     __builtin_amdgcn_s_barrier();
     for (int g = wave; g < G; g += 4) {
-        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * G + g) * kHeadDim;
+        if (g >= p.Gq) {                       // an idle head slot (group of 3 in the kernel of 4, ...): a query of zeros
+            if (lane == 0) { qsum[g] = 0.f; qs[g] = 0.f; }
+            continue;
+        }
+        const size_t qoff = ((size_t)b * p.Hq + (size_t)h * p.Gq + g) * kHeadDim;
         const float q0 = a_ld16(p.q, qoff + lane, p.dtype), q1 = a_ld16(p.q, qoff + 64 + lane, p.dtype);
         const float mx = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
         const float sm = wave_sum(q0 + q1);
@@ -880,8 +890,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     if (p.dynamic && tid == 0) {
         uint32_t *done = p.counters + n_heads + bh;
         if (atomicAdd(done, 1u) + 1u == (uint32_t)p.nsplit) {
-            p.counters[bh] = 0u;
-            *done = 0u;
+            atomicExch(p.counters + bh, 0u);
+            atomicExch(done, 0u);
         }
     }
 
@@ -904,7 +914,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         const int ch = 64 * j + 32 * w + t;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const size_t hq = (size_t)b * p.Hq + (size_t)h * G + g;
+            if (g >= p.Gq) break;
+            const size_t hq = (size_t)b * p.Hq + (size_t)h * p.Gq + g;
             // fields were consumed as fp16 subnormals (delta * 2^-24)
             const float val = (acc[g >> 2][g & 3] * 16777216.f + st_z[g]) * wscale_inv;
             if (p.direct_out) {                // one split and no window: this is the result, no merge launch follows

@@ -35,7 +35,8 @@ struct Workspace {
     bool encoded;           // an encoder has run on this stream: ptr[kScratchEncoder] starts with its ScanState
 };
 std::vector<Workspace> g_ws;
-std::vector<void *> g_retired;      // superseded buffers, kept until the process ends
+struct Retired { int dev; hipStream_t stream; void *ptr; };
+std::vector<Retired> g_retired;     // superseded buffers, kept until their stream is released (a captured graph may hold them)
 std::mutex g_ws_mu;
 
 int workspace_for(hipStream_t s, Workspace **out) {     // caller holds g_ws_mu
@@ -77,7 +78,7 @@ int scratch_get(size_t bytes, hipStream_t s, void **out, int kind) {
         const size_t want = scratch_grown_size(w->bytes[kind], bytes);
         void *fresh = nullptr;
         PKV_HIP_CHECK(hipMalloc(&fresh, want));
-        if (w->ptr[kind]) g_retired.push_back(w->ptr[kind]);
+        if (w->ptr[kind]) g_retired.push_back(Retired{w->dev, s, w->ptr[kind]});
         w->ptr[kind] = fresh;
         w->bytes[kind] = want;
     }
@@ -112,6 +113,38 @@ int attn_counters_get(hipStream_t s, uint32_t **out) {
         w->counters = (uint32_t *)c;
     }
     *out = w->counters;
+    return PKV_OK;
+}
+
+// Gives back everything the library holds for (current device, stream `s`): waits for the stream, frees its scratch
+// buffers, its tile counters and the buffers it has outgrown, and forgets the stream.
+int stream_release(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    int dev = 0;
+    PKV_HIP_CHECK(hipGetDevice(&dev));
+    PKV_REQUIRE(!capturing(s), PKV_ERR_INVALID, "the stream is capturing a graph");
+    size_t at = g_ws.size();
+    for (size_t i = 0; i < g_ws.size(); i++)
+        if (g_ws[i].dev == dev && g_ws[i].stream == s) at = i;
+    bool any = at < g_ws.size();
+    for (const Retired &r : g_retired) any = any || (r.dev == dev && r.stream == s);
+    if (!any) return PKV_OK;
+    PKV_HIP_CHECK(hipStreamSynchronize(s));
+    if (at < g_ws.size()) {
+        Workspace &w = g_ws[at];
+        for (int k = 0; k < 2; k++)
+            if (w.ptr[k]) PKV_HIP_CHECK(hipFree(w.ptr[k]));
+        if (w.counters) PKV_HIP_CHECK(hipFree(w.counters));
+        g_ws.erase(g_ws.begin() + (long)at);
+    }
+    for (size_t i = 0; i < g_retired.size();) {
+        if (g_retired[i].dev == dev && g_retired[i].stream == s) {
+            PKV_HIP_CHECK(hipFree(g_retired[i].ptr));
+            g_retired.erase(g_retired.begin() + (long)i);
+        } else {
+            i++;
+        }
+    }
     return PKV_OK;
 }
 
@@ -173,3 +206,5 @@ int pkv_abi_version(void) { return PKV_ABI_VERSION; }
 const char *pkv_last_error(void) { return pkv::g_error; }
 
 }  // extern "C"
+
+extern "C" int pkv_stream_release(pkv_stream_t s) { return pkv::stream_release((hipStream_t)s); }

@@ -25,6 +25,7 @@ size_t scratch_grown_size(size_t have, size_t want);
 // allocated on first use; the attention kernel leaves every counter it used at zero again.
 constexpr int kAttnCounters = 65536;
 int attn_counters_get(hipStream_t s, uint32_t **out);
+int stream_release(hipStream_t s);
 
 // Per-call timing: records start/stop events on `stream` around fn() and returns elapsed ms
 // after synchronising on the stop event (mirrors the reference launchers, which time every

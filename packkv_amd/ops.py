@@ -141,6 +141,16 @@ def _decode(is_k, stream, info, codes, ctx_len, hidden_dim, ctx_blk, hid_blk, bi
     return float(ms.value) if timed else None
 
 
+def stream_release(stream=None):
+    """Gives back the device memory the library keeps for `stream` (a torch.cuda.Stream; default: the current one) --
+    scratch buffers, tile counters and the buffers it has outgrown.  For callers that create and destroy streams:
+    call it before the stream goes away, and only when no HIP graph captured on it will be replayed again."""
+    st = torch.cuda.current_stream() if stream is None else stream
+    with torch.cuda.device(st.device):
+        rc = _lib.load().pkv_stream_release(ctypes.c_void_p(st.cuda_stream))
+    _lib.check(rc)
+
+
 def encode_status(device=None, bits=0):
     """Stream size of the last encode launched on the current stream of `device` with want_size=False; waits for the
     stream and raises what the encode would have raised (a stream that did not fit, a code wider than `bits`)."""

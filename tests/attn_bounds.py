@@ -10,13 +10,15 @@ Two kinds of kernel are held to it:
 * the checking mode of the plain kernel (variant 1 with ref_rounding, fp32 result): it forms the very elements the
   reference stores, so it must meet the contract as it stands, for fp16 and bf16 alike, on every case;
 * the fast kernels never form those 16-bit elements -- they fold scale and zero into the scores and weights and so
-  skip the reference's rounding of K-hat and V-hat.  They are held (i) to exact arithmetic: fp64 attention on the
+  skip the reference's rounding of K-hat and V-hat.  They are held to exact arithmetic: fp64 attention on the
   unrounded (code + zero) * scale, within the kernel's own rounding (weights handed to the matrix cores as fp16,
-  and the rounding of a 16-bit result); and (ii) to the reference path within a bound that the test computes from
-  the oracle for that very case: the distance between the reference path and exact arithmetic -- what the
-  reference's own rounding moved -- plus the same kernel allowance.  Nothing the kernel adds beyond the
-  reference's own rounding passes (ii).  Where the contract itself holds for a fast kernel (the benchmark
-  shapes in fp16) it is asserted directly as well.
+  and the rounding of a 16-bit result).  Their distance to the reference path is then at most that allowance plus
+  what the reference's own rounding moved (|ref - exact|, which the oracle gives for the very case) -- a consequence
+  of the first bound, not a second test, so it is printed, not asserted: every check prints "fast kernel vs
+  reference path: X, contract: Y" with X the measured distance and Y the largest value the contract allows.
+  Where the contract itself holds for a fast kernel -- the benchmark shapes in fp16 -- it is asserted directly
+  (contract_holds).  In bf16 the reference's own rounding of K-hat / V-hat alone is 4e-3 .. 3e-2, so the literal
+  contract is met by the checking mode, not by the fast kernels.
 """
 import numpy as np
 import torch
@@ -55,15 +57,17 @@ def check_reference_mode(got_f32, ref, label=""):
 
 
 def check_fast(got, ref, exact, dtype, variant=0, out_f32=False, label=""):
-    """A fast kernel against exact arithmetic and against the reference path (bound computed from the oracle)."""
+    """A fast kernel against exact arithmetic (asserted); its distance to the reference path beside what the contract
+    allows and what the reference's own rounding moved (printed and recorded)."""
     got, ref, exact = _np(got), _np(ref), _np(exact)
     allow = KERNEL_SLACK[variant] + (0.0 if out_f32 else 1.05 * HALF_ULP[dtype] * np.abs(exact))
     e_exact = np.abs(got - exact)
     own = np.abs(ref - exact)                      # what the reference's rounding of K-hat / V-hat moved
     e_ref = np.abs(got - ref)
-    say("   %s vs exact arithmetic: max|err| = %.3e;  vs reference path: max|err| = %.3e "
-        "(the reference's own rounding: %.3e)" % (label, e_exact.max(), e_ref.max(), own.max()))
+    contract = ABS_TOL + REL_TOL * np.abs(ref)
+    say("   %s vs exact arithmetic: max|err| = %.3e;  fast kernel vs reference path: %.3e, contract: %.3e (%s; the "
+        "reference's own rounding: %.3e)" % (label, e_exact.max(), e_ref.max(), contract.max(),
+                                              "met" if (e_ref <= contract).all() else "not met", own.max()))
     ROWS.append((label, "fast vs exact", float(e_exact.max()), float(allow.max() if np.ndim(allow) else allow)))
     ROWS.append((label, "fast vs reference", float(e_ref.max()), float(own.max())))
     assert (e_exact <= allow).all()
-    assert (e_ref <= own + allow).all()

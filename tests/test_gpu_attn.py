@@ -16,8 +16,8 @@ pytestmark = pytest.mark.gpu
 
 
 def _parity(cuda, q, ke, ve, ref, exact, dtype, variants, k_win=None, v_win=None, label="", contract_too=False):
-    """The checking mode against the reference path at the contract; every fast variant against exact arithmetic
-    and against the reference path within the bound computed from (ref, exact)."""
+    """The checking mode against the reference path at the contract; every fast variant against exact arithmetic,
+    its distance to the reference path printed beside the contract (asserted where `contract_too` says it holds)."""
     qd = q.to(cuda)
     chk = ops.attn_decode(qd, ke, ve, k_win, v_win, variant=1, ref_rounding=True, out_f32=True)
     check_reference_mode(chk, ref, label)
@@ -122,6 +122,24 @@ def test_attn_decode_with_tail_window(cuda, variant):
             exact = oq.attention_f64_np(q.unsqueeze(2), kw, vw).squeeze(2)
             ke = ve = None
         _parity(cuda, q, ke, ve, want, exact, dtype, [variant], kw.to(cuda), vw.to(cuda), label="T=%d+%d" % (T, Tw))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_attn_decode_group_sizes_that_are_no_power_of_two(cuda, dtype, variant):
+    """3, 5, 6 and 7 query heads per KV head (24 q / 8 KV, 28 q / 4 KV, ...): the kernels of 4 and 8 with idle head
+    slots.  Same bars as every other case, with and without a tail window."""
+    for (B, Hq, Hkv, T, Tw) in ((2, 24, 8, 512, 0), (1, 28, 4, 1024, 37), (2, 10, 2, 384, 0), (1, 12, 2, 640, 130), (1, 3, 1, 256, 0)):
+        _say("odd group case", dtype, "variant", variant, B, Hq, Hkv, T, Tw)
+        k, v = synth.make_kv(B, Hkv, T + Tw, seed=520 + Hq, dtype=dtype)
+        q = synth.make_q(B, Hq, seed=521, dtype=dtype)
+        kc, vc = k[:, :, :T].contiguous(), v[:, :, :T].contiguous()
+        kw, vw = (k[:, :, T:].contiguous(), v[:, :, T:].contiguous()) if Tw else (None, None)
+        want = _reference(q, kc, vc, 0.1, 0.1, kw, vw)
+        exact = _exact(q, kc, vc, 0.1, 0.1, kw, vw)
+        ke, ve = ops.k_quant_encode(kc.to(cuda), 0.1), ops.v_quant_encode(vc.to(cuda), 0.1)
+        _parity(cuda, q, ke, ve, want, exact, dtype, [variant], kw.to(cuda) if Tw else None, vw.to(cuda) if Tw else None,
+                label="group of %d" % (Hq // Hkv))
 
 
 def test_attn_decode_close_to_reference_fp16_eager(cuda):
@@ -308,6 +326,53 @@ def test_two_streams_do_not_share_scratch(cuda):
     for e in encs:
         assert torch.equal(e["stream"][:n], want_enc["stream"][:n])
         assert torch.equal(e["info"].view(torch.int32), want_enc["info"].view(torch.int32))
+
+
+def test_stream_release_gives_the_scratch_back(cuda):
+    """A stream's workspace (partials, tile counters, encoder state, outgrown buffers) is freed by
+    pkv_stream_release and allocated afresh on the next call; results do not change, and a hundred streams that
+    come and go leave no memory behind."""
+    B, Hq, Hkv, T = 4, 32, 8, 4096
+    k, v = synth.make_kv(B, Hkv, T, seed=310, device=cuda)
+    q = synth.make_q(B, Hq, seed=311, device=cuda)
+    ke, ve = ops.k_quant_encode(k, 0.1), ops.v_quant_encode(v, 0.1)
+    want = ops.attn_decode(q, ke, ve)
+    torch.cuda.synchronize()
+    ops.stream_release(torch.cuda.Stream())                 # a stream the library has never seen: not an error
+
+    def one_stream():
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            got = ops.attn_decode(q, ke, ve)
+            enc = ops.k_quant_encode(k, 0.1)
+        st.synchronize()
+        ops.stream_release(st)
+        return got, enc
+
+    got, enc = one_stream()
+    assert torch.equal(got, want) and enc["size"] == ke["size"]
+    del got, enc
+    for _ in range(40):                                      # torch hands out streams from a pool of 32 that it creates
+        one_stream()                                         # lazily, and the runtime allocates for every new stream
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()           # torch caches freed blocks per stream: take them out of the picture
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(100):
+        got, enc = one_stream()
+        del got, enc
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    leaked = free0 - torch.cuda.mem_get_info()[0]
+    _say("   100 streams created, used and released: free memory moved by %d bytes" % leaked)
+    assert leaked < (8 << 20)                                # an unreleased workspace is > 1 MiB per stream
+    st = torch.cuda.Stream()                                 # released and used again
+    with torch.cuda.stream(st):
+        a = ops.attn_decode(q, ke, ve)
+        ops.stream_release(st)
+        b = ops.attn_decode(q, ke, ve)
+    st.synchronize()
+    assert torch.equal(a, want) and torch.equal(b, want)
+    ops.stream_release(st)
 
 
 @pytest.mark.parametrize("rel,bits", [(0.05, 5), (0.03, 6)])

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 def _attend_parity(cache, layer, q, wk, wv, ek, ev, dtype, cuda, label):
     """cache.attend in the checking mode against the reference path at the contract, and the fast decode step
-    against exact arithmetic / the reference path within the bound the oracle gives (tests/attn_bounds.py).
+    against exact arithmetic, its distance to the reference path printed beside the contract (tests/attn_bounds.py).
     wk, wv: what the reference's update returns; ek, ev: the same tokens before their rounding to 16 bits (fp64).
     Only the tokens already in the streams are attended unrounded: a pending 64-token cut sits in the 16-bit window
     in dequantised form, like the buffer."""

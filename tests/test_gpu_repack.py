@@ -265,7 +265,7 @@ def test_median_repack_inside_the_fused_encode_equals_the_code_matrix_path(cuda,
     the same permutation, streams, block_info and parameters.  The permutation is also checked against the NumPy
     restatement on the restated quantiser's codes."""
     cases = [(2, 4, 512, 0.1, 0.1, 64), (3, 8, 256, 0.2, 0.05, 64), (1, 2, 1024, 0.1, 0.2, 128), (2, 8, 512, 0.05, 0.1, 256),
-             (1, 1, 256, 0.5, 0.1, 64)]
+             (1, 1, 256, 0.5, 0.1, 64), (2, 8, 256, 0.03, 0.03, 64)]      # the last: 6-bit codes, the widest the fused path takes
     for n, (B, H, T, k_rel, v_rel, bs) in enumerate(cases):
         _say("fused median case", dtype, B, H, T, k_rel, v_rel, bs)
         k, v = synth.make_kv(B, H, T, seed=300 + n)

@@ -37,6 +37,29 @@ def test_noalloc_entry_point_matches_the_allocating_one(cuda):
                 assert torch.equal(got, w)
 
 
+def test_noalloc_entry_point_with_tiles_handed_out_by_counter(cuda):
+    """A step whose members take tiles from the heads' counters (8 members x 16 tiles) with the counters in the fixed
+    array, behind the partials: twice in a row, then a smaller step, then again -- every launch must leave the
+    counters at zero for the next.  Which member takes which tile depends on timing, and with it the running maxima
+    against which the softmax weights are rounded to fp16, so two runs of such a step differ by that rounding (a few
+    1e-5) and by a rounding of the 16-bit output; they are held to that, not to the bit (the small step has fixed
+    shares and is compared bit for bit)."""
+    big = _case(cuda, 16, 32, 8, 16384, 0, seed=730)
+    small = _case(cuda, 2, 16, 4, 1024, 0, seed=740)
+    want_big, want_small = ops.attn_decode(*big), ops.attn_decode(*small)
+    torch.cuda.synchronize()
+    for c, w in ((big, want_big), (big, want_big), (small, want_small), (big, want_big)):
+        print("no-alloc case with tile counters: batch", c[0].shape[0], "tokens", c[1]["scale"].shape[1], flush=True)
+        got = ops.attn_decode(*c, noalloc=True)
+        torch.cuda.synchronize()
+        if c is small:
+            assert torch.equal(got, w)
+        else:
+            err = (got.float() - w.float()).abs()
+            print("   largest difference between two runs of the step: %.3e" % err.max().item(), flush=True)
+            assert bool((err <= 2.0 ** -10 * w.float().abs() + 2e-4).all())     # a lost or repeated tile would move them by 1e-2
+
+
 def test_noalloc_entry_point_rejects_what_does_not_fit(cuda):
     """8 MiB hold B * Hq * partials * 520 bytes: batch 64 x 64 query heads with a window (2 x 2 partials... ) fits, a
     step with 64 sequences x 64 heads x 2 x 32 partials does not -- and says so instead of overrunning the array."""
