@@ -23,11 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the decode kernel on the default workload, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 208311 and WRITE_SIZE 3141 KiB per dispatch), each scaled by what the same counter read
-# for a plain 256 MiB device copy in the same run (131088 -> factor 1.99976; 262144 -> factor 1.0);
+# (FETCH_SIZE 208456 and WRITE_SIZE 2542 KiB per dispatch), each scaled by what the same counter read
+# for a plain 256 MiB device copy in the same run (131093 -> factor 1.99969; 262144 -> factor 1.0);
 # the summary with the commands is profiles/attn_dma_kernel_config1.md.  It is a recorded
 # measurement, not something this script can observe, so it is reported for that workload only.
-DEFAULT_TRAFFIC_BYTES = int((208311 * (262144 / 131088) + 3141 * 1.0) * 1024)
+DEFAULT_TRAFFIC_BYTES = int((208456 * (262144 / 131093) + 2542 * 1.0) * 1024)
 TRAFFIC_SOURCE = ("recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measurement of this workload "
                   "(profiles/attn_dma_kernel_config1.md), not observed by this run")
 
@@ -499,7 +499,32 @@ def main():
             "median_repack_ms": rp_ms, "median_repack_gbs": 5 * Tc * hidden / (rp_ms * 1e-3) / 1e9,   # V read twice, K once, both written
             "bit_pack_size_ms": bp_ms, "bit_pack_size_gbs": Tc * hidden / (bp_ms * 1e-3) / 1e9,
         }
-        del codes, codes_v
+        # packs longer than 16 tokens (this build's extension of the format) on the same 2 x 512 MiB of codes: the real
+        # codec at every pack length, beside the 16-token codec's figures above (K decode 1.0 = as fast as that one)
+        long_packs = {}
+        back = torch.empty_like(codes)
+        for pack in (32, 64, 128, 256):
+            row = {}
+            for name, is_k, mat, ref_enc, ref_dec in (("k", True, codes, ck_ms, uk_ms), ("v", False, codes_v, cv_ms, uv_ms)):
+                ctx_blk, hid_blk = ops.long_block_shape(is_k, pack)
+                if Tc % ctx_blk:
+                    continue
+                info_p = torch.empty((Tc // ctx_blk) * (hidden // hid_blk), 2, dtype=torch.uint32, device=dev)
+                stream_p = ke["stream"] if is_k else ve["stream"]
+                if stream_p.numel() < info_p.shape[0] * ops.block_bound_p(pack, bits):
+                    stream_p = torch.empty(info_p.shape[0] * ops.block_bound_p(pack, bits), dtype=torch.uint8, device=dev)
+                size_p = ops.encode_p(is_k, mat, stream_p, info_p, pack, bits)
+                e_ms = event_time_ms(torch, lambda: ops.encode_p(is_k, mat, stream_p, info_p, pack, bits, want_size=False), 3)
+                d_ms = event_time_ms(torch, lambda: ops.decode_p(is_k, stream_p, info_p, back, pack, bits), 3)
+                row.update({name + "_encode_ms": e_ms, name + "_decode_ms": d_ms, name + "_stream_bytes": size_p,
+                            name + "_encode_vs_16": ref_enc / e_ms, name + "_decode_vs_16": ref_dec / d_ms})
+                del info_p
+            long_packs["pack %d" % pack] = row
+        # (the long-pack encodes overwrote the streams: put the 16-token streams back for what follows)
+        ops.k_quant_encode(kc, args.rel, bits, ke["stream"], ke["info"], want_size=False)
+        ops.v_quant_encode(vc, args.rel, bits, ve["stream"], ve["info"], want_size=False)
+        result["long_packs"] = long_packs
+        del codes, codes_v, back
         # median repacking inside the encode: the order from V itself (V's parameters kept), then the fused encoders
         # on the permuted rows -- against the plain fused encode above, all on preallocated buffers
         if Hkv <= 8 and bits <= 6:

@@ -35,11 +35,7 @@ namespace pkv {
 // to fewer resident workgroups: with three (groups of 8) equal priorities are best (197 us against 218), with two
 // (widths 5 and 6) the K stage first (211 us against 218).
 template <int G, bool WIDE> struct StagePrio {                       // 4 workgroups per CU
-#ifdef PKV_PRIO_K
-    static constexpr int K = PKV_PRIO_K, S = PKV_PRIO_S, D = PKV_PRIO_D, V = PKV_PRIO_V;
-#else
     static constexpr int K = 1, S = 2, D = 0, V = 3;                 // K stage, parse + softmax, copy issue and waits, V stage
-#endif
 };
 template <int G> struct StagePrio<G, true> { static constexpr int K = 2, S = 1, D = 0, V = 0; };
 template <> struct StagePrio<8, false> { static constexpr int K = 0, S = 0, D = 0, V = 0; };
@@ -869,11 +865,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
         if (take) request(batch_of(cur_base));                // collected at the wait above, a step or more from now
         __builtin_amdgcn_s_setprio(Prio::V);
         if (!(PKV_ATTN_PROBE & 8)) v_stage(slot_c, vcur);
-#ifdef PKV_PRIO_TOP
-        __builtin_amdgcn_s_setprio(PKV_PRIO_TOP);
-#else
         __builtin_amdgcn_s_setprio(0);
-#endif
         t_cur = t1; t1 = t2; t2 = t3; t3 = t4;
         i1 = i2; i2 = pack_info(i3);
         s++;

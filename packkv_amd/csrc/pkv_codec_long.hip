@@ -317,6 +317,252 @@ __global__ void __launch_bounds__(1024) unpack_long_kernel(const uint8_t *__rest
     }
 }
 
+// ---- decoders that stage the stream through LDS ----------------------------------------------------------------
+// A pack of P tokens is P / 16 sub-words of the 16-token shape, so sub-word s of all packs of a unit is a 16-token
+// unit whose words sit at payload + off[i] * nsub + s * 2 len[i] instead of payload + off[i]: decoded with the
+// windows of the 16-token codec (sub_codes), 16 tokens x 4 slots per lane at a time.  What differs from the kernel
+// above is where the bytes come from and go to: the unit (K) or one slot of four units (V) is copied into LDS in
+// aligned 16-byte pieces first -- a lane's pack is a contiguous run of up to 256 bytes in the stream, so lanes that
+// fetch their own words touch a cache line each per load -- and V, whose units are 32 channels wide, goes through
+// an LDS tile of 128 channels (two adjacent blocks) so that whole 128-byte lines are written.
+
+// codes of sub-word `word_off` (LDS byte offsets, even) of the lane's four packs: c4[k] = the four slots' codes of
+// token k, one per byte.  W <= 4: words of at most 8 bytes, 16-bit windows of four tokens; else field by field.
+__device__ __forceinline__ void sub_codes(const uint8_t *lds, const uint32_t word_off[4], const uint32_t len[4], const uint32_t mn[4],
+                                          bool wide, uint32_t c4[16]) {
+    typedef unsigned short u16pair __attribute__((ext_vector_type(2)));
+    if (!wide) {
+        uint32_t hlf[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint64_t w = lds_load64(lds, word_off[i]);
+            hlf[i][0] = (uint32_t)(w >> (8u * len[i]));   // tokens 0..7
+            hlf[i][1] = (uint32_t)w;                      // tokens 8..15
+        }
+        const uint32_t len01 = len[0] | (len[1] << 16), len23 = len[2] | (len[3] << 16);
+        const uint32_t mq = ((1u << len[0]) - 1u) | (((1u << len[1]) - 1u) << 8) | (((1u << len[2]) - 1u) << 16) |
+                            (((1u << len[3]) - 1u) << 24);
+        const uint32_t minq = mn[0] | (mn[1] << 8) | (mn[2] << 16) | (mn[3] << 24);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            uint32_t qd[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t src = hlf[i][q >> 1];
+                qd[i] = (q & 1) ? src : (src >> (4u * len[i]));
+            }
+            const uint32_t w01 = __builtin_amdgcn_perm(qd[1], qd[0], 0x05040100u);   // tokens 4q..4q+3 of packs 0 | 1
+            const uint32_t w23 = __builtin_amdgcn_perm(qd[3], qd[2], 0x05040100u);
+#pragma unroll
+            for (int pp = 0; pp < 4; pp++) {
+                const u16pair s01 = __builtin_bit_cast(u16pair, len01 * (uint32_t)(3 - pp));
+                const u16pair s23 = __builtin_bit_cast(u16pair, len23 * (uint32_t)(3 - pp));
+                const uint32_t x01 = __builtin_bit_cast(uint32_t, (u16pair)(__builtin_bit_cast(u16pair, w01) >> s01));
+                const uint32_t x23 = __builtin_bit_cast(uint32_t, (u16pair)(__builtin_bit_cast(u16pair, w23) >> s23));
+                c4[4 * q + pp] = (__builtin_amdgcn_perm(x23, x01, 0x06040200u) & mq) + minq;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) c4[k] = 0u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint64_t lo = lds_load64(lds, word_off[i]), hi = lds_load64(lds, word_off[i] + 8u);
+            uint32_t d0 = (uint32_t)lo, d1 = (uint32_t)(lo >> 32), d2 = (uint32_t)hi, d3 = (uint32_t)(hi >> 32);
+            const uint32_t mask = (1u << len[i]) - 1u, sh = len[i];
+#pragma unroll
+            for (int k = 15; k >= 0; k--) {
+                c4[k] |= (((d0 & mask) + mn[i]) & 0xFFu) << (8 * i);
+                d0 = __builtin_amdgcn_alignbit(d1, d0, sh);
+                d1 = __builtin_amdgcn_alignbit(d2, d1, sh);
+                d2 = __builtin_amdgcn_alignbit(d3, d2, sh);
+                d3 >>= sh;
+            }
+        }
+    }
+}
+
+// codes of one 16-token sub-word of a single pack (V works slot by slot: a lane's four packs are four token groups)
+__device__ __forceinline__ void sub_codes1(const uint8_t *lds, uint32_t word_off, uint32_t len, uint32_t mn, bool wide, uint32_t c[16]) {
+    const uint32_t mask = (1u << len) - 1u;
+    if (!wide) {
+        const uint64_t w = lds_load64(lds, word_off);
+#pragma unroll
+        for (int k = 0; k < 16; k++) c[k] = ((uint32_t)(w >> ((15 - k) * len)) & mask) + mn;
+    } else {
+        const uint64_t lo = lds_load64(lds, word_off), hi = lds_load64(lds, word_off + 8u);
+        uint32_t d0 = (uint32_t)lo, d1 = (uint32_t)(lo >> 32), d2 = (uint32_t)hi, d3 = (uint32_t)(hi >> 32);
+#pragma unroll
+        for (int k = 15; k >= 0; k--) {
+            c[k] = (d0 & mask) + mn;
+            d0 = __builtin_amdgcn_alignbit(d1, d0, len);
+            d1 = __builtin_amdgcn_alignbit(d2, d1, len);
+            d2 = __builtin_amdgcn_alignbit(d3, d2, len);
+            d3 >>= len;
+        }
+    }
+}
+
+// Where unit u of block b lies in the stream, made safe: false when block_info or the header cannot be right
+// (the codes of the unit then stay as they are).  ustart / ubytes: offset inside the block and size of the unit.
+__device__ __forceinline__ bool long_unit_span(const uint8_t *stream, uint64_t stream_bytes, const uint32_t *info, uint32_t b, int u,
+                                               int P, uint32_t meta, uint64_t &boff, uint32_t &ustart, uint32_t &ubytes) {
+    boff = info[2 * (size_t)b];
+    const uint32_t bsize = info[2 * (size_t)b + 1];
+    if (boff + bsize > stream_bytes || bsize < 8u + 4u * meta) return false;
+    const uint16_t *hdr = reinterpret_cast<const uint16_t *>(stream + boff);
+    const uint32_t gran = P == 16 ? 1u : 4u;
+    ustart = 8u + (u ? (uint32_t)hdr[u - 1] * gran : 0u);
+    const uint32_t uend = 8u + (uint32_t)hdr[u] * gran;
+    if (!(ustart + meta <= uend && uend <= bsize)) return false;
+    ubytes = uend - ustart;
+    return true;
+}
+
+// K: one workgroup per unit (P tokens x 128 channels); half-wavefront h decodes sub-words h, h + nhw, ... and
+// writes their 16 rows of 128 bytes.  Dynamic LDS: the unit's bytes + 48.
+__global__ void __launch_bounds__(256) unpack_long_k_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+                                                           uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
+                                                           uint64_t stream_bytes, uint32_t unit_cap) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, hw = tid >> 5, nhw = (int)blockDim.x >> 5, t = tid & 31;
+    const uint32_t b = blockIdx.x >> 2;
+    const int u = (int)(blockIdx.x & 3u);
+    const int n_hid = hidden_dim / 128;
+    const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    uint64_t boff;
+    uint32_t ustart, ubytes;
+    if (!long_unit_span(stream, stream_bytes, info, b, u, P, meta, boff, ustart, ubytes)) return;      // uniform
+    ubytes = min(ubytes, unit_cap);
+    const uint32_t phase = stage_to_lds(stream + boff + ustart, ubytes, lds, tid, (int)blockDim.x);
+    __syncthreads();
+    const uint32_t minsw = lds_meta_word(lds + phase, t, W);
+    const uint32_t lensw = lds_meta_word(lds + phase + g.mins_bytes, t, g.LB);
+    uint32_t mn[4], len[4], off[4], payload;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        mn[i] = (minsw >> (i * W)) & ((1u << W) - 1u);
+        len[i] = min((lensw >> (i * g.LB)) & ((1u << g.LB) - 1u), (uint32_t)kMaxBits);
+    }
+    pack_offsets(len, off, payload);
+    const uint32_t nsub = (uint32_t)P / 16u;
+    if (meta + payload * nsub > ubytes) return;                    // (uniform) widths that overrun the unit
+    const uint32_t pay = phase + meta;
+    uint8_t *tile = codes + (size_t)cb * (4 * P) * hidden_dim + (size_t)hb * 128 + (size_t)(u * P) * hidden_dim + 4 * t;
+    for (uint32_t s = (uint32_t)hw; s < nsub; s += (uint32_t)nhw) {
+        uint32_t wo[4], c4[16];
+#pragma unroll
+        for (int i = 0; i < 4; i++) wo[i] = pay + off[i] * nsub + s * 2u * len[i];
+        sub_codes(lds, wo, len, mn, W > 4, c4);
+        uint8_t *row = tile + (size_t)(P - 16 * (int)(s + 1)) * hidden_dim;
+#pragma unroll
+        for (int k = 0; k < 16; k++) *reinterpret_cast<uint32_t *>(row + (size_t)k * hidden_dim) = c4[k];
+    }
+}
+
+// V: one workgroup of 256 threads per (pair of adjacent blocks, token half `seg`): half-wavefront h serves unit
+// q = h % 4 of the pair (block q / 2, channel half q % 2) and the sub-words of parity h / 4.  The bytes of `sps`
+// slots of the four units (all four when they fit the staging area, one at a time for the longest packs) go to LDS;
+// then, slot by slot, every half-wavefront decodes `R` sub-words per step into tiles of 16 tokens x 128 channels
+// (double-buffered) that are written out as whole lines.  Dynamic LDS: 4 staging regions, 2 x 2 R tiles, metadata.
+template <int R>
+__global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+                                                           uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
+                                                           uint64_t stream_bytes, uint32_t stage_cap, int sps) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, hw = tid >> 5, t = tid & 31;
+    const int q = hw & 3, sp = hw >> 2;                    // unit of the pair, parity of the sub-words
+    const int seg = (int)(blockIdx.x & 1u);
+    const uint32_t pair = blockIdx.x >> 1;
+    const int n_pair = hidden_dim / 128;
+    const uint32_t cb = pair / (uint32_t)n_pair, hp = pair % (uint32_t)n_pair;
+    const uint32_t b = cb * (uint32_t)(2 * n_pair) + 2u * hp + (uint32_t)(q >> 1);
+    const int u = 2 * (q & 1) + seg;                       // unit of block b: channel half q % 2, token half seg
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const uint32_t region = stage_cap + 48u;               // LDS bytes of one unit's staged slots
+    constexpr int kTileBytes = 16 * 128, kBuf = 2 * R * kTileBytes;
+    uint8_t *tiles = lds + 4 * region;                     // [2 buffers][2 parities][R][16 tokens][128 channels]
+    uint8_t *metas = tiles + 2 * kBuf;                     // [4 units][meta rounded up to 16 + 32]
+    const uint32_t meta_stride = ((meta + 15u) & ~15u) + 32u;
+    uint64_t boff = 0;
+    uint32_t ustart = 0, ubytes = 0;
+    bool ok = long_unit_span(stream, stream_bytes, info, b, u, P, meta, boff, ustart, ubytes);          // uniform per half-wavefront
+    // metadata of the four units -> LDS (the two half-wavefronts of a unit share the copy)
+    uint32_t mphase = 0;
+    if (ok) mphase = stage_to_lds(stream + boff + ustart, meta, metas + q * meta_stride, t + 32 * sp, 64);
+    __syncthreads();
+    uint32_t mn[4], len[4], off[4], payload = 0;
+    {
+        const uint8_t *m = metas + q * meta_stride + mphase;
+        const uint32_t minsw = ok ? lds_meta_word(m, t, W) : 0u;
+        const uint32_t lensw = ok ? lds_meta_word(m + g.mins_bytes, t, g.LB) : 0u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            mn[i] = (minsw >> (i * W)) & ((1u << W) - 1u);
+            len[i] = min((lensw >> (i * g.LB)) & ((1u << g.LB) - 1u), (uint32_t)kMaxBits);
+        }
+        pack_offsets(len, off, payload);                   // (whole wavefronts: every lane takes part)
+    }
+    const uint32_t nsub = (uint32_t)P / 16u;
+    ok = ok && meta + payload * nsub <= ubytes;            // widths that overrun the unit
+    // slot i of this unit: bytes [base[i], base[i + 1]) * nsub of the payload; the slot bases are the offsets of the
+    // half-wavefront's first lane (swizzle within 32 lanes: every lane reads lane 0 of its half)
+    uint32_t base[5];
+#pragma unroll
+    for (int i = 0; i < 4; i++) base[i] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[i], 0);
+    base[4] = payload;
+    uint8_t *out = codes + (size_t)cb * (8 * P) * hidden_dim + (size_t)hp * 128;
+    uint8_t *reg = lds + q * region;
+    int buf = 0;
+    uint32_t sphase = 0, b_stage = 0;                      // phase of the staged bytes, payload offset (/ nsub) they start at
+#pragma unroll 1
+    for (int i = 0; i < 4; i++) {
+        uint32_t len_i = len[0], mn_i = mn[0], off_i = off[0];                  // (selected, not indexed: the arrays stay in registers)
+        if (i == 1) { len_i = len[1]; mn_i = mn[1]; off_i = off[1]; }
+        if (i == 2) { len_i = len[2]; mn_i = mn[2]; off_i = off[2]; }
+        if (i == 3) { len_i = len[3]; mn_i = mn[3]; off_i = off[3]; }
+        if (i % sps == 0) {                                // (uniform) the next sps slots' bytes
+            const uint32_t b_lo = i == 0 ? base[0] : i == 1 ? base[1] : i == 2 ? base[2] : base[3];
+            const int ie = i + sps;
+            const uint32_t b_hi = ie == 1 ? base[1] : ie == 2 ? base[2] : ie == 3 ? base[3] : base[4];
+            const uint32_t sbytes = min((b_hi - b_lo) * nsub, stage_cap);
+            __syncthreads();                               // the bytes staged before are no longer read
+            if (ok) sphase = stage_to_lds(stream + boff + ustart + meta + b_lo * nsub, sbytes, reg, t + 32 * sp, 64);
+            b_stage = b_lo;
+            __syncthreads();
+        }
+        const size_t tok_slot = (size_t)(seg * 4 + i) * P;
+#pragma unroll 1
+        for (uint32_t s0 = 0; s0 < nsub; s0 += 2 * R) {    // sub-words s0 .. s0 + 2 R - 1: parity sp takes s0 + sp, s0 + sp + 2, ...
+            if (ok) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const uint32_t s = s0 + (uint32_t)sp + 2u * (uint32_t)r;
+                    uint8_t *tile = tiles + buf * kBuf + (sp * R + r) * kTileBytes;
+                    uint32_t c[16];
+                    sub_codes1(reg, sphase + (off_i - b_stage) * nsub + s * 2u * len_i, len_i, mn_i, W > 4, c);
+#pragma unroll
+                    for (int k = 0; k < 16; k++) tile[k * 128 + 32 * q + t] = (uint8_t)c[k];
+                }
+            }
+            __syncthreads();                               // the tiles of this buffer are complete
+            // 2 R tiles of 16 rows x 128 bytes = 256 R pieces of 16 bytes: R per thread
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int idx = tid + 256 * r;
+                const int tl = idx >> 7, row = (idx >> 3) & 15, c16 = idx & 7;      // tile (parity * R + r'), row, piece
+                const uint32_t sw = s0 + (uint32_t)(tl / R) + 2u * (uint32_t)(tl % R);
+                const uint4 v = *reinterpret_cast<const uint4 *>(tiles + buf * kBuf + tl * kTileBytes + row * 128 + 16 * c16);
+                *reinterpret_cast<uint4 *>(out + (tok_slot + (size_t)(P - 16 * (int)(sw + 1)) + row) * hidden_dim + 16 * c16) = v;
+            }
+            buf ^= 1;                                      // the next step writes the other buffer while this one is read
+        }
+    }
+}
+
 static int check_long(bool is_k, const void *codes, const void *stream, const void *info, int ctx_len, int hidden_dim,
                       int P, int bits) {
     PKV_REQUIRE(codes && stream && info, PKV_ERR_INVALID, "null pointer argument");
@@ -360,9 +606,29 @@ static int run_unpack_long(bool is_k, const uint8_t *stream, uint64_t stream_byt
     const uint32_t nblocks = (uint32_t)(ctx_len / ((is_k ? 4 : 8) * P)) * (uint32_t)(hidden_dim / (is_k ? 128 : 64));
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    const int threads = 128 * long_chunks(P);
-    if (is_k) unpack_long_kernel<true><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
-    else unpack_long_kernel<false><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    const uint32_t meta = 16u * (uint32_t)(bits + len_field_bits(bits));
+    const uint32_t slot_cap = 4u * (uint32_t)P * (uint32_t)bits;              // 32 packs of P tokens at full width
+    if (is_k) {
+        // a workgroup per unit, staged through LDS; a half-wavefront per sub-word, at most eight
+        const uint32_t unit_cap = meta + 4u * slot_cap;
+        const int threads = 32 * (P / 16 < 8 ? P / 16 : 8);
+        unpack_long_k_kernel<<<4 * nblocks, threads < 64 ? 64 : threads, unit_cap + 48u, s>>>(stream, info, codes, hidden_dim, P, bits,
+                                                                                          stream_bytes, unit_cap);
+    } else if (hidden_dim % 128 == 0) {
+        // pairs of adjacent blocks (whole 128-byte lines), a workgroup per token half; all four slots of a unit are
+        // staged at once while they fit 8 KiB per unit, else one slot at a time
+        const int sps = 4u * slot_cap <= 8192u ? 4 : 2u * slot_cap <= 8192u ? 2 : 1;
+        const uint32_t stage_cap = (uint32_t)sps * slot_cap;
+        const int R = P >= 64 ? 2 : 1;                               // sub-words per half-wavefront and step
+        const uint32_t lds_bytes = 4u * (stage_cap + 48u) + 2u * 2u * (uint32_t)R * 2048u + 4u * (((meta + 15u) & ~15u) + 32u);
+        const void *fn = R == 2 ? reinterpret_cast<const void *>(unpack_long_v_kernel<2>) : reinterpret_cast<const void *>(unpack_long_v_kernel<1>);
+        PKV_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        if (R == 2) unpack_long_v_kernel<2><<<nblocks, 256, lds_bytes, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes, stage_cap, sps);
+        else unpack_long_v_kernel<1><<<nblocks, 256, lds_bytes, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes, stage_cap, sps);
+    } else {
+        const int threads = 128 * long_chunks(P);
+        unpack_long_kernel<false><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+    }
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }
