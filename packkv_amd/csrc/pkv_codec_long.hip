@@ -12,12 +12,14 @@
 //            metadata bit arrays and the slot-major, lane-minor payload order of the reference's format;
 //   header   four u16 cumulative unit sizes, counted in 4-byte words for P >= 32 (every unit size is then a
 //            multiple of 4; in bytes a unit of 256-token packs would not fit 16 bits).
-// One workgroup per block: 128 threads -- one 32-lane half-wavefront per unit, lane t <-> 4 packs -- times the number
-// of CHUNKS a pack is cut into (P / 16 of them, at most 8: 256 .. 1024 threads), since a long pack is a row of
-// independent 16-token sub-words and blocks of long packs are few.  A thread handles its chunk's sub-words of its
-// four packs; minima and widths are combined over the chunks through LDS.  The encoder reads the block's codes twice
-// (minima / widths, then the words; the second time from L2), obtains the block's offset by the same ticket +
-// look-back as the 16-token codec and writes the words straight into the stream.
+// Encoders: K keeps the thread layout of the 16-token codec (half-wavefront per unit, lane <-> 4 channels) times the
+// CHUNKS a pack is cut into (P / 16 of them, at most 8: a long pack is a row of independent 16-token sub-words), V
+// gives a wavefront to each of a block's eight (segment, slot) token ranges; both read the codes once, keep them in
+// registers, build the block in LDS as it will lie in the stream, take its offset from the same ticket + look-back
+// as the 16-token codec and copy it out in aligned 16-byte stores.  Decoders stage the stream through LDS and write
+// whole 128-byte rows (V: two adjacent blocks per workgroup).  The two *_plain kernels serve V code matrices whose
+// rows are no multiple of 128 channels or that do not start at a 16-byte boundary: a workgroup per block, the lane
+// layout of the format itself, byte loads and 2-byte stores.
 #include "pkv_block.hpp"
 #include "pkv_runtime.hpp"
 
@@ -71,8 +73,7 @@ constexpr int kLongMetaWords = 52;      // 16 * (8 + 4) bytes of metadata at mos
 constexpr int kLongMaxChunks = 8;
 __host__ __device__ inline int long_chunks(int P) { return P / 16 < kLongMaxChunks ? P / 16 : kLongMaxChunks; }
 
-template <bool IS_K>
-__global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+__global__ void __launch_bounds__(1024) pack_long_v_plain_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                         uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
                                                         int hidden_dim, int P, int W, uint32_t nblocks) {
     __shared__ uint32_t s_idx;
@@ -89,7 +90,7 @@ __global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restri
     __syncthreads();
     const uint32_t b = s_idx;
     if (b >= nblocks) return;
-    const int hid_blk = IS_K ? 128 : 64, ctx_blk = (IS_K ? 4 : 8) * P;
+    const int hid_blk = 64, ctx_blk = 8 * P;
     const int n_hid = hidden_dim / hid_blk;
     const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
     const uint8_t *tile = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
@@ -98,41 +99,7 @@ __global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restri
 
     // ---- minima and widths of the lane's four packs ----
     uint32_t mn[4], len[4];
-    if (IS_K) {     // one dword per token row holds the four channels
-        const uint8_t *col = tile + (size_t)(u * P) * hidden_dim + 4 * t;
-        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-        u16x2 amn2 = {255, 255}, amx2 = {0, 0}, bmn2 = {255, 255}, bmx2 = {0, 0};   // channels (0, 2) and (1, 3) as 16-bit pairs
-        for (int k = k0; k < k1; k += 8) {
-            uint32_t d[8];
-#pragma unroll
-            for (int q = 0; q < 8; q++) d[q] = *reinterpret_cast<const uint32_t *>(col + (size_t)(k + q) * hidden_dim);
-#pragma unroll
-            for (int q = 0; q < 8; q++) {
-                const u16x2 a = __builtin_bit_cast(u16x2, d[q] & 0x00FF00FFu), c = __builtin_bit_cast(u16x2, (d[q] >> 8) & 0x00FF00FFu);
-                amn2 = __builtin_elementwise_min(amn2, a);
-                amx2 = __builtin_elementwise_max(amx2, a);
-                bmn2 = __builtin_elementwise_min(bmn2, c);
-                bmx2 = __builtin_elementwise_max(bmx2, c);
-            }
-        }
-        s_mm[chunk][tid & 127] = make_uint4(__builtin_bit_cast(uint32_t, amn2), __builtin_bit_cast(uint32_t, amx2),
-                                            __builtin_bit_cast(uint32_t, bmn2), __builtin_bit_cast(uint32_t, bmx2));
-        __syncthreads();
-        for (int c = 0; c < nch; c++) {
-            const uint4 o = s_mm[c][tid & 127];
-            amn2 = __builtin_elementwise_min(amn2, __builtin_bit_cast(u16x2, o.x));
-            amx2 = __builtin_elementwise_max(amx2, __builtin_bit_cast(u16x2, o.y));
-            bmn2 = __builtin_elementwise_min(bmn2, __builtin_bit_cast(u16x2, o.z));
-            bmx2 = __builtin_elementwise_max(bmx2, __builtin_bit_cast(u16x2, o.w));
-        }
-        const uint32_t amn = __builtin_bit_cast(uint32_t, amn2), amx = __builtin_bit_cast(uint32_t, amx2),
-                       bmn = __builtin_bit_cast(uint32_t, bmn2), bmx = __builtin_bit_cast(uint32_t, bmx2);
-        mn[0] = amn & 0xFFFFu; mn[2] = amn >> 16; mn[1] = bmn & 0xFFFFu; mn[3] = bmn >> 16;
-        len[0] = (uint32_t)bit_length_u32((amx & 0xFFFFu) - mn[0]);
-        len[2] = (uint32_t)bit_length_u32((amx >> 16) - mn[2]);
-        len[1] = (uint32_t)bit_length_u32((bmx & 0xFFFFu) - mn[1]);
-        len[3] = (uint32_t)bit_length_u32((bmx >> 16) - mn[3]);
-    } else {
+    {
         uint32_t lohi[4];                                  // minimum | maximum << 16 of each pack over the chunk
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -212,21 +179,7 @@ __global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restri
             reinterpret_cast<uint16_t *>(dst_u)[q] = reinterpret_cast<const uint16_t *>(area)[q];
     // ---- the words: sub-word s of a pack holds its tokens P - 16 (s + 1) .. P - 16 s - 1 ----
     uint8_t *pay = dst_u + meta;
-    if (IS_K) {
-        for (uint32_t s = s0; s < s1; s++) {
-            const uint8_t *row = tile + (size_t)(u * P + P - 16 * (int)(s + 1)) * hidden_dim + 4 * t;
-            uint32_t d[16];
-#pragma unroll
-            for (int k = 0; k < 16; k++) d[k] = *reinterpret_cast<const uint32_t *>(row + (size_t)k * hidden_dim);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint32_t c[16];
-#pragma unroll
-                for (int k = 0; k < 16; k++) c[k] = ((d[k] >> (8 * i)) & 0xFFu) - mn[i];
-                long_put_sub(reinterpret_cast<uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
-            }
-        }
-    } else {
+    {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             int tok0, ch;
@@ -242,15 +195,278 @@ __global__ void __launch_bounds__(1024) pack_long_kernel(const uint8_t *__restri
     }
 }
 
-template <bool IS_K>
-__global__ void __launch_bounds__(1024) unpack_long_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
+// ---- encoders that keep the codes in registers and build the block in LDS ------------------------------------------
+// The kernel above reads a block's codes twice (V: byte by byte, 64 bytes per wavefront load) and writes every
+// sub-word to the stream in 2-byte stores.  These two read the codes once with whole-row loads, keep them in
+// registers between the pass that finds minima and widths and the pass that forms the words, put the block together
+// in LDS exactly as it will lie in the stream, and copy it out in aligned 16-byte stores while the look-back of the
+// first wavefront runs beside the second pass.
+
+// n bytes (even) of LDS (src 16-byte aligned, readable 20 bytes past n) -> global memory (dst 2-byte aligned) by the whole
+// workgroup: head to the first 16-byte boundary and tail in 2-byte pieces, the body as aligned 16-byte stores fed by
+// aligned LDS reads and byte funnel shifts
+__device__ __forceinline__ void long_copy_out(uint8_t *dst, const uint8_t *src, uint32_t n, int tid, int nthreads) {
+    const uint32_t head = min(n, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
+    const uint32_t nq = (n - head) >> 4;
+    for (uint32_t i = (uint32_t)tid; i < (head >> 1); i += (uint32_t)nthreads)
+        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(src)[i];
+    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(src + (head & ~3u));
+    for (uint32_t i = (uint32_t)tid; i < nq; i += (uint32_t)nthreads) {
+        const uint32_t *q = src32 + 4 * i;
+        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+        uint4 v;
+        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
+        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
+        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
+        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+        *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
+    }
+    const uint32_t done = head + 16u * nq;
+    for (uint32_t i = (uint32_t)tid; i < ((n - done) >> 1); i += (uint32_t)nthreads)
+        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(src + done)[i];
+}
+
+// K: the thread layout of pack_long_kernel (half-wavefront per unit, lane <-> 4 channels, times the chunks of a
+// pack); a thread holds the NT = P / chunks tokens of its chunk as one dword (four channels) per token.
+template <int NT>
+__global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                                                          uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                                                          int hidden_dim, int P, int W, uint32_t nblocks) {
+    extern __shared__ __align__(16) uint8_t image[];       // the block as it will lie in the stream (+ 32 bytes of slack)
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t s_unit[4];
+    __shared__ uint32_t s_meta[4][kLongMetaWords];
+    __shared__ uint4 s_mm[kLongMaxChunks][128];            // minima and maxima of a thread's four packs over its chunk
+    const int tid = threadIdx.x, u = (tid >> 5) & 3, t = tid & 31;
+    const int chunk = tid >> 7, nch = (int)blockDim.x >> 7;
+    const uint32_t nsub = (uint32_t)P / 16u;
+    const uint32_t s1 = nsub * (uint32_t)(chunk + 1) / (uint32_t)nch;     // its sub-words end here; NT / 16 of them
+    const int k0 = P - 16 * (int)s1;                                     // ... and hold tokens k0 .. k0 + NT - 1 of the pack
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    if (chunk == 0) {
+        s_meta[u][t] = 0u;
+        if (t < kLongMetaWords - 32) s_meta[u][32 + t] = 0u;
+    }
+    __syncthreads();
+    const uint32_t b = s_idx;
+    if (b >= nblocks) return;
+    const int n_hid = hidden_dim / 128;
+    const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+    const uint8_t *tile = codes + (size_t)cb * (4 * P) * hidden_dim + (size_t)hb * 128;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    // ---- the codes, minima and widths ----
+    uint32_t d[NT];
+    const uint8_t *col = tile + (size_t)(u * P + k0) * hidden_dim + 4 * t;
+#pragma unroll
+    for (int q = 0; q < NT; q++) d[q] = *reinterpret_cast<const uint32_t *>(col + (size_t)q * hidden_dim);
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    u16x2 amn2 = {255, 255}, amx2 = {0, 0}, bmn2 = {255, 255}, bmx2 = {0, 0};   // channels (0, 2) and (1, 3) as 16-bit pairs
+#pragma unroll
+    for (int q = 0; q < NT; q++) {
+        const u16x2 a = __builtin_bit_cast(u16x2, d[q] & 0x00FF00FFu), c = __builtin_bit_cast(u16x2, (d[q] >> 8) & 0x00FF00FFu);
+        amn2 = __builtin_elementwise_min(amn2, a);
+        amx2 = __builtin_elementwise_max(amx2, a);
+        bmn2 = __builtin_elementwise_min(bmn2, c);
+        bmx2 = __builtin_elementwise_max(bmx2, c);
+    }
+    s_mm[chunk][tid & 127] = make_uint4(__builtin_bit_cast(uint32_t, amn2), __builtin_bit_cast(uint32_t, amx2),
+                                        __builtin_bit_cast(uint32_t, bmn2), __builtin_bit_cast(uint32_t, bmx2));
+    __syncthreads();
+    for (int c = 0; c < nch; c++) {
+        const uint4 o = s_mm[c][tid & 127];
+        amn2 = __builtin_elementwise_min(amn2, __builtin_bit_cast(u16x2, o.x));
+        amx2 = __builtin_elementwise_max(amx2, __builtin_bit_cast(u16x2, o.y));
+        bmn2 = __builtin_elementwise_min(bmn2, __builtin_bit_cast(u16x2, o.z));
+        bmx2 = __builtin_elementwise_max(bmx2, __builtin_bit_cast(u16x2, o.w));
+    }
+    const uint32_t amn = __builtin_bit_cast(uint32_t, amn2), amx = __builtin_bit_cast(uint32_t, amx2),
+                   bmn = __builtin_bit_cast(uint32_t, bmn2), bmx = __builtin_bit_cast(uint32_t, bmx2);
+    uint32_t mn[4], len[4];
+    mn[0] = amn & 0xFFFFu; mn[2] = amn >> 16; mn[1] = bmn & 0xFFFFu; mn[3] = bmn >> 16;
+    len[0] = (uint32_t)bit_length_u32((amx & 0xFFFFu) - mn[0]);
+    len[2] = (uint32_t)bit_length_u32((amx >> 16) - mn[2]);
+    len[1] = (uint32_t)bit_length_u32((bmx & 0xFFFFu) - mn[1]);
+    len[3] = (uint32_t)bit_length_u32((bmx >> 16) - mn[3]);
+    uint32_t off[4], payload;
+    pack_offsets(len, off, payload);
+    payload *= nsub;
+    if (t == 0 && chunk == 0) s_unit[u] = meta + payload;
+    if (chunk == 0) {
+        uint32_t minsw = 0, lensw = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            minsw |= (mn[i] & ((1u << W) - 1u)) << (i * W);
+            lensw |= len[i] << (i * g.LB);
+        }
+        long_put_meta(s_meta[u], t, W, minsw);
+        long_put_meta(s_meta[u] + g.mins_bytes / 4, t, g.LB, lensw);
+    }
+    __syncthreads();
+    const uint32_t bytes = 8u + s_unit[0] + s_unit[1] + s_unit[2] + s_unit[3];
+    if (tid == 0) lookback_publish(st, b, bytes);
+    // ---- the block in LDS: header, metadata, words ----
+    if (tid < 4) {
+        uint32_t cum = 0;
+        for (int q = 0; q <= tid; q++) cum += s_unit[q];
+        reinterpret_cast<uint16_t *>(image)[tid] = (uint16_t)(cum >> 2);
+    }
+    uint32_t ustart = 8u;
+    for (int q = 0; q < u; q++) ustart += s_unit[q];
+    if (chunk == 0)
+        for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
+            reinterpret_cast<uint32_t *>(image + ustart)[q] = s_meta[u][q];
+    uint8_t *pay = image + ustart + meta;
+#pragma unroll
+    for (int j = 0; j < NT / 16; j++) {
+        const uint32_t s = s1 - 1u - (uint32_t)j;           // tokens k0 + 16 j .. + 15 are sub-word s1 - 1 - j
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t c[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) c[k] = ((d[16 * j + k] >> (8 * i)) & 0xFFu) - mn[i];
+            long_put_sub(reinterpret_cast<uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+        }
+    }
+    if (tid < 64) {
+        const uint64_t o = lookback_offset(st, b, bytes, true);
+        if (tid == 0) {
+            s_off = o;
+            info[2 * (size_t)b] = (uint32_t)o;
+            info[2 * (size_t)b + 1] = bytes;
+            if (b == nblocks - 1) st->total = o + bytes;
+            if (o + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t o = s_off;
+    if (o + bytes > capacity) return;
+    long_copy_out(stream + o, image, bytes, tid, (int)blockDim.x);
+}
+
+// V: a workgroup of eight wavefronts per block, wavefront r <-> the P tokens of slot r % 4 of segment r / 4, lane <->
+// channel (the lower half-wavefront belongs to the unit of channels 0..31, the upper to that of channels 32..63).  A
+// 16-token x 64-channel tile is one 16-byte load per lane (four lanes per 64-byte row piece) and goes through LDS
+// to turn rows into the lane's column; the lane keeps its P codes four to a register.
+template <int P>
+__global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                                                         uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                                                         int hidden_dim, int W, uint32_t nblocks) {
+    constexpr int NSUB = P / 16;
+    constexpr int kRow = 80;                               // tile rows padded: 16-byte aligned, spread over the banks
+    extern __shared__ __align__(16) uint8_t image[];
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t s_unit[4];
+    __shared__ uint32_t s_meta[4][kLongMetaWords];
+    __shared__ uint8_t s_len[8][64];
+    __shared__ __align__(16) uint8_t s_tile[8][16 * kRow];
+    const int tid = threadIdx.x, r = tid >> 6, c = tid & 63;
+    const int seg = r >> 2, slot = r & 3, u = (c >> 5) * 2 + seg, t = c & 31;
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    if (tid < 4 * kLongMetaWords) (&s_meta[0][0])[tid] = 0u;
+    __syncthreads();
+    const uint32_t b = s_idx;
+    if (b >= nblocks) return;
+    const int n_hid = hidden_dim / 64;
+    const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    // ---- the codes, minimum and width of the lane's pack ----
+    const uint8_t *rows = codes + ((size_t)cb * (8 * P) + (size_t)r * P + (size_t)(c >> 2)) * hidden_dim + (size_t)hb * 64 + 16 * (c & 3);
+    uint8_t *mine = s_tile[r];
+    uint32_t pk[P / 4];
+    uint32_t lo = 255u, hi = 0u;
+    constexpr int kBatch = NSUB < 4 ? NSUB : 4;             // tiles requested at a time
+#pragma unroll
+    for (int j0 = 0; j0 < NSUB; j0 += kBatch) {
+        uint4 v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; j++) v[j] = *reinterpret_cast<const uint4 *>(rows + (size_t)(16 * (j0 + j)) * hidden_dim);
+#pragma unroll
+        for (int j = 0; j < kBatch; j++) {
+            *reinterpret_cast<uint4 *>(mine + (c >> 2) * kRow + 16 * (c & 3)) = v[j];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            uint32_t e[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) e[k] = mine[k * kRow + c];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int k = 0; k < 16; k++) { lo = min(lo, e[k]); hi = max(hi, e[k]); }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                pk[4 * (j0 + j) + q] = e[4 * q] | (e[4 * q + 1] << 8) | (e[4 * q + 2] << 16) | (e[4 * q + 3] << 24);
+                asm volatile("" : "+v"(pk[4 * (j0 + j) + q]));          // (kept packed: the compiler would carry the bytes apart)
+            }
+        }
+        asm volatile("" ::: "memory");                    // the next batch is requested here, not all batches up front
+    }
+    const uint32_t mn = lo, len = (uint32_t)bit_length_u32(hi - lo);
+    s_len[r][c] = (uint8_t)len;
+    __syncthreads();
+    uint32_t len4[4], off4[4], payload;
+#pragma unroll
+    for (int i = 0; i < 4; i++) len4[i] = s_len[seg * 4 + i][c];
+    pack_offsets(len4, off4, payload);
+    payload *= (uint32_t)NSUB;
+    if (slot == 0 && t == 0) s_unit[u] = meta + payload;
+    long_put_meta(s_meta[u], t, W, (mn & ((1u << W) - 1u)) << (slot * W));
+    long_put_meta(s_meta[u] + g.mins_bytes / 4, t, g.LB, len << (slot * g.LB));
+    __syncthreads();
+    const uint32_t bytes = 8u + s_unit[0] + s_unit[1] + s_unit[2] + s_unit[3];
+    if (tid == 0) lookback_publish(st, b, bytes);
+    // ---- the block in LDS: header, metadata, words ----
+    if (tid < 4) {
+        uint32_t cum = 0;
+        for (int q = 0; q <= tid; q++) cum += s_unit[q];
+        reinterpret_cast<uint16_t *>(image)[tid] = (uint16_t)(cum >> 2);
+    }
+    uint32_t ustart = 8u;
+    for (int q = 0; q < u; q++) ustart += s_unit[q];
+    if (slot == 0)
+        for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
+            reinterpret_cast<uint32_t *>(image + ustart)[q] = s_meta[u][q];
+    uint8_t *pay = image + ustart + meta + off4[slot] * (uint32_t)NSUB;
+    const uint32_t mn4 = mn * 0x01010101u;
+#pragma unroll
+    for (int j = 0; j < NSUB; j++) {
+        uint32_t e[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t w = pk[4 * j + q] - mn4;         // no byte borrows: every code is at least the minimum
+            e[4 * q] = w & 0xFFu; e[4 * q + 1] = (w >> 8) & 0xFFu; e[4 * q + 2] = (w >> 16) & 0xFFu; e[4 * q + 3] = w >> 24;
+        }
+        long_put_sub(reinterpret_cast<uint16_t *>(pay + (uint32_t)(NSUB - 1 - j) * 2u * len), e, len);   // tokens 16 j .. are sub-word NSUB - 1 - j
+    }
+    if (tid < 64) {
+        const uint64_t o = lookback_offset(st, b, bytes, true);
+        if (tid == 0) {
+            s_off = o;
+            info[2 * (size_t)b] = (uint32_t)o;
+            info[2 * (size_t)b + 1] = bytes;
+            if (b == nblocks - 1) st->total = o + bytes;
+            if (o + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t o = s_off;
+    if (o + bytes > capacity) return;
+    long_copy_out(stream + o, image, bytes, tid, 512);
+}
+
+__global__ void __launch_bounds__(1024) unpack_long_v_plain_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
                                                           uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
                                                           uint64_t stream_bytes) {
     __shared__ uint32_t s_meta[4][kLongMetaWords];
     const int tid = threadIdx.x, u = (tid >> 5) & 3, t = tid & 31;
     const int chunk = tid >> 7, nch = (int)blockDim.x >> 7;       // as in the encoder
     const uint32_t b = blockIdx.x;
-    const int hid_blk = IS_K ? 128 : 64, ctx_blk = (IS_K ? 4 : 8) * P;
+    const int hid_blk = 64, ctx_blk = 8 * P;
     const int n_hid = hidden_dim / hid_blk;
     const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
     uint8_t *tile = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
@@ -285,23 +501,7 @@ __global__ void __launch_bounds__(1024) unpack_long_kernel(const uint8_t *__rest
     if (ustart + meta + payload * nsub > uend) return;             // (uniform) widths that overrun the unit
     const uint32_t s0 = nsub * (uint32_t)chunk / (uint32_t)nch, s1 = nsub * (uint32_t)(chunk + 1) / (uint32_t)nch;
     const uint8_t *pay = src_u + meta;
-    if (IS_K) {
-        for (uint32_t s = s0; s < s1; s++) {
-            uint32_t d[16];
-#pragma unroll
-            for (int k = 0; k < 16; k++) d[k] = 0u;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint32_t c[16];
-                long_get_sub(reinterpret_cast<const uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
-#pragma unroll
-                for (int k = 0; k < 16; k++) d[k] |= ((c[k] + mn[i]) & 0xFFu) << (8 * i);
-            }
-            uint8_t *row = tile + (size_t)(u * P + P - 16 * (int)(s + 1)) * hidden_dim + 4 * t;
-#pragma unroll
-            for (int k = 0; k < 16; k++) *reinterpret_cast<uint32_t *>(row + (size_t)k * hidden_dim) = d[k];
-        }
-    } else {
+    {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             int tok0, ch;
@@ -463,17 +663,21 @@ __global__ void __launch_bounds__(256) unpack_long_k_kernel(const uint8_t *__res
 }
 
 // V: one workgroup of 256 threads per (pair of adjacent blocks, token half `seg`): half-wavefront h serves unit
-// q = h % 4 of the pair (block q / 2, channel half q % 2) and the sub-words of parity h / 4.  The bytes of `sps`
-// slots of the four units (all four when they fit the staging area, one at a time for the longest packs) go to LDS;
-// then, slot by slot, every half-wavefront decodes `R` sub-words per step into tiles of 16 tokens x 128 channels
-// (double-buffered) that are written out as whole lines.  Dynamic LDS: 4 staging regions, 2 x 2 R tiles, metadata.
-template <int R>
+// q = h % 4 of the pair (block q / 2, channel half q % 2).  The bytes of `sps` slots of the four units (the whole
+// unit with its metadata when all four slots fit the staging area, one or two slots at a time for the longest packs,
+// the next stage requested into registers while the current one is decoded) go to LDS.  A unit's work is cut into
+// items (slot, sub-word) of 16 tokens x 32 channels; a lane decodes FOUR ADJACENT CHANNELS of one item -- it reads
+// their (offset, width, minimum) from a table the unit's lanes fill after the offset scan -- so the codes come out
+// as the 16-token codec's K side produces them, a dword of four channels per token, and go into the tile as dwords.
+// A step is eight items per unit (the two half-wavefronts of a unit take four each): eight tiles of 16 tokens x 128
+// channels that are written out as whole lines.  Dynamic LDS: 4 staging regions, 8 tiles, the table, metadata.
+constexpr int kLongVTile = 16 * 128 + 32;                  // tile pitch: 32 bytes of padding keep the four items of a half-wavefront on different banks
 __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
                                                            uint8_t *__restrict__ codes, int hidden_dim, int P, int W,
                                                            uint64_t stream_bytes, uint32_t stage_cap, int sps) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, hw = tid >> 5, t = tid & 31;
-    const int q = hw & 3, sp = hw >> 2;                    // unit of the pair, parity of the sub-words
+    const int q = hw & 3, sp = hw >> 2;                    // unit of the pair, half of a step's items
     const int seg = (int)(blockIdx.x & 1u);
     const uint32_t pair = blockIdx.x >> 1;
     const int n_pair = hidden_dim / 128;
@@ -482,21 +686,29 @@ __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__res
     const int u = 2 * (q & 1) + seg;                       // unit of block b: channel half q % 2, token half seg
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
-    const uint32_t region = stage_cap + 48u;               // LDS bytes of one unit's staged slots
-    constexpr int kTileBytes = 16 * 128, kBuf = 2 * R * kTileBytes;
-    uint8_t *tiles = lds + 4 * region;                     // [2 buffers][2 parities][R][16 tokens][128 channels]
-    uint8_t *metas = tiles + 2 * kBuf;                     // [4 units][meta rounded up to 16 + 32]
-    const uint32_t meta_stride = ((meta + 15u) & ~15u) + 32u;
+    const uint32_t meta16 = (meta + 15u) & ~15u;
+    const uint32_t region = stage_cap + meta16 + 48u;      // LDS bytes of one unit's staged slots (with its metadata when the unit is staged whole)
+    uint8_t *tiles = lds + 4 * region;                     // [8 items][16 tokens][128 channels], padded
+    uint32_t *table = reinterpret_cast<uint32_t *>(tiles + 8 * kLongVTile);     // [4 units][4 slots][32 channels]: offset | width << 16 | minimum << 24
+    uint8_t *metas = reinterpret_cast<uint8_t *>(table + 4 * 4 * 32);          // [4 units][meta rounded up to 16 + 32]
+    const uint32_t meta_stride = meta16 + 32u;
     uint64_t boff = 0;
     uint32_t ustart = 0, ubytes = 0;
     bool ok = long_unit_span(stream, stream_bytes, info, b, u, P, meta, boff, ustart, ubytes);          // uniform per half-wavefront
-    // metadata of the four units -> LDS (the two half-wavefronts of a unit share the copy)
+    uint8_t *reg = lds + q * region;
+    const int l64 = t + 32 * sp;
+    // all four slots fit the staging area: the unit goes to LDS in one piece, metadata and words (one trip to memory
+    // instead of two); else the metadata first (the two half-wavefronts of a unit share the copies)
+    const bool whole = sps == 4;
     uint32_t mphase = 0;
-    if (ok) mphase = stage_to_lds(stream + boff + ustart, meta, metas + q * meta_stride, t + 32 * sp, 64);
+    if (ok) mphase = whole ? stage_to_lds(stream + boff + ustart, min(ubytes, meta + stage_cap), reg, l64, 64)
+                           : stage_to_lds(stream + boff + ustart, meta, metas + q * meta_stride, l64, 64);
     __syncthreads();
-    uint32_t mn[4], len[4], off[4], payload = 0;
+    const uint32_t nsub = (uint32_t)P / 16u;
+    uint32_t base[5];
     {
-        const uint8_t *m = metas + q * meta_stride + mphase;
+        uint32_t mn[4], len[4], off[4], payload = 0;
+        const uint8_t *m = (whole ? reg : metas + q * meta_stride) + mphase;
         const uint32_t minsw = ok ? lds_meta_word(m, t, W) : 0u;
         const uint32_t lensw = ok ? lds_meta_word(m + g.mins_bytes, t, g.LB) : 0u;
 #pragma unroll
@@ -505,60 +717,96 @@ __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__res
             len[i] = min((lensw >> (i * g.LB)) & ((1u << g.LB) - 1u), (uint32_t)kMaxBits);
         }
         pack_offsets(len, off, payload);                   // (whole wavefronts: every lane takes part)
+        ok = ok && meta + payload * nsub <= ubytes;        // widths that overrun the unit
+        if (sp == 0)
+#pragma unroll
+            for (int i = 0; i < 4; i++) table[(q * 4 + i) * 32 + t] = off[i] | (len[i] << 16) | (mn[i] << 24);
+        // slot i of this unit: bytes [base[i], base[i + 1]) * nsub of the payload; the slot bases are the offsets of the
+        // half-wavefront's first lane (swizzle within 32 lanes: every lane reads lane 0 of its half)
+#pragma unroll
+        for (int i = 0; i < 4; i++) base[i] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[i], 0);
+        base[4] = payload;
     }
-    const uint32_t nsub = (uint32_t)P / 16u;
-    ok = ok && meta + payload * nsub <= ubytes;            // widths that overrun the unit
-    // slot i of this unit: bytes [base[i], base[i + 1]) * nsub of the payload; the slot bases are the offsets of the
-    // half-wavefront's first lane (swizzle within 32 lanes: every lane reads lane 0 of its half)
-    uint32_t base[5];
-#pragma unroll
-    for (int i = 0; i < 4; i++) base[i] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[i], 0);
-    base[4] = payload;
     uint8_t *out = codes + (size_t)cb * (8 * P) * hidden_dim + (size_t)hp * 128;
-    uint8_t *reg = lds + q * region;
-    int buf = 0;
-    uint32_t sphase = 0, b_stage = 0;                      // phase of the staged bytes, payload offset (/ nsub) they start at
-#pragma unroll 1
-    for (int i = 0; i < 4; i++) {
-        uint32_t len_i = len[0], mn_i = mn[0], off_i = off[0];                  // (selected, not indexed: the arrays stay in registers)
-        if (i == 1) { len_i = len[1]; mn_i = mn[1]; off_i = off[1]; }
-        if (i == 2) { len_i = len[2]; mn_i = mn[2]; off_i = off[2]; }
-        if (i == 3) { len_i = len[3]; mn_i = mn[3]; off_i = off[3]; }
-        if (i % sps == 0) {                                // (uniform) the next sps slots' bytes
-            const uint32_t b_lo = i == 0 ? base[0] : i == 1 ? base[1] : i == 2 ? base[2] : base[3];
-            const int ie = i + sps;
-            const uint32_t b_hi = ie == 1 ? base[1] : ie == 2 ? base[2] : ie == 3 ? base[3] : base[4];
-            const uint32_t sbytes = min((b_hi - b_lo) * nsub, stage_cap);
-            __syncthreads();                               // the bytes staged before are no longer read
-            if (ok) sphase = stage_to_lds(stream + boff + ustart + meta + b_lo * nsub, sbytes, reg, t + 32 * sp, 64);
-            b_stage = b_lo;
-            __syncthreads();
+    uint32_t sphase = mphase + meta, b_stage = 0;          // phase of the staged words, payload offset (/ nsub) they start at
+    // Longer packs are staged `sps` slots at a time.  The 16-byte pieces of the next stage are requested into
+    // registers before the current one is decoded (up to kPre per thread: 64 threads x 5 x 16 bytes cover 4 KiB and
+    // the phase), so that the trip to memory runs under the decode; larger stages are fetched when they are needed.
+    constexpr int kPre = 5;
+    const bool pre = !whole && stage_cap + 16u <= 64u * kPre * 16u;
+    uint4 pv[kPre];
+    uint32_t ld_phase = 0, ld_n16 = 0, ld_b = 0;
+    auto slot_base = [&](int i) { return i == 0 ? base[0] : i == 1 ? base[1] : i == 2 ? base[2] : i == 3 ? base[3] : base[4]; };
+    auto pre_load = [&](int i) {
+        const uint32_t b_lo = slot_base(i), b_hi = slot_base(i + sps);
+        const uint32_t sbytes = min((b_hi - b_lo) * nsub, stage_cap);
+        const uint8_t *src = stream + boff + ustart + meta + b_lo * nsub;
+        ld_phase = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
+        ld_n16 = ok ? (ld_phase + sbytes + 15u) >> 4 : 0u;
+        ld_b = b_lo;
+        const uint4 *s16 = reinterpret_cast<const uint4 *>(src - ld_phase);
+#pragma unroll
+        for (int v = 0; v < kPre; v++) {
+            const uint32_t idx = (uint32_t)l64 + 64u * (uint32_t)v;
+            pv[v] = idx < ld_n16 ? s16[idx] : make_uint4(0u, 0u, 0u, 0u);
         }
-        const size_t tok_slot = (size_t)(seg * 4 + i) * P;
+    };
+    if (pre) pre_load(0);
+    const int m4 = t & 7, sel = t >> 3;                    // the lane's four channels 4 m4 .. 4 m4 + 3 and which of the half-wavefront's four items
+    const uint32_t steps_per_stage = nsub * (uint32_t)sps / 8u;      // (the launcher sees to nsub * sps >= 8)
 #pragma unroll 1
-        for (uint32_t s0 = 0; s0 < nsub; s0 += 2 * R) {    // sub-words s0 .. s0 + 2 R - 1: parity sp takes s0 + sp, s0 + sp + 2, ...
-            if (ok) {
+    for (int i0 = 0; i0 < 4; i0 += sps) {                  // a stage: slots i0 .. i0 + sps - 1
+        if (!whole) {
+            __syncthreads();                               // the bytes staged before are no longer read
+            if (pre) {
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    const uint32_t s = s0 + (uint32_t)sp + 2u * (uint32_t)r;
-                    uint8_t *tile = tiles + buf * kBuf + (sp * R + r) * kTileBytes;
-                    uint32_t c[16];
-                    sub_codes1(reg, sphase + (off_i - b_stage) * nsub + s * 2u * len_i, len_i, mn_i, W > 4, c);
-#pragma unroll
-                    for (int k = 0; k < 16; k++) tile[k * 128 + 32 * q + t] = (uint8_t)c[k];
+                for (int v = 0; v < kPre; v++) {
+                    const uint32_t idx = (uint32_t)l64 + 64u * (uint32_t)v;
+                    if (idx < ld_n16) reinterpret_cast<uint4 *>(reg)[idx] = pv[v];
                 }
+                sphase = ld_phase;
+                b_stage = ld_b;
+            } else {
+                const uint32_t b_lo = slot_base(i0), b_hi = slot_base(i0 + sps);
+                const uint32_t sbytes = min((b_hi - b_lo) * nsub, stage_cap);
+                if (ok) sphase = stage_to_lds(stream + boff + ustart + meta + b_lo * nsub, sbytes, reg, l64, 64);
+                b_stage = b_lo;
             }
-            __syncthreads();                               // the tiles of this buffer are complete
-            // 2 R tiles of 16 rows x 128 bytes = 256 R pieces of 16 bytes: R per thread
+        }
+        __syncthreads();                                   // the stage and the table are there
+        if (pre && i0 + sps < 4) pre_load(i0 + sps);
+#pragma unroll 1
+        for (uint32_t j = 0; j < steps_per_stage; j++) {
+            const uint32_t item0 = (uint32_t)i0 * nsub + 8u * j;            // the step's first item: slot item / nsub, sub-word item % nsub
+            if (ok) {
+                const uint32_t item = item0 + 4u * (uint32_t)sp + (uint32_t)sel;
+                const uint32_t i = item / nsub, s = item % nsub;
+                const uint4 tb = *reinterpret_cast<const uint4 *>(table + (q * 4 + (int)i) * 32 + 4 * m4);
+                const uint32_t e4[4] = {tb.x, tb.y, tb.z, tb.w};
+                uint32_t wo[4], len[4], mn[4], c4[16];
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const int idx = tid + 256 * r;
-                const int tl = idx >> 7, row = (idx >> 3) & 15, c16 = idx & 7;      // tile (parity * R + r'), row, piece
-                const uint32_t sw = s0 + (uint32_t)(tl / R) + 2u * (uint32_t)(tl % R);
-                const uint4 v = *reinterpret_cast<const uint4 *>(tiles + buf * kBuf + tl * kTileBytes + row * 128 + 16 * c16);
-                *reinterpret_cast<uint4 *>(out + (tok_slot + (size_t)(P - 16 * (int)(sw + 1)) + row) * hidden_dim + 16 * c16) = v;
+                for (int c = 0; c < 4; c++) {
+                    len[c] = (e4[c] >> 16) & 0xFFu;
+                    mn[c] = e4[c] >> 24;
+                    wo[c] = sphase + ((e4[c] & 0xFFFFu) - b_stage) * nsub + s * 2u * len[c];
+                }
+                sub_codes(reg, wo, len, mn, W > 4, c4);
+                uint8_t *tile = tiles + (4 * sp + sel) * kLongVTile + 32 * q + 4 * m4;
+#pragma unroll
+                for (int k = 0; k < 16; k++) *reinterpret_cast<uint32_t *>(tile + k * 128) = c4[k];
             }
-            buf ^= 1;                                      // the next step writes the other buffer while this one is read
+            __syncthreads();                               // the tiles are complete
+            // 8 tiles of 16 rows x 128 bytes = 1024 pieces of 16 bytes: four per thread
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int idx = tid + 256 * r;
+                const int tl = idx >> 7, row = (idx >> 3) & 15, c16 = idx & 7;
+                const uint32_t item = item0 + (uint32_t)tl;
+                const uint32_t i = item / nsub, s = item % nsub;
+                const uint4 v = *reinterpret_cast<const uint4 *>(tiles + tl * kLongVTile + row * 128 + 16 * c16);
+                *reinterpret_cast<uint4 *>(out + ((size_t)(seg * 4 + (int)i) * P + (size_t)(P - 16 * (int)(s + 1)) + row) * hidden_dim + 16 * c16) = v;
+            }
+            __syncthreads();                               // ... and read before the next step writes them
         }
     }
 }
@@ -592,8 +840,30 @@ static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint6
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     const int threads = 128 * long_chunks(P);
-    if (is_k) pack_long_kernel<true><<<nblocks, threads, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
-    else pack_long_kernel<false><<<nblocks, threads, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    // the block image in LDS: the block's bound and what the copy reads past the last byte
+    const uint32_t image_bytes = (uint32_t)pkv_block_bound_p(P, bits) + 32u;
+    if (is_k) {
+        const int nt = P / long_chunks(P);                            // tokens of a pack per thread: 16, or 32 for P = 256
+        const void *fn = nt == 32 ? reinterpret_cast<const void *>(pack_long_k_kernel<32>) : reinterpret_cast<const void *>(pack_long_k_kernel<16>);
+        PKV_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)image_bytes));
+        if (nt == 32) pack_long_k_kernel<32><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+        else pack_long_k_kernel<16><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    } else if ((reinterpret_cast<uintptr_t>(codes) & 15u) == 0) {
+#define PKV_LAUNCH_LONG_V(PP)                                                                                                  \
+    do {                                                                                                                       \
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pack_long_v_kernel<PP>),                               \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)image_bytes));                       \
+        pack_long_v_kernel<PP><<<nblocks, 512, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, bits, nblocks); \
+    } while (0)
+        if (P == 32) PKV_LAUNCH_LONG_V(32);
+        else if (P == 64) PKV_LAUNCH_LONG_V(64);
+        else if (P == 128) PKV_LAUNCH_LONG_V(128);
+        else PKV_LAUNCH_LONG_V(256);
+#undef PKV_LAUNCH_LONG_V
+    } else {
+        // a code matrix that does not start at a 16-byte boundary: the plain kernel (byte loads)
+        pack_long_v_plain_kernel<<<nblocks, threads, 0, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+    }
     PKV_HIP_CHECK(hipGetLastError());
     if ((rc = tm.end(ms_out))) return rc;
     return finish_encode(st, size_out, 0, s);
@@ -614,20 +884,22 @@ static int run_unpack_long(bool is_k, const uint8_t *stream, uint64_t stream_byt
         const int threads = 32 * (P / 16 < 8 ? P / 16 : 8);
         unpack_long_k_kernel<<<4 * nblocks, threads < 64 ? 64 : threads, unit_cap + 48u, s>>>(stream, info, codes, hidden_dim, P, bits,
                                                                                           stream_bytes, unit_cap);
-    } else if (hidden_dim % 128 == 0) {
+    } else if (hidden_dim % 128 == 0 && (reinterpret_cast<uintptr_t>(codes) & 15u) == 0) {
         // pairs of adjacent blocks (whole 128-byte lines), a workgroup per token half; all four slots of a unit are
-        // staged at once while they fit 8 KiB per unit, else one slot at a time
-        const int sps = 4u * slot_cap <= 8192u ? 4 : 2u * slot_cap <= 8192u ? 2 : 1;
+        // staged at once while they fit 4 KiB per unit, else two or one at a time -- but never less than the eight
+        // (slot, sub-word) items of a step
+        const uint32_t stage_max = 4096u;        // (8 KiB: 5 % slower at 128 and 256 tokens, two trips to memory per stage; 2 KiB: 15 % slower at 64)
+        int sps = 4u * slot_cap <= stage_max ? 4 : 2u * slot_cap <= stage_max ? 2 : 1;
+        while (sps * (P / 16) < 8) sps *= 2;
         const uint32_t stage_cap = (uint32_t)sps * slot_cap;
-        const int R = P >= 64 ? 2 : 1;                               // sub-words per half-wavefront and step
-        const uint32_t lds_bytes = 4u * (stage_cap + 48u) + 2u * 2u * (uint32_t)R * 2048u + 4u * (((meta + 15u) & ~15u) + 32u);
-        const void *fn = R == 2 ? reinterpret_cast<const void *>(unpack_long_v_kernel<2>) : reinterpret_cast<const void *>(unpack_long_v_kernel<1>);
-        PKV_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        if (R == 2) unpack_long_v_kernel<2><<<nblocks, 256, lds_bytes, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes, stage_cap, sps);
-        else unpack_long_v_kernel<1><<<nblocks, 256, lds_bytes, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes, stage_cap, sps);
+        const uint32_t meta16 = (meta + 15u) & ~15u;
+        const uint32_t lds_bytes = 4u * (stage_cap + meta16 + 48u) + 8u * (uint32_t)kLongVTile + 4u * 4u * 32u * 4u + 4u * (meta16 + 32u);
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(unpack_long_v_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        unpack_long_v_kernel<<<nblocks, 256, lds_bytes, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes, stage_cap, sps);
     } else {
         const int threads = 128 * long_chunks(P);
-        unpack_long_kernel<false><<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
+        unpack_long_v_plain_kernel<<<nblocks, threads, 0, s>>>(stream, info, codes, hidden_dim, P, bits, stream_bytes);
     }
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);

@@ -258,6 +258,29 @@ def test_long_packs_bit_exact_vs_oracle(cuda, oracle_codec, is_k, P):
             assert torch.equal(back, d_codes)
 
 
+def test_long_v_packs_from_a_code_matrix_that_is_not_16_byte_aligned(cuda):
+    """V's long-pack encoder loads 16 bytes per lane; a code matrix that starts elsewhere takes the plain kernel and
+    must give the same stream."""
+    g = torch.Generator().manual_seed(11)
+    for P, W in ((32, 4), (128, 3), (256, 6)):
+        ctx_blk, hid_blk = ops.long_block_shape(0, P)
+        T, H = 2 * ctx_blk, 3 * hid_blk
+        c = torch.randint(0, 1 << W, (T, H), generator=g, dtype=torch.uint8).to(cuda)
+        buf = torch.empty(T * H + 16, dtype=torch.uint8, device=cuda)
+        shifted = buf[3:3 + T * H].view(T, H)
+        shifted.copy_(c)
+        assert shifted.data_ptr() % 16 != 0 and shifted.is_contiguous()
+        nblk = (T // ctx_blk) * (H // hid_blk)
+        out = []
+        for m in (c, shifted):
+            stream = torch.zeros(nblk * ops.block_bound_p(P, W), dtype=torch.uint8, device=cuda)
+            info = torch.zeros(nblk, 2, dtype=torch.uint32, device=cuda)
+            size = ops.encode_p(0, m, stream, info, P, W)
+            out.append((size, stream[:size].clone(), info.clone()))
+        assert out[0][0] == out[1][0]
+        assert torch.equal(out[0][1], out[1][1]) and torch.equal(out[0][2].view(torch.int32), out[1][2].view(torch.int32))
+
+
 def test_long_packs_of_16_tokens_forward_to_the_reference_format(cuda, oracle_codec):
     rng = np.random.default_rng(77)
     for is_k, (cb, hb) in ((1, (64, 128)), (0, (128, 64))):
