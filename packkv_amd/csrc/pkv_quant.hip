@@ -378,8 +378,7 @@ __device__ __forceinline__ f16x2 pk_max_h(f16x2 a, f16x2 b) {
 // l16 == 0 writes the token's scale and zero and its constants for quant4.  `rows` is x at (sequence, head 0, the
 // round's first token) and uniform, so the eight loads are one 32-bit lane offset on eight scalar bases.
 template <int DT>
-__device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
-                                                   uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
+__device__ __forceinline__ void round_token_minmax(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float &mn, float &mx) {
     const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;          // bytes
     uint4 v[8];
     v[0] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows) + lane_off);
@@ -388,7 +387,6 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
         if (i < H) v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)i * head_stride) + lane_off);
         else v[i] = v[0];
     }
-    float mn, mx;
     if (DT == PKV_F16) {               // packed fp16 comparisons all the way down to one word each
         f16x2 lo[8], hi[8];
 #pragma unroll
@@ -413,6 +411,13 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
         for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
     }
     row16_minmax(mn, mx);
+}
+
+template <int DT>
+__device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
+                                                   uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
+    float mn, mx;
+    round_token_minmax<DT>(rows, head_stride, H, tt, l16, mn, mx);
     if (l16 == 0) {
         const float range = round_t<DT>(mx - mn);
         const float sc = round_t<DT>(range * rel);
@@ -422,6 +427,7 @@ __device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t 
         *par_out = token_par<DT>(sc, zb, false);
     }
 }
+
 
 // The same for groups of up to four heads (several of which share a workgroup): only the rows that exist are
 // fetched and compared.
@@ -640,87 +646,8 @@ __device__ __forceinline__ void unit_emit_any(uint8_t *blk, uint32_t unit_off, i
     for (int i = 0; i < 4; i++) put_pack(reinterpret_cast<uint16_t *>(pay + u.off[i]), u, i);
 }
 
-// V blocks: a wavefront's 64 cells (round 4 sg + i, channels 4 g .. 4 g + 3; lane = 16 i + g) cover
-// one segment sg of the block; V units want lane c = channel c holding the packs of rounds
-// 4 sg .. 4 sg + 3.  The packs change lanes inside the wavefront through a 1 KiB LDS area, one
-// 32-bit field at a time: every lane stores its four channels as one 16-byte word (area[lane][slot]
-// = area[round i][channel 4 g + slot]), then lane c reads area[i][c] for i = 0..3 -- both sides
-// touch consecutive dwords, no bank conflicts.  LDS serves a wavefront's accesses in order, so
-// only the compiler needs fencing.
-__device__ __forceinline__ void v_exchange(UnitPacks &u, uint8_t *area, int lane) {
-    uint32_t *a = reinterpret_cast<uint32_t *>(area);
-    uint32_t f[3][4];
-#pragma unroll
-    for (int sl = 0; sl < 4; sl++) {
-        f[0][sl] = (uint32_t)u.word[sl];
-        f[1][sl] = (uint32_t)(u.word[sl] >> 32);
-        f[2][sl] = u.mn[sl] | (u.len[sl] << 8);
-    }
-#pragma unroll
-    for (int kind = 0; kind < 3; kind++) {
-        *reinterpret_cast<uint4 *>(a + 4 * lane) = make_uint4(f[kind][0], f[kind][1], f[kind][2], f[kind][3]);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int i = 0; i < 4; i++) f[kind][i] = a[64 * i + lane];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-#pragma unroll
-    for (int sl = 0; sl < 4; sl++) {
-        u.word[sl] = ((uint64_t)f[1][sl] << 32) | f[0][sl];
-        u.mn[sl] = f[2][sl] & 0xFFu;
-        u.len[sl] = f[2][sl] >> 8;
-    }
-}
-
-// the same exchange for the two-halves pack words of widths 5 and 6
-__device__ __forceinline__ void v_exchange(UnitPacksW &u, uint8_t *area, int lane) {
-    uint32_t *a = reinterpret_cast<uint32_t *>(area);
-    uint32_t f[5][4];
-#pragma unroll
-    for (int sl = 0; sl < 4; sl++) {
-        f[0][sl] = (uint32_t)u.lo[sl];
-        f[1][sl] = (uint32_t)(u.lo[sl] >> 32);
-        f[2][sl] = (uint32_t)u.hi[sl];
-        f[3][sl] = (uint32_t)(u.hi[sl] >> 32);
-        f[4][sl] = u.mn[sl] | (u.len[sl] << 8);
-    }
-#pragma unroll
-    for (int kind = 0; kind < 5; kind++) {
-        *reinterpret_cast<uint4 *>(a + 4 * lane) = make_uint4(f[kind][0], f[kind][1], f[kind][2], f[kind][3]);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int i = 0; i < 4; i++) f[kind][i] = a[64 * i + lane];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-#pragma unroll
-    for (int sl = 0; sl < 4; sl++) {
-        u.lo[sl] = ((uint64_t)f[1][sl] << 32) | f[0][sl];
-        u.hi[sl] = ((uint64_t)f[3][sl] << 32) | f[2][sl];
-        u.mn[sl] = f[4][sl] & 0xFFu;
-        u.len[sl] = f[4][sl] >> 8;
-    }
-}
-
-// ---- fused parameters + quantize + encode, one workgroup per sub-group ---------------------
-// A group is the run of blocks that share one (context block, sequence): H blocks for K, 2 H for
-// V, consecutive in stream order; a sub-group is up to eight consecutive blocks of a group.  One
-// workgroup of 256 threads (two blocks at a time)
-//   1. reads the group's x for the per-token min / max over ALL heads (sub-groups of one group
-//      repeat this read; they run at the same time, so the repeats are served by the caches);
-//      the first sub-group writes scale / zero;
-//   2. re-reads its own blocks (cache-hot) cell by cell, quantizes and encodes them into LDS;
-//   3. obtains the sub-group's stream offset with ONE look-back (one ticket and one status word
-//      per sub-group) and writes its bytes, contiguous in the stream, in one sweep of aligned
-//      16-byte stores.
-// So x crosses HBM once, and the ordered-ticket / look-back traffic shrinks eightfold.
+// A group is the run of blocks that share one (context block, sequence): H blocks for K, 2 H for V, consecutive in
+// stream order.  The encoders below give a workgroup the blocks of up to eight heads of a group.
 constexpr int kSubBlocks = 8;
 
 // Wave priorities (s_setprio) of the round-major encoders' phases: the parameter pass goes first, so that its rows
@@ -732,185 +659,6 @@ constexpr int kSubBlocks = 8;
 #define PKV_EPRIO_EMIT 2
 #endif
 
-template <bool IS_K, int DT, bool WIDE>
-__global__ void __launch_bounds__(256) quant_encode_group_kernel(
-    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
-    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t nsub, uint32_t bound, uint64_t base, int par_stride) {
-    constexpr int CTX = IS_K ? 64 : 128;
-    extern __shared__ __align__(16) uint8_t gbuf[];        // the sub-group's encoded bytes (8 x block bound)
-    __shared__ uint32_t s_idx;
-    __shared__ uint64_t s_off;
-    __shared__ uint32_t unit_bytes[2][4];
-    __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the sub-group
-    __shared__ __attribute__((aligned(16))) TokPar s_par[CTX];
-    const int tid = threadIdx.x;
-    const int HB = IS_K ? H : 2 * H;                      // blocks per group
-    const int SG = (HB + kSubBlocks - 1) / kSubBlocks;    // sub-groups per group
-    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
-    __syncthreads();
-    const uint32_t sidx = s_idx;
-    if (sidx >= nsub) return;
-    const uint32_t gidx = sidx / (uint32_t)SG, sg = sidx % (uint32_t)SG;
-    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
-    const size_t tok0 = (size_t)cb * CTX;
-    const int jbase = (int)sg * kSubBlocks;               // first block of the sub-group inside the group
-    const int nb = min(kSubBlocks, HB - jbase);
-
-    // ---- 1. per-token parameters ----
-    // Sub-group 0 of a group computes them (16 lanes x 8 channels per token, all heads) and
-    // publishes each token's (scale, zero) as ONE 64-bit word (valid bit | scale | zero) behind the
-    // status words -- single relaxed agent-scope atomics like the look-back, no fence, so no cache
-    // write-back.  Later sub-groups of the group, whose tickets are younger (so sub-group 0 is
-    // already running and never waits for them), poll those words instead of reading all heads
-    // again.  A wait that expires falls back to computing.
-    uint64_t *tokw = st->status + nsub + ((size_t)b * T + tok0);
-    __shared__ int s_miss;
-    if (tid == 0) s_miss = 0;
-    __syncthreads();
-    if (sg != 0) {
-        if (tid < CTX) {
-            uint64_t w = __hip_atomic_load(tokw + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            int spins = 0;
-            while ((w >> 63) == 0 && spins < kSpinLimit) {
-                __builtin_amdgcn_s_sleep(16);
-                w = __hip_atomic_load(tokw + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                spins++;
-            }
-            if ((w >> 63) == 0) s_miss = 1;
-            else s_par[tid] = token_par<DT>(T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu), (uint32_t)w & 0xFFFFu);
-        }
-        __syncthreads();
-    }
-    if (sg == 0 || s_miss)
-    for (int tt = tid >> 4; tt < CTX; tt += 16) {
-        const int l16 = tid & 15;
-        float mn = INFINITY, mx = -INFINITY;
-        // eight rows in flight at a time (head indices clamped: a repeated row changes no min / max)
-        for (int h0 = 0; h0 < H; h0 += 8) {
-            uint4 v[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                v[i] = *reinterpret_cast<const uint4 *>(
-                    x + (((size_t)b * H + min(h0 + i, H - 1)) * T + tok0 + tt) * kHeadDim + l16 * 8);
-#pragma unroll
-            for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
-        }
-#pragma unroll
-        for (int d = 8; d >= 1; d >>= 1) {
-            mn = fminf(mn, __shfl_xor(mn, d, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, d, 16));
-        }
-        if (l16 == 0) {
-            const float range = round_t<DT>(mx - mn);
-            const float sc = round_t<DT>(range * rel);
-            const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-            if (sg == 0) {
-                scale[(size_t)b * par_stride + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
-                zero[(size_t)b * par_stride + tok0 + tt] = (uint16_t)zb;
-                if (SG > 1)
-                    __hip_atomic_store(tokw + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(sc) << 16) | (uint64_t)zb,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            s_par[tt] = token_par<DT>(sc, zb);
-        }
-    }
-    if (tid == 0) blk_off[0] = 0;
-    __syncthreads();
-
-    // ---- 2. encode, two blocks at a time ----
-    const UnitGeom g = unit_geom(W);
-    const int jl = tid >> 7, ct = tid & 127;             // local block, cell
-    const int round = IS_K ? ct >> 5 : ct >> 4;
-    const int cgrp = IS_K ? ct & 31 : ct & 15;
-    const int unit = IS_K ? ct >> 5 : 2 * ((ct >> 5) & 1) + (ct >> 6);
-    const int t = tid & 31;
-    uint32_t cmax_all = 0;
-    for (int j0 = 0; j0 < nb; j0 += 2) {
-        const int jj = j0 + jl;                           // block inside the sub-group
-        const bool active = jj < nb;
-        const int j = jbase + min(jj, nb - 1);            // block inside the group (clamped: loads are unconditional)
-        const int h = IS_K ? j : j >> 1, d0 = IS_K ? 0 : (j & 1) * 64;
-        uint2 xr[16];
-        cell_load(x + (((size_t)b * H + h) * T + tok0 + 16 * round) * kHeadDim + d0 + 4 * cgrp, xr);
-        typename PacksOf<WIDE>::type u;
-        uint32_t cmax;
-        cell_packs<DT>(xr, s_par + 16 * round, u, cmax);
-        if (active) {
-            cmax_all = max(cmax_all, cmax);
-            // V: the exchange area (1 KiB per wavefront) sits in the block's own worst-case slot,
-            // which lies behind everything encoded so far
-            if (!IS_K) v_exchange(u, gbuf + (((size_t)jj * bound + 15) & ~(size_t)15) + ((tid >> 6) & 1) * 1024, tid & 63);
-            pack_offsets(u.len, u.off, u.payload);
-            if (t == 0) unit_bytes[jl][unit] = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
-        }
-        __syncthreads();
-        if (tid == 0) {                                   // block sizes of this pair -> offsets inside the sub-group
-            uint32_t off = blk_off[j0];
-            off += 8u + unit_bytes[0][0] + unit_bytes[0][1] + unit_bytes[0][2] + unit_bytes[0][3];
-            blk_off[j0 + 1] = off;
-            if (j0 + 1 < nb) blk_off[j0 + 2] = off + 8u + unit_bytes[1][0] + unit_bytes[1][1] + unit_bytes[1][2] + unit_bytes[1][3];
-            // the sub-group's size is known here, before its last pair is written: the successors' look-backs wait less
-            if (j0 + 2 >= nb) lookback_publish(st, sidx, blk_off[nb]);
-        }
-        __syncthreads();
-        if (active) {
-            uint8_t *blk = gbuf + blk_off[jj];
-            uint32_t base = 8u;
-#pragma unroll
-            for (int q = 0; q < 4; q++) base += q < unit ? unit_bytes[jl][q] : 0u;
-            if (t == 0) reinterpret_cast<uint16_t *>(blk)[unit] = (uint16_t)(base - 8u + unit_bytes[jl][unit]);
-            unit_emit_any(blk, base, t, g, u);
-        }
-        __syncthreads();
-    }
-    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
-        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
-    }
-
-    // ---- 3. one look-back for the whole sub-group, then one contiguous copy ----
-    const uint32_t bytes = blk_off[nb];
-    if (tid < 64) {
-        const uint64_t off = base + lookback_offset(st, sidx, bytes, true);
-        if (tid == 0) {
-            s_off = off;
-            if (sidx == nsub - 1) st->total = off + bytes;
-            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
-        }
-    }
-    __syncthreads();
-    const uint64_t off = s_off;
-    if (off + bytes > capacity) return;
-    if (tid < nb) {
-        const uint32_t first = cb * (uint32_t)(B * HB) + b * (uint32_t)HB + (uint32_t)jbase;   // stream index of the first block
-        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
-        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
-    }
-    // head (to the first 16-byte boundary of the stream) and tail in 2-byte pieces, the body as
-    // aligned 16-byte stores fed by aligned LDS reads and byte funnel shifts
-    uint8_t *dst = stream + off;
-    const uint32_t head = min(bytes, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
-    const uint32_t nq = (bytes - head) >> 4;
-    for (uint32_t i = tid; i < (head >> 1); i += 256)
-        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(gbuf)[i];
-    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(gbuf + (head & ~3u));
-    for (uint32_t i = tid; i < nq; i += 256) {
-        const uint32_t *q = src32 + 4 * i;
-        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
-        uint4 v;
-        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
-        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
-        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
-        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
-        *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
-    }
-    const uint32_t done = head + 16u * nq;
-    for (uint32_t i = tid; i < ((bytes - done) >> 1); i += 256)
-        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(gbuf + done)[i];
-}
-
 // ---- K, all heads in one workgroup: round-major single trip over x --------------------------
 // For H <= 8 the eight blocks of a (context block, sequence) group are the eight heads, so one
 // workgroup of 256 threads (head j = tid / 32, lane t = tid % 32) can go through the group ROUND BY
@@ -921,12 +669,13 @@ __global__ void __launch_bounds__(256) quant_encode_group_kernel(
 // PERM: the tokens are encoded in the order of a repacking -- position p of the output holds token
 // (p / perm_block) * perm_block + perm[p] of x (perm_block a multiple of 64) -- so a round's rows are gathered; scale
 // and zero are written in the output order.
-template <int DT, bool WIDE, bool PERM>
+template <int DT, bool WIDE, bool PERM, bool XCH = false>
 __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
-    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger, int gpw, uint32_t ngroups_total) {
+    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger, int gpw, uint32_t ngroups_total,
+    int nsg = 1, uint64_t *xw = nullptr) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -938,6 +687,16 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     __syncthreads();
     const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);   // uniform: the rows' addresses become scalar
     if (gidx >= ngroups) return;
+    // XCH (more than eight heads): a group's heads are cut into nsg runs of eight, one workgroup (one ticket) each,
+    // consecutive in the stream.  A workgroup reads only its own heads: it forms the round's minima and maxima over
+    // them, publishes them per token as one 64-bit word (valid | min | max, a relaxed agent-scope atomic like the
+    // look-back's status words) and takes the other runs' words to form the token parameters, which are therefore
+    // the same bits in every run.  The runs of a group hold consecutive tickets, so all of them are running or next
+    // in line: the oldest unfinished group is always complete on the machine and the waits end.  H_all = all heads.
+    const int H_all = H;
+    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
+    const int hbase = XCH ? 8 * (int)sgi : 0;
+    if (XCH) H = min(8, H_all - hbase);
     // Fewer than five heads: a workgroup takes gpw = 8 / H (rounded down) consecutive groups -- consecutive in the
     // stream too -- so that its eight half-wavefronts all have a block; `ngroups` then counts workgroups and
     // `ngroups_all` groups.  Half-wavefront j serves head j % H of group gidx * gpw + j / H; everything below that is
@@ -948,7 +707,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint32_t grp_first = gidx * (uint32_t)gpw;
     const int ng = (int)min((uint32_t)gpw, ngroups_all - grp_first);          // groups of this workgroup
     const int nblk = gpw > 1 ? ng * H : H;                // blocks of this workgroup
-    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : gidx;
+    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : XCH ? gidx / (uint32_t)nsg : gidx;
     const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 64;
     const UnitGeom g = unit_geom(W);
@@ -974,6 +733,46 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
                 const uint32_t src = r == 0 ? src_tok[0] : r == 1 ? src_tok[1] : r == 2 ? src_tok[2] : src_tok[3];
                 round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
                                        (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
+            } else if (XCH) {
+                float mn, mx;
+                round_token_minmax<DT>(x + (((size_t)b * H_all + hbase) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, mn, mx);
+                uint64_t *words = xw + ((size_t)(gidx - sgi) * 4 + r) * 16;       // [run][round][token] of this group
+                if (l16 == 0)
+                    __hip_atomic_store(words + (size_t)sgi * 64 + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(mn) << 16) | (uint64_t)T16<DT>::to_bits(mx),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // the first wavefront collects: lane = (run, token) for up to four runs at a time
+                if (tid < 64) {
+                    float amn = INFINITY, amx = -INFINITY;
+                    for (int s0 = 0; s0 < nsg; s0 += 4) {
+                        const int run = s0 + (tid >> 4);
+                        if (run < nsg) {
+                            const uint64_t *wp = words + (size_t)run * 64 + (tid & 15);
+                            uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            int spins = 0;
+                            while ((w >> 63) == 0 && spins < kSpinLimit) {
+                                __builtin_amdgcn_s_sleep(8);
+                                w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                spins++;
+                            }
+                            if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
+                            amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
+                            amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
+                        }
+                    }
+                    amn = fminf(amn, __shfl_xor(amn, 16, 64)); amx = fmaxf(amx, __shfl_xor(amx, 16, 64));
+                    amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
+                    if (tid < 16) {
+                        const float range = round_t<DT>(amx - amn);
+                        const float sc = round_t<DT>(range * rel);
+                        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
+                        if (sgi == 0) {
+                            const size_t tk = (size_t)b * par_stride + tok0 + 16 * r + tid;
+                            scale[tk] = (uint16_t)T16<DT>::to_bits(sc);
+                            zero[tk] = (uint16_t)zb;
+                        }
+                        s_par[tid] = token_par<DT>(sc, zb, false);
+                    }
+                }
             } else if (gpw == 1) {
                 round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
                                        scale + tok, zero + tok, s_par + tt);
@@ -994,7 +793,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
             cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 16 * r, (uint32_t)perm_block - 1u,
                            (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
         } else {
-            cell_load(x + (((size_t)b * H + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
+            cell_load(x + (((size_t)b * H_all + hbase + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
         }
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
@@ -1042,7 +841,7 @@ __global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < nblk) {
-        const uint32_t first = (gpw > 1 ? grp_first : gidx) * (uint32_t)H;      // block index = group * H + head
+        const uint32_t first = XCH ? grp * (uint32_t)H_all + (uint32_t)hbase : (gpw > 1 ? grp_first : gidx) * (uint32_t)H;      // block index = group * H + head
         info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
         info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
@@ -1132,13 +931,13 @@ __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, con
 // unit (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight
 // threads of a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed
 // in with LDS atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.
-template <int DT, bool WIDE, bool PERM>
+template <int DT, bool WIDE, bool PERM, bool XCH = false>
 __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
     const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
-    const uint16_t *__restrict__ zero_in, const Stagger stagger, int gpw, uint32_t ngroups_total) {
+    const uint16_t *__restrict__ zero_in, const Stagger stagger, int gpw, uint32_t ngroups_total, int nsg, uint64_t *xw) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1152,6 +951,12 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     __syncthreads();
     const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
     if (gidx >= ngroups) return;
+    // XCH (more than eight heads): runs of eight heads, one workgroup each, that exchange the minima and maxima of
+    // their rows per token, as in the K kernel; a run's words are [iteration][token of the iteration]
+    const int H_all = H;
+    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
+    const int hbase = XCH ? 8 * (int)sgi : 0;
+    if (XCH) H = min(8, H_all - hbase);
     // Fewer than five heads: gpw = 8 / H (rounded down) consecutive groups to a workgroup, as in the K kernel --
     // `ngroups` counts workgroups, `ngroups_total` groups; head slot j serves head j % H of group gidx * gpw + j / H.
     const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31;
@@ -1159,7 +964,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint32_t grp_first = gidx * (uint32_t)gpw;
     const int ng = (int)min((uint32_t)gpw, ngroups_total - grp_first);        // groups of this workgroup
     const int nheads = gpw > 1 ? ng * H : H;              // head slots in use
-    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : gidx;
+    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : XCH ? gidx / (uint32_t)nsg : gidx;
     const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
     const UnitGeom g = unit_geom(W);
@@ -1198,6 +1003,42 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
                     round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
                                            (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
                 }
+            } else if (XCH) {
+                float mn, mx;
+                round_token_minmax<DT>(x + (((size_t)b * H_all + hbase) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, mn, mx);
+                uint64_t *words = xw + (size_t)(gidx - sgi) * 128 + 32 * it;      // [run][iteration][token] of this group
+                if (l16 == 0)
+                    __hip_atomic_store(words + (size_t)sgi * 128 + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(mn) << 16) | (uint64_t)T16<DT>::to_bits(mx),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // the first wavefront collects: lane = (parity of the run, token)
+                if (tid < 64) {
+                    float amn = INFINITY, amx = -INFINITY;
+                    for (int run = tid >> 5; run < nsg; run += 2) {
+                        const uint64_t *wp = words + (size_t)run * 128 + (tid & 31);
+                        uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        int spins = 0;
+                        while ((w >> 63) == 0 && spins < kSpinLimit) {
+                            __builtin_amdgcn_s_sleep(8);
+                            w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            spins++;
+                        }
+                        if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
+                        amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
+                        amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
+                    }
+                    amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
+                    if (tid < 32) {
+                        const float range = round_t<DT>(amx - amn);
+                        const float sc = round_t<DT>(range * rel);
+                        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
+                        if (sgi == 0) {
+                            const size_t tk = (size_t)b * par_stride + tok0 + 32 * it + tid;
+                            scale[tk] = (uint16_t)T16<DT>::to_bits(sc);
+                            zero[tk] = (uint16_t)zb;
+                        }
+                        s_par[tid] = token_par<DT>(sc, zb, false);
+                    }
+                }
             } else if (gpw == 1) {
                 round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
                                        scale + tok, zero + tok, s_par + tt);
@@ -1219,7 +1060,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
             cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 32 * it + 16 * rps, (uint32_t)perm_block - 1u,
                            (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
         } else {
-            cell_load(x + (((size_t)b * H + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
+            cell_load(x + (((size_t)b * H_all + hbase + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
         }
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
@@ -1293,7 +1134,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < nblk) {
-        const uint32_t first = grp_first * (uint32_t)(2 * H);                 // block index = group * 2 H + 2 head + half
+        const uint32_t first = XCH ? grp * (uint32_t)(2 * H_all) + (uint32_t)(2 * hbase) : grp_first * (uint32_t)(2 * H);    // block index = group * 2 H + 2 head + half
         info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
         info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
@@ -1505,15 +1346,19 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
     if (capacity > (1ull << 32)) capacity = 1ull << 32;
     PKV_REQUIRE(base <= capacity, PKV_ERR_CAPACITY, "stream offset beyond 4 GiB: block_info offsets are 32 bits");
     ScanState *st = nullptr;
-    // One workgroup per sub-group of up to eight consecutive blocks that share (context block, sequence).
+    // One workgroup per run of up to eight heads of a (context block, sequence) group -- K: its up to eight blocks;
+    // V: its up to sixteen -- or, with fewer than five heads, per 8 / H groups.
     {
         const int HB = IS_K ? H : 2 * H;
         const uint32_t bound = IS_K ? (uint32_t)k_block_bound(ctx_blk, bits) : (uint32_t)v_block_bound(hid_blk, bits);
-        const uint32_t gbytes = (uint32_t)kSubBlocks * bound + 32u;
         const uint32_t nsub = (uint32_t)(T / ctx_blk) * (uint32_t)B * (uint32_t)((HB + kSubBlocks - 1) / kSubBlocks);
-        const bool shared_params = (HB > kSubBlocks);            // sub-groups of a group hand the token parameters on
-        PKV_REQUIRE((uint64_t)nsub + (uint64_t)B * (uint64_t)T < (1ull << 31), PKV_ERR_UNSUPPORTED, "batch x tokens too large");
-        if ((rc = prepare_scan_state(nsub + (shared_params ? (uint32_t)B * (uint32_t)T : 0u), &st, s))) return rc;   // status words, then one word per token
+        // status words (one per ticket; nsub bounds the tickets of every kernel below), then, with more than eight
+        // heads, the words the runs of a group exchange: one per (run, token)
+        const int nruns = (H + kSubBlocks - 1) / kSubBlocks;                // runs of eight heads per group
+        const uint32_t nruns_all = (uint32_t)(T / ctx_blk) * (uint32_t)B * (uint32_t)nruns;
+        PKV_REQUIRE((uint64_t)nsub + (uint64_t)nruns_all * (uint64_t)ctx_blk < (1ull << 31), PKV_ERR_UNSUPPORTED, "batch x tokens too large");
+        const uint32_t xwords = H <= kSubBlocks ? 0u : nruns_all * (uint32_t)ctx_blk;
+        if ((rc = prepare_scan_state(nsub + xwords, &st, s))) return rc;
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
         if (!IS_K && H <= 8) {               // one workgroup per group of 2 H blocks
@@ -1537,7 +1382,7 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
             kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
                                            stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
-                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all);
+                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all, 1, nullptr);
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
             // up to four heads: 8 / H groups to a workgroup, so that all eight half-wavefronts have a block
@@ -1555,14 +1400,34 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             Stagger sg;
             if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
             kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                       capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub);
-        } else {
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, true>
-                                                      : quant_encode_group_kernel<IS_K, PKV_BF16, true>)
-                                 : (dtype == PKV_F16 ? quant_encode_group_kernel<IS_K, PKV_F16, false>
-                                                      : quant_encode_group_kernel<IS_K, PKV_BF16, false>);
-            kern<<<nsub, 256, gbytes, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                           capacity, info, st, bits, nsub, bound, base, par_stride);
+                                       capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub, 1, nullptr);
+        } else if (IS_K) {                           // more than eight heads: runs of eight, one workgroup each, that exchange their minima and maxima
+            const uint32_t slot = (bound + 15u) & ~15u;
+            const uint32_t lds = (uint32_t)kSubBlocks * slot + 32u;
+            const int nsg = (H + kSubBlocks - 1) / kSubBlocks;
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false, true>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true, false, true>)
+                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false, true>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false, false, true>);
+            Stagger sg;
+            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nsub, &sg))) return rc;
+            kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                        capacity, info, st, bits, nsub, slot, base, par_stride, nullptr, 0, sg, 1, nsub, nsg,
+                                        st->status + nsub);
+        } else {                                     // V, more than eight heads: the same runs of eight
+            const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
+            const uint32_t lds = 64u * unit_slot + 64u;
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false, true>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true, false, true>)
+                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false, true>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false, false, true>);
+            PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            Stagger sg;
+            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, nruns_all, &sg))) return rc;
+            kern<<<nruns_all, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
+                                             stream, capacity, info, st, bits, nruns_all, unit_slot, base, par_stride, nullptr, 0,
+                                             nullptr, nullptr, sg, 1, nruns_all, nruns, st->status + nruns_all);
         }
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;

@@ -60,6 +60,29 @@ def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
             assert torch.equal(r["zero"].cpu().view(torch.int16), z.reshape(B, T).view(torch.int16))
 
 
+def test_fused_quant_encode_more_than_eight_heads(cuda, oracle_codec):
+    """More than eight KV heads: the heads of a (context block, sequence) are cut into runs of eight, one workgroup
+    each, that exchange their minima and maxima through memory; hundreds of runs in flight, groups of 3, 4 and 5 runs,
+    a last run of fewer than eight heads."""
+    for (B, H, T, rel, dtype) in ((4, 32, 2048, 0.1, torch.float16), (2, 24, 1024, 0.2, torch.bfloat16),
+                                  (1, 40, 512, 0.1, torch.float16), (3, 20, 512, 0.05, torch.float16)):
+        k, v = synth.make_kv(B, H, T, seed=3 + H, dtype=dtype)
+        for is_k, x in ((1, k), (0, v)):
+            _say("fused quant+encode, many heads", "K" if is_k else "V", dtype, B, H, T, rel)
+            c, z, s = oq.quant_ints(x, 64, rel)
+            cm = oq.code_matrix(c).numpy()
+            W = ops.bits_for_rel(rel)
+            cb, hb = (64, 128) if is_k else (128, 64)
+            so, io, zo = oracle_codec.encode(is_k, cm, cb, hb, W)
+            for rep in range(2):                      # (twice: the exchange words of the first call must not leak into the second)
+                r = (ops.k_quant_encode if is_k else ops.v_quant_encode)(x.to(cuda), rel, W)
+                assert r["size"] == zo
+                assert np.array_equal(r["info"].cpu().numpy(), io)
+                assert np.array_equal(r["stream"][:zo].cpu().numpy(), so[:zo])
+                assert torch.equal(r["scale"].cpu().view(torch.int16), s.reshape(B, T).view(torch.int16))
+                assert torch.equal(r["zero"].cpu().view(torch.int16), z.reshape(B, T).view(torch.int16))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_fused_quant_encode_offset_rows_bit_exact(cuda, oracle_codec, dtype):
     """Rows far from zero: the zero point is large (here about -750 and +750, and a few hundred for the smaller
