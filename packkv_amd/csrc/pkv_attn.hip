@@ -714,13 +714,16 @@ int pkv::attn_decode_impl(const pkv_attn_args *a, float *ms_out, hipStream_t s, 
     const int n_tiles = a->T_c / kTile;
     int nsplit = 0, tps = 0;
     if (n_tiles > 0) {
-        // Members per (sequence, KV head): about PKV_SPLIT_TARGET workgroups in all -- four resident on each of 256
+        // Members per (sequence, KV head): about PKV_SPLIT_TARGET workgroups in all for the reference's widths -- four resident on each of 256
         // CUs.  When the heads do not divide that number, rounding the members up leaves a few workgroups over that
         // only start once others have finished, each with a full share of tiles (12 sequences x 8 heads: 11 members,
         // 1056 workgroups, 115 us per step against 99 us with 10 members); so both roundings are priced as
         // generations x tiles per member and the cheaper one is taken, the finer cut on a tie.
         const int pairs = a->B * a->Hkv;
-        const int target = PKV_SPLIT_TARGET;
+        // (as many members as are resident at once: widths 5 and 6 run two workgroups per CU -- 193 us per step with
+        // 512 members against 199 us with 1024 in two generations, 6 bits 201 against 218 us -- and groups of eight
+        // query heads three: 156 against 165 us)
+        const int target = PKV_SPLIT_TARGET / 4 * PKV_DMA_WAVES((a->k_bits > a->v_bits ? a->k_bits : a->v_bits), G);
         long best_cost = -1;
         for (int up = 1; up >= 0; up--) {
             int want = up ? (target + pairs - 1) / pairs : target / pairs;
