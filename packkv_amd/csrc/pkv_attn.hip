@@ -530,8 +530,10 @@ static int launch_dma(const AttnParams &p, hipStream_t s) {
 template <int G>
 static int launch_dma_bits(const AttnParams &p, hipStream_t s) {
 #ifdef PKV_ATTN_MINIMAL
-#if PKV_ATTN_MINIMAL == 55     // (-DPKV_ATTN_MINIMAL=55: the 5-bit kernel instead)
+#if PKV_ATTN_MINIMAL == 55     // (-DPKV_ATTN_MINIMAL=55: the 5-bit kernel instead, =33: the 3-bit kernel)
     if constexpr (G == 4) { if (p.k_bits == 5 && p.v_bits == 5) return launch_dma<G, 5, 5>(p, s); }
+#elif PKV_ATTN_MINIMAL == 33
+    if constexpr (G == 4) { if (p.k_bits == 3 && p.v_bits == 3) return launch_dma<G, 3, 3>(p, s); }
 #else
     if constexpr (G == 4 || G == 1) { if (p.k_bits == 4 && p.v_bits == 4) return launch_dma<G, 4, 4>(p, s); }
 #endif

@@ -799,20 +799,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PKV_DM
     const int n_dyn = n_tiles - 5 * p.nsplit;                   // tiles that are handed out by counter
     uint32_t fetched = 0u;        // wave 0, lane 0: old counter value of the request in flight
     int pend_n = 0, cur_base = 0, cur_left = 0;                 // size of that request; the batch being drawn on
-    // (the index goes through a vector register the compiler cannot see into: with an address it knows to be the
-    // same in every lane it rewrites the atomic as a reduction over the active lanes whose epilogue waits for the
-    // answer on the spot -- and with it for the copies just issued)
-    uint32_t ctr_idx = (uint32_t)bh;
-    asm volatile("" : "+v"(ctr_idx));
     auto batch_of = [&](int handed) -> int {
         int n = (n_dyn - handed) >> p.batch_shift;
         n = max(n, 1);
         PKV_SCALAR(n);
         return min(n, 4);
     };
+    // (the counter's index goes through a vector register the compiler cannot see into: with an address it knows to be
+    // the same in every lane it rewrites the atomic as a reduction over the active lanes whose epilogue waits for the
+    // answer on the spot -- and with it for the copies just issued.  And it does so where it is used: an address
+    // formed once before the loop is a register pair that lives through it, and the 3-bit kernels spilled it, which
+    // put a scratch reload and its wait for every outstanding copy in here)
     auto request = [&](int n) {
-        if (wave == 0 && lane == 0)
+        if (wave == 0 && lane == 0) {
+            uint32_t ctr_idx = (uint32_t)bh;
+            asm volatile("" : "+v"(ctr_idx));
             fetched = __hip_atomic_fetch_add(p.counters + ctr_idx, (uint32_t)n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         pend_n = n;
     };
     if (p.dynamic) request(batch_of(0));

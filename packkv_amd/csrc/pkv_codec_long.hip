@@ -378,33 +378,32 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
     uint8_t *mine = s_tile[r];
     uint32_t pk[P / 4];
     uint32_t lo = 255u, hi = 0u;
-    constexpr int kBatch = NSUB < 4 ? NSUB : 4;             // tiles requested at a time
+    // two tiles are requested ahead of the one being turned (named registers: an array here ends up in scratch memory)
+    uint4 t0 = *reinterpret_cast<const uint4 *>(rows);
+    uint4 t1 = *reinterpret_cast<const uint4 *>(rows + (size_t)16 * hidden_dim);          // (NSUB >= 2)
 #pragma unroll
-    for (int j0 = 0; j0 < NSUB; j0 += kBatch) {
-        uint4 v[kBatch];
+    for (int j = 0; j < NSUB; j++) {
+        uint4 t2 = t1;
+        if (j + 2 < NSUB) t2 = *reinterpret_cast<const uint4 *>(rows + (size_t)(16 * (j + 2)) * hidden_dim);
+        *reinterpret_cast<uint4 *>(mine + (c >> 2) * kRow + 16 * (c & 3)) = t0;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        uint32_t e[16];
 #pragma unroll
-        for (int j = 0; j < kBatch; j++) v[j] = *reinterpret_cast<const uint4 *>(rows + (size_t)(16 * (j0 + j)) * hidden_dim);
+        for (int k = 0; k < 16; k++) e[k] = mine[k * kRow + c];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int j = 0; j < kBatch; j++) {
-            *reinterpret_cast<uint4 *>(mine + (c >> 2) * kRow + 16 * (c & 3)) = v[j];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            uint32_t e[16];
+        for (int k = 0; k < 16; k++) { lo = min(lo, e[k]); hi = max(hi, e[k]); }
 #pragma unroll
-            for (int k = 0; k < 16; k++) e[k] = mine[k * kRow + c];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-            for (int k = 0; k < 16; k++) { lo = min(lo, e[k]); hi = max(hi, e[k]); }
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                pk[4 * (j0 + j) + q] = e[4 * q] | (e[4 * q + 1] << 8) | (e[4 * q + 2] << 16) | (e[4 * q + 3] << 24);
-                asm volatile("" : "+v"(pk[4 * (j0 + j) + q]));          // (kept packed: the compiler would carry the bytes apart)
-            }
+        for (int q = 0; q < 4; q++) {
+            pk[4 * j + q] = e[4 * q] | (e[4 * q + 1] << 8) | (e[4 * q + 2] << 16) | (e[4 * q + 3] << 24);
+            asm volatile("" : "+v"(pk[4 * j + q]));          // (kept packed: the compiler would carry the bytes apart)
         }
-        asm volatile("" ::: "memory");                    // the next batch is requested here, not all batches up front
+        t0 = t1;
+        t1 = t2;
     }
     const uint32_t mn = lo, len = (uint32_t)bit_length_u32(hi - lo);
     s_len[r][c] = (uint8_t)len;
@@ -431,7 +430,8 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
     if (slot == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
             reinterpret_cast<uint32_t *>(image + ustart)[q] = s_meta[u][q];
-    uint8_t *pay = image + ustart + meta + off4[slot] * (uint32_t)NSUB;
+    const uint32_t my_off = slot == 0 ? off4[0] : slot == 1 ? off4[1] : slot == 2 ? off4[2] : off4[3];
+    uint8_t *pay = image + ustart + meta + my_off * (uint32_t)NSUB;
     const uint32_t mn4 = mn * 0x01010101u;
 #pragma unroll
     for (int j = 0; j < NSUB; j++) {
@@ -705,7 +705,7 @@ __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__res
                            : stage_to_lds(stream + boff + ustart, meta, metas + q * meta_stride, l64, 64);
     __syncthreads();
     const uint32_t nsub = (uint32_t)P / 16u;
-    uint32_t base[5];
+    uint32_t base0, base1, base2, base3, base4;       // (scalars, not an array: indexed by the stage below it would live in scratch memory)
     {
         uint32_t mn[4], len[4], off[4], payload = 0;
         const uint8_t *m = (whole ? reg : metas + q * meta_stride) + mphase;
@@ -723,9 +723,11 @@ __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__res
             for (int i = 0; i < 4; i++) table[(q * 4 + i) * 32 + t] = off[i] | (len[i] << 16) | (mn[i] << 24);
         // slot i of this unit: bytes [base[i], base[i + 1]) * nsub of the payload; the slot bases are the offsets of the
         // half-wavefront's first lane (swizzle within 32 lanes: every lane reads lane 0 of its half)
-#pragma unroll
-        for (int i = 0; i < 4; i++) base[i] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[i], 0);
-        base[4] = payload;
+        base0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[0], 0);
+        base1 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[1], 0);
+        base2 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[2], 0);
+        base3 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)off[3], 0);
+        base4 = payload;
     }
     uint8_t *out = codes + (size_t)cb * (8 * P) * hidden_dim + (size_t)hp * 128;
     uint32_t sphase = mphase + meta, b_stage = 0;          // phase of the staged words, payload offset (/ nsub) they start at
@@ -736,7 +738,7 @@ __global__ void __launch_bounds__(256) unpack_long_v_kernel(const uint8_t *__res
     const bool pre = !whole && stage_cap + 16u <= 64u * kPre * 16u;
     uint4 pv[kPre];
     uint32_t ld_phase = 0, ld_n16 = 0, ld_b = 0;
-    auto slot_base = [&](int i) { return i == 0 ? base[0] : i == 1 ? base[1] : i == 2 ? base[2] : i == 3 ? base[3] : base[4]; };
+    auto slot_base = [&](int i) { return i == 0 ? base0 : i == 1 ? base1 : i == 2 ? base2 : i == 3 ? base3 : base4; };
     auto pre_load = [&](int i) {
         const uint32_t b_lo = slot_base(i), b_hi = slot_base(i + sps);
         const uint32_t sbytes = min((b_hi - b_lo) * nsub, stage_cap);

@@ -1162,7 +1162,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
 // (hist[level][thread]: one LDS add per value, no two threads on one word).  At the end the columns of a token are
 // summed per level and the level that reaches rank (n - 1) / 2 is the median.  H <= 8, code width <= 6 bits.
 template <int DT>
-__global__ void __launch_bounds__(256, DT == PKV_F16 ? 8 : 5) token_median_from_x_kernel(const uint16_t *__restrict__ x, int B, int H, int T, float rel,
+__global__ void __launch_bounds__(256, DT == PKV_F16 ? 8 : 4) token_median_from_x_kernel(const uint16_t *__restrict__ x, int B, int H, int T, float rel,
                                                                   int W, uint8_t *__restrict__ median,
                                                                   uint16_t *__restrict__ scale_out, uint16_t *__restrict__ zero_out) {
     extern __shared__ uint32_t hist[];                     // [1 << W][256]
@@ -1171,6 +1171,7 @@ __global__ void __launch_bounds__(256, DT == PKV_F16 ? 8 : 5) token_median_from_
     // workgroups go round-robin over the 8 XCDs: each XCD takes a contiguous eighth of the tokens
     const uint32_t wg = (gridDim.x & 7u) == 0u ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     const size_t tok0 = (size_t)wg * 16;
+    const uint32_t tok_idx = (uint32_t)tok0 + (uint32_t)tt;
     for (int l = 0; l < levels; l++) hist[l * 256 + tid] = 0u;       // the thread's own column: no barrier needed
     const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;
     typedef __attribute__((address_space(3))) uint32_t *lds_u32_ptr;
@@ -1224,8 +1225,12 @@ __global__ void __launch_bounds__(256, DT == PKV_F16 ? 8 : 5) token_median_from_
         // a wavefront holds four tokens: it takes the usual quantisation sequence when all four can, else the general
         // one for all (quant4 branches on the first lane's constants)
         if (scale_out && l16 == 0) {                       // the parameters pkv_quant_params would write, for the encoder
-            scale_out[(size_t)b * T + tok0 + tt] = (uint16_t)T16<DT>::to_bits(sc);
-            zero_out[(size_t)b * T + tok0 + tt] = (uint16_t)zb;
+            // (a uniform row pointer and a 32-bit offset, written out as the store itself: the compiler kept 64-bit
+            // per-lane addresses across the loop and spilled them, with a reload and a full wait in every sequence)
+            uint16_t *srow = scale_out + (size_t)b * T, *zrow = zero_out + (size_t)b * T;
+            const uint32_t boff = 2u * tok_idx, sbits = T16<DT>::to_bits(sc);
+            asm volatile("global_store_short %0, %1, %2" : : "v"(boff), "v"(sbits), "s"(srow) : "memory");
+            asm volatile("global_store_short %0, %1, %2" : : "v"(boff), "v"(zb), "s"(zrow) : "memory");
         }
         TokPar tp = token_par<DT>(sc, zb, false);
         const bool wave_usual = !__any(tp.sub2 == 0u);
