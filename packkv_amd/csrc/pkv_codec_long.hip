@@ -199,31 +199,54 @@ __global__ void __launch_bounds__(1024) pack_long_v_plain_kernel(const uint8_t *
 // The kernel above reads a block's codes twice (V: byte by byte, 64 bytes per wavefront load) and writes every
 // sub-word to the stream in 2-byte stores.  These two read the codes once with whole-row loads, keep them in
 // registers between the pass that finds minima and widths and the pass that forms the words, put the block together
-// in LDS exactly as it will lie in the stream, and copy it out in aligned 16-byte stores while the look-back of the
+// in LDS byte for byte as it will lie in the stream (bank-swizzled, below), and copy it out in aligned 16-byte stores while the look-back of the
 // first wavefront runs beside the second pass.
 
-// n bytes (even) of LDS (src 16-byte aligned, readable 20 bytes past n) -> global memory (dst 2-byte aligned) by the whole
-// workgroup: head to the first 16-byte boundary and tail in 2-byte pieces, the body as aligned 16-byte stores fed by
-// aligned LDS reads and byte funnel shifts
-__device__ __forceinline__ void long_copy_out(uint8_t *dst, const uint8_t *src, uint32_t n, int tid, int nthreads) {
+// The block image in LDS is bank-swizzled: byte a of the block lies at a ^ (((a >> 7) & 31) << 2), i.e. the dword's
+// bank is XOR-ed with the number of its 128-byte row.  A lane's pack is a run of 2 len P / 16 bytes, so with 4-bit
+// widths and packs of 128 or 256 tokens the lanes' runs start 64 or 128 bytes apart and their 2-byte stores of one
+// instruction would all land on one or two banks (123 M conflict cycles per launch at 256 tokens, more than half
+// of the kernel's time); rows that differ now take different banks.
+__device__ __forceinline__ uint32_t long_swz(uint32_t a) { return a ^ (((a >> 7) & 31u) << 2); }
+
+// the 2 * len bytes of one 16-token sub-word into the swizzled image at byte offset `off` (even)
+__device__ __forceinline__ void long_put_sub_swz(uint8_t *image, uint32_t off, const uint32_t c[16], uint32_t len) {
+    uint64_t hi = 0, lo = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        hi = (hi << len) | c[k];
+        lo = (lo << len) | c[8 + k];
+    }
+    unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
+    for (uint32_t q = 0; q < len; q++) {
+        *reinterpret_cast<uint16_t *>(image + long_swz(off + 2u * q)) = (uint16_t)wd;
+        wd >>= 16;
+    }
+}
+
+// n bytes (even) of the swizzled image -> global memory (dst 2-byte aligned) by the whole workgroup: head to the first
+// 16-byte boundary and tail in 2-byte pieces, the body as aligned 16-byte stores fed by dword LDS reads and byte
+// funnel shifts (the image is readable 20 bytes past n)
+__device__ __forceinline__ void long_copy_out(uint8_t *dst, const uint8_t *image, uint32_t n, int tid, int nthreads) {
     const uint32_t head = min(n, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
     const uint32_t nq = (n - head) >> 4;
     for (uint32_t i = (uint32_t)tid; i < (head >> 1); i += (uint32_t)nthreads)
-        reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(src)[i];
-    const uint32_t *src32 = reinterpret_cast<const uint32_t *>(src + (head & ~3u));
+        reinterpret_cast<uint16_t *>(dst)[i] = *reinterpret_cast<const uint16_t *>(image + long_swz(2u * i));
+    const uint32_t a0 = head & ~3u;
     for (uint32_t i = (uint32_t)tid; i < nq; i += (uint32_t)nthreads) {
-        const uint32_t *q = src32 + 4 * i;
-        const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+        uint32_t d[5];
+#pragma unroll
+        for (int k = 0; k < 5; k++) d[k] = *reinterpret_cast<const uint32_t *>(image + long_swz(a0 + 16u * i + 4u * (uint32_t)k));
         uint4 v;
-        v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
-        v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
-        v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
-        v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
+        v.x = __builtin_amdgcn_alignbyte(d[1], d[0], head);
+        v.y = __builtin_amdgcn_alignbyte(d[2], d[1], head);
+        v.z = __builtin_amdgcn_alignbyte(d[3], d[2], head);
+        v.w = __builtin_amdgcn_alignbyte(d[4], d[3], head);
         *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
     }
     const uint32_t done = head + 16u * nq;
     for (uint32_t i = (uint32_t)tid; i < ((n - done) >> 1); i += (uint32_t)nthreads)
-        reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(src + done)[i];
+        reinterpret_cast<uint16_t *>(dst + done)[i] = *reinterpret_cast<const uint16_t *>(image + long_swz(done + 2u * i));
 }
 
 // K: the thread layout of pack_long_kernel (half-wavefront per unit, lane <-> 4 channels, times the chunks of a
@@ -310,14 +333,14 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
     if (tid < 4) {
         uint32_t cum = 0;
         for (int q = 0; q <= tid; q++) cum += s_unit[q];
-        reinterpret_cast<uint16_t *>(image)[tid] = (uint16_t)(cum >> 2);
+        *reinterpret_cast<uint16_t *>(image + long_swz(2u * (uint32_t)tid)) = (uint16_t)(cum >> 2);
     }
     uint32_t ustart = 8u;
     for (int q = 0; q < u; q++) ustart += s_unit[q];
     if (chunk == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
-            reinterpret_cast<uint32_t *>(image + ustart)[q] = s_meta[u][q];
-    uint8_t *pay = image + ustart + meta;
+            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[u][q];
+    const uint32_t pay = ustart + meta;                   // byte offset of the unit's payload inside the block
 #pragma unroll
     for (int j = 0; j < NT / 16; j++) {
         const uint32_t s = s1 - 1u - (uint32_t)j;           // tokens k0 + 16 j .. + 15 are sub-word s1 - 1 - j
@@ -326,7 +349,7 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
             uint32_t c[16];
 #pragma unroll
             for (int k = 0; k < 16; k++) c[k] = ((d[16 * j + k] >> (8 * i)) & 0xFFu) - mn[i];
-            long_put_sub(reinterpret_cast<uint16_t *>(pay + off[i] * nsub + s * 2u * len[i]), c, len[i]);
+            long_put_sub_swz(image, pay + off[i] * nsub + s * 2u * len[i], c, len[i]);
         }
     }
     if (tid < 64) {
@@ -423,15 +446,15 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
     if (tid < 4) {
         uint32_t cum = 0;
         for (int q = 0; q <= tid; q++) cum += s_unit[q];
-        reinterpret_cast<uint16_t *>(image)[tid] = (uint16_t)(cum >> 2);
+        *reinterpret_cast<uint16_t *>(image + long_swz(2u * (uint32_t)tid)) = (uint16_t)(cum >> 2);
     }
     uint32_t ustart = 8u;
     for (int q = 0; q < u; q++) ustart += s_unit[q];
     if (slot == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
-            reinterpret_cast<uint32_t *>(image + ustart)[q] = s_meta[u][q];
+            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[u][q];
     const uint32_t my_off = slot == 0 ? off4[0] : slot == 1 ? off4[1] : slot == 2 ? off4[2] : off4[3];
-    uint8_t *pay = image + ustart + meta + my_off * (uint32_t)NSUB;
+    const uint32_t pay = ustart + meta + my_off * (uint32_t)NSUB;      // byte offset of the lane's pack inside the block
     const uint32_t mn4 = mn * 0x01010101u;
 #pragma unroll
     for (int j = 0; j < NSUB; j++) {
@@ -441,7 +464,7 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
             const uint32_t w = pk[4 * j + q] - mn4;         // no byte borrows: every code is at least the minimum
             e[4 * q] = w & 0xFFu; e[4 * q + 1] = (w >> 8) & 0xFFu; e[4 * q + 2] = (w >> 16) & 0xFFu; e[4 * q + 3] = w >> 24;
         }
-        long_put_sub(reinterpret_cast<uint16_t *>(pay + (uint32_t)(NSUB - 1 - j) * 2u * len), e, len);   // tokens 16 j .. are sub-word NSUB - 1 - j
+        long_put_sub_swz(image, pay + (uint32_t)(NSUB - 1 - j) * 2u * len, e, len);     // tokens 16 j .. are sub-word NSUB - 1 - j
     }
     if (tid < 64) {
         const uint64_t o = lookback_offset(st, b, bytes, true);
@@ -843,7 +866,7 @@ static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint6
     if ((rc = tm.begin())) return rc;
     const int threads = 128 * long_chunks(P);
     // the block image in LDS: the block's bound and what the copy reads past the last byte
-    const uint32_t image_bytes = (uint32_t)pkv_block_bound_p(P, bits) + 32u;
+    const uint32_t image_bytes = ((uint32_t)pkv_block_bound_p(P, bits) + 32u + 127u) & ~127u;      // (whole 128-byte rows: the swizzle stays inside a row)
     if (is_k) {
         const int nt = P / long_chunks(P);                            // tokens of a pack per thread: 16, or 32 for P = 256
         const void *fn = nt == 32 ? reinterpret_cast<const void *>(pack_long_k_kernel<32>) : reinterpret_cast<const void *>(pack_long_k_kernel<16>);
