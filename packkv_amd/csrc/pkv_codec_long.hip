@@ -372,33 +372,36 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
 // channel (the lower half-wavefront belongs to the unit of channels 0..31, the upper to that of channels 32..63).  A
 // 16-token x 64-channel tile is one 16-byte load per lane (four lanes per 64-byte row piece) and goes through LDS
 // to turn rows into the lane's column; the lane keeps its P codes four to a register.
-template <int P>
-__global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
-                                                         uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
-                                                         int hidden_dim, int W, uint32_t nblocks) {
+template <int P, int NB>
+__global__ void __launch_bounds__(512 * NB) pack_long_v_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
+                                                              uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
+                                                              int hidden_dim, int W, uint32_t ntickets) {
+    // NB = 2: two adjacent blocks (consecutive in the stream as well) per workgroup and ticket, eight wavefronts each --
+    // together their rows are whole 128-byte lines, and the tickets, which retire one after the other, are half as many
     constexpr int NSUB = P / 16;
     constexpr int kRow = 80;                               // tile rows padded: 16-byte aligned, spread over the banks
     extern __shared__ __align__(16) uint8_t image[];
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
-    __shared__ uint32_t s_unit[4];
-    __shared__ uint32_t s_meta[4][kLongMetaWords];
-    __shared__ uint8_t s_len[8][64];
-    __shared__ __align__(16) uint8_t s_tile[8][16 * kRow];
-    const int tid = threadIdx.x, r = tid >> 6, c = tid & 63;
+    __shared__ uint32_t s_unit[NB][4];
+    __shared__ uint32_t s_meta[NB][4][kLongMetaWords];
+    __shared__ uint8_t s_len[NB][8][64];
+    __shared__ __align__(16) uint8_t s_tile[NB * 8][16 * kRow];
+    const int tid = threadIdx.x, bw = tid >> 9, r = (tid >> 6) & 7, c = tid & 63;
     const int seg = r >> 2, slot = r & 3, u = (c >> 5) * 2 + seg, t = c & 31;
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
-    if (tid < 4 * kLongMetaWords) (&s_meta[0][0])[tid] = 0u;
+    if (tid < NB * 4 * kLongMetaWords) (&s_meta[0][0][0])[tid] = 0u;
     __syncthreads();
-    const uint32_t b = s_idx;
-    if (b >= nblocks) return;
+    const uint32_t tk = s_idx;
+    if (tk >= ntickets) return;
+    const uint32_t b = tk * (uint32_t)NB + (uint32_t)bw;   // (the launcher pairs blocks only when every row of blocks is even)
     const int n_hid = hidden_dim / 64;
     const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
     // ---- the codes, minimum and width of the lane's pack ----
     const uint8_t *rows = codes + ((size_t)cb * (8 * P) + (size_t)r * P + (size_t)(c >> 2)) * hidden_dim + (size_t)hb * 64 + 16 * (c & 3);
-    uint8_t *mine = s_tile[r];
+    uint8_t *mine = s_tile[bw * 8 + r];
     uint32_t pk[P / 4];
     uint32_t lo = 255u, hi = 0u;
     // two tiles are requested ahead of the one being turned (named registers: an array here ends up in scratch memory)
@@ -429,32 +432,39 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
         t1 = t2;
     }
     const uint32_t mn = lo, len = (uint32_t)bit_length_u32(hi - lo);
-    s_len[r][c] = (uint8_t)len;
+    s_len[bw][r][c] = (uint8_t)len;
     __syncthreads();
     uint32_t len4[4], off4[4], payload;
 #pragma unroll
-    for (int i = 0; i < 4; i++) len4[i] = s_len[seg * 4 + i][c];
+    for (int i = 0; i < 4; i++) len4[i] = s_len[bw][seg * 4 + i][c];
     pack_offsets(len4, off4, payload);
     payload *= (uint32_t)NSUB;
-    if (slot == 0 && t == 0) s_unit[u] = meta + payload;
-    long_put_meta(s_meta[u], t, W, (mn & ((1u << W) - 1u)) << (slot * W));
-    long_put_meta(s_meta[u] + g.mins_bytes / 4, t, g.LB, len << (slot * g.LB));
+    if (slot == 0 && t == 0) s_unit[bw][u] = meta + payload;
+    long_put_meta(s_meta[bw][u], t, W, (mn & ((1u << W) - 1u)) << (slot * W));
+    long_put_meta(s_meta[bw][u] + g.mins_bytes / 4, t, g.LB, len << (slot * g.LB));
     __syncthreads();
-    const uint32_t bytes = 8u + s_unit[0] + s_unit[1] + s_unit[2] + s_unit[3];
-    if (tid == 0) lookback_publish(st, b, bytes);
-    // ---- the block in LDS: header, metadata, words ----
-    if (tid < 4) {
-        uint32_t cum = 0;
-        for (int q = 0; q <= tid; q++) cum += s_unit[q];
-        *reinterpret_cast<uint16_t *>(image + long_swz(2u * (uint32_t)tid)) = (uint16_t)(cum >> 2);
+    // the blocks lie one behind the other in the image, as in the stream
+    uint32_t blk_bytes[NB], bytes = 0, blk0 = 0;
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        blk_bytes[j] = 8u + s_unit[j][0] + s_unit[j][1] + s_unit[j][2] + s_unit[j][3];
+        if (j < bw) blk0 += blk_bytes[j];
+        bytes += blk_bytes[j];
     }
-    uint32_t ustart = 8u;
-    for (int q = 0; q < u; q++) ustart += s_unit[q];
+    if (tid == 0) lookback_publish(st, tk, bytes);
+    // ---- the blocks in LDS: header, metadata, words ----
+    if (r == 0 && c < 4) {
+        uint32_t cum = 0;
+        for (int q = 0; q <= c; q++) cum += s_unit[bw][q];
+        *reinterpret_cast<uint16_t *>(image + long_swz(blk0 + 2u * (uint32_t)c)) = (uint16_t)(cum >> 2);
+    }
+    uint32_t ustart = blk0 + 8u;
+    for (int q = 0; q < u; q++) ustart += s_unit[bw][q];
     if (slot == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
-            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[u][q];
+            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[bw][u][q];
     const uint32_t my_off = slot == 0 ? off4[0] : slot == 1 ? off4[1] : slot == 2 ? off4[2] : off4[3];
-    const uint32_t pay = ustart + meta + my_off * (uint32_t)NSUB;      // byte offset of the lane's pack inside the block
+    const uint32_t pay = ustart + meta + my_off * (uint32_t)NSUB;      // byte offset of the lane's pack inside the image
     const uint32_t mn4 = mn * 0x01010101u;
 #pragma unroll
     for (int j = 0; j < NSUB; j++) {
@@ -467,19 +477,24 @@ __global__ void __launch_bounds__(512) pack_long_v_kernel(const uint8_t *__restr
         long_put_sub_swz(image, pay + (uint32_t)(NSUB - 1 - j) * 2u * len, e, len);     // tokens 16 j .. are sub-word NSUB - 1 - j
     }
     if (tid < 64) {
-        const uint64_t o = lookback_offset(st, b, bytes, true);
+        const uint64_t o = lookback_offset(st, tk, bytes, true);
         if (tid == 0) {
             s_off = o;
-            info[2 * (size_t)b] = (uint32_t)o;
-            info[2 * (size_t)b + 1] = bytes;
-            if (b == nblocks - 1) st->total = o + bytes;
+            uint32_t run = 0;
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                info[2 * (size_t)(tk * NB + j)] = (uint32_t)(o + run);
+                info[2 * (size_t)(tk * NB + j) + 1] = blk_bytes[j];
+                run += blk_bytes[j];
+            }
+            if (tk == ntickets - 1) st->total = o + bytes;
             if (o + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
         }
     }
     __syncthreads();
     const uint64_t o = s_off;
     if (o + bytes > capacity) return;
-    long_copy_out(stream + o, image, bytes, tid, 512);
+    long_copy_out(stream + o, image, bytes, tid, 512 * NB);
 }
 
 __global__ void __launch_bounds__(1024) unpack_long_v_plain_kernel(const uint8_t *__restrict__ stream, const uint32_t *__restrict__ info,
@@ -874,11 +889,23 @@ static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint6
         if (nt == 32) pack_long_k_kernel<32><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
         else pack_long_k_kernel<16><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
     } else if ((reinterpret_cast<uintptr_t>(codes) & 15u) == 0) {
+        // two adjacent blocks per workgroup for packs of 32 and 64 tokens when every row of blocks is even (512 MiB of
+        // 4-bit codes: 0.42 -> 0.32 ms and 0.27 -> 0.23 ms; longer packs lose by it -- 0.23 -> 0.26 ms at 128 tokens,
+        // 0.27 -> 0.29 ms at 256 -- because two images leave one workgroup per CU)
+        const bool pair = hidden_dim % 128 == 0 && P <= 64;
+        const uint32_t lds_v = pair ? 2u * image_bytes : image_bytes;
 #define PKV_LAUNCH_LONG_V(PP)                                                                                                  \
     do {                                                                                                                       \
-        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pack_long_v_kernel<PP>),                               \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)image_bytes));                       \
-        pack_long_v_kernel<PP><<<nblocks, 512, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, bits, nblocks); \
+        if (pair) {                                                                                                            \
+            PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pack_long_v_kernel<PP, 2>),                        \
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_v));                         \
+            pack_long_v_kernel<PP, 2><<<nblocks / 2, 1024, lds_v, s>>>(codes, stream, capacity, info, st, hidden_dim, bits,      \
+                                                                       nblocks / 2);                                           \
+        } else {                                                                                                               \
+            PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pack_long_v_kernel<PP, 1>),                        \
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_v));                         \
+            pack_long_v_kernel<PP, 1><<<nblocks, 512, lds_v, s>>>(codes, stream, capacity, info, st, hidden_dim, bits, nblocks); \
+        }                                                                                                                      \
     } while (0)
         if (P == 32) PKV_LAUNCH_LONG_V(32);
         else if (P == 64) PKV_LAUNCH_LONG_V(64);

@@ -240,7 +240,9 @@ def test_long_packs_bit_exact_vs_oracle(cuda, oracle_codec, is_k, P):
     ctx_blk, hid_blk = ops.long_block_shape(is_k, P)
     for W in (2, 3, 4, 5, 6, 7, 8):
         for kind in ("uniform", "const", "narrow", "gauss"):
-            T, H = ctx_blk * (3 if P <= 64 else 2), hid_blk * 5
+            # five blocks to a row: V rows of 320 channels (one block per workgroup, plain decoder); six: whole 128-byte
+            # lines (two V blocks per workgroup in the encoder, the staged decoder)
+            T, H = ctx_blk * (3 if P <= 64 else 2), hid_blk * (5 if kind in ("uniform", "narrow") else 6)
             _say("long-pack case", "K" if is_k else "V", "pack", P, "bits", W, kind, (T, H))
             c = _rand_codes(rng, T, H, W, kind)
             so, io, zo = codec.long_encode(is_k, c, P, W)
