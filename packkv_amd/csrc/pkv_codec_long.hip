@@ -251,29 +251,33 @@ __device__ __forceinline__ void long_copy_out(uint8_t *dst, const uint8_t *image
 
 // K: the thread layout of pack_long_kernel (half-wavefront per unit, lane <-> 4 channels, times the chunks of a
 // pack); a thread holds the NT = P / chunks tokens of its chunk as one dword (four channels) per token.
-template <int NT>
+template <int NT, int NB>
 __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                           uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
-                                                          int hidden_dim, int P, int W, uint32_t nblocks) {
+                                                          int hidden_dim, int P, int W, uint32_t ntickets) {
     extern __shared__ __align__(16) uint8_t image[];       // the block as it will lie in the stream (+ 32 bytes of slack)
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
-    __shared__ uint32_t s_unit[4];
-    __shared__ uint32_t s_meta[4][kLongMetaWords];
+    __shared__ uint32_t s_unit[NB][4];
+    __shared__ uint32_t s_meta[NB][4][kLongMetaWords];
     __shared__ uint4 s_mm[kLongMaxChunks][128];            // minima and maxima of a thread's four packs over its chunk
-    const int tid = threadIdx.x, u = (tid >> 5) & 3, t = tid & 31;
-    const int chunk = tid >> 7, nch = (int)blockDim.x >> 7;
+    // NB consecutive blocks per workgroup and ticket (short packs: a block is small and the tickets, which retire
+    // one after the other, would set the pace): block bw is served by threads [bw, bw + 1) * blockDim / NB
+    const int tid = threadIdx.x, nthr = (int)blockDim.x / NB, bw = tid / nthr, ltid = tid % nthr;
+    const int u = (ltid >> 5) & 3, t = ltid & 31;
+    const int chunk = ltid >> 7, nch = nthr >> 7;
     const uint32_t nsub = (uint32_t)P / 16u;
     const uint32_t s1 = nsub * (uint32_t)(chunk + 1) / (uint32_t)nch;     // its sub-words end here; NT / 16 of them
     const int k0 = P - 16 * (int)s1;                                     // ... and hold tokens k0 .. k0 + NT - 1 of the pack
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     if (chunk == 0) {
-        s_meta[u][t] = 0u;
-        if (t < kLongMetaWords - 32) s_meta[u][32 + t] = 0u;
+        s_meta[bw][u][t] = 0u;
+        if (t < kLongMetaWords - 32) s_meta[bw][u][32 + t] = 0u;
     }
     __syncthreads();
-    const uint32_t b = s_idx;
-    if (b >= nblocks) return;
+    const uint32_t tk = s_idx;
+    if (tk >= ntickets) return;
+    const uint32_t b = tk * (uint32_t)NB + (uint32_t)bw;     // (the launcher sees to NB dividing the number of blocks)
     const int n_hid = hidden_dim / 128;
     const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
     const uint8_t *tile = codes + (size_t)cb * (4 * P) * hidden_dim + (size_t)hb * 128;
@@ -294,11 +298,11 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
         bmn2 = __builtin_elementwise_min(bmn2, c);
         bmx2 = __builtin_elementwise_max(bmx2, c);
     }
-    s_mm[chunk][tid & 127] = make_uint4(__builtin_bit_cast(uint32_t, amn2), __builtin_bit_cast(uint32_t, amx2),
+    s_mm[bw * nch + chunk][ltid & 127] = make_uint4(__builtin_bit_cast(uint32_t, amn2), __builtin_bit_cast(uint32_t, amx2),
                                         __builtin_bit_cast(uint32_t, bmn2), __builtin_bit_cast(uint32_t, bmx2));
     __syncthreads();
     for (int c = 0; c < nch; c++) {
-        const uint4 o = s_mm[c][tid & 127];
+        const uint4 o = s_mm[bw * nch + c][ltid & 127];
         amn2 = __builtin_elementwise_min(amn2, __builtin_bit_cast(u16x2, o.x));
         amx2 = __builtin_elementwise_max(amx2, __builtin_bit_cast(u16x2, o.y));
         bmn2 = __builtin_elementwise_min(bmn2, __builtin_bit_cast(u16x2, o.z));
@@ -315,7 +319,7 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
     uint32_t off[4], payload;
     pack_offsets(len, off, payload);
     payload *= nsub;
-    if (t == 0 && chunk == 0) s_unit[u] = meta + payload;
+    if (t == 0 && chunk == 0) s_unit[bw][u] = meta + payload;
     if (chunk == 0) {
         uint32_t minsw = 0, lensw = 0;
 #pragma unroll
@@ -323,23 +327,30 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
             minsw |= (mn[i] & ((1u << W) - 1u)) << (i * W);
             lensw |= len[i] << (i * g.LB);
         }
-        long_put_meta(s_meta[u], t, W, minsw);
-        long_put_meta(s_meta[u] + g.mins_bytes / 4, t, g.LB, lensw);
+        long_put_meta(s_meta[bw][u], t, W, minsw);
+        long_put_meta(s_meta[bw][u] + g.mins_bytes / 4, t, g.LB, lensw);
     }
     __syncthreads();
-    const uint32_t bytes = 8u + s_unit[0] + s_unit[1] + s_unit[2] + s_unit[3];
-    if (tid == 0) lookback_publish(st, b, bytes);
-    // ---- the block in LDS: header, metadata, words ----
-    if (tid < 4) {
-        uint32_t cum = 0;
-        for (int q = 0; q <= tid; q++) cum += s_unit[q];
-        *reinterpret_cast<uint16_t *>(image + long_swz(2u * (uint32_t)tid)) = (uint16_t)(cum >> 2);
+    // the blocks lie one behind the other in the image, as in the stream
+    uint32_t blk_bytes[NB], bytes = 0, blk0 = 0;
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        blk_bytes[j] = 8u + s_unit[j][0] + s_unit[j][1] + s_unit[j][2] + s_unit[j][3];
+        if (j < bw) blk0 += blk_bytes[j];
+        bytes += blk_bytes[j];
     }
-    uint32_t ustart = 8u;
-    for (int q = 0; q < u; q++) ustart += s_unit[q];
+    if (tid == 0) lookback_publish(st, tk, bytes);
+    // ---- the block in LDS: header, metadata, words ----
+    if (ltid < 4) {
+        uint32_t cum = 0;
+        for (int q = 0; q <= ltid; q++) cum += s_unit[bw][q];
+        *reinterpret_cast<uint16_t *>(image + long_swz(blk0 + 2u * (uint32_t)ltid)) = (uint16_t)(cum >> 2);
+    }
+    uint32_t ustart = blk0 + 8u;
+    for (int q = 0; q < u; q++) ustart += s_unit[bw][q];
     if (chunk == 0)
         for (uint32_t q = (uint32_t)t; q < meta / 4u; q += 32u)
-            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[u][q];
+            *reinterpret_cast<uint32_t *>(image + long_swz(ustart + 4u * q)) = s_meta[bw][u][q];
     const uint32_t pay = ustart + meta;                   // byte offset of the unit's payload inside the block
 #pragma unroll
     for (int j = 0; j < NT / 16; j++) {
@@ -353,12 +364,17 @@ __global__ void __launch_bounds__(1024) pack_long_k_kernel(const uint8_t *__rest
         }
     }
     if (tid < 64) {
-        const uint64_t o = lookback_offset(st, b, bytes, true);
+        const uint64_t o = lookback_offset(st, tk, bytes, true);
         if (tid == 0) {
             s_off = o;
-            info[2 * (size_t)b] = (uint32_t)o;
-            info[2 * (size_t)b + 1] = bytes;
-            if (b == nblocks - 1) st->total = o + bytes;
+            uint32_t run = 0;
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                info[2 * (size_t)(tk * NB + j)] = (uint32_t)(o + run);
+                info[2 * (size_t)(tk * NB + j) + 1] = blk_bytes[j];
+                run += blk_bytes[j];
+            }
+            if (tk == ntickets - 1) st->total = o + bytes;
             if (o + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
         }
     }
@@ -883,11 +899,23 @@ static int run_pack_long(bool is_k, const uint8_t *codes, uint8_t *stream, uint6
     // the block image in LDS: the block's bound and what the copy reads past the last byte
     const uint32_t image_bytes = ((uint32_t)pkv_block_bound_p(P, bits) + 32u + 127u) & ~127u;      // (whole 128-byte rows: the swizzle stays inside a row)
     if (is_k) {
-        const int nt = P / long_chunks(P);                            // tokens of a pack per thread: 16, or 32 for P = 256
-        const void *fn = nt == 32 ? reinterpret_cast<const void *>(pack_long_k_kernel<32>) : reinterpret_cast<const void *>(pack_long_k_kernel<16>);
-        PKV_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)image_bytes));
-        if (nt == 32) pack_long_k_kernel<32><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
-        else pack_long_k_kernel<16><<<nblocks, threads, image_bytes, s>>>(codes, stream, capacity, info, st, hidden_dim, P, bits, nblocks);
+        // packs of 32 tokens: four consecutive blocks per workgroup (1024 threads) while the number of blocks allows --
+        // 0.41 -> 0.28 ms per 512 MiB; at 64 tokens two blocks per workgroup lose, 0.25 -> 0.28 ms.  NT = tokens of a
+        // pack per thread: 16, or 32 for packs of 256
+        const int nb = P != 32 ? 1 : nblocks % 4 == 0 ? 4 : nblocks % 2 == 0 ? 2 : 1;
+        const uint32_t lds_k = (uint32_t)nb * (((uint32_t)pkv_block_bound_p(P, bits) + 127u) & ~127u) + 128u;
+#define PKV_LAUNCH_LONG_K(NT_, NB_)                                                                                            \
+    do {                                                                                                                       \
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pack_long_k_kernel<NT_, NB_>),                          \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_k));                             \
+        pack_long_k_kernel<NT_, NB_><<<nblocks / NB_, threads * NB_, lds_k, s>>>(codes, stream, capacity, info, st, hidden_dim, \
+                                                                                P, bits, nblocks / NB_);                        \
+    } while (0)
+        if (P == 256) PKV_LAUNCH_LONG_K(32, 1);
+        else if (nb == 4) PKV_LAUNCH_LONG_K(16, 4);
+        else if (nb == 2) PKV_LAUNCH_LONG_K(16, 2);
+        else PKV_LAUNCH_LONG_K(16, 1);
+#undef PKV_LAUNCH_LONG_K
     } else if ((reinterpret_cast<uintptr_t>(codes) & 15u) == 0) {
         // two adjacent blocks per workgroup for packs of 32 and 64 tokens when every row of blocks is even (512 MiB of
         // 4-bit codes: 0.42 -> 0.32 ms and 0.27 -> 0.23 ms; longer packs lose by it -- 0.23 -> 0.26 ms at 128 tokens,
