@@ -242,7 +242,10 @@ def test_long_packs_bit_exact_vs_oracle(cuda, oracle_codec, is_k, P):
         for kind in ("uniform", "const", "narrow", "gauss"):
             # five blocks to a row: V rows of 320 channels (one block per workgroup, plain decoder); six: whole 128-byte
             # lines (two V blocks per workgroup in the encoder, the staged decoder)
-            T, H = ctx_blk * (3 if P <= 64 else 2), hid_blk * (5 if kind in ("uniform", "narrow") else 6)
+            # (packs of 32 tokens, K: 20 or 24 blocks at even widths -- four to a workgroup -- and 15 or 18 at odd widths,
+            # one or two to a workgroup)
+            rows_of_blocks = (4 if W % 2 == 0 else 3) if P == 32 else 3 if P == 64 else 2
+            T, H = ctx_blk * rows_of_blocks, hid_blk * (5 if kind in ("uniform", "narrow") else 6)
             _say("long-pack case", "K" if is_k else "V", "pack", P, "bits", W, kind, (T, H))
             c = _rand_codes(rng, T, H, W, kind)
             so, io, zo = codec.long_encode(is_k, c, P, W)
