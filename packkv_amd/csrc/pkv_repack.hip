@@ -10,6 +10,10 @@
 // of equal medians to the backend.  Here ties keep their original order (a stable descending sort).
 #include "pkv_common.hpp"
 #include "pkv_runtime.hpp"
+#include "pkv_block.hpp"
+
+#include <map>
+#include <mutex>
 
 namespace pkv {
 
@@ -307,6 +311,324 @@ __global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint
     }
 }
 
+// ---- greedy order of blocks of up to 64 tokens: the block's rows stay in registers, sliced by channel ----
+// A workgroup of 256 threads holds 2048 channels of all the tokens of a block (thread = 8 adjacent channels, one
+// dword pair per token, in registers for the whole block), so a pick re-reads nothing from memory.  The
+// ceil(2 * hidden / 2048) workgroups that cover a block form a group: every step (a seed or a pick) each member
+// sums its slice per token, publishes the partial sums as (step number << 32 | value) words, reads the words of
+// all members and finds the winner for itself; the words of two consecutive steps live in two buffers, and a member
+// can be at most one step ahead of another, so a word is never overwritten before it was read.  Workgroups take
+// tickets in the order they start and a group is a run of consecutive tickets: whenever a member waits, the members
+// it waits for run already or start as soon as a complete group ahead of them leaves; the launch never holds more
+// groups than fit the device.  The waits are bounded all the same (kGreedySpinLimit, error word of the state).
+//
+// The remaining tokens occupy register slots 0 .. n_alive - 1 (the winner's slot takes the rows of the last slot;
+// lane l of every wavefront knows which token slot l holds), so a step walks a prefix of the slots without a test
+// per token and two tokens are priced side by side.
+//
+// Pricing a token: min and max as packed 16-bit lanes, r = max - min, then bit_length(r) is the exponent of
+// (2 r + 1) 2^-10 as a half: one packed fma on r read as a subnormal half (r 2^-24 * 2^15 + 2^-10, exact), the
+// exponent fields masked and added by a sum of absolute differences -- 3.5 vector instructions per channel.  The
+// constant bias of the exponent (5 per channel) is common to all tokens.
+constexpr int kSlicedThreads = 256;
+constexpr int kSlicedChannels = 8 * kSlicedThreads;      // per workgroup
+constexpr int kSlicedTokens = 64;
+constexpr int kGreedySpinLimit = 1 << 22;
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// Even / odd bytes of a dword as 16-bit lanes, with the mask and the byte selector as operands: the kernel below
+// makes these two constants opaque once per step, so that nothing derived from the packed rows -- which stay in
+// registers for a whole block -- is kept in registers of its own from step to step.
+__device__ __forceinline__ uint32_t even_bytes(uint32_t x, uint32_t mask_00ff00ff) { return x & mask_00ff00ff; }
+__device__ __forceinline__ uint32_t odd_bytes(uint32_t x, uint32_t sel_0c030c01) { return __builtin_amdgcn_perm(0u, x, sel_0c030c01); }
+
+// exponent fields (<< 10, both halves) of (2 r + 1) 2^-10, r = max(x, mx) - min(x, mn) per 16-bit lane
+__device__ __forceinline__ uint32_t range_exponents(uint32_t x, uint32_t mn, uint32_t mx) {
+    const ushort2v r = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, x), __builtin_bit_cast(ushort2v, mx)) -
+                       __builtin_elementwise_min(__builtin_bit_cast(ushort2v, x), __builtin_bit_cast(ushort2v, mn));
+    const half2v f = __builtin_elementwise_fma(__builtin_bit_cast(half2v, r), (half2v){(_Float16)32768.0f, (_Float16)32768.0f},
+                                               (half2v){(_Float16)0.0009765625f, (_Float16)0.0009765625f});
+    return __builtin_bit_cast(uint32_t, f) & 0x7C007C00u;
+}
+// sum over the 8 channels of a dword pair of the exponent fields, << 10
+__device__ __forceinline__ uint32_t price8(uint32_t x0, uint32_t x1, const uint32_t (&mn)[4], const uint32_t (&mx)[4],
+                                           uint32_t k_even, uint32_t k_odd) {
+    uint32_t a = __builtin_amdgcn_sad_u16(range_exponents(even_bytes(x0, k_even), mn[0], mx[0]), 0u, 0u);
+    a = __builtin_amdgcn_sad_u16(range_exponents(odd_bytes(x0, k_odd), mn[1], mx[1]), 0u, a);
+    a = __builtin_amdgcn_sad_u16(range_exponents(even_bytes(x1, k_even), mn[2], mx[2]), 0u, a);
+    return __builtin_amdgcn_sad_u16(range_exponents(odd_bytes(x1, k_odd), mn[3], mx[3]), 0u, a);
+}
+
+// data-parallel-primitive moves between the lanes of a row of 16 (0x100 | n: from lane + n, 0x110 | n: from lane - n,
+// 0x142 / 0x143: lane 15 / 31 to the following rows, below 0x100: a permutation of every four lanes)
+template <int CTRL, int ROW_MASK, bool ZERO_FILL>
+__device__ __forceinline__ uint32_t lane_move(uint32_t old, uint32_t src) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, ROW_MASK, 0xF, ZERO_FILL);
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {      // the minimum over the wavefront, uniform
+    v = min(v, lane_move<0x111, 0xF, false>(0xFFFFFFFFu, v));
+    v = min(v, lane_move<0x112, 0xF, false>(0xFFFFFFFFu, v));
+    v = min(v, lane_move<0x114, 0xF, false>(0xFFFFFFFFu, v));
+    v = min(v, lane_move<0x118, 0xF, false>(0xFFFFFFFFu, v));
+    v = min(v, lane_move<0x142, 0xA, false>(0xFFFFFFFFu, v));
+    v = min(v, lane_move<0x143, 0xC, false>(0xFFFFFFFFu, v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ __forceinline__ uint32_t quad_sum(uint32_t v) {          // every lane: the sum over its four lanes
+    v += lane_move<0xB1, 0xF, false>(0u, v);
+    return v + lane_move<0x4E, 0xF, false>(0u, v);
+}
+__device__ __forceinline__ uint32_t sum8_down(uint32_t v) {         // lanes 0, 8, ..: the sum over lanes l .. l + 7
+    v += lane_move<0x101, 0xF, true>(0u, v);
+    v += lane_move<0x102, 0xF, true>(0u, v);
+    return v + lane_move<0x104, 0xF, true>(0u, v);
+}
+
+// one statement per register slot: switches over these cases keep every index of the register arrays a constant
+#define PKV_SLOTS16(M, b) M(b + 0) M(b + 1) M(b + 2) M(b + 3) M(b + 4) M(b + 5) M(b + 6) M(b + 7) M(b + 8) M(b + 9) M(b + 10) \
+    M(b + 11) M(b + 12) M(b + 13) M(b + 14) M(b + 15)
+#define PKV_SLOTS64(M) PKV_SLOTS16(M, 0) PKV_SLOTS16(M, 16) PKV_SLOTS16(M, 32) PKV_SLOTS16(M, 48)
+
+// Sum over the members first, first + stride, .. of word `idx` of their 128 published words, four loads in flight.
+__device__ __forceinline__ unsigned long long gather_words(const uint64_t *words, uint32_t idx, uint32_t first, uint32_t stride,
+                                                           uint32_t members, uint32_t seq, ScanState *st) {
+    unsigned long long sum = 0ull;
+    for (uint32_t m0 = first; m0 < members; m0 += 4 * stride) {
+        const uint64_t *p = words + (size_t)m0 * 128 + idx;
+        uint64_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            w[i] = m0 + i * stride < members ? __hip_atomic_load(p + (size_t)i * stride * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                             : (uint64_t)seq << 32;
+        int spins = 0;
+        while (((uint32_t)(w[0] >> 32) != seq || (uint32_t)(w[1] >> 32) != seq || (uint32_t)(w[2] >> 32) != seq ||
+                (uint32_t)(w[3] >> 32) != seq) && spins < kGreedySpinLimit) {
+            __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if ((uint32_t)(w[i] >> 32) != seq)
+                    w[i] = __hip_atomic_load(p + (size_t)i * stride * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            spins++;
+        }
+        if (spins >= kGreedySpinLimit) st->error = (uint32_t)PKV_ERR_INTERNAL;
+        sum += (unsigned long long)(uint32_t)w[0] + (uint32_t)w[1] + (uint32_t)w[2] + (uint32_t)w[3];
+    }
+    return sum;
+}
+
+__global__ void __launch_bounds__(kSlicedThreads, 2)
+greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *__restrict__ v_codes, int hidden, int N,
+                           int pack_len, uint32_t nblocks, uint32_t members, uint32_t groups,
+                           uint32_t *__restrict__ perm, ScanState *st) {
+    __shared__ uint32_t s_acc[2][32 * 32];           // picks: [buffer][pair of slots][adder]
+    __shared__ uint32_t s_seed[128 * 32];            // seeds: [2 * slot + (0: dot, 1: squared norm)][adder]
+    __shared__ uint32_t s_tot[4][64];                // picks: sums over a quarter of the members
+    __shared__ unsigned long long s_tot64[2][128];   // seeds: sums over half of the members
+    __shared__ uint32_t s_ticket;
+    const int tid = threadIdx.x, lane = tid & 63;
+    if (tid == 0) s_ticket = atomicAdd(&st->ticket, 1u);
+    for (int i = tid; i < 2 * 32 * 32; i += kSlicedThreads) (&s_acc[0][0])[i] = 0u;
+    __syncthreads();
+    const uint32_t ticket = s_ticket;
+    const uint32_t grp = ticket / members, mem = ticket - grp * members;
+    if (grp >= groups) return;
+    uint64_t *xw = st->status + (size_t)grp * 2 * members * 128;      // [buffer][member][128]
+    const int D2 = 2 * hidden;
+    const int ch = ((int)mem * kSlicedThreads + tid) * 8;             // first of the thread's 8 channels
+    const uint8_t *col = ch < hidden ? k_codes + ch : v_codes + (ch - hidden);
+    const bool have = ch < D2;
+    const int adder = (tid >> 2) & 31;               // the LDS word that takes the sums of the thread's four lanes
+    const bool quad_first = (tid & 3) == 0;
+    uint32_t seq = 0;
+    int flip = 0, ab = 0;
+
+    for (uint32_t blk = grp; blk < nblocks; blk += groups) {
+        const size_t row0 = (size_t)blk * N;
+        uint32_t x0[kSlicedTokens], x1[kSlicedTokens];
+#pragma unroll
+        for (int t = 0; t < kSlicedTokens; t++) {
+            uint2 v = make_uint2(0u, 0u);
+            if (t < N && have) v = *reinterpret_cast<const uint2 *>(col + (row0 + t) * (size_t)hidden);
+            x0[t] = v.x;
+            x1[t] = v.y;
+        }
+        uint32_t orig = (uint32_t)lane;          // the token in slot `lane`
+        int n_alive = N, picked = 0;
+        uint32_t mn[4], mx[4];       // even / odd bytes of dword 0, even / odd bytes of dword 1, as 16-bit lanes
+
+        for (int step = 0; step < N / pack_len * pack_len; step++) {
+            const bool seed = step % pack_len == 0;
+            int sel = -1;
+            uint32_t k_even = 0x00FF00FFu, k_odd = 0x0C030C01u, k_zero = 0u;     // opaque from here on: see even_bytes
+            asm volatile("" : "+s"(k_even), "+s"(k_odd), "+v"(k_zero));
+            if (seed) {
+            // ---- seed: rounded mean of the remaining tokens, then the best cosine ----
+            uint32_t sum[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int t8 = 0; t8 < kSlicedTokens; t8 += 8) {
+                if (t8 < n_alive) {
+#pragma unroll
+                    for (int t = t8; t < t8 + 8; t++)
+                        if (t < n_alive) {
+                            sum[0] += even_bytes(x0[t], k_even); sum[1] += odd_bytes(x0[t], k_odd);
+                            sum[2] += even_bytes(x1[t], k_even); sum[3] += odd_bytes(x1[t], k_odd);
+                        }
+                }
+            }
+            uint32_t mean[2];
+#pragma unroll
+            for (int d = 0; d < 2; d++) {      // mean(dim=1).round(): fp32 quotient, round half to even
+                const float na = (float)n_alive;
+                const uint32_t e_lo = (uint32_t)rintf((float)(sum[2 * d] & 0xFFFFu) / na), e_hi = (uint32_t)rintf((float)(sum[2 * d] >> 16) / na);
+                const uint32_t o_lo = (uint32_t)rintf((float)(sum[2 * d + 1] & 0xFFFFu) / na), o_hi = (uint32_t)rintf((float)(sum[2 * d + 1] >> 16) / na);
+                mean[d] = e_lo | (o_lo << 8) | (e_hi << 16) | (o_hi << 24);
+            }
+            for (int i = tid; i < 128 * 32; i += kSlicedThreads) s_seed[i] = 0u;
+            __syncthreads();
+#pragma unroll
+            for (int t8 = 0; t8 < kSlicedTokens; t8 += 8) {
+                if (t8 < n_alive) {
+#pragma unroll
+                    for (int t = t8; t < t8 + 8; t++)
+                        if (t < n_alive) {
+                            const uint32_t dot = quad_sum(__builtin_amdgcn_udot4(x0[t], mean[0], __builtin_amdgcn_udot4(x1[t], mean[1], 0u, false), false));
+                            const uint32_t nx = quad_sum(__builtin_amdgcn_udot4(x0[t], x0[t], __builtin_amdgcn_udot4(x1[t], x1[t], k_zero, false), false));
+                            if (quad_first) {
+                                atomicAdd(&s_seed[(2 * t) * 32 + adder], dot);
+                                atomicAdd(&s_seed[(2 * t + 1) * 32 + adder], nx);
+                            }
+                        }
+                }
+            }
+            __syncthreads();
+            seq++;
+            {   // value v = tid >> 1: two threads add 16 adders each
+                const int v = tid >> 1, part = tid & 1;
+                uint32_t a = 0u;
+#pragma unroll
+                for (int i = 0; i < 16; i++) a += s_seed[v * 32 + part * 16 + i];
+                a += lane_move<0xB1, 0xF, false>(0u, a);
+                if (part == 0 && v < 2 * n_alive) {
+                    if (members > 1)
+                        __hip_atomic_store(xw + ((size_t)flip * members + mem) * 128 + v, ((uint64_t)seq << 32) | a,
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else
+                        s_tot64[0][v] = a;
+                }
+            }
+            if (members > 1) {
+                const int v = tid & 127, q = tid >> 7;
+                s_tot64[q][v] = v < 2 * n_alive ? gather_words(xw + (size_t)flip * members * 128, (uint32_t)v, (uint32_t)q, 2u, members, seq, st) : 0ull;
+                flip ^= 1;
+            }
+            __syncthreads();
+            {
+                unsigned long long bd = 0, bn = 0;
+                uint32_t bo = orig;
+                if (lane < n_alive) {
+                    sel = lane;
+                    bd = s_tot64[0][2 * lane];
+                    bn = s_tot64[0][2 * lane + 1];
+                    if (members > 1) { bd += s_tot64[1][2 * lane]; bn += s_tot64[1][2 * lane + 1]; }
+                }
+#pragma unroll
+                for (int d = 32; d >= 1; d >>= 1) {      // equal cosines: the earlier token
+                    const int os = __shfl_xor(sel, d, 64);
+                    const uint32_t oo = __shfl_xor(bo, d, 64);
+                    const unsigned long long od = __shfl_xor(bd, d, 64), on = __shfl_xor(bn, d, 64);
+                    if (os >= 0 && (sel < 0 || cos_greater(od, on, bd, bn) || (!cos_greater(bd, bn, od, on) && oo < bo))) {
+                        sel = os; bo = oo; bd = od; bn = on;
+                    }
+                }
+                sel = __builtin_amdgcn_readfirstlane(sel);
+            }
+            } else {
+            // ---- the pack's other tokens: fewest bits after the pick ----
+                uint32_t *acc = s_acc[ab];
+#pragma unroll
+                for (int k4 = 0; k4 < kSlicedTokens / 2; k4 += 4) {
+                    if (2 * k4 < n_alive) {
+#pragma unroll
+                        for (int k = k4; k < k4 + 4; k++)
+                            if (2 * k < n_alive) {
+                                // (with an odd count the slot past the last one is priced as well: a bounded sum nobody reads)
+                                const uint32_t a0 = price8(x0[2 * k], x1[2 * k], mn, mx, k_even, k_odd), a1 = price8(x0[2 * k + 1], x1[2 * k + 1], mn, mx, k_even, k_odd);
+                                const uint32_t c = quad_sum((a0 >> 10) | (a1 << 6));      // sums of fields at bit 10: a 16-bit lane per slot
+                                if (quad_first) atomicAdd(&acc[k * 32 + adder], c);
+                            }
+                    }
+                }
+                __syncthreads();
+                seq++;
+                {   // pair k = tid >> 3: eight threads add 4 adders each; then the other buffer is cleared for the next pick
+                    const int k = tid >> 3, part = tid & 7;
+                    const uint32_t a = sum8_down(acc[k * 32 + part * 4] + acc[k * 32 + part * 4 + 1] + acc[k * 32 + part * 4 + 2] +
+                                                 acc[k * 32 + part * 4 + 3]);
+                    if (part == 0 && 2 * k < n_alive) {
+                        if (members > 1) {
+                            uint64_t *dst = xw + ((size_t)flip * members + mem) * 128 + 2 * k;
+                            __hip_atomic_store(dst, ((uint64_t)seq << 32) | (a & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            __hip_atomic_store(dst + 1, ((uint64_t)seq << 32) | (a >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        } else {
+                            s_tot[0][2 * k] = a & 0xFFFFu;
+                            s_tot[0][2 * k + 1] = a >> 16;
+                        }
+                    }
+                    ab ^= 1;
+                    uint32_t *other = s_acc[ab];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) other[tid * 4 + i] = 0u;
+                }
+                if (members > 1) {
+                    const int q = tid >> 6;
+                    s_tot[q][lane] = lane < n_alive ? (uint32_t)gather_words(xw + (size_t)flip * members * 128, (uint32_t)lane, (uint32_t)q, 4u, members, seq, st) : 0u;
+                    flip ^= 1;
+                }
+                __syncthreads();
+                uint32_t key = 0xFFFFFFFFu;            // (cost, token) in one word: the minimum is the first cheapest token
+                if (lane < n_alive) {
+                    uint32_t a = s_tot[0][lane];
+                    if (members > 1) a += s_tot[1][lane] + s_tot[2][lane] + s_tot[3][lane];
+                    key = (a << 8) | orig;
+                }
+                const uint32_t best = wave_min_u32(key);
+                sel = (int)__builtin_ctzll(__ballot(key == best));
+            }
+            // the winner in slot `sel` leaves: its rows widen the pack's ranges and the last slot moves into `sel`
+            const int last = n_alive - 1;
+            const uint32_t tok = (uint32_t)__builtin_amdgcn_readlane((int)orig, sel);
+            const uint32_t moved = (uint32_t)__builtin_amdgcn_readlane((int)orig, last);
+            if (lane == sel) orig = moved;
+            uint32_t l0 = 0u, l1 = 0u, w0 = 0u, w1 = 0u;
+            switch (last) {
+#define PKV_SLOT_READ(t) case t: l0 = x0[t]; l1 = x1[t]; break;
+                PKV_SLOTS64(PKV_SLOT_READ)
+#undef PKV_SLOT_READ
+            }
+            switch (sel) {
+            // (the rows are replaced where they are: left to the compiler, the 64 cases become chains of register copies)
+#define PKV_SLOT_SWAP(t) case t: w0 = x0[t]; w1 = x1[t]; \
+    asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "+v"(x0[t]), "+v"(x1[t]) : "v"(l0), "v"(l1)); break;
+                PKV_SLOTS64(PKV_SLOT_SWAP)
+#undef PKV_SLOT_SWAP
+            }
+            if (mem == 0 && tid == 0) perm[row0 + picked] = tok;
+            picked++;
+            n_alive--;
+            if (seed) {
+                mn[0] = mx[0] = even_bytes(w0, k_even); mn[1] = mx[1] = odd_bytes(w0, k_odd);
+                mn[2] = mx[2] = even_bytes(w1, k_even); mn[3] = mx[3] = odd_bytes(w1, k_odd);
+            } else {
+                mn[0] = pk_min_u16(mn[0], even_bytes(w0, k_even)); mx[0] = pk_max_u16(mx[0], even_bytes(w0, k_even));
+                mn[1] = pk_min_u16(mn[1], odd_bytes(w0, k_odd)); mx[1] = pk_max_u16(mx[1], odd_bytes(w0, k_odd));
+                mn[2] = pk_min_u16(mn[2], even_bytes(w1, k_even)); mx[2] = pk_max_u16(mx[2], even_bytes(w1, k_even));
+                mn[3] = pk_min_u16(mn[3], odd_bytes(w1, k_odd)); mx[3] = pk_max_u16(mx[3], odd_bytes(w1, k_odd));
+            }
+        }
+    }
+}
+
 // ---- out row r = in row perm[r], for K and V at once: grid (ctx_len), 256 threads ----
 __global__ void __launch_bounds__(256) gather_rows_kernel(const uint8_t *__restrict__ k_in, const uint8_t *__restrict__ v_in,
                                                           uint8_t *__restrict__ k_out, uint8_t *__restrict__ v_out,
@@ -473,18 +795,55 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
                 "ctx_len must be divisible by a block size of at most 256 tokens");
     PKV_REQUIRE(block_size % pack_len == 0, PKV_ERR_INVALID,
                 "block_size must be a multiple of pack_len (the reference drops the tokens of an incomplete pack)");
-    // the cost word holds (bits << 8 | token): bits <= 8 * 2 * hidden_dim must stay below 2^24
+    const uint32_t nblocks = (uint32_t)(ctx_len / block_size);
+    // blocks of up to 64 tokens: register-resident channel slices, as many groups of workgroups as fit the device
+    uint32_t members = (uint32_t)((2 * (size_t)hidden_dim + kSlicedChannels - 1) / kSlicedChannels), groups = 0;
+    if (block_size <= kSlicedTokens) {
+        int dev = 0;
+        PKV_HIP_CHECK(hipGetDevice(&dev));
+        static std::mutex mu;
+        static std::map<int, uint32_t> resident;      // workgroups of the sliced kernel that fit the device at once
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = resident.find(dev);
+        if (it == resident.end()) {
+            int cus = 0, per_cu = 0;
+            PKV_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+            PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                &per_cu, reinterpret_cast<const void *>(greedy_order_sliced_kernel), kSlicedThreads, 0));
+            it = resident.emplace(dev, (uint32_t)(cus > 0 && per_cu > 0 ? cus * per_cu : 0)).first;
+        }
+        groups = it->second / members;
+        if (groups > nblocks) groups = nblocks;
+    }
+    int rc;
+    if (groups > 0) {
+        ScanState *st = nullptr;
+        if ((rc = prepare_scan_state(groups * 2u * members * 128u, &st, s))) return rc;
+        LaunchTimer tm(s, ms_out != nullptr);
+        if ((rc = tm.begin())) return rc;
+        greedy_order_sliced_kernel<<<groups * members, kSlicedThreads, 0, s>>>(k_codes, v_codes, hidden_dim, block_size, pack_len,
+                                                                               nblocks, members, groups, perm, st);
+        gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
+        PKV_HIP_CHECK(hipGetLastError());
+        if ((rc = tm.end(ms_out))) return rc;
+        if (ms_out) {                                  // a timed call has waited for the kernels: look at the error word
+            uint32_t head[2] = {0u, 0u};
+            PKV_HIP_CHECK(hipMemcpyAsync(head, st, sizeof(head), hipMemcpyDeviceToHost, s));
+            PKV_HIP_CHECK(hipStreamSynchronize(s));
+            PKV_REQUIRE(head[1] == 0u, PKV_ERR_INTERNAL, "greedy order: a workgroup waited too long for the sums of its group");
+        }
+        return PKV_OK;
+    }
+    // longer blocks: the cost word holds (bits << 8 | token): bits <= 8 * 2 * hidden_dim must stay below 2^24
     const size_t lds = 4 * (size_t)hidden_dim + kGreedyMaxTokens * (8 + 8 + 8 + 1);
     PKV_REQUIRE(hidden_dim <= 32768 && lds <= 160 * 1024, PKV_ERR_UNSUPPORTED,
-                "not supported: the greedy order keeps 4 * hidden_dim bytes in LDS (hidden_dim <= 32768)");
+                "not supported: the greedy order of blocks of more than 64 tokens keeps 4 * hidden_dim bytes in LDS (hidden_dim <= 32768)");
     if (lds > 48 * 1024)
         PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(greedy_order_kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     LaunchTimer tm(s, ms_out != nullptr);
-    int rc;
     if ((rc = tm.begin())) return rc;
-    greedy_order_kernel<<<(unsigned)(ctx_len / block_size), kGreedyThreads, lds, s>>>(k_codes, v_codes, hidden_dim, block_size,
-                                                                                    pack_len, perm);
+    greedy_order_kernel<<<nblocks, kGreedyThreads, lds, s>>>(k_codes, v_codes, hidden_dim, block_size, pack_len, perm);
     gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
