@@ -315,12 +315,14 @@ __global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint
 // A workgroup of 256 threads holds 2048 channels of all the tokens of a block (thread = 8 adjacent channels, one
 // dword pair per token, in registers for the whole block), so a pick re-reads nothing from memory.  The
 // ceil(2 * hidden / 2048) workgroups that cover a block form a group: every step (a seed or a pick) each member
-// sums its slice per token, publishes the partial sums as (step number << 32 | value) words, reads the words of
-// all members and finds the winner for itself; the words of two consecutive steps live in two buffers, and a member
-// can be at most one step ahead of another, so a word is never overwritten before it was read.  Workgroups take
-// tickets in the order they start and a group is a run of consecutive tickets: whenever a member waits, the members
-// it waits for run already or start as soon as a complete group ahead of them leaves; the launch never holds more
-// groups than fit the device.  The waits are bounded all the same (kGreedySpinLimit, error word of the state).
+// sums its slice per token (every thread leaves its sums in LDS, eight threads per pair of tokens add them up),
+// publishes the sums as (step number << 32 | value) words -- a pick: one word per pair of tokens, two 16-bit sums;
+// a seed: dot product and squared norm per token -- reads the words of all members and finds the winner for itself.
+// The words of two consecutive steps live in two buffers, and a member can be at most one step ahead of another, so
+// a word is never overwritten before it was read.  Workgroups take tickets in the order they start and a group is a
+// run of consecutive tickets: whenever a member waits, the members it waits for run already or start as soon as a
+// complete group ahead of them leaves; the launch never holds more groups than fit the device.  The waits are
+// bounded all the same (kGreedySpinLimit, error word of the state).
 //
 // The remaining tokens occupy register slots 0 .. n_alive - 1 (the winner's slot takes the rows of the last slot;
 // lane l of every wavefront knows which token slot l holds), so a step walks a prefix of the slots without a test
@@ -328,12 +330,14 @@ __global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint
 //
 // Pricing a token: min and max as packed 16-bit lanes, r = max - min, then bit_length(r) is the exponent of
 // (2 r + 1) 2^-10 as a half: one packed fma on r read as a subnormal half (r 2^-24 * 2^15 + 2^-10, exact), the
-// exponent fields masked and added by a sum of absolute differences -- 3.5 vector instructions per channel.  The
-// constant bias of the exponent (5 per channel) is common to all tokens.
+// exponent fields masked and added by a sum of absolute differences -- 3.7 vector instructions per channel.  The
+// constant bias of the exponent (5 per channel) is common to all tokens.  A step of a group of 16 takes ~6.5 us on
+// an MI355X, about half of it pricing; the two workgroups a CU holds fill each other's waits.
 constexpr int kSlicedThreads = 256;
 constexpr int kSlicedChannels = 8 * kSlicedThreads;      // per workgroup
 constexpr int kSlicedTokens = 64;
 constexpr int kGreedySpinLimit = 1 << 22;
+constexpr int kPartStride = 8 * 36 + 4;                 // words per row of the per-thread sums (8 runs of 32 + 4, then + 4)
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
@@ -343,21 +347,35 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t even_bytes(uint32_t x, uint32_t mask_00ff00ff) { return x & mask_00ff00ff; }
 __device__ __forceinline__ uint32_t odd_bytes(uint32_t x, uint32_t sel_0c030c01) { return __builtin_amdgcn_perm(0u, x, sel_0c030c01); }
 
-// exponent fields (<< 10, both halves) of (2 r + 1) 2^-10, r = max(x, mx) - min(x, mn) per 16-bit lane
-__device__ __forceinline__ uint32_t range_exponents(uint32_t x, uint32_t mn, uint32_t mx) {
-    const ushort2v r = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, x), __builtin_bit_cast(ushort2v, mx)) -
-                       __builtin_elementwise_min(__builtin_bit_cast(ushort2v, x), __builtin_bit_cast(ushort2v, mn));
-    const half2v f = __builtin_elementwise_fma(__builtin_bit_cast(half2v, r), (half2v){(_Float16)32768.0f, (_Float16)32768.0f},
-                                               (half2v){(_Float16)0.0009765625f, (_Float16)0.0009765625f});
-    return __builtin_bit_cast(uint32_t, f) & 0x7C007C00u;
-}
-// sum over the 8 channels of a dword pair of the exponent fields, << 10
-__device__ __forceinline__ uint32_t price8(uint32_t x0, uint32_t x1, const uint32_t (&mn)[4], const uint32_t (&mx)[4],
-                                           uint32_t k_even, uint32_t k_odd) {
-    uint32_t a = __builtin_amdgcn_sad_u16(range_exponents(even_bytes(x0, k_even), mn[0], mx[0]), 0u, 0u);
-    a = __builtin_amdgcn_sad_u16(range_exponents(odd_bytes(x0, k_odd), mn[1], mx[1]), 0u, a);
-    a = __builtin_amdgcn_sad_u16(range_exponents(even_bytes(x1, k_even), mn[2], mx[2]), 0u, a);
-    return __builtin_amdgcn_sad_u16(range_exponents(odd_bytes(x1, k_odd), mn[3], mx[3]), 0u, a);
+// Two tokens (a, b), 8 channels each: sums of the exponent fields, << 10.  Stage by stage over the eight independent
+// chains, so that no instruction waits for the one before it.
+__device__ __forceinline__ void price8x2(uint32_t x0a, uint32_t x1a, uint32_t x0b, uint32_t x1b, const uint32_t (&mn)[4],
+                                         const uint32_t (&mx)[4], uint32_t k_even, uint32_t k_odd, uint32_t &sum_a, uint32_t &sum_b) {
+    const uint32_t v[8] = {even_bytes(x0a, k_even), even_bytes(x0b, k_even), odd_bytes(x0a, k_odd), odd_bytes(x0b, k_odd),
+                           even_bytes(x1a, k_even), even_bytes(x1b, k_even), odd_bytes(x1a, k_odd), odd_bytes(x1b, k_odd)};
+    ushort2v hi[8], lo[8];
+    uint32_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) hi[i] = __builtin_elementwise_max(__builtin_bit_cast(ushort2v, v[i]), __builtin_bit_cast(ushort2v, mx[i >> 1]));
+#pragma unroll
+    for (int i = 0; i < 8; i++) lo[i] = __builtin_elementwise_min(__builtin_bit_cast(ushort2v, v[i]), __builtin_bit_cast(ushort2v, mn[i >> 1]));
+#pragma unroll
+    for (int i = 0; i < 8; i++) hi[i] -= lo[i];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const half2v f = __builtin_elementwise_fma(__builtin_bit_cast(half2v, hi[i]), (half2v){(_Float16)32768.0f, (_Float16)32768.0f},
+                                                   (half2v){(_Float16)0.0009765625f, (_Float16)0.0009765625f});
+        e[i] = __builtin_bit_cast(uint32_t, f);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) e[i] &= 0x7C007C00u;
+    sum_a = __builtin_amdgcn_sad_u16(e[0], 0u, 0u);
+    sum_b = __builtin_amdgcn_sad_u16(e[1], 0u, 0u);
+#pragma unroll
+    for (int i = 1; i < 4; i++) {
+        sum_a = __builtin_amdgcn_sad_u16(e[2 * i], 0u, sum_a);
+        sum_b = __builtin_amdgcn_sad_u16(e[2 * i + 1], 0u, sum_b);
+    }
 }
 
 // data-parallel-primitive moves between the lanes of a row of 16 (0x100 | n: from lane + n, 0x110 | n: from lane - n,
@@ -390,45 +408,44 @@ __device__ __forceinline__ uint32_t sum8_down(uint32_t v) {         // lanes 0, 
     M(b + 11) M(b + 12) M(b + 13) M(b + 14) M(b + 15)
 #define PKV_SLOTS64(M) PKV_SLOTS16(M, 0) PKV_SLOTS16(M, 16) PKV_SLOTS16(M, 32) PKV_SLOTS16(M, 48)
 
-// Sum over the members first, first + stride, .. of word `idx` of their 128 published words, four loads in flight.
-__device__ __forceinline__ unsigned long long gather_words(const uint64_t *words, uint32_t idx, uint32_t first, uint32_t stride,
-                                                           uint32_t members, uint32_t seq, ScanState *st) {
-    unsigned long long sum = 0ull;
+// Word `idx` of the 128 published words of the members first, first + stride, ..: up to four loads in flight, all of
+// them repeated until every word carries the step number.  `take(w)` gets the low halves.
+template <typename F>
+__device__ __forceinline__ void gather_words(const uint64_t *words, uint32_t idx, uint32_t first, uint32_t stride, uint32_t members,
+                                             uint32_t seq, ScanState *st, F &&take) {
     for (uint32_t m0 = first; m0 < members; m0 += 4 * stride) {
         const uint64_t *p = words + (size_t)m0 * 128 + idx;
-        uint64_t w[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            w[i] = m0 + i * stride < members ? __hip_atomic_load(p + (size_t)i * stride * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                             : (uint64_t)seq << 32;
+        const bool on1 = m0 + stride < members, on2 = m0 + 2 * stride < members, on3 = m0 + 3 * stride < members;
+        const uint64_t *p1 = on1 ? p + (size_t)stride * 128 : p, *p2 = on2 ? p + (size_t)2 * stride * 128 : p,
+                       *p3 = on3 ? p + (size_t)3 * stride * 128 : p;
+        uint64_t w0, w1, w2, w3;
         int spins = 0;
-        while (((uint32_t)(w[0] >> 32) != seq || (uint32_t)(w[1] >> 32) != seq || (uint32_t)(w[2] >> 32) != seq ||
-                (uint32_t)(w[3] >> 32) != seq) && spins < kGreedySpinLimit) {
-            __builtin_amdgcn_s_sleep(1);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if ((uint32_t)(w[i] >> 32) != seq)
-                    w[i] = __hip_atomic_load(p + (size_t)i * stride * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            spins++;
-        }
+        do {
+            w0 = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            w1 = __hip_atomic_load(p1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            w2 = __hip_atomic_load(p2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            w3 = __hip_atomic_load(p3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } while (((uint32_t)(w0 >> 32) != seq || (uint32_t)(w1 >> 32) != seq || (uint32_t)(w2 >> 32) != seq ||
+                  (uint32_t)(w3 >> 32) != seq) && ++spins < kGreedySpinLimit);
         if (spins >= kGreedySpinLimit) st->error = (uint32_t)PKV_ERR_INTERNAL;
-        sum += (unsigned long long)(uint32_t)w[0] + (uint32_t)w[1] + (uint32_t)w[2] + (uint32_t)w[3];
+        take((uint32_t)w0);
+        if (on1) take((uint32_t)w1);
+        if (on2) take((uint32_t)w2);
+        if (on3) take((uint32_t)w3);
     }
-    return sum;
 }
 
 __global__ void __launch_bounds__(kSlicedThreads, 2)
 greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *__restrict__ v_codes, int hidden, int N,
                            int pack_len, uint32_t nblocks, uint32_t members, uint32_t groups,
                            uint32_t *__restrict__ perm, ScanState *st) {
-    __shared__ uint32_t s_acc[2][32 * 32];           // picks: [buffer][pair of slots][adder]
+    __shared__ __attribute__((aligned(16))) uint32_t s_part[32 * kPartStride];   // picks: [pair of slots][thread], padded
     __shared__ uint32_t s_seed[128 * 32];            // seeds: [2 * slot + (0: dot, 1: squared norm)][adder]
-    __shared__ uint32_t s_tot[4][64];                // picks: sums over a quarter of the members
+    __shared__ uint32_t s_tot[8][64];                // picks: sums over an eighth of the members
     __shared__ unsigned long long s_tot64[2][128];   // seeds: sums over half of the members
     __shared__ uint32_t s_ticket;
     const int tid = threadIdx.x, lane = tid & 63;
     if (tid == 0) s_ticket = atomicAdd(&st->ticket, 1u);
-    for (int i = tid; i < 2 * 32 * 32; i += kSlicedThreads) (&s_acc[0][0])[i] = 0u;
     __syncthreads();
     const uint32_t ticket = s_ticket;
     const uint32_t grp = ticket / members, mem = ticket - grp * members;
@@ -441,7 +458,10 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
     const int adder = (tid >> 2) & 31;               // the LDS word that takes the sums of the thread's four lanes
     const bool quad_first = (tid & 3) == 0;
     uint32_t seq = 0;
-    int flip = 0, ab = 0;
+    int flip = 0;
+    // a thread's word in a row of s_part and, as a reader, where the 32 words it adds start: rows and runs of 32 are
+    // padded so that the 16-byte reads of a wavefront spread over all banks
+    const int part_word = (tid >> 5) * 36 + (tid & 31), part_read = (tid >> 3) * kPartStride + (tid & 7) * 36;
 
     for (uint32_t blk = grp; blk < nblocks; blk += groups) {
         const size_t row0 = (size_t)blk * N;
@@ -519,7 +539,10 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
             }
             if (members > 1) {
                 const int v = tid & 127, q = tid >> 7;
-                s_tot64[q][v] = v < 2 * n_alive ? gather_words(xw + (size_t)flip * members * 128, (uint32_t)v, (uint32_t)q, 2u, members, seq, st) : 0ull;
+                unsigned long long a = 0ull;
+                if (v < 2 * n_alive)
+                    gather_words(xw + (size_t)flip * members * 128, (uint32_t)v, (uint32_t)q, 2u, members, seq, st, [&](uint32_t w) { a += w; });
+                s_tot64[q][v] = a;
                 flip ^= 1;
             }
             __syncthreads();
@@ -545,7 +568,6 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
             }
             } else {
             // ---- the pack's other tokens: fewest bits after the pick ----
-                uint32_t *acc = s_acc[ab];
 #pragma unroll
                 for (int k4 = 0; k4 < kSlicedTokens / 2; k4 += 4) {
                     if (2 * k4 < n_alive) {
@@ -553,43 +575,50 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                         for (int k = k4; k < k4 + 4; k++)
                             if (2 * k < n_alive) {
                                 // (with an odd count the slot past the last one is priced as well: a bounded sum nobody reads)
-                                const uint32_t a0 = price8(x0[2 * k], x1[2 * k], mn, mx, k_even, k_odd), a1 = price8(x0[2 * k + 1], x1[2 * k + 1], mn, mx, k_even, k_odd);
-                                const uint32_t c = quad_sum((a0 >> 10) | (a1 << 6));      // sums of fields at bit 10: a 16-bit lane per slot
-                                if (quad_first) atomicAdd(&acc[k * 32 + adder], c);
+                                uint32_t a0, a1;
+                                price8x2(x0[2 * k], x1[2 * k], x0[2 * k + 1], x1[2 * k + 1], mn, mx, k_even, k_odd, a0, a1);
+                                s_part[k * kPartStride + part_word] = (a0 >> 10) | (a1 << 6);   // sums of fields at bit 10: a 16-bit lane per slot
                             }
                     }
                 }
                 __syncthreads();
                 seq++;
-                {   // pair k = tid >> 3: eight threads add 4 adders each; then the other buffer is cleared for the next pick
+                {   // pair k = tid >> 3: eight threads add 32 words each
                     const int k = tid >> 3, part = tid & 7;
-                    const uint32_t a = sum8_down(acc[k * 32 + part * 4] + acc[k * 32 + part * 4 + 1] + acc[k * 32 + part * 4 + 2] +
-                                                 acc[k * 32 + part * 4 + 3]);
+                    const uint4 *src = reinterpret_cast<const uint4 *>(s_part + part_read);
+                    uint32_t a = 0u;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const uint4 w = src[i];
+                        a += w.x + w.y + w.z + w.w;
+                    }
+                    a = sum8_down(a);
                     if (part == 0 && 2 * k < n_alive) {
-                        if (members > 1) {
-                            uint64_t *dst = xw + ((size_t)flip * members + mem) * 128 + 2 * k;
-                            __hip_atomic_store(dst, ((uint64_t)seq << 32) | (a & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            __hip_atomic_store(dst + 1, ((uint64_t)seq << 32) | (a >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (members > 1) {      // both slots of the pair in one word
+                            __hip_atomic_store(xw + ((size_t)flip * members + mem) * 128 + k, ((uint64_t)seq << 32) | a, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
                         } else {
                             s_tot[0][2 * k] = a & 0xFFFFu;
                             s_tot[0][2 * k + 1] = a >> 16;
                         }
                     }
-                    ab ^= 1;
-                    uint32_t *other = s_acc[ab];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) other[tid * 4 + i] = 0u;
                 }
-                if (members > 1) {
-                    const int q = tid >> 6;
-                    s_tot[q][lane] = lane < n_alive ? (uint32_t)gather_words(xw + (size_t)flip * members * 128, (uint32_t)lane, (uint32_t)q, 4u, members, seq, st) : 0u;
+                if (members > 1) {       // pair k = tid & 31 of the members q, q + 8, ..
+                    const int k = tid & 31, q = tid >> 5;
+                    uint32_t a_lo = 0u, a_hi = 0u;
+                    if (2 * k < n_alive)
+                        gather_words(xw + (size_t)flip * members * 128, (uint32_t)k, (uint32_t)q, 8u, members, seq, st,
+                                     [&](uint32_t w) { a_lo += w & 0xFFFFu; a_hi += w >> 16; });
+                    s_tot[q][2 * k] = a_lo;
+                    s_tot[q][2 * k + 1] = a_hi;
                     flip ^= 1;
                 }
                 __syncthreads();
                 uint32_t key = 0xFFFFFFFFu;            // (cost, token) in one word: the minimum is the first cheapest token
                 if (lane < n_alive) {
                     uint32_t a = s_tot[0][lane];
-                    if (members > 1) a += s_tot[1][lane] + s_tot[2][lane] + s_tot[3][lane];
+                    if (members > 1)
+                        a += s_tot[1][lane] + s_tot[2][lane] + s_tot[3][lane] + s_tot[4][lane] + s_tot[5][lane] + s_tot[6][lane] + s_tot[7][lane];
                     key = (a << 8) | orig;
                 }
                 const uint32_t best = wave_min_u32(key);
