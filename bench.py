@@ -492,7 +492,7 @@ def main():
         cv_ms = event_time_ms(torch, lambda: ops.v_encode(codes_v, ve["stream"], ve["info"], 128, 64, bits, want_size=False), 3)
         rp_ms = event_time_ms(torch, lambda: ops.median_repacking(codes, codes_v, 64), 3)
         bp_ms = event_time_ms(torch, lambda: ops.bit_pack_bytes(codes, 16), 3)
-        g_rows = min(Tc, 8192)      # the greedy order re-reads a block once per pick: a slice of the workload is enough
+        g_rows = min(Tc, 8192)      # 128 blocks of 64 tokens x 2 x 16384 channels: the shape the kernel's figures are quoted on
         gr_ms = event_time_ms(torch, lambda: ops.greedy_repacking(codes[:g_rows], codes_v[:g_rows], 16, 64), 2)
         result["repack"] = {
             "greedy_repack_ms": gr_ms, "greedy_repack_rows": g_rows,

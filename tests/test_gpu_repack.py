@@ -137,7 +137,10 @@ def test_greedy_repacking_matches_restatement(cuda):
         kc, vc = _codes(B, H, T, 0.1, seed=240 + B + H)
         cases.append((kc, vc, bs, pack, "quantised %dx%dx%d" % (B, H, T)))
     g = torch.Generator(device="cpu").manual_seed(241)
-    for (T, hid, top, bs, pack) in ((64, 16, 4, 16, 4), (128, 48, 2, 64, 16), (256, 2064, 200, 256, 32), (64, 32768, 16, 64, 16)):
+    # (the last two have more blocks than the device holds at once as groups of workgroups: 72 blocks of 8 slices and
+    # 520 blocks of one slice, so a group walks several blocks)
+    for (T, hid, top, bs, pack) in ((64, 16, 4, 16, 4), (128, 48, 2, 64, 16), (256, 2064, 200, 256, 32), (64, 32768, 16, 64, 16),
+                                    (576, 8192, 6, 8, 4), (33280, 128, 6, 64, 16)):
         kc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
         vc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
         cases.append((kc, vc, bs, pack, "random %dx%d below %d" % (T, hid, top)))
