@@ -312,9 +312,9 @@ __global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint
 }
 
 // ---- greedy order of blocks of up to 64 tokens: the block's rows stay in registers, sliced by channel ----
-// A workgroup of 256 threads holds 2048 channels of all the tokens of a block (thread = 8 adjacent channels, one
-// dword pair per token, in registers for the whole block), so a pick re-reads nothing from memory.  The
-// ceil(2 * hidden / 2048) workgroups that cover a block form a group: every step (a seed or a pick) each member
+// A workgroup of 512 threads holds 4096 channels of all the tokens of a block (thread = 8 adjacent channels, one
+// dword pair per token, in registers for the whole block), so a pick re-reads nothing from memory; rows of up to
+// 2048 channels take workgroups of 256 threads, two per CU.  The workgroups that cover a block form a group: every step (a seed or a pick) each member
 // sums its slice per token (every thread leaves its sums in LDS, eight threads per pair of tokens add them up),
 // publishes the sums as (step number << 32 | value) words -- a pick: one word per pair of tokens, two 16-bit sums;
 // a seed: dot product and squared norm per token -- reads the words of all members and finds the winner for itself.
@@ -331,13 +331,14 @@ __global__ void __launch_bounds__(kGreedyThreads) greedy_order_kernel(const uint
 // Pricing a token: min and max as packed 16-bit lanes, r = max - min, then bit_length(r) is the exponent of
 // (2 r + 1) 2^-10 as a half: one packed fma on r read as a subnormal half (r 2^-24 * 2^15 + 2^-10, exact), the
 // exponent fields masked and added by a sum of absolute differences -- 3.7 vector instructions per channel.  The
-// constant bias of the exponent (5 per channel) is common to all tokens.  A step of a group of 16 takes ~6.5 us on
-// an MI355X, about half of it pricing; the two workgroups a CU holds fill each other's waits.
-constexpr int kSlicedThreads = 256;
-constexpr int kSlicedChannels = 8 * kSlicedThreads;      // per workgroup
+// constant bias of the exponent (5 per channel) is common to all tokens.  A step of a group of eight wide
+// workgroups takes ~6.5 us on an MI355X: 3.8 us of pricing at the full rate of the vector ALUs, the rest the sums,
+// the exchange, the winner and the slot move, which nothing overlaps.
+constexpr int kSlicedThreadsWide = 512;                 // one workgroup per CU, two wavefronts per SIMD: rows of two or more slices
+constexpr int kSlicedThreadsNarrow = 256;               // two workgroups per CU: rows of up to 2048 channels
 constexpr int kSlicedTokens = 64;
 constexpr int kGreedySpinLimit = 1 << 22;
-constexpr int kPartStride = 8 * 36 + 4;                 // words per row of the per-thread sums (8 runs of 32 + 4, then + 4)
+// words per row of the per-thread sums: runs of 32 threads, each + 4, then + 4
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
@@ -435,14 +436,16 @@ __device__ __forceinline__ void gather_words(const uint64_t *words, uint32_t idx
     }
 }
 
-__global__ void __launch_bounds__(kSlicedThreads, 2)
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS, 2)
 greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *__restrict__ v_codes, int hidden, int N,
                            int pack_len, uint32_t nblocks, uint32_t members, uint32_t groups,
                            uint32_t *__restrict__ perm, ScanState *st) {
+    constexpr int kRuns = THREADS / 32, kPartStride = kRuns * 36 + 4, kSeedParts = THREADS / 128;
     __shared__ __attribute__((aligned(16))) uint32_t s_part[32 * kPartStride];   // picks: [pair of slots][thread], padded
     __shared__ uint32_t s_seed[128 * 32];            // seeds: [2 * slot + (0: dot, 1: squared norm)][adder]
-    __shared__ uint32_t s_tot[8][64];                // picks: sums over an eighth of the members
-    __shared__ unsigned long long s_tot64[2][128];   // seeds: sums over half of the members
+    __shared__ uint32_t s_tot[kRuns][64];            // picks: sums over the members q, q + kRuns, ..
+    __shared__ unsigned long long s_tot64[kSeedParts][128];   // seeds: sums over the members q, q + kSeedParts, ..
     __shared__ uint32_t s_ticket;
     const int tid = threadIdx.x, lane = tid & 63;
     if (tid == 0) s_ticket = atomicAdd(&st->ticket, 1u);
@@ -452,7 +455,7 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
     if (grp >= groups) return;
     uint64_t *xw = st->status + (size_t)grp * 2 * members * 128;      // [buffer][member][128]
     const int D2 = 2 * hidden;
-    const int ch = ((int)mem * kSlicedThreads + tid) * 8;             // first of the thread's 8 channels
+    const int ch = ((int)mem * THREADS + tid) * 8;                    // first of the thread's 8 channels
     const uint8_t *col = ch < hidden ? k_codes + ch : v_codes + (ch - hidden);
     const bool have = ch < D2;
     const int adder = (tid >> 2) & 31;               // the LDS word that takes the sums of the thread's four lanes
@@ -461,7 +464,7 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
     int flip = 0;
     // a thread's word in a row of s_part and, as a reader, where the 32 words it adds start: rows and runs of 32 are
     // padded so that the 16-byte reads of a wavefront spread over all banks
-    const int part_word = (tid >> 5) * 36 + (tid & 31), part_read = (tid >> 3) * kPartStride + (tid & 7) * 36;
+    const int part_word = (tid >> 5) * 36 + (tid & 31), part_read = (tid / kRuns) * kPartStride + (tid % kRuns) * 36;
 
     for (uint32_t blk = grp; blk < nblocks; blk += groups) {
         const size_t row0 = (size_t)blk * N;
@@ -504,7 +507,7 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                 const uint32_t o_lo = (uint32_t)rintf((float)(sum[2 * d + 1] & 0xFFFFu) / na), o_hi = (uint32_t)rintf((float)(sum[2 * d + 1] >> 16) / na);
                 mean[d] = e_lo | (o_lo << 8) | (e_hi << 16) | (o_hi << 24);
             }
-            for (int i = tid; i < 128 * 32; i += kSlicedThreads) s_seed[i] = 0u;
+            for (int i = tid; i < 128 * 32; i += THREADS) s_seed[i] = 0u;
             __syncthreads();
 #pragma unroll
             for (int t8 = 0; t8 < kSlicedTokens; t8 += 8) {
@@ -523,12 +526,13 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
             }
             __syncthreads();
             seq++;
-            {   // value v = tid >> 1: two threads add 16 adders each
-                const int v = tid >> 1, part = tid & 1;
+            {   // value v: two or four adjacent threads add 16 or 8 adders each
+                const int v = tid / kSeedParts, part = tid % kSeedParts;
                 uint32_t a = 0u;
 #pragma unroll
-                for (int i = 0; i < 16; i++) a += s_seed[v * 32 + part * 16 + i];
+                for (int i = 0; i < 32 / kSeedParts; i++) a += s_seed[v * 32 + part * (32 / kSeedParts) + i];
                 a += lane_move<0xB1, 0xF, false>(0u, a);
+                if (kSeedParts == 4) a += lane_move<0x4E, 0xF, false>(0u, a);
                 if (part == 0 && v < 2 * n_alive) {
                     if (members > 1)
                         __hip_atomic_store(xw + ((size_t)flip * members + mem) * 128 + v, ((uint64_t)seq << 32) | a,
@@ -541,7 +545,8 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                 const int v = tid & 127, q = tid >> 7;
                 unsigned long long a = 0ull;
                 if (v < 2 * n_alive)
-                    gather_words(xw + (size_t)flip * members * 128, (uint32_t)v, (uint32_t)q, 2u, members, seq, st, [&](uint32_t w) { a += w; });
+                    gather_words(xw + (size_t)flip * members * 128, (uint32_t)v, (uint32_t)q, (uint32_t)kSeedParts, members, seq, st,
+                                 [&](uint32_t w) { a += w; });
                 s_tot64[q][v] = a;
                 flip ^= 1;
             }
@@ -553,7 +558,10 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                     sel = lane;
                     bd = s_tot64[0][2 * lane];
                     bn = s_tot64[0][2 * lane + 1];
-                    if (members > 1) { bd += s_tot64[1][2 * lane]; bn += s_tot64[1][2 * lane + 1]; }
+                    if (members > 1) {
+#pragma unroll
+                        for (int q = 1; q < kSeedParts; q++) { bd += s_tot64[q][2 * lane]; bn += s_tot64[q][2 * lane + 1]; }
+                    }
                 }
 #pragma unroll
                 for (int d = 32; d >= 1; d >>= 1) {      // equal cosines: the earlier token
@@ -583,8 +591,8 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                 }
                 __syncthreads();
                 seq++;
-                {   // pair k = tid >> 3: eight threads add 32 words each
-                    const int k = tid >> 3, part = tid & 7;
+                {   // pair k: kRuns adjacent threads add 32 words each
+                    const int k = tid / kRuns, part = tid % kRuns;
                     const uint4 *src = reinterpret_cast<const uint4 *>(s_part + part_read);
                     uint32_t a = 0u;
 #pragma unroll
@@ -593,6 +601,7 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                         a += w.x + w.y + w.z + w.w;
                     }
                     a = sum8_down(a);
+                    if (kRuns == 16) a += lane_move<0x108, 0xF, true>(0u, a);
                     if (part == 0 && 2 * k < n_alive) {
                         if (members > 1) {      // both slots of the pair in one word
                             __hip_atomic_store(xw + ((size_t)flip * members + mem) * 128 + k, ((uint64_t)seq << 32) | a, __ATOMIC_RELAXED,
@@ -603,11 +612,11 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                         }
                     }
                 }
-                if (members > 1) {       // pair k = tid & 31 of the members q, q + 8, ..
+                if (members > 1) {       // pair k = tid & 31 of the members q, q + kRuns, ..
                     const int k = tid & 31, q = tid >> 5;
                     uint32_t a_lo = 0u, a_hi = 0u;
                     if (2 * k < n_alive)
-                        gather_words(xw + (size_t)flip * members * 128, (uint32_t)k, (uint32_t)q, 8u, members, seq, st,
+                        gather_words(xw + (size_t)flip * members * 128, (uint32_t)k, (uint32_t)q, (uint32_t)kRuns, members, seq, st,
                                      [&](uint32_t w) { a_lo += w & 0xFFFFu; a_hi += w >> 16; });
                     s_tot[q][2 * k] = a_lo;
                     s_tot[q][2 * k + 1] = a_hi;
@@ -617,8 +626,10 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                 uint32_t key = 0xFFFFFFFFu;            // (cost, token) in one word: the minimum is the first cheapest token
                 if (lane < n_alive) {
                     uint32_t a = s_tot[0][lane];
-                    if (members > 1)
-                        a += s_tot[1][lane] + s_tot[2][lane] + s_tot[3][lane] + s_tot[4][lane] + s_tot[5][lane] + s_tot[6][lane] + s_tot[7][lane];
+                    if (members > 1) {
+#pragma unroll
+                        for (int q = 1; q < kRuns; q++) a += s_tot[q][lane];
+                    }
                     key = (a << 8) | orig;
                 }
                 const uint32_t best = wave_min_u32(key);
@@ -825,21 +836,29 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
     PKV_REQUIRE(block_size % pack_len == 0, PKV_ERR_INVALID,
                 "block_size must be a multiple of pack_len (the reference drops the tokens of an incomplete pack)");
     const uint32_t nblocks = (uint32_t)(ctx_len / block_size);
-    // blocks of up to 64 tokens: register-resident channel slices, as many groups of workgroups as fit the device
-    uint32_t members = (uint32_t)((2 * (size_t)hidden_dim + kSlicedChannels - 1) / kSlicedChannels), groups = 0;
+    // blocks of up to 64 tokens: register-resident channel slices, as many groups of workgroups as fit the device;
+    // rows of more than one narrow slice go to the wide workgroups, which have a CU to themselves: two members of a
+    // group on one CU, or another group's member in the same phase, would price at half speed and hold up their group
+    const bool wide = 2 * (size_t)hidden_dim > 8u * kSlicedThreadsNarrow;
+    const uint32_t slice = 8u * (wide ? kSlicedThreadsWide : kSlicedThreadsNarrow);
+    uint32_t members = (uint32_t)((2 * (size_t)hidden_dim + slice - 1) / slice), groups = 0;
     if (block_size <= kSlicedTokens) {
         int dev = 0;
         PKV_HIP_CHECK(hipGetDevice(&dev));
         static std::mutex mu;
-        static std::map<int, uint32_t> resident;      // workgroups of the sliced kernel that fit the device at once
+        static std::map<std::pair<int, bool>, uint32_t> resident;      // workgroups of the sliced kernel that fit the device at once
         std::lock_guard<std::mutex> lock(mu);
-        auto it = resident.find(dev);
+        auto it = resident.find({dev, wide});
         if (it == resident.end()) {
             int cus = 0, per_cu = 0;
             PKV_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-            PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                &per_cu, reinterpret_cast<const void *>(greedy_order_sliced_kernel), kSlicedThreads, 0));
-            it = resident.emplace(dev, (uint32_t)(cus > 0 && per_cu > 0 ? cus * per_cu : 0)).first;
+            if (wide)
+                PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &per_cu, reinterpret_cast<const void *>(greedy_order_sliced_kernel<kSlicedThreadsWide>), kSlicedThreadsWide, 0));
+            else
+                PKV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &per_cu, reinterpret_cast<const void *>(greedy_order_sliced_kernel<kSlicedThreadsNarrow>), kSlicedThreadsNarrow, 0));
+            it = resident.emplace(std::make_pair(dev, wide), (uint32_t)(cus > 0 && per_cu > 0 ? cus * per_cu : 0)).first;
         }
         groups = it->second / members;
         if (groups > nblocks) groups = nblocks;
@@ -850,8 +869,12 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
         if ((rc = prepare_scan_state(groups * 2u * members * 128u, &st, s))) return rc;
         LaunchTimer tm(s, ms_out != nullptr);
         if ((rc = tm.begin())) return rc;
-        greedy_order_sliced_kernel<<<groups * members, kSlicedThreads, 0, s>>>(k_codes, v_codes, hidden_dim, block_size, pack_len,
-                                                                               nblocks, members, groups, perm, st);
+        if (wide)
+            greedy_order_sliced_kernel<kSlicedThreadsWide><<<groups * members, kSlicedThreadsWide, 0, s>>>(
+                k_codes, v_codes, hidden_dim, block_size, pack_len, nblocks, members, groups, perm, st);
+        else
+            greedy_order_sliced_kernel<kSlicedThreadsNarrow><<<groups * members, kSlicedThreadsNarrow, 0, s>>>(
+                k_codes, v_codes, hidden_dim, block_size, pack_len, nblocks, members, groups, perm, st);
         gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
