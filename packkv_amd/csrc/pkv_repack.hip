@@ -404,11 +404,6 @@ __device__ __forceinline__ uint32_t sum8_down(uint32_t v) {         // lanes 0, 
     return v + lane_move<0x104, 0xF, true>(0u, v);
 }
 
-// one statement per register slot: switches over these cases keep every index of the register arrays a constant
-#define PKV_SLOTS16(M, b) M(b + 0) M(b + 1) M(b + 2) M(b + 3) M(b + 4) M(b + 5) M(b + 6) M(b + 7) M(b + 8) M(b + 9) M(b + 10) \
-    M(b + 11) M(b + 12) M(b + 13) M(b + 14) M(b + 15)
-#define PKV_SLOTS64(M) PKV_SLOTS16(M, 0) PKV_SLOTS16(M, 16) PKV_SLOTS16(M, 32) PKV_SLOTS16(M, 48)
-
 // Word `idx` of the 128 published words of the members first, first + stride, ..: up to four loads in flight, all of
 // them repeated until every word carries the step number.  `take(w)` gets the low halves.
 template <typename F>
@@ -435,6 +430,10 @@ __device__ __forceinline__ void gather_words(const uint64_t *words, uint32_t idx
         if (on3) take((uint32_t)w3);
     }
 }
+
+// The rows of a thread: 64 slots as two vectors of 32 registers, which the slot move indexes with a uniform run-time
+// index (register-indexed moves); every other access is by constant.
+typedef uint32_t u32x32 __attribute__((ext_vector_type(32)));
 
 template <int THREADS>
 __global__ void __launch_bounds__(THREADS, 2)
@@ -468,13 +467,15 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
 
     for (uint32_t blk = grp; blk < nblocks; blk += groups) {
         const size_t row0 = (size_t)blk * N;
-        uint32_t x0[kSlicedTokens], x1[kSlicedTokens];
+        u32x32 x0v[2], x1v[2];
+#define x0(t) x0v[(t) >> 5][(t) & 31]
+#define x1(t) x1v[(t) >> 5][(t) & 31]
 #pragma unroll
         for (int t = 0; t < kSlicedTokens; t++) {
             uint2 v = make_uint2(0u, 0u);
             if (t < N && have) v = *reinterpret_cast<const uint2 *>(col + (row0 + t) * (size_t)hidden);
-            x0[t] = v.x;
-            x1[t] = v.y;
+            x0(t) = v.x;
+            x1(t) = v.y;
         }
         uint32_t orig = (uint32_t)lane;          // the token in slot `lane`
         int n_alive = N, picked = 0;
@@ -494,8 +495,8 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
 #pragma unroll
                     for (int t = t8; t < t8 + 8; t++)
                         if (t < n_alive) {
-                            sum[0] += even_bytes(x0[t], k_even); sum[1] += odd_bytes(x0[t], k_odd);
-                            sum[2] += even_bytes(x1[t], k_even); sum[3] += odd_bytes(x1[t], k_odd);
+                            sum[0] += even_bytes(x0(t), k_even); sum[1] += odd_bytes(x0(t), k_odd);
+                            sum[2] += even_bytes(x1(t), k_even); sum[3] += odd_bytes(x1(t), k_odd);
                         }
                 }
             }
@@ -515,8 +516,8 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
 #pragma unroll
                     for (int t = t8; t < t8 + 8; t++)
                         if (t < n_alive) {
-                            const uint32_t dot = quad_sum(__builtin_amdgcn_udot4(x0[t], mean[0], __builtin_amdgcn_udot4(x1[t], mean[1], 0u, false), false));
-                            const uint32_t nx = quad_sum(__builtin_amdgcn_udot4(x0[t], x0[t], __builtin_amdgcn_udot4(x1[t], x1[t], k_zero, false), false));
+                            const uint32_t dot = quad_sum(__builtin_amdgcn_udot4(x0(t), mean[0], __builtin_amdgcn_udot4(x1(t), mean[1], 0u, false), false));
+                            const uint32_t nx = quad_sum(__builtin_amdgcn_udot4(x0(t), x0(t), __builtin_amdgcn_udot4(x1(t), x1(t), k_zero, false), false));
                             if (quad_first) {
                                 atomicAdd(&s_seed[(2 * t) * 32 + adder], dot);
                                 atomicAdd(&s_seed[(2 * t + 1) * 32 + adder], nx);
@@ -584,7 +585,7 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
                             if (2 * k < n_alive) {
                                 // (with an odd count the slot past the last one is priced as well: a bounded sum nobody reads)
                                 uint32_t a0, a1;
-                                price8x2(x0[2 * k], x1[2 * k], x0[2 * k + 1], x1[2 * k + 1], mn, mx, k_even, k_odd, a0, a1);
+                                price8x2(x0(2 * k), x1(2 * k), x0(2 * k + 1), x1(2 * k + 1), mn, mx, k_even, k_odd, a0, a1);
                                 s_part[k * kPartStride + part_word] = (a0 >> 10) | (a1 << 6);   // sums of fields at bit 10: a 16-bit lane per slot
                             }
                     }
@@ -640,19 +641,17 @@ greedy_order_sliced_kernel(const uint8_t *__restrict__ k_codes, const uint8_t *_
             const uint32_t tok = (uint32_t)__builtin_amdgcn_readlane((int)orig, sel);
             const uint32_t moved = (uint32_t)__builtin_amdgcn_readlane((int)orig, last);
             if (lane == sel) orig = moved;
-            uint32_t l0 = 0u, l1 = 0u, w0 = 0u, w1 = 0u;
-            switch (last) {
-#define PKV_SLOT_READ(t) case t: l0 = x0[t]; l1 = x1[t]; break;
-                PKV_SLOTS64(PKV_SLOT_READ)
-#undef PKV_SLOT_READ
-            }
-            switch (sel) {
-            // (the rows are replaced where they are: left to the compiler, the 64 cases become chains of register copies)
-#define PKV_SLOT_SWAP(t) case t: w0 = x0[t]; w1 = x1[t]; \
-    asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "+v"(x0[t]), "+v"(x1[t]) : "v"(l0), "v"(l1)); break;
-                PKV_SLOTS64(PKV_SLOT_SWAP)
-#undef PKV_SLOT_SWAP
-            }
+            // (both halves of the slot arrays are read and written at the index modulo 32, with what they hold unless
+            // the slot lies in them: no branch, so the arrays stay where they are)
+            const int li = last & 31, si = sel & 31;
+            const uint32_t la0 = x0v[0][li], la1 = x1v[0][li], lb0 = x0v[1][li], lb1 = x1v[1][li];
+            const uint32_t l0 = last < 32 ? la0 : lb0, l1 = last < 32 ? la1 : lb1;
+            const uint32_t sa0 = x0v[0][si], sa1 = x1v[0][si], sb0 = x0v[1][si], sb1 = x1v[1][si];
+            const uint32_t w0 = sel < 32 ? sa0 : sb0, w1 = sel < 32 ? sa1 : sb1;
+            x0v[0][si] = sel < 32 ? l0 : sa0;
+            x1v[0][si] = sel < 32 ? l1 : sa1;
+            x0v[1][si] = sel < 32 ? sb0 : l0;
+            x1v[1][si] = sel < 32 ? sb1 : l1;
             if (mem == 0 && tid == 0) perm[row0 + picked] = tok;
             picked++;
             n_alive--;
