@@ -140,7 +140,9 @@ def test_greedy_repacking_matches_restatement(cuda):
     # (the last two have more blocks than the device holds at once as groups of workgroups: 72 blocks of 8 slices and
     # 520 blocks of one slice, so a group walks several blocks)
     for (T, hid, top, bs, pack) in ((64, 16, 4, 16, 4), (128, 48, 2, 64, 16), (256, 2064, 200, 256, 32), (64, 32768, 16, 64, 16),
-                                    (576, 8192, 6, 8, 4), (33280, 128, 6, 64, 16)):
+                                    (576, 8192, 6, 8, 4), (33280, 128, 6, 64, 16),
+                                    # two slices with blocks of 32 tokens; a last slice of 32 channels only; 8-bit codes in two slices
+                                    (96, 4096, 5, 32, 8), (128, 2064, 9, 64, 16), (64, 4096, 256, 64, 32)):
         kc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
         vc = torch.randint(0, top, (T, hid), dtype=torch.uint8, generator=g)
         cases.append((kc, vc, bs, pack, "random %dx%d below %d" % (T, hid, top)))
