@@ -210,7 +210,8 @@ int pkv_median_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
  *   every tie to the earlier token (the reference computes both criteria in fp32 and leaves ties to the backend).
  *   Same outputs as pkv_median_repack.  Blocks of up to 64 tokens keep their rows in registers (any hidden_dim whose
  *   channel slices fit the device at once as one group of workgroups); longer blocks need hidden_dim <= 32768.
- *   With ms_out the call waits for the kernels and also reports a device-side failure of the group exchange. */
+ *   With ms_out the call waits for the kernels and also reports a device-side failure of the group exchange.
+ *   k_out = v_out = NULL: the order only (perm), for the fused encoders' pkv_*_quant_encode_perm. */
 int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k_out, uint8_t *v_out, uint32_t *perm,
                       int ctx_len, int hidden_dim, int block_size, int pack_len, float *ms_out, pkv_stream_t s);
 

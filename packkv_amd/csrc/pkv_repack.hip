@@ -824,8 +824,9 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
                       int ctx_len, int hidden_dim, int block_size, int pack_len, float *ms_out, pkv_stream_t s_) {
     using namespace pkv;
     hipStream_t s = (hipStream_t)s_;
-    PKV_REQUIRE(k_codes && v_codes && k_out && v_out && perm, PKV_ERR_INVALID, "null pointer argument");
+    PKV_REQUIRE(k_codes && v_codes && perm && (k_out != nullptr) == (v_out != nullptr), PKV_ERR_INVALID, "null pointer argument");
     PKV_REQUIRE(k_codes != k_out && v_codes != v_out, PKV_ERR_INVALID, "repacking cannot run in place");
+    const bool rows = k_out != nullptr;               // without outputs: the order only
     PKV_REQUIRE(ctx_len > 0 && hidden_dim > 0 && block_size > 0 && pack_len > 0, PKV_ERR_INVALID, "sizes must be positive");
     PKV_REQUIRE(hidden_dim % 16 == 0 && ((reinterpret_cast<uintptr_t>(k_codes) | reinterpret_cast<uintptr_t>(v_codes) |
                                           reinterpret_cast<uintptr_t>(k_out) | reinterpret_cast<uintptr_t>(v_out)) & 15u) == 0,
@@ -874,7 +875,7 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
         else
             greedy_order_sliced_kernel<kSlicedThreadsNarrow><<<groups * members, kSlicedThreadsNarrow, 0, s>>>(
                 k_codes, v_codes, hidden_dim, block_size, pack_len, nblocks, members, groups, perm, st);
-        gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
+        if (rows) gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
         if (ms_out) {                                  // a timed call has waited for the kernels: look at the error word
@@ -895,7 +896,7 @@ int pkv_greedy_repack(const uint8_t *k_codes, const uint8_t *v_codes, uint8_t *k
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
     greedy_order_kernel<<<nblocks, kGreedyThreads, lds, s>>>(k_codes, v_codes, hidden_dim, block_size, pack_len, perm);
-    gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
+    if (rows) gather_rows_kernel<<<(unsigned)ctx_len, 256, 0, s>>>(k_codes, v_codes, k_out, v_out, perm, block_size, hidden_dim);
     PKV_HIP_CHECK(hipGetLastError());
     return tm.end(ms_out);
 }

@@ -522,6 +522,21 @@ def greedy_repacking(k_codes, v_codes, pack_len=16, block_size=64, timed=False):
     return (k_out, v_out, perm, float(ms.value)) if timed else (k_out, v_out, perm)
 
 
+def greedy_order(k_codes, v_codes, pack_len=16, block_size=64):
+    """perm [ctx] int32 of greedy_repacking without the repacked matrices (for the fused encoders, which gather the
+    rows of K and V themselves)."""
+    _check_code_matrix(k_codes, "k_codes")
+    _check_code_matrix(v_codes, "v_codes")
+    _require(k_codes.shape == v_codes.shape, "K and V code matrices must have one shape")
+    ctx, hidden = k_codes.shape
+    perm = torch.empty(ctx, dtype=torch.int32, device=k_codes.device)
+    with torch.cuda.device(k_codes.device):
+        rc = _lib.load().pkv_greedy_repack(_ptr(k_codes), _ptr(v_codes), None, None, _ptr(perm), ctx, hidden,
+                                           int(block_size), int(pack_len), None, _stream(k_codes.device))
+    _lib.check(rc)
+    return perm
+
+
 def repack_and_encode(k_codes, v_codes, pack_size, repack_method="none", block_size=64):
     """`repack_and_encode` (utils/compute.py:329-357) on code matrices: (k_size_pre, v_size_pre, k_size_aft,
     v_size_aft) in bytes.  repack_method: "none", "median" or "greedy"."""
@@ -560,21 +575,34 @@ def repack_quant_encode(k, v, k_rel, v_rel, repack_method="median", block_size=6
     perm): dicts like k_quant_encode / v_quant_encode -- stream, info, scale, zero in the REPACKED token order, so
     attn_decode takes them as they are (attention does not depend on the order of the cached tokens) -- and the
     permutation [T] int32 (perm[blk * block_size + r] = position inside the block the token at r came from).
-    `fused` (default: whenever it applies -- median method, H <= 8, codes of at most 6 bits) takes the order from V
-    itself (median_order) and runs the fused encoders on the permuted tokens; fused=False goes through the code
-    matrices (quantize, repack, block codec), which gives the same streams."""
+    `fused` (default: whenever it applies -- median or greedy method, H <= 8, codes of at most 6 bits) runs the fused
+    encoders on the permuted tokens: the median order is counted from V itself (median_order, no code matrix at all),
+    the greedy order from the code matrices (greedy_order), which are then dropped instead of being repacked and
+    encoded; fused=False goes through the code matrices (quantize, repack, block codec), which gives the same streams."""
     B, H, T = _check_x(k)
     _require(v.shape == k.shape and v.dtype == k.dtype and v.is_cuda and v.is_contiguous(), "K and V must have one shape")
     _require(T % 128 == 0 and T % block_size == 0, "the token count must be a multiple of 128 and of block_size")
     k_bits, v_bits = k_bits or bits_for_rel(k_rel), v_bits or bits_for_rel(v_rel)
-    can_fuse = repack_method == "median" and H <= 8 and max(k_bits, v_bits) <= 6 and block_size % 64 == 0 and block_size <= 1024
+    can_fuse = (repack_method in ("median", "greedy") and H <= 8 and max(k_bits, v_bits) <= 6 and block_size % 64 == 0 and
+                block_size <= (1024 if repack_method == "median" else 256))
     if fused is None:
         fused = can_fuse
     if fused:
         # the order from V itself, then the fused encoders on the tokens in that order: no code matrix in HBM
-        _require(can_fuse, "the fused path takes the median method, at most 8 KV heads, codes of at most 6 bits and blocks "
-                           "of a multiple of 64 tokens")
-        perm, vs, vz = median_order(v, v_rel, v_bits, block_size, want_params=True)
+        _require(can_fuse, "the fused path takes the median or greedy method, at most 8 KV heads, codes of at most 6 bits and "
+                           "blocks of a multiple of 64 tokens")
+        if repack_method == "median":
+            perm, vs, vz = median_order(v, v_rel, v_bits, block_size, want_params=True)
+        else:
+            ks, kz = quant_params(k, k_rel)
+            vs, vz = quant_params(v, v_rel)
+            kc, kmx = quantize(k, ks, kz)
+            vc, vmx = quantize(v, vs, vz)
+            for mx, bits in ((kmx, k_bits), (vmx, v_bits)):
+                if mx >= (1 << bits):
+                    raise PackKVError(1, "not supported: code %d does not fit bits_len %d" % (mx, bits))
+            perm = greedy_order(kc, vc, 16, block_size)      # the codecs' packs are 16 tokens
+            del kc, vc
         ke = _quant_encode(True, k, k_rel, k_bits, None, None, True, False, perm, block_size)
         ve = _quant_encode(False, v, v_rel, v_bits, None, None, True, False, perm, block_size, (vs, vz))
         return ke, ve, perm

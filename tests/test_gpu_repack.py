@@ -304,6 +304,32 @@ def test_median_repack_inside_the_fused_encode_equals_the_code_matrix_path(cuda,
         ops.repack_quant_encode(k.to(cuda), v.to(cuda), 0.1, 0.0125, "median", fused=True)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_greedy_order_inside_the_fused_encode_equals_the_code_matrix_path(cuda, dtype):
+    """repack_quant_encode("greedy") with the fused encoders gathering the rows in the greedy order (the code matrices
+    serve the order only) against the path that repacks the code matrices and runs the block codec: the same
+    permutation, streams, block_info and parameters; the permutation also against the restatement."""
+    cases = [(2, 4, 512, 0.1, 0.1, 64), (1, 8, 256, 0.2, 0.05, 64), (1, 2, 512, 0.1, 0.2, 128), (3, 8, 256, 0.1, 0.1, 256)]
+    for n, (B, H, T, k_rel, v_rel, bs) in enumerate(cases):
+        _say("fused greedy case", dtype, B, H, T, k_rel, v_rel, bs)
+        k, v = synth.make_kv(B, H, T, seed=500 + n)
+        g = torch.Generator().manual_seed(600 + n)
+        v = v.float() * 0.4 + torch.randn(1, 1, T, 1, generator=g) * 1.5       # token-wise level shifts: an order that matters
+        k, v = k.to(dtype), v.to(dtype)
+        kd, vd = k.to(cuda), v.to(cuda)
+        kf, vf, pf = ops.repack_quant_encode(kd, vd, k_rel, v_rel, "greedy", bs, fused=True)
+        km, vm, pm = ops.repack_quant_encode(kd, vd, k_rel, v_rel, "greedy", bs, fused=False)
+        assert torch.equal(pf.view(torch.int32), pm.view(torch.int32))
+        assert not torch.equal(pf.view(-1, bs), torch.arange(bs, dtype=torch.int32, device=cuda).expand(T // bs, bs))
+        _same_encoding(kf, km, "K")
+        _same_encoding(vf, vm, "V")
+        cv, _, _ = oq.quant_ints(v, 64, v_rel)
+        ck, _, _ = oq.quant_ints(k, 64, k_rel)
+        blocks = orp.blocks_from_code_matrices(oq.code_matrix(ck).numpy(), oq.code_matrix(cv).numpy(), bs)
+        _, order = orp.greedy_repacking(blocks, 16)
+        assert np.array_equal(pf.cpu().numpy().reshape(-1, bs), order)
+
+
 def test_fused_median_repack_at_the_benchmark_shape(cuda):
     """16 sequences x 8 KV heads x 32768 tokens: the fused path's streams decode (unpack kernels) to codes whose
     every 64-token block is the natural-order block permuted by perm, and the medians along the new order descend."""
