@@ -166,25 +166,32 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
     const int jl = tid >> 7, lt = tid & 127, unit = lt >> 5, t = tid & 31;
     const uint8_t *tile = lds + jl * tile_bytes;
     const int row16 = hid_blk >> 4, n16 = ctx_blk * row16;
+    // the tile of a thread's block of the pair that starts at block j0: four 16-byte pieces (tiles are 8 KiB: 512
+    // pieces over the 128 threads of a block), loaded a pair ahead so that the loads fly while the current pair is
+    // analysed and emitted
+#define PKV_FETCH_PAIR(j0_)                                                                                              \
+    {                                                                                                                    \
+        const uint32_t b = b0 + (uint32_t)min((j0_) + jl, nb - 1); /* clamped: the loads are unconditional */           \
+        const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;                                               \
+        const uint8_t *src = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;                           \
+        const int i0 = min(lt, n16 - 1), i1 = min(lt + 128, n16 - 1), i2 = min(lt + 256, n16 - 1), i3 = min(lt + 384, n16 - 1); \
+        a0 = *reinterpret_cast<const uint4 *>(src + (size_t)(i0 / row16) * hidden_dim + 16 * (i0 % row16));              \
+        a1 = *reinterpret_cast<const uint4 *>(src + (size_t)(i1 / row16) * hidden_dim + 16 * (i1 % row16));              \
+        a2 = *reinterpret_cast<const uint4 *>(src + (size_t)(i2 / row16) * hidden_dim + 16 * (i2 % row16));              \
+        a3 = *reinterpret_cast<const uint4 *>(src + (size_t)(i3 / row16) * hidden_dim + 16 * (i3 % row16));              \
+    }
+    uint4 a0, a1, a2, a3;
+    PKV_FETCH_PAIR(0)
     for (int j0 = 0; j0 < nb; j0 += 2) {
         const int jj = j0 + jl;
         const bool active = jj < nb;
-        const uint32_t b = b0 + (uint32_t)min(jj, nb - 1);            // clamped: the loads are unconditional
-        const uint32_t cb = b / (uint32_t)n_hid, hb = b % (uint32_t)n_hid;
-        const uint8_t *src = codes + (size_t)cb * ctx_blk * hidden_dim + (size_t)hb * hid_blk;
         uint4 *t16 = reinterpret_cast<uint4 *>(lds + jl * tile_bytes);
-        for (int i = lt; i < n16; i += 4 * 128) {                     // four loads in flight
-            uint4 v[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int idx = min(i + 128 * u, n16 - 1);
-                v[u] = *reinterpret_cast<const uint4 *>(src + (size_t)(idx / row16) * hidden_dim + 16 * (idx % row16));
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++)
-                if (i + 128 * u < n16) t16[i + 128 * u] = v[u];
-        }
+        if (lt < n16) t16[lt] = a0;
+        if (lt + 128 < n16) t16[lt + 128] = a1;
+        if (lt + 256 < n16) t16[lt + 256] = a2;
+        if (lt + 384 < n16) t16[lt + 384] = a3;
         __syncthreads();
+        if (j0 + 2 < nb) PKV_FETCH_PAIR(j0 + 2)
         UnitPacks u;
         constexpr bool wide = WIDE;                       // the field-by-field code of the extension widths (W > 4)
         if (active) {
@@ -216,6 +223,7 @@ __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restri
         }
         __syncthreads();
     }
+#undef PKV_FETCH_PAIR
     const uint32_t bytes = blk_off[nb];
     if (tid < 64) {
         const uint64_t off = lookback_offset(st, gidx, bytes, true);
