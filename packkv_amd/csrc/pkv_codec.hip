@@ -143,8 +143,11 @@ constexpr int kPackGroup = 8;
 template <bool IS_K, bool WIDE>
 __global__ void __launch_bounds__(256) pack_group_kernel(const uint8_t *__restrict__ codes, uint8_t *__restrict__ stream,
                                                          uint64_t capacity, uint32_t *__restrict__ info, ScanState *st,
-                                                         int hidden_dim, int ctx_blk, int hid_blk, int W, uint32_t nblocks,
+                                                         int hidden_dim, int /* ctx_blk */, int /* hid_blk */, int W, uint32_t nblocks,
                                                          uint32_t ngroups, const Stagger stagger) {
+    // blocks of four units are 64 tokens x 128 channels (K) or 128 tokens x 64 channels (V): as constants, the tile
+    // offsets of a lane's codes are immediates of its loads instead of an address register each
+    constexpr int ctx_blk = IS_K ? 64 : 128, hid_blk = IS_K ? 128 : 64;
     extern __shared__ __align__(16) uint8_t lds[];         // two code tiles | the group's bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
