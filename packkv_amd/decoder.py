@@ -31,8 +31,10 @@ class DecoderShape:
 
 
 def _rms(x, w, eps):
-    v = x.float()
-    return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+    """RMS norm over the last dimension in fp32, one library kernel (models/qwen3.py:53-58 rounds to the storage
+    dtype before the weight multiply; the two agree wherever the weight is exactly representable times the value,
+    as for the unit weights used here)."""
+    return F.rms_norm(x, (x.size(-1),), w, eps)
 
 
 class ShapedDecoder:
@@ -52,13 +54,17 @@ class ShapedDecoder:
         self.final_norm = one(s.hidden)
         self.blocks = []
         for _ in range(s.layers):
-            self.blocks.append({
-                "in_norm": one(s.hidden), "post_norm": one(s.hidden),
-                "q": w(s.q_heads * s.head_dim, s.hidden), "k": w(s.kv_heads * s.head_dim, s.hidden),
-                "v": w(s.kv_heads * s.head_dim, s.hidden), "o": w(s.hidden, s.q_heads * s.head_dim),
-                "q_norm": one(s.head_dim), "k_norm": one(s.head_dim),
-                "gate": w(s.mlp, s.hidden), "up": w(s.mlp, s.hidden), "down": w(s.hidden, s.mlp),
-            })
+            # q, k, v projections as one weight [Hq*128 + 2*Hkv*128, hidden] and gate, up as one [2*mlp, hidden]:
+            # a decode step is launch-bound around the cache, so every projection pair that shares its input is
+            # one library GEMM
+            blk = {"in_norm": one(s.hidden), "post_norm": one(s.hidden)}
+            blk["qkv"] = torch.cat((w(s.q_heads * s.head_dim, s.hidden), w(s.kv_heads * s.head_dim, s.hidden),
+                                    w(s.kv_heads * s.head_dim, s.hidden)), dim=0)
+            blk["o"] = w(s.hidden, s.q_heads * s.head_dim)
+            blk["q_norm"], blk["k_norm"] = one(s.head_dim), one(s.head_dim)
+            blk["gate_up"] = torch.cat((w(s.mlp, s.hidden), w(s.mlp, s.hidden)), dim=0)
+            blk["down"] = w(s.hidden, s.mlp)
+            self.blocks.append(blk)
         inv = 1.0 / (s.rope_theta ** (torch.arange(0, s.head_dim, 2, device=self.device, dtype=torch.float32) / s.head_dim))
         self.inv_freq = inv
 
@@ -73,6 +79,15 @@ class ShapedDecoder:
         emb = torch.cat((f, f), dim=-1)
         cos, sin = emb.cos().to(self.dtype), emb.sin().to(self.dtype)
         return cos.unsqueeze(0).expand(batch, n, -1), sin.unsqueeze(0).expand(batch, n, -1)
+
+    @staticmethod
+    def _rotate_q(q, cos, sin_signed):
+        """q [B, n, Hq, 128] * cos + rotate_half(q) * sin with the reference's roundings (each product rounded,
+        then the sum; utils/compute.py:35-43): rotate_half(q) * sin = roll(q, 64) * (-sin | sin), sign changes
+        being exact."""
+        t = q * cos.unsqueeze(2)
+        t += torch.roll(q, q.size(-1) // 2, -1) * sin_signed.unsqueeze(2)
+        return t
 
     def _dense_attention(self, q, k, v, scaling):
         """Decode step (one query token): the reference's eager attention (models/llama.py:189-212: fp32 softmax
@@ -102,16 +117,20 @@ class ShapedDecoder:
         cos, sin = self._rotary(pos0, n, B)
         fused = attention == "fused" and n == 1
         scaling = 1.0 / math.sqrt(s.head_dim)
-        h = self.embed[ids]
+        half = s.head_dim // 2
+        sin_signed = torch.cat((-sin[..., :half], sin[..., half:]), dim=-1)
+        nq = s.q_heads * s.head_dim
+        kw = {"cos": cos, "sin": sin}
+        h = self.embed[ids].view(B * n, s.hidden)
         for li, blk in enumerate(self.blocks):
             x = _rms(h, blk["in_norm"], s.rms_eps)
-            q = F.linear(x, blk["q"]).view(B, n, s.q_heads, s.head_dim).transpose(1, 2)
-            k = F.linear(x, blk["k"]).view(B, n, s.kv_heads, s.head_dim).transpose(1, 2)
-            v = F.linear(x, blk["v"]).view(B, n, s.kv_heads, s.head_dim).transpose(1, 2)
+            qkv = F.linear(x, blk["qkv"]).view(B, n, s.q_heads + 2 * s.kv_heads, s.head_dim)
+            q, k, v = qkv[:, :, :s.q_heads], qkv[:, :, s.q_heads:s.q_heads + s.kv_heads], qkv[:, :, s.q_heads + s.kv_heads:]
             if s.head_norm:
                 q, k = _rms(q, blk["q_norm"], s.rms_eps), _rms(k, blk["k_norm"], s.rms_eps)
-            q = q * cos.unsqueeze(1) + rotate_half(q) * sin.unsqueeze(1)
-            kw = {"cos": cos, "sin": sin}
+                v = v.contiguous()                        # the cache reads K and V with one set of strides
+            q = self._rotate_q(q, cos, sin_signed).transpose(1, 2)                 # [B, Hq, n, 128]
+            k, v = k.transpose(1, 2), v.transpose(1, 2)
             if fused:
                 cache.update(k, v, li, kw, return_dense=False)
                 a = cache.attend(q, li, sm_scale=scaling)                          # [B, Hq, 1, 128]
@@ -120,9 +139,11 @@ class ShapedDecoder:
                 a = self._dense_attention(q, kd, vd, scaling)
             if taps is not None:
                 taps.append((q, a))
-            h = h + F.linear(a.transpose(1, 2).reshape(B, n, s.q_heads * s.head_dim), blk["o"])
+            h = torch.addmm(h, a.transpose(1, 2).reshape(B * n, nq), blk["o"].t())
             x = _rms(h, blk["post_norm"], s.rms_eps)
-            h = h + F.linear(F.silu(F.linear(x, blk["gate"])) * F.linear(x, blk["up"]), blk["down"])
+            gu = F.linear(x, blk["gate_up"])
+            h = torch.addmm(h, F.silu(gu[:, :s.mlp]) * gu[:, s.mlp:], blk["down"].t())
+        h = h.view(B, n, s.hidden)
         h = _rms(h[:, -1], self.final_norm, s.rms_eps)
         return F.linear(h, self.lm_head).float()
 
