@@ -522,6 +522,29 @@ __device__ __forceinline__ bool round_all_fast(const TokPar *par) {
     return !__any(sub2 == 0u);
 }
 
+// The codes of a loaded cell (rows xr, the 16 tokens' constants at par) as pairs of 16-bit integers.
+template <int DT>
+__device__ __forceinline__ void cell_quant(const uint2 xr[16], const TokPar *par, uint32_t c01[16], uint32_t c23[16]) {
+    if (DT == PKV_F16 && round_all_fast(par)) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) quant4_f16_fast(xr[k], par[k], c01[k], c23[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+    }
+}
+
+// The four packs of a cell's codes: words, minima, widths.
+__device__ __forceinline__ void cell_build(const uint32_t c01[16], const uint32_t c23[16], UnitPacks &u, uint32_t &cmax) {
+    uint32_t mn01, mn23, len01, len23, mx01, mx23;
+    build_pair(c01, mn01, len01, mx01, u.word[0], u.word[1]);
+    build_pair(c23, mn23, len23, mx23, u.word[2], u.word[3]);
+    const u16x2 m = __builtin_elementwise_max(as_u16x2(mx01), as_u16x2(mx23));
+    cmax = max((uint32_t)m[0], (uint32_t)m[1]);
+    u.mn[0] = mn01 & 0xFFFFu; u.mn[1] = mn01 >> 16; u.mn[2] = mn23 & 0xFFFFu; u.mn[3] = mn23 >> 16;
+    u.len[0] = len01 & 0xFFFFu; u.len[1] = len01 >> 16; u.len[2] = len23 & 0xFFFFu; u.len[3] = len23 >> 16;
+}
+
 // The four packs of a loaded cell (rows xr, the 16 tokens' constants at par): words, minima, widths.
 template <int DT>
 __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par, UnitPacks &u, uint32_t &cmax) {
@@ -590,6 +613,16 @@ __device__ __forceinline__ void build_pair_wide(const uint32_t c[16], uint32_t &
     lo_a = join4(ew[4] & 0xFFFFu, ew[5] & 0xFFFFu, ew[6] & 0xFFFFu, ew[7] & 0xFFFFu, l0);
     hi_b = join4(ew[0] >> 16, ew[1] >> 16, ew[2] >> 16, ew[3] >> 16, l1);
     lo_b = join4(ew[4] >> 16, ew[5] >> 16, ew[6] >> 16, ew[7] >> 16, l1);
+}
+
+__device__ __forceinline__ void cell_build(const uint32_t c01[16], const uint32_t c23[16], UnitPacksW &u, uint32_t &cmax) {
+    uint32_t mn01, mn23, len01, len23, mx01, mx23;
+    build_pair_wide(c01, mn01, len01, mx01, u.lo[0], u.hi[0], u.lo[1], u.hi[1]);
+    build_pair_wide(c23, mn23, len23, mx23, u.lo[2], u.hi[2], u.lo[3], u.hi[3]);
+    const u16x2 m = __builtin_elementwise_max(as_u16x2(mx01), as_u16x2(mx23));
+    cmax = max((uint32_t)m[0], (uint32_t)m[1]);
+    u.mn[0] = mn01 & 0xFFFFu; u.mn[1] = mn01 >> 16; u.mn[2] = mn23 & 0xFFFFu; u.mn[3] = mn23 >> 16;
+    u.len[0] = len01 & 0xFFFFu; u.len[1] = len01 >> 16; u.len[2] = len23 & 0xFFFFu; u.len[3] = len23 >> 16;
 }
 
 template <int DT>
@@ -896,6 +929,187 @@ __device__ __forceinline__ void copy_out32(uint8_t *dst, const uint8_t *src, uin
         reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(src + done)[i];
 }
 
+// Minimum and maximum of every token of a round over a wavefront's cells (fp16).  Lane's cell: rows xr[k] = token
+// k, four channels.  The 16 per-token values of a lane are reduced and transposed at once: each step exchanges half
+// of the registers with the lane 32, 16, 8, 4 positions away and keeps the other half, so the register count halves
+// while the lanes behind a value double -- v_permlane32_swap / v_permlane16_swap trade whole half-wavefronts and
+// rows between two registers, the two steps inside a row are DPP moves under bank masks.  Afterwards lane l holds
+// token l / 4 (all four lanes of a quad the same): ~120 vector instructions instead of a second pass over the rows.
+// (The packed min / max are written as instructions, see pk_min_h; a lane exchange must not read a register that a
+// vector instruction wrote less than two instructions earlier, and the compiler does not see into the assembly, so
+// these carry their own two wait states.)
+template <bool MAX>
+__device__ __forceinline__ f16x2 pk_sel_x(f16x2 a, f16x2 b) {
+    f16x2 r;
+    if (MAX) asm("v_pk_max_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+    else asm("v_pk_min_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+template <bool MAX>
+__device__ __forceinline__ f16x2 swap32_sel(f16x2 a, f16x2 b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, (uint32_t)r[0]), __builtin_bit_cast(f16x2, (uint32_t)r[1]));
+}
+template <bool MAX>
+__device__ __forceinline__ f16x2 swap16_sel(f16x2 a, f16x2 b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, (uint32_t)r[0]), __builtin_bit_cast(f16x2, (uint32_t)r[1]));
+}
+// lanes whose bank is in HI_BANKS keep b and meet the partner's b, the others keep a and meet the partner's a;
+// CTRL_LO / CTRL_HI: how the low / high banks read their partner
+template <bool MAX, int CTRL_LO, int CTRL_HI, int HI_BANKS>
+__device__ __forceinline__ f16x2 row_step_sel(f16x2 a, f16x2 b) {
+    const int ai = __builtin_bit_cast(int, a), bi = __builtin_bit_cast(int, b);
+    const int mine = __builtin_amdgcn_update_dpp(ai, bi, 0xE4, 0xF, HI_BANKS, false);
+    int theirs = __builtin_amdgcn_update_dpp(0, ai, CTRL_LO, 0xF, 0xF ^ HI_BANKS, false);
+    theirs = __builtin_amdgcn_update_dpp(theirs, bi, CTRL_HI, 0xF, HI_BANKS, false);
+    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, mine), __builtin_bit_cast(f16x2, theirs));
+}
+// one side (minimum or maximum) of cell_token_minmax_f16 as packed halves: lane l holds token l / 4, two channel parities
+template <bool MAX>
+__device__ __forceinline__ f16x2 cell_token_side_f16(const uint2 xr[16]) {
+    f16x2 v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) v[k] = pk_sel_x<MAX>(__builtin_bit_cast(f16x2, xr[k].x), __builtin_bit_cast(f16x2, xr[k].y));
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = swap32_sel<MAX>(v[k], v[k + 8]);          // lanes 0..31: token k, lanes 32..63: token k + 8
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = swap16_sel<MAX>(v[k], v[k + 4]);          // row rho: token k + 4 rho
+#pragma unroll
+    for (int k = 0; k < 2; k++) v[k] = row_step_sel<MAX, 0x128, 0x128, 0xC>(v[k], v[k + 2]);   // lanes 8..15 of a row: token k + 2 + 4 rho
+    return row_step_sel<MAX, 0x104, 0x114, 0xA>(v[0], v[1]);                     // banks 1, 3: the odd token; token = lane / 4
+}
+__device__ __forceinline__ void cell_token_minmax_f16(const uint2 xr[16], float &mn, float &mx) {
+    const f16x2 lo = cell_token_side_f16<false>(xr);
+    __builtin_amdgcn_sched_barrier(0);                     // (one side after the other: 16 registers in flight, not 32)
+    const f16x2 hi = cell_token_side_f16<true>(xr);
+    mn = fminf((float)lo[0], (float)lo[1]);
+    mx = fmaxf((float)hi[0], (float)hi[1]);
+    asm("s_nop 1\n\t"
+        "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf"
+        : "+v"(mn), "+v"(mx));
+}
+
+// ---- K, all heads in one workgroup, fp16, x read ONCE as cells --------------------------------
+// The round-major encoder above reads a round's rows twice: once row-wise for the token parameters (the trip that
+// goes to HBM and whose latency every round waits out) and again as cells.  Here a round is read as cells only; the
+// token minima and maxima come from the cell registers (cell_token_minmax_f16: per wavefront, then four partial
+// results per token through LDS, from which every wavefront forms the round's parameters for itself, so a round
+// has one barrier), and the next round's cells are requested as soon as this round's are quantized -- into the same
+// registers -- so that they travel while the packs are formed and emitted.  For 5..8 heads (one group per
+// workgroup), tokens in their own order.  Same stream, parameters and block_info as the round-major kernel.
+template <bool WIDE>
+__global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride, const Stagger stagger) {
+    constexpr int DT = PKV_F16;
+    extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[kSubBlocks + 1];
+    __shared__ __attribute__((aligned(16))) TokPar s_par[4 * 16];       // [wavefront][token of the round]
+    __shared__ float2 s_mm[2][4][16];                                    // [round parity][wavefront][token]: (min, max)
+    const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);
+    if (gidx >= ngroups) return;
+    const int j = tid >> 5, t = tid & 31, wave = tid >> 6, lane = tid & 63;
+    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * 64;
+    const UnitGeom g = unit_geom(W);
+    const bool active = j < H;
+    const int jc = min(j, H - 1);                          // (a repeated head changes no minimum or maximum)
+    const TokPar *my_par = s_par + 16 * wave;
+    uint8_t *blk = gbuf + (size_t)j * bound;
+    uint32_t my_off = 8u;
+    uint32_t cmax_all = 0;
+    const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0) * kHeadDim + 4 * t;
+    uint2 xr[16];
+    cell_load(cells, xr);
+#pragma unroll 1
+    for (int r = 0; r < 4; r++) {
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
+        {
+            float mn, mx;
+            cell_token_minmax_f16(xr, mn, mx);
+            if ((lane & 3) == 0) s_mm[r & 1][wave][lane >> 2] = make_float2(mn, mx);
+        }
+        __syncthreads();
+        if (lane < 16) {
+            const float2 p0 = s_mm[r & 1][0][lane], p1 = s_mm[r & 1][1][lane], p2 = s_mm[r & 1][2][lane], p3 = s_mm[r & 1][3][lane];
+            const float mn = fminf(fminf(p0.x, p1.x), fminf(p2.x, p3.x)), mx = fmaxf(fmaxf(p0.y, p1.y), fmaxf(p2.y, p3.y));
+            const float range = round_t<DT>(mx - mn);
+            const float sc = round_t<DT>(range * rel);
+            const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+            if (wave == 0) {
+                const size_t tok = (size_t)b * par_stride + tok0 + 16 * r + lane;
+                scale[tok] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[tok] = (uint16_t)zb;
+            }
+            s_par[16 * wave + lane] = token_par<DT>(sc, zb, false);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
+        uint32_t c01[16], c23[16];
+        cell_quant<DT>(xr, my_par, c01, c23);
+        if (r < 3) cell_load(cells + (size_t)(r + 1) * 16 * kHeadDim, xr);      // travels while the packs are formed
+        typename PacksOf<WIDE>::type u;
+        uint32_t cmax;
+        cell_build(c01, c23, u, cmax);
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+        pack_offsets(u.len, u.off, u.payload);
+        const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        if (r == 3) {
+            // every block's final size is known before its last unit is written: the group's size is published now
+            if (active && t == 0) blk_off[j + 1] = my_off + usz;
+            if (tid == 0) blk_off[0] = 0;
+            __syncthreads();
+            if (tid == 0) {
+                for (int q = 1; q <= H; q++) blk_off[q] += blk_off[q - 1];
+                lookback_publish(st, gidx, blk_off[H]);
+            }
+        }
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
+            unit_emit_any(blk, my_off, t, g, u);
+            my_off += usz;
+        }
+    }
+    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+    __syncthreads();
+    const uint32_t bytes = blk_off[H];
+    if (tid < 64) {
+        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < H) {
+        info[2 * (size_t)(gidx * (uint32_t)H + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(gidx * (uint32_t)H + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    if (active) copy_out32(stream + off + blk_off[j], blk, my_off, t);
+}
+
 // OR the FB-bit fields f[0..3] of four adjacent lanes 4m..4m+3, slot i, into a unit's LSB-first metadata array
 // (field of lane c, slot i at bit (4c + i) * FB).  The 16 * FB bits of the four lanes start at byte 2 * FB * m.
 __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, const uint32_t f[4]) {
@@ -1153,6 +1367,164 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     }
 }
 
+// ---- V, all heads in one workgroup, fp16, x read ONCE as cells --------------------------------
+// The V counterpart of k_quant_encode_cells_kernel: the 16 wavefronts-halves of the round-major V encoder keep their
+// roles (thread = round parity rp, head j, cell lane t), but an iteration's 32 tokens are read as cells only.  A
+// wavefront holds two heads of one round, so its cell registers give that round's 16 token minima and maxima over
+// its heads; the four wavefronts of a round exchange them through LDS and each forms the round's parameters for
+// itself.  For 5..8 heads, tokens in their own order; same stream, parameters and block_info as the round-major kernel.
+template <bool WIDE>
+__global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride, const Stagger stagger) {
+    constexpr int DT = PKV_F16;
+    extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[17];
+    __shared__ uint32_t s_tot[2][8][4];
+    __shared__ uint16_t s_usz[16][4];
+    __shared__ __attribute__((aligned(16))) TokPar s_par[8 * 16];       // [wavefront][token of its round]
+    __shared__ float2 s_mm[2][8][16];                                    // [iteration parity][wavefront][token]: (min, max)
+    const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = s_idx;
+    if (gidx >= ngroups) return;
+    const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31, wave = tid >> 6, lane = tid & 63;
+    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * 128;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const bool active = j < H;
+    const int jc = min(j, H - 1);
+    const TokPar *my_par = s_par + 16 * wave;
+    const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
+    for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)                 // metadata areas start as zeros
+        reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
+    uint32_t run_off = 0;
+    uint32_t cmax_all = 0;
+    const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0 + 16 * rp) * kHeadDim + 4 * t;
+#pragma unroll 1
+    for (int it = 0; it < 4; it++) {
+        // (no request ahead as in the K kernel: placing the packs holds too many registers to keep 16 rows in flight)
+        uint2 xr[16];
+        cell_load(cells + (size_t)it * 32 * kHeadDim, xr);
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
+        {
+            float mn, mx;
+            cell_token_minmax_f16(xr, mn, mx);
+            if ((lane & 3) == 0) s_mm[it & 1][wave][lane >> 2] = make_float2(mn, mx);
+        }
+        __syncthreads();
+        if (lane < 16) {
+            const int w0 = wave & 4;                                         // the four wavefronts of this round
+            const float2 p0 = s_mm[it & 1][w0][lane], p1 = s_mm[it & 1][w0 + 1][lane], p2 = s_mm[it & 1][w0 + 2][lane],
+                         p3 = s_mm[it & 1][w0 + 3][lane];
+            const float mn = fminf(fminf(p0.x, p1.x), fminf(p2.x, p3.x)), mx = fmaxf(fmaxf(p0.y, p1.y), fmaxf(p2.y, p3.y));
+            const float range = round_t<DT>(mx - mn);
+            const float sc = round_t<DT>(range * rel);
+            const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
+            if ((wave & 3) == 0) {
+                const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + 16 * rp + lane;
+                scale[tok] = (uint16_t)T16<DT>::to_bits(sc);
+                zero[tok] = (uint16_t)zb;
+            }
+            s_par[16 * wave + lane] = token_par<DT>(sc, zb, false);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
+        uint32_t c01[16], c23[16];
+        cell_quant<DT>(xr, my_par, c01, c23);
+        typename PacksOf<WIDE>::type u;
+        uint32_t cmax;
+        cell_build(c01, c23, u, cmax);
+        const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
+        uint32_t inc = pb;
+#pragma unroll
+        for (int d = 1; d < 8; d <<= 1) {
+            const uint32_t up = __shfl_up(inc, d, 8);
+            if (m >= d) inc += up;
+        }
+        const uint32_t tot = __shfl(inc, 7, 8);
+        if (m == 0) s_tot[rp][j][t >> 3] = tot;
+        __syncthreads();
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+        const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
+        if (it == 3) {
+            if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
+            __syncthreads();
+            if (tid == 0) {
+                uint32_t run = 0;
+                for (int q = 0; q < 2 * H; q++) {
+                    blk_off[q] = run;
+                    run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
+                }
+                blk_off[2 * H] = run;
+                lookback_publish(st, gidx, run);
+            }
+        }
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            const int sg = it >> 1, slot = 2 * (it & 1) + rp;
+            uint8_t *unit = gbuf + (size_t)(blkid * 4 + 2 * w + sg) * unit_slot;
+            meta_or4(unit, m, g.W, slot, u.mn);
+            meta_or4(unit + g.mins_bytes, m, g.LB, slot, u.len);
+            uint32_t o = meta + run_off + (rp ? tot_even : 0u) + (inc - pb);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                put_pack(reinterpret_cast<uint16_t *>(unit + o), u, k);
+                o += 2u * u.len[k];
+            }
+        }
+        run_off += tot_even + tot_odd;
+        if (it & 1) {
+            if (it == 1 && active && rp == 0 && m == 0) s_usz[blkid][2 * w] = (uint16_t)(meta + run_off);
+            run_off = 0;
+        }
+        // (s_tot is rewritten only after the next iteration's first barrier, which every thread reaches after these reads)
+    }
+    if (__any(cmax_all >= (1u << W))) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+    __syncthreads();
+    const int nblk = 2 * H;
+    const uint32_t bytes = blk_off[nblk];
+    if (tid < 64) {
+        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < nblk) {
+        info[2 * (size_t)(gidx * (uint32_t)nblk + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(gidx * (uint32_t)nblk + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    const int q = tid >> 5;
+    if (q < nblk) {
+        uint8_t *dst = stream + off + blk_off[q];
+        uint32_t cum = 0;
+#pragma unroll
+        for (int un = 0; un < 4; un++) {
+            const uint32_t n = s_usz[q][un];
+            copy_out32(dst + 8 + cum, gbuf + (size_t)(q * 4 + un) * unit_slot, n, t);
+            cum += n;
+            if (t == un) reinterpret_cast<uint16_t *>(dst)[un] = (uint16_t)cum;
+        }
+    }
+}
+
 // ---- per-token median of the V codes, straight from V -----------------------------------------------------------
 // `median_repacking` (utils/compute.py:262-270) orders the tokens of a block by the lower median of each token's
 // V codes over ALL channels of all sequences and heads.  This kernel gets those medians without a code matrix: a
@@ -1384,10 +1756,19 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             Stagger sg;
-            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
-            kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
-                                           stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
-                                           (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all, 1, nullptr);
+            if (!perm && dtype == PKV_F16 && gpw == 1) {        // fp16 in its own token order: x read once, as cells
+                auto cells = bits > 4 ? v_quant_encode_cells_kernel<true> : v_quant_encode_cells_kernel<false>;
+                PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(cells),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 512, lds, ngroups, &sg))) return rc;
+                cells<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
+                                                stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, sg);
+            } else {
+                if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
+                kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
+                                               stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
+                                               (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all, 1, nullptr);
+            }
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
             // up to four heads: 8 / H groups to a workgroup, so that all eight half-wavefronts have a block
@@ -1403,9 +1784,16 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
                                          : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
                                                              : k_quant_encode_rounds_kernel<PKV_BF16, false, false>));
             Stagger sg;
-            if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
-            kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                       capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub, 1, nullptr);
+            if (!perm && dtype == PKV_F16 && gpw == 1) {        // fp16 in its own token order: x read once, as cells
+                auto cells = bits > 4 ? k_quant_encode_cells_kernel<true> : k_quant_encode_cells_kernel<false>;
+                if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 256, lds, nwg, &sg))) return rc;
+                cells<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                            capacity, info, st, bits, nwg, slot, base, par_stride, sg);
+            } else {
+                if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
+                kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
+                                           capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub, 1, nullptr);
+            }
         } else if (IS_K) {                           // more than eight heads: runs of eight, one workgroup each, that exchange their minima and maxima
             const uint32_t slot = (bound + 15u) & ~15u;
             const uint32_t lds = (uint32_t)kSubBlocks * slot + 32u;
