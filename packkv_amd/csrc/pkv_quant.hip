@@ -1137,6 +1137,20 @@ __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, con
     if (FB > 2) atomicOr(w + 1, (uint32_t)(v >> 32));
 }
 
+// Inclusive prefix sum over each run of eight lanes (m = lane % 8) on the DPP data path; `total` receives the run's
+// sum in all eight lanes.
+__device__ __forceinline__ uint32_t oct_incl_scan(uint32_t v, int m, uint32_t &total) {
+    uint32_t x = v;
+    const uint32_t u1 = __builtin_amdgcn_update_dpp(0u, x, 0x111, 0xF, 0xF, true);      // row_shr:1
+    x += m >= 1 ? u1 : 0u;
+    const uint32_t u2 = __builtin_amdgcn_update_dpp(0u, x, 0x112, 0xF, 0xF, true);      // row_shr:2
+    x += m >= 2 ? u2 : 0u;
+    x += __builtin_amdgcn_update_dpp(0u, x, 0x114, 0xF, 0xA, false);                    // row_shr:4 into lanes 4..7 of a run
+    const uint32_t last = __builtin_amdgcn_update_dpp(0u, x, 0xFF, 0xF, 0xF, false);    // every quad: its lane 3
+    total = __builtin_amdgcn_update_dpp(last, last, 0x104, 0xF, 0x5, false);            // first quad of a run: the second quad's
+    return x;
+}
+
 // ---- V, all heads in one workgroup: round-major single trip over x --------------------------
 // For H <= 8 one workgroup of 512 threads owns the 2 H blocks of a (128-token context block, sequence) group and
 // goes through it 32 tokens (two rounds) at a time: read the rows of all heads for the token parameters, then at
@@ -1283,13 +1297,8 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         cell_packs<DT>(xr, my_par, u, cmax);
         // bytes of the thread's four packs, their offsets inside the (unit, slot) and the slot's total
         const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
-        uint32_t inc = pb;
-#pragma unroll
-        for (int d = 1; d < 8; d <<= 1) {
-            const uint32_t up = __shfl_up(inc, d, 8);
-            if (m >= d) inc += up;
-        }
-        const uint32_t tot = __shfl(inc, 7, 8);
+        uint32_t tot;
+        const uint32_t inc = oct_incl_scan(pb, m, tot);
         if (m == 0) s_tot[rp][j][t >> 3] = tot;
         __syncthreads();                                  // s_par is rewritten by the next iteration; s_tot is published
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
@@ -1444,17 +1453,18 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
         uint32_t cmax;
         cell_build(c01, c23, u, cmax);
         const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
-        uint32_t inc = pb;
-#pragma unroll
-        for (int d = 1; d < 8; d <<= 1) {
-            const uint32_t up = __shfl_up(inc, d, 8);
-            if (m >= d) inc += up;
-        }
-        const uint32_t tot = __shfl(inc, 7, 8);
+        uint32_t tot;
+        const uint32_t inc = oct_incl_scan(pb, m, tot);
         if (m == 0) s_tot[rp][j][t >> 3] = tot;
+#ifndef PKV_PROBE_NOB2
         __syncthreads();
+#endif
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+#ifdef PKV_PROBE_NOB2
+        const uint32_t tot_even = tot, tot_odd = tot;
+#else
         const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
+#endif
         if (it == 3) {
             if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
             __syncthreads();
