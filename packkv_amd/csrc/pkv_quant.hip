@@ -929,7 +929,7 @@ __device__ __forceinline__ void copy_out32(uint8_t *dst, const uint8_t *src, uin
         reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(src + done)[i];
 }
 
-// Minimum and maximum of every token of a round over a wavefront's cells (fp16).  Lane's cell: rows xr[k] = token
+// Minimum and maximum of every token of a round over a wavefront's cells.  Lane's cell: rows xr[k] = token
 // k, four channels.  The 16 per-token values of a lane are reduced and transposed at once: each step exchanges half
 // of the registers with the lane 32, 16, 8, 4 positions away and keeps the other half, so the register count halves
 // while the lanes behind a value double -- v_permlane32_swap / v_permlane16_swap trade whole half-wavefronts and
@@ -938,53 +938,70 @@ __device__ __forceinline__ void copy_out32(uint8_t *dst, const uint8_t *src, uin
 // (The packed min / max are written as instructions, see pk_min_h; a lane exchange must not read a register that a
 // vector instruction wrote less than two instructions earlier, and the compiler does not see into the assembly, so
 // these carry their own two wait states.)
-template <bool MAX>
-__device__ __forceinline__ f16x2 pk_sel_x(f16x2 a, f16x2 b) {
-    f16x2 r;
-    if (MAX) asm("v_pk_max_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
-    else asm("v_pk_min_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+// KEYS: the operands are order keys of bf16 values (bf16_keys), compared as signed 16-bit integers.
+template <bool MAX, bool KEYS>
+__device__ __forceinline__ uint32_t pk_sel_x(uint32_t a, uint32_t b) {
+    uint32_t r;
+    if (KEYS) {
+        if (MAX) asm("v_pk_max_i16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+        else asm("v_pk_min_i16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+    } else {
+        if (MAX) asm("v_pk_max_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+        else asm("v_pk_min_f16 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(a), "v"(b));
+    }
     return r;
 }
-template <bool MAX>
-__device__ __forceinline__ f16x2 swap32_sel(f16x2 a, f16x2 b) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
-    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, (uint32_t)r[0]), __builtin_bit_cast(f16x2, (uint32_t)r[1]));
+// bf16 has no packed min / max: both halves of a word become 16-bit integers that order like the values (negative
+// values have their magnitude bits flipped); the map is its own inverse.
+__device__ __forceinline__ uint32_t bf16_keys(uint32_t w) {
+    typedef short i16x2 __attribute__((ext_vector_type(2)));
+    const i16x2 v = __builtin_bit_cast(i16x2, w);
+    const i16x2 m = (v >> (short)15) & (short)0x7FFF;
+    return __builtin_bit_cast(uint32_t, (i16x2)(v ^ m));
 }
-template <bool MAX>
-__device__ __forceinline__ f16x2 swap16_sel(f16x2 a, f16x2 b) {
-    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
-    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, (uint32_t)r[0]), __builtin_bit_cast(f16x2, (uint32_t)r[1]));
+template <bool MAX, bool KEYS>
+__device__ __forceinline__ uint32_t swap32_sel(uint32_t a, uint32_t b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    return pk_sel_x<MAX, KEYS>((uint32_t)r[0], (uint32_t)r[1]);
+}
+template <bool MAX, bool KEYS>
+__device__ __forceinline__ uint32_t swap16_sel(uint32_t a, uint32_t b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+    return pk_sel_x<MAX, KEYS>((uint32_t)r[0], (uint32_t)r[1]);
 }
 // lanes whose bank is in HI_BANKS keep b and meet the partner's b, the others keep a and meet the partner's a;
 // CTRL_LO / CTRL_HI: how the low / high banks read their partner
-template <bool MAX, int CTRL_LO, int CTRL_HI, int HI_BANKS>
-__device__ __forceinline__ f16x2 row_step_sel(f16x2 a, f16x2 b) {
-    const int ai = __builtin_bit_cast(int, a), bi = __builtin_bit_cast(int, b);
-    const int mine = __builtin_amdgcn_update_dpp(ai, bi, 0xE4, 0xF, HI_BANKS, false);
-    int theirs = __builtin_amdgcn_update_dpp(0, ai, CTRL_LO, 0xF, 0xF ^ HI_BANKS, false);
-    theirs = __builtin_amdgcn_update_dpp(theirs, bi, CTRL_HI, 0xF, HI_BANKS, false);
-    return pk_sel_x<MAX>(__builtin_bit_cast(f16x2, mine), __builtin_bit_cast(f16x2, theirs));
+template <bool MAX, bool KEYS, int CTRL_LO, int CTRL_HI, int HI_BANKS>
+__device__ __forceinline__ uint32_t row_step_sel(uint32_t a, uint32_t b) {
+    const int mine = __builtin_amdgcn_update_dpp((int)a, (int)b, 0xE4, 0xF, HI_BANKS, false);
+    int theirs = __builtin_amdgcn_update_dpp(0, (int)a, CTRL_LO, 0xF, 0xF ^ HI_BANKS, false);
+    theirs = __builtin_amdgcn_update_dpp(theirs, (int)b, CTRL_HI, 0xF, HI_BANKS, false);
+    return pk_sel_x<MAX, KEYS>((uint32_t)mine, (uint32_t)theirs);
 }
-// one side (minimum or maximum) of cell_token_minmax_f16 as packed halves: lane l holds token l / 4, two channel parities
-template <bool MAX>
-__device__ __forceinline__ f16x2 cell_token_side_f16(const uint2 xr[16]) {
-    f16x2 v[16];
+// one side (minimum or maximum) of cell_token_minmax as packed halves: lane l holds token l / 4, two channel parities
+template <int DT, bool MAX>
+__device__ __forceinline__ uint32_t cell_token_side(const uint2 xr[16]) {
+    constexpr bool KEYS = DT != PKV_F16;
+    uint32_t v[16];
 #pragma unroll
-    for (int k = 0; k < 16; k++) v[k] = pk_sel_x<MAX>(__builtin_bit_cast(f16x2, xr[k].x), __builtin_bit_cast(f16x2, xr[k].y));
+    for (int k = 0; k < 16; k++)
+        v[k] = KEYS ? pk_sel_x<MAX, true>(bf16_keys(xr[k].x), bf16_keys(xr[k].y)) : pk_sel_x<MAX, false>(xr[k].x, xr[k].y);
 #pragma unroll
-    for (int k = 0; k < 8; k++) v[k] = swap32_sel<MAX>(v[k], v[k + 8]);          // lanes 0..31: token k, lanes 32..63: token k + 8
+    for (int k = 0; k < 8; k++) v[k] = swap32_sel<MAX, KEYS>(v[k], v[k + 8]);          // lanes 0..31: token k, lanes 32..63: token k + 8
 #pragma unroll
-    for (int k = 0; k < 4; k++) v[k] = swap16_sel<MAX>(v[k], v[k + 4]);          // row rho: token k + 4 rho
+    for (int k = 0; k < 4; k++) v[k] = swap16_sel<MAX, KEYS>(v[k], v[k + 4]);          // row rho: token k + 4 rho
 #pragma unroll
-    for (int k = 0; k < 2; k++) v[k] = row_step_sel<MAX, 0x128, 0x128, 0xC>(v[k], v[k + 2]);   // lanes 8..15 of a row: token k + 2 + 4 rho
-    return row_step_sel<MAX, 0x104, 0x114, 0xA>(v[0], v[1]);                     // banks 1, 3: the odd token; token = lane / 4
+    for (int k = 0; k < 2; k++) v[k] = row_step_sel<MAX, KEYS, 0x128, 0x128, 0xC>(v[k], v[k + 2]);   // lanes 8..15 of a row: token k + 2 + 4 rho
+    const uint32_t r = row_step_sel<MAX, KEYS, 0x104, 0x114, 0xA>(v[0], v[1]);         // banks 1, 3: the odd token; token = lane / 4
+    return KEYS ? bf16_keys(r) : r;
 }
-__device__ __forceinline__ void cell_token_minmax_f16(const uint2 xr[16], float &mn, float &mx) {
-    const f16x2 lo = cell_token_side_f16<false>(xr);
+template <int DT>
+__device__ __forceinline__ void cell_token_minmax(const uint2 xr[16], float &mn, float &mx) {
+    const uint32_t lo = cell_token_side<DT, false>(xr);
     __builtin_amdgcn_sched_barrier(0);                     // (one side after the other: 16 registers in flight, not 32)
-    const f16x2 hi = cell_token_side_f16<true>(xr);
-    mn = fminf((float)lo[0], (float)lo[1]);
-    mx = fmaxf((float)hi[0], (float)hi[1]);
+    const uint32_t hi = cell_token_side<DT, true>(xr);
+    mn = fminf(T16<DT>::from_bits(lo & 0xFFFFu), T16<DT>::from_bits(lo >> 16));
+    mx = fmaxf(T16<DT>::from_bits(hi & 0xFFFFu), T16<DT>::from_bits(hi >> 16));
     asm("s_nop 1\n\t"
         "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
         "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
@@ -994,20 +1011,20 @@ __device__ __forceinline__ void cell_token_minmax_f16(const uint2 xr[16], float 
         : "+v"(mn), "+v"(mx));
 }
 
-// ---- K, all heads in one workgroup, fp16, x read ONCE as cells --------------------------------
+// ---- K, all heads in one workgroup, x read ONCE as cells ----------------------------------------
 // The round-major encoder above reads a round's rows twice: once row-wise for the token parameters (the trip that
 // goes to HBM and whose latency every round waits out) and again as cells.  Here a round is read as cells only; the
-// token minima and maxima come from the cell registers (cell_token_minmax_f16: per wavefront, then four partial
+// token minima and maxima come from the cell registers (cell_token_minmax: per wavefront, then four partial
 // results per token through LDS, from which every wavefront forms the round's parameters for itself, so a round
 // has one barrier), and the next round's cells are requested as soon as this round's are quantized -- into the same
 // registers -- so that they travel while the packs are formed and emitted.  For 5..8 heads (one group per
-// workgroup), tokens in their own order.  Same stream, parameters and block_info as the round-major kernel.
-template <bool WIDE>
+// workgroup); PERM as in the round-major kernel.  Same stream, parameters and block_info as that kernel.
+template <int DT, bool WIDE, bool PERM>
 __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride, const Stagger stagger) {
-    constexpr int DT = PKV_F16;
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
+    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1031,14 +1048,26 @@ __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
     uint32_t my_off = 8u;
     uint32_t cmax_all = 0;
     const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0) * kHeadDim + 4 * t;
+    // PERM: the rows of a round are tokens perm[...] of the repacking block that holds this context block
+    const uint16_t *pseq = x + (((size_t)b * H) * T + (tok0 / (size_t)(PERM ? perm_block : 1)) * (size_t)(PERM ? perm_block : 1)) * kHeadDim;
+    const uint32_t plane = (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2);
+    // (bf16 with the wide packs would need more than 128 registers to keep a round in flight: it asks at the top)
+    constexpr bool AHEAD = !(WIDE && DT != PKV_F16);
     uint2 xr[16];
-    cell_load(cells, xr);
+    if (AHEAD) {
+        if (PERM) cell_load_rows(pseq, perm + tok0, (uint32_t)perm_block - 1u, plane, xr);
+        else cell_load(cells, xr);
+    }
 #pragma unroll 1
     for (int r = 0; r < 4; r++) {
+        if (!AHEAD) {
+            if (PERM) cell_load_rows(pseq, perm + tok0 + 16 * r, (uint32_t)perm_block - 1u, plane, xr);
+            else cell_load(cells + (size_t)r * 16 * kHeadDim, xr);
+        }
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             float mn, mx;
-            cell_token_minmax_f16(xr, mn, mx);
+            cell_token_minmax<DT>(xr, mn, mx);
             if ((lane & 3) == 0) s_mm[r & 1][wave][lane >> 2] = make_float2(mn, mx);
         }
         __syncthreads();
@@ -1061,7 +1090,10 @@ __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         uint32_t c01[16], c23[16];
         cell_quant<DT>(xr, my_par, c01, c23);
-        if (r < 3) cell_load(cells + (size_t)(r + 1) * 16 * kHeadDim, xr);      // travels while the packs are formed
+        if (AHEAD && r < 3) {                              // travels while the packs are formed
+            if (PERM) cell_load_rows(pseq, perm + tok0 + 16 * (r + 1), (uint32_t)perm_block - 1u, plane, xr);
+            else cell_load(cells + (size_t)(r + 1) * 16 * kHeadDim, xr);
+        }
         typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_build(c01, c23, u, cmax);
@@ -1376,18 +1408,17 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     }
 }
 
-// ---- V, all heads in one workgroup, fp16, x read ONCE as cells --------------------------------
+// ---- V, all heads in one workgroup, x read ONCE as cells ----------------------------------------
 // The V counterpart of k_quant_encode_cells_kernel: the 16 wavefronts-halves of the round-major V encoder keep their
 // roles (thread = round parity rp, head j, cell lane t), but an iteration's 32 tokens are read as cells only.  A
 // wavefront holds two heads of one round, so its cell registers give that round's 16 token minima and maxima over
 // its heads; the four wavefronts of a round exchange them through LDS and each forms the round's parameters for
 // itself.  For 5..8 heads, tokens in their own order; same stream, parameters and block_info as the round-major kernel.
-template <bool WIDE>
+template <int DT, bool WIDE>
 __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride, const Stagger stagger) {
-    constexpr int DT = PKV_F16;
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1424,7 +1455,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             float mn, mx;
-            cell_token_minmax_f16(xr, mn, mx);
+            cell_token_minmax<DT>(xr, mn, mx);
             if ((lane & 3) == 0) s_mm[it & 1][wave][lane >> 2] = make_float2(mn, mx);
         }
         __syncthreads();
@@ -1766,8 +1797,9 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             Stagger sg;
-            if (!perm && dtype == PKV_F16 && gpw == 1) {        // fp16 in its own token order: x read once, as cells
-                auto cells = bits > 4 ? v_quant_encode_cells_kernel<true> : v_quant_encode_cells_kernel<false>;
+            if (!perm && gpw == 1) {                // tokens in their own order: x read once, as cells
+                auto cells = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, true> : v_quant_encode_cells_kernel<PKV_BF16, true>)
+                                      : (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, false> : v_quant_encode_cells_kernel<PKV_BF16, false>);
                 PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(cells),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
                 if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 512, lds, ngroups, &sg))) return rc;
@@ -1785,24 +1817,29 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             const int gpw = (H <= 4 && !perm) ? kSubBlocks / H : 1;
             const uint32_t nwg = (nsub + (uint32_t)gpw - 1u) / (uint32_t)gpw;
             const uint32_t lds = (uint32_t)(gpw * H) * slot + 32u;
-            auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, true>
-                                                             : k_quant_encode_rounds_kernel<PKV_BF16, true, true>)
-                                         : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, true>
-                                                             : k_quant_encode_rounds_kernel<PKV_BF16, false, true>))
-                             : (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false>
-                                                             : k_quant_encode_rounds_kernel<PKV_BF16, true, false>)
-                                         : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
-                                                             : k_quant_encode_rounds_kernel<PKV_BF16, false, false>));
+            // (a token order always comes with gpw == 1, i.e. the cells kernel: the round-major kernel serves groups of
+            // up to four heads in their own order)
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true, false>)
+                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false, false>);
             Stagger sg;
-            if (!perm && dtype == PKV_F16 && gpw == 1) {        // fp16 in its own token order: x read once, as cells
-                auto cells = bits > 4 ? k_quant_encode_cells_kernel<true> : k_quant_encode_cells_kernel<false>;
+            if (gpw == 1) {                         // five to eight heads: x read once, as cells
+                auto cells = perm ? (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, true, true>
+                                                                  : k_quant_encode_cells_kernel<PKV_BF16, true, true>)
+                                              : (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, false, true>
+                                                                  : k_quant_encode_cells_kernel<PKV_BF16, false, true>))
+                                  : (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, true, false>
+                                                                  : k_quant_encode_cells_kernel<PKV_BF16, true, false>)
+                                              : (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, false, false>
+                                                                  : k_quant_encode_cells_kernel<PKV_BF16, false, false>));
                 if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 256, lds, nwg, &sg))) return rc;
                 cells<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                            capacity, info, st, bits, nwg, slot, base, par_stride, sg);
+                                            capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg);
             } else {
                 if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
                 kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                           capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, gpw, nsub, 1, nullptr);
+                                           capacity, info, st, bits, nwg, slot, base, par_stride, nullptr, 0, sg, gpw, nsub, 1, nullptr);
             }
         } else if (IS_K) {                           // more than eight heads: runs of eight, one workgroup each, that exchange their minima and maxima
             const uint32_t slot = (bound + 15u) & ~15u;
