@@ -193,7 +193,9 @@ __device__ __forceinline__ uint32_t pk_u16(u16x2 v) { return __builtin_bit_cast(
 __device__ __forceinline__ u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
 
 // codes of four adjacent channels of one token as two pairs of 16-bit integers
-template <int DT>
+// (UNIFORM: every lane of the wavefront holds the same token constants, so the choice of the sequence is a uniform
+// branch; otherwise each lane chooses for itself)
+template <int DT, bool UNIFORM = true>
 __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01, uint32_t &c23) {
     if (DT == PKV_F16) {
         const f16x2 x01 = __builtin_bit_cast(f16x2, xw.x), x23 = __builtin_bit_cast(f16x2, xw.y);
@@ -205,8 +207,7 @@ __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01,
         };
         const f16x2 h01 = {quot(x01[0]), quot(x01[1])}, h23 = {quot(x23[0]), quot(x23[1])};
         const f16x2 add = __builtin_bit_cast(f16x2, tp.add2);
-        // every lane of the wavefront holds the same token constants: a uniform branch
-        if (__builtin_amdgcn_readfirstlane(tp.sub2) != 0u) {
+        if ((UNIFORM ? (uint32_t)__builtin_amdgcn_readfirstlane(tp.sub2) : tp.sub2) != 0u) {
             const u16x2 sub = as_u16x2(tp.sub2);
             c01 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h01 + add)) - sub));
             c23 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h23 + add)) - sub));
@@ -216,7 +217,7 @@ __device__ __forceinline__ void quant4(uint2 xw, const TokPar tp, uint32_t &c01,
             c01 = __builtin_bit_cast(uint32_t, (f16x2)(d01 + magic)) & 0x00FF00FFu;
             c23 = __builtin_bit_cast(uint32_t, (f16x2)(d23 + magic)) & 0x00FF00FFu;
         }
-    } else if (__builtin_amdgcn_readfirstlane(tp.sub2) != 0u) {
+    } else if ((UNIFORM ? (uint32_t)__builtin_amdgcn_readfirstlane(tp.sub2) : tp.sub2) != 0u) {
         // bf16, zero point of moderate size: the same three-instruction quotient (a quotient of two 8-bit
         // significands is either exactly a bf16 rounding midpoint or at least 2^-17 away from every one), rounded to
         // bf16 by the hardware conversion; rint(h) and rint(h) - zero are then exact in fp32 (bf16 values of 256 and
@@ -523,14 +524,14 @@ __device__ __forceinline__ bool round_all_fast(const TokPar *par) {
 }
 
 // The codes of a loaded cell (rows xr, the 16 tokens' constants at par) as pairs of 16-bit integers.
-template <int DT>
+template <int DT, bool UNIFORM = true>
 __device__ __forceinline__ void cell_quant(const uint2 xr[16], const TokPar *par, uint32_t c01[16], uint32_t c23[16]) {
     if (DT == PKV_F16 && round_all_fast(par)) {
 #pragma unroll
         for (int k = 0; k < 16; k++) quant4_f16_fast(xr[k], par[k], c01[k], c23[k]);
     } else {
 #pragma unroll
-        for (int k = 0; k < 16; k++) quant4<DT>(xr[k], par[k], c01[k], c23[k]);
+        for (int k = 0; k < 16; k++) quant4<DT, UNIFORM>(xr[k], par[k], c01[k], c23[k]);
     }
 }
 
@@ -1011,6 +1012,42 @@ __device__ __forceinline__ void cell_token_minmax(const uint2 xr[16], float &mn,
         : "+v"(mn), "+v"(mx));
 }
 
+// The same for a wavefront whose two halves hold different rounds (lanes 0..31 the tokens of one round, lanes 32..63
+// those of the next): the reduction stays inside the halves -- rows, then 8, 4 and 2 lanes -- and lane l ends up
+// with token l / 2 of the 32.
+template <int DT, bool MAX>
+__device__ __forceinline__ uint32_t cell_token_side_halves(const uint2 xr[16], bool odd_pair) {
+    constexpr bool KEYS = DT != PKV_F16;
+    uint32_t v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+        v[k] = KEYS ? pk_sel_x<MAX, true>(bf16_keys(xr[k].x), bf16_keys(xr[k].y)) : pk_sel_x<MAX, false>(xr[k].x, xr[k].y);
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = swap16_sel<MAX, KEYS>(v[k], v[k + 8]);          // odd rows: token k + 8
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = row_step_sel<MAX, KEYS, 0x128, 0x128, 0xC>(v[k], v[k + 4]);   // lanes 8..15 of a row: + 4
+#pragma unroll
+    for (int k = 0; k < 2; k++) v[k] = row_step_sel<MAX, KEYS, 0x104, 0x114, 0xA>(v[k], v[k + 2]);   // banks 1, 3: + 2
+    // lanes 2, 3 of a quad: + 1 (no bank mask reaches inside a quad: selects, and the exchange as a quad permute)
+    const uint32_t mine = odd_pair ? v[1] : v[0], send = odd_pair ? v[0] : v[1];
+    const uint32_t theirs = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0x4E, 0xF, 0xF, false);
+    const uint32_t r = pk_sel_x<MAX, KEYS>(mine, theirs);
+    return KEYS ? bf16_keys(r) : r;
+}
+template <int DT>
+__device__ __forceinline__ void cell_token_minmax_halves(const uint2 xr[16], float &mn, float &mx) {
+    const bool odd_pair = (threadIdx.x & 2) != 0;
+    const uint32_t lo = cell_token_side_halves<DT, false>(xr, odd_pair);
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t hi = cell_token_side_halves<DT, true>(xr, odd_pair);
+    mn = fminf(T16<DT>::from_bits(lo & 0xFFFFu), T16<DT>::from_bits(lo >> 16));
+    mx = fmaxf(T16<DT>::from_bits(hi & 0xFFFFu), T16<DT>::from_bits(hi >> 16));
+    asm("s_nop 1\n\t"
+        "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"
+        : "+v"(mn), "+v"(mx));
+}
+
 // ---- K, all heads in one workgroup, x read ONCE as cells ----------------------------------------
 // The round-major encoder above reads a round's rows twice: once row-wise for the token parameters (the trip that
 // goes to HBM and whose latency every round waits out) and again as cells.  Here a round is read as cells only; the
@@ -1409,11 +1446,14 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
 }
 
 // ---- V, all heads in one workgroup, x read ONCE as cells ----------------------------------------
-// The V counterpart of k_quant_encode_cells_kernel: the 16 wavefronts-halves of the round-major V encoder keep their
-// roles (thread = round parity rp, head j, cell lane t), but an iteration's 32 tokens are read as cells only.  A
-// wavefront holds two heads of one round, so its cell registers give that round's 16 token minima and maxima over
-// its heads; the four wavefronts of a round exchange them through LDS and each forms the round's parameters for
-// itself.  For 5..8 heads, tokens in their own order; same stream, parameters and block_info as the round-major kernel.
+// The V counterpart of k_quant_encode_cells_kernel: the threads keep the roles of the round-major V encoder (round
+// parity rp, head j, cell lane t), but an iteration's 32 tokens are read as cells only, and a wavefront is ONE head
+// with both rounds of the iteration (lanes 0..31 the even round, lanes 32..63 the odd one).  Everything a head's
+// blocks need from each other -- the payload bytes the even round puts in front of the odd one -- is then an
+// exchange between the halves of a wavefront, and the only thing wavefronts share is the token minima and maxima:
+// each forms those of its head from the cell registers, the eight partial results per token go through LDS, and
+// every wavefront forms the 32 tokens' parameters for itself.  One barrier per iteration.  For 5..8 heads, tokens
+// in their own order; same stream, parameters and block_info as the round-major kernel.
 template <int DT, bool WIDE>
 __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
@@ -1423,24 +1463,23 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
     __shared__ uint32_t blk_off[17];
-    __shared__ uint32_t s_tot[2][8][4];
     __shared__ uint16_t s_usz[16][4];
-    __shared__ __attribute__((aligned(16))) TokPar s_par[8 * 16];       // [wavefront][token of its round]
-    __shared__ float2 s_mm[2][8][16];                                    // [iteration parity][wavefront][token]: (min, max)
+    __shared__ __attribute__((aligned(16))) TokPar s_par[8 * 32];       // [wavefront][token of the iteration]
+    __shared__ uint32_t s_mm[2][8][32];                                  // [iteration parity][wavefront][token]: min | max << 16 (16-bit patterns)
     const int tid = threadIdx.x;
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
     const uint32_t gidx = s_idx;
     if (gidx >= ngroups) return;
-    const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31, wave = tid >> 6, lane = tid & 63;
+    const int j = tid >> 6, rp = (tid >> 5) & 1, t = tid & 31, wave = j, lane = tid & 63;
     const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
     const bool active = j < H;
     const int jc = min(j, H - 1);
-    const TokPar *my_par = s_par + 16 * wave;
+    const TokPar *my_par = s_par + 32 * wave + 16 * rp;
     const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
     for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)                 // metadata areas start as zeros
         reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
@@ -1455,47 +1494,43 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             float mn, mx;
-            cell_token_minmax<DT>(xr, mn, mx);
-            if ((lane & 3) == 0) s_mm[it & 1][wave][lane >> 2] = make_float2(mn, mx);
+            cell_token_minmax_halves<DT>(xr, mn, mx);
+            if ((lane & 1) == 0) s_mm[it & 1][wave][lane >> 1] = T16<DT>::to_bits(mn) | (T16<DT>::to_bits(mx) << 16);
         }
         __syncthreads();
-        if (lane < 16) {
-            const int w0 = wave & 4;                                         // the four wavefronts of this round
-            const float2 p0 = s_mm[it & 1][w0][lane], p1 = s_mm[it & 1][w0 + 1][lane], p2 = s_mm[it & 1][w0 + 2][lane],
-                         p3 = s_mm[it & 1][w0 + 3][lane];
-            const float mn = fminf(fminf(p0.x, p1.x), fminf(p2.x, p3.x)), mx = fmaxf(fmaxf(p0.y, p1.y), fmaxf(p2.y, p3.y));
+        if (lane < 32) {
+            float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const uint32_t p = s_mm[it & 1][q][lane];
+                mn = fminf(mn, T16<DT>::from_bits(p & 0xFFFFu));
+                mx = fmaxf(mx, T16<DT>::from_bits(p >> 16));
+            }
             const float range = round_t<DT>(mx - mn);
             const float sc = round_t<DT>(range * rel);
             const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-            if ((wave & 3) == 0) {
-                const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + 16 * rp + lane;
+            if (wave == 0) {
+                const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + lane;
                 scale[tok] = (uint16_t)T16<DT>::to_bits(sc);
                 zero[tok] = (uint16_t)zb;
             }
-            s_par[16 * wave + lane] = token_par<DT>(sc, zb, false);
+            s_par[32 * wave + lane] = token_par<DT>(sc, zb, false);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         uint32_t c01[16], c23[16];
-        cell_quant<DT>(xr, my_par, c01, c23);
+        cell_quant<DT, false>(xr, my_par, c01, c23);          // (the halves of the wavefront hold different tokens)
         typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_build(c01, c23, u, cmax);
         const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
         uint32_t tot;
         const uint32_t inc = oct_incl_scan(pb, m, tot);
-        if (m == 0) s_tot[rp][j][t >> 3] = tot;
-#ifndef PKV_PROBE_NOB2
-        __syncthreads();
-#endif
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
-#ifdef PKV_PROBE_NOB2
-        const uint32_t tot_even = tot, tot_odd = tot;
-#else
-        const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
-#endif
+        const auto halves = __builtin_amdgcn_permlane32_swap(tot, tot, false, false);      // the even round's total, the odd round's
+        const uint32_t tot_even = halves[0], tot_odd = halves[1];
         if (it == 3) {
             if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
             __syncthreads();
@@ -1527,7 +1562,6 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
             if (it == 1 && active && rp == 0 && m == 0) s_usz[blkid][2 * w] = (uint16_t)(meta + run_off);
             run_off = 0;
         }
-        // (s_tot is rewritten only after the next iteration's first barrier, which every thread reaches after these reads)
     }
     if (__any(cmax_all >= (1u << W))) {
 #pragma unroll
