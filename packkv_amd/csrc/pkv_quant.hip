@@ -486,6 +486,20 @@ __device__ __forceinline__ void cell_load_rows(const uint16_t *seq, const uint32
         xr[k] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(seq + (size_t)min(rows[k], last_row) * kHeadDim) + lane_off);
 }
 
+// The same when the lanes of a wavefront do not share their rows (`rows` differs between lanes; 64-byte aligned): the
+// 16 indices are loaded by the lane itself and the row offsets are per-lane 32-bit offsets on the uniform base.
+__device__ __forceinline__ void cell_load_rows_lanes(const uint16_t *seq, const uint32_t *rows, uint32_t last_row, uint32_t lane_off, uint2 xr[16]) {
+    uint4 idx[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) idx[q] = reinterpret_cast<const uint4 *>(rows)[q];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const uint4 v = idx[k >> 2];
+        const uint32_t row = min((k & 3) == 0 ? v.x : (k & 3) == 1 ? v.y : (k & 3) == 2 ? v.z : v.w, last_row);
+        xr[k] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(seq) + (row * (uint32_t)(kHeadDim * 2) + lane_off));
+    }
+}
+
 // (general_form: the constants of the general sequence whatever the zero point -- for callers whose wavefronts hold
 // several tokens and must take one path for all of them)
 template <int DT>
@@ -1454,11 +1468,16 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
 // each forms those of its head from the cell registers, the eight partial results per token go through LDS, and
 // every wavefront forms the 32 tokens' parameters for itself.  One barrier per iteration.  For 5..8 heads, tokens
 // in their own order; same stream, parameters and block_info as the round-major kernel.
-template <int DT, bool WIDE>
+// PERM: the tokens in the order of a repacking, as in the round-major kernel; with scale_in / zero_in (the tokens'
+// parameters in the order of x, known from the pass that made the order) nothing is left to exchange and an
+// iteration has no barrier at all.
+template <int DT, bool WIDE, bool PERM>
 __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride, const Stagger stagger) {
+    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
+    const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
+    const uint16_t *__restrict__ zero_in, const Stagger stagger) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1470,7 +1489,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    const uint32_t gidx = s_idx;
+    const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
     if (gidx >= ngroups) return;
     const int j = tid >> 6, rp = (tid >> 5) & 1, t = tid & 31, wave = j, lane = tid & 63;
     const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
@@ -1486,12 +1505,30 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     uint32_t run_off = 0;
     uint32_t cmax_all = 0;
     const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0 + 16 * rp) * kHeadDim + 4 * t;
+    const uint32_t plane = (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2);
+    const bool known = PERM && scale_in != nullptr;              // uniform
+    if (known) __syncthreads();                                  // the metadata zeros are in place before the first OR (no barrier below)
 #pragma unroll 1
     for (int it = 0; it < 4; it++) {
         // (no request ahead as in the K kernel: placing the packs holds too many registers to keep 16 rows in flight)
         uint2 xr[16];
-        cell_load(cells + (size_t)it * 32 * kHeadDim, xr);
+        // PERM: (the 32 tokens of an iteration lie in one repacking block: perm_block is a multiple of 64)
+        const size_t rb = PERM ? ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block : 0;
+        if (PERM) cell_load_rows_lanes(x + (((size_t)b * H) * T + rb) * kHeadDim, perm + tok0 + 32 * it + 16 * rp, (uint32_t)perm_block - 1u, plane, xr);
+        else cell_load(cells + (size_t)it * 32 * kHeadDim, xr);
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
+        if (known) {
+            if (lane < 32) {
+                const uint32_t src = min(perm[tok0 + 32 * it + lane], (uint32_t)perm_block - 1u);
+                const uint32_t sb = scale_in[(size_t)b * T + rb + src], zb = zero_in[(size_t)b * T + rb + src];
+                if (wave == 0) {
+                    const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + lane;
+                    scale[tok] = (uint16_t)sb;
+                    zero[tok] = (uint16_t)zb;
+                }
+                s_par[32 * wave + lane] = token_par<DT>(T16<DT>::from_bits(sb), zb, false);
+            }
+        } else {
         {
             float mn, mx;
             cell_token_minmax_halves<DT>(xr, mn, mx);
@@ -1515,6 +1552,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
                 zero[tok] = (uint16_t)zb;
             }
             s_par[32 * wave + lane] = token_par<DT>(sc, zb, false);
+        }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -1820,30 +1858,34 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             // up to four heads: 8 / H groups to a workgroup, so that all eight head slots have blocks
             const int gpw = (H <= 4 && !perm) ? kSubBlocks / H : 1;
             const uint32_t ngroups = (ngroups_all + (uint32_t)gpw - 1u) / (uint32_t)gpw;
-            auto kern = perm ? (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, true>
-                                                             : v_quant_encode_rounds_kernel<PKV_BF16, true, true>)
-                                         : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, true>
-                                                             : v_quant_encode_rounds_kernel<PKV_BF16, false, true>))
-                             : (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false>
-                                                             : v_quant_encode_rounds_kernel<PKV_BF16, true, false>)
-                                         : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false>
-                                                             : v_quant_encode_rounds_kernel<PKV_BF16, false, false>));
+            // (a token order always comes with gpw == 1, i.e. the cells kernel)
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true, false>)
+                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false, false>);
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             Stagger sg;
-            if (!perm && gpw == 1) {                // tokens in their own order: x read once, as cells
-                auto cells = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, true> : v_quant_encode_cells_kernel<PKV_BF16, true>)
-                                      : (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, false> : v_quant_encode_cells_kernel<PKV_BF16, false>);
+            if (gpw == 1) {                         // five to eight heads, or any token order: x read once, as cells
+                auto cells = perm ? (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, true, true>
+                                                                  : v_quant_encode_cells_kernel<PKV_BF16, true, true>)
+                                              : (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, false, true>
+                                                                  : v_quant_encode_cells_kernel<PKV_BF16, false, true>))
+                                  : (bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, true, false>
+                                                                  : v_quant_encode_cells_kernel<PKV_BF16, true, false>)
+                                              : (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, false, false>
+                                                                  : v_quant_encode_cells_kernel<PKV_BF16, false, false>));
                 PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(cells),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
                 if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 512, lds, ngroups, &sg))) return rc;
                 cells<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
-                                                stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, sg);
+                                                stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
+                                                (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg);
             } else {
                 if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
                 kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
-                                               stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
-                                               (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, gpw, ngroups_all, 1, nullptr);
+                                               stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, nullptr, 0,
+                                               nullptr, nullptr, sg, gpw, ngroups_all, 1, nullptr);
             }
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
