@@ -86,77 +86,6 @@ __global__ void quant_params_kernel(const uint16_t *__restrict__ x, int H, int T
     }
 }
 
-// ---- x -> uint8 code matrix [T, B*H*128] -----------------------------------------------
-// grid (T/16, H, B), 256 threads.
-template <int DT>
-__global__ void quantize_kernel(const uint16_t *__restrict__ x, int H, int T,
-                                const uint16_t *__restrict__ scale, const uint16_t *__restrict__ zero,
-                                uint8_t *__restrict__ codes, uint32_t *max_code_out) {
-    const int b = blockIdx.z, h = blockIdx.y;
-    const int B = gridDim.z;
-    const int tok = blockIdx.x * 16 + (threadIdx.x >> 4);
-    const int l16 = threadIdx.x & 15;
-    uint32_t cmax = 0;
-    if (tok < T) {
-        const float sc = T16<DT>::from_bits(scale[(size_t)b * T + tok]);
-        const float z = T16<DT>::from_bits(zero[(size_t)b * T + tok]);
-        const uint4 v = *reinterpret_cast<const uint4 *>(
-            x + (((size_t)b * H + h) * T + tok) * kHeadDim + l16 * 8);
-        float f[8];
-        unpack8<DT>(v, f);
-        uint32_t lo = 0, hi = 0;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t c0 = (uint32_t)(int)quant_code<DT>(f[i], sc, z) & 0xFFu;
-            const uint32_t c1 = (uint32_t)(int)quant_code<DT>(f[4 + i], sc, z) & 0xFFu;
-            lo |= c0 << (8 * i);
-            hi |= c1 << (8 * i);
-            cmax = max(cmax, max(c0, c1));
-        }
-        const size_t hidden = (size_t)B * H * kHeadDim;
-        uint2 *dst = reinterpret_cast<uint2 *>(codes + (size_t)tok * hidden +
-                                               ((size_t)b * H + h) * kHeadDim + l16 * 8);
-        *dst = make_uint2(lo, hi);
-    }
-    if (max_code_out) {
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) cmax = max(cmax, __shfl_xor(cmax, d, 64));
-        // a read first: once the largest code has been seen nobody writes any more (a million atomics on one
-        // address would cost milliseconds)
-        if ((threadIdx.x & 63) == 0 && cmax > __hip_atomic_load(max_code_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-            atomicMax(max_code_out, cmax);
-    }
-}
-
-// ---- uint8 code matrix -> x_hat [B, H, T, 128] -----------------------------------------
-template <int DT>
-__global__ void dequantize_kernel(const uint8_t *__restrict__ codes, int H, int T,
-                                  const uint16_t *__restrict__ scale, const uint16_t *__restrict__ zero,
-                                  uint16_t *__restrict__ x) {
-    const int b = blockIdx.z, h = blockIdx.y;
-    const int B = gridDim.z;
-    const int tok = blockIdx.x * 16 + (threadIdx.x >> 4);
-    const int l16 = threadIdx.x & 15;
-    if (tok >= T) return;
-    const float sc = T16<DT>::from_bits(scale[(size_t)b * T + tok]);
-    const float z = T16<DT>::from_bits(zero[(size_t)b * T + tok]);
-    const size_t hidden = (size_t)B * H * kHeadDim;
-    const uint2 c = *reinterpret_cast<const uint2 *>(codes + (size_t)tok * hidden +
-                                                    ((size_t)b * H + h) * kHeadDim + l16 * 8);
-    uint32_t out[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t w = i < 2 ? c.x : c.y;
-        const float a0 = (float)((w >> (16 * (i & 1))) & 0xFFu);
-        const float a1 = (float)((w >> (16 * (i & 1) + 8)) & 0xFFu);
-        const uint32_t r0 = T16<DT>::to_bits(round_t<DT>(a0 + z) * sc);
-        const uint32_t r1 = T16<DT>::to_bits(round_t<DT>(a1 + z) * sc);
-        out[i] = r0 | (r1 << 16);
-    }
-    *reinterpret_cast<uint4 *>(x + (((size_t)b * H + h) * T + tok) * kHeadDim + l16 * 8) =
-        make_uint4(out[0], out[1], out[2], out[3]);
-}
-
 // ---- fused quantize + encode: the cell ---------------------------------------------------
 // 128 threads work on one block.  Thread = "cell": 16 tokens (one round) x 4 adjacent channels,
 // i.e. four packs.  The cell is loaded straight from x (8 bytes per token row, rows of a
@@ -188,6 +117,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 //   sub2 == 0: add2 = (-zero, -zero) for the general sequence rint(h) + (-zero).
 // bf16: sub2 != 0 (|zero| <= 2^20): add2 = 2^23 - zero as fp32 bits; sub2 == 0: add2 = zero as fp32 bits.
 struct TokPar { float s, r; uint32_t add2, sub2; };
+template <int DT> __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits, bool general_form = false);
 
 __device__ __forceinline__ uint32_t pk_u16(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
@@ -273,6 +203,92 @@ __device__ __forceinline__ void quant4_f16_fast(uint2 xw, const TokPar tp, uint3
     c23 = pk_u16((u16x2)(__builtin_bit_cast(u16x2, (f16x2)(h23 + add)) - sub));
 }
 
+// ---- x -> uint8 code matrix [T, B*H*128] -----------------------------------------------
+// grid (T/16, ceil(H / 4), B), 256 threads: 16 lanes per token, 8 channels per lane, up to four heads per thread with
+// all of their rows requested before the first is used; the quotient as in the fused encoders (quant4: the lanes of a
+// wavefront hold four different tokens, so each chooses its sequence for itself).
+constexpr int kQuantHeads = 4;
+template <int DT>
+__global__ void __launch_bounds__(256) quantize_kernel(const uint16_t *__restrict__ x, int H, int T,
+                                                       const uint16_t *__restrict__ scale, const uint16_t *__restrict__ zero,
+                                                       uint8_t *__restrict__ codes, uint32_t *max_code_out) {
+    const int b = blockIdx.z, h0 = blockIdx.y * kQuantHeads;
+    const int B = gridDim.z;
+    const int tok = blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int l16 = threadIdx.x & 15;
+    const int nh = min(kQuantHeads, H - h0);               // uniform
+    uint32_t cmax = 0;
+    if (tok < T) {
+        uint4 v[kQuantHeads];
+#pragma unroll
+        for (int i = 0; i < kQuantHeads; i++)
+            if (i < nh) v[i] = *reinterpret_cast<const uint4 *>(x + (((size_t)b * H + h0 + i) * T + tok) * kHeadDim + l16 * 8);
+        const TokPar tp = token_par<DT>(T16<DT>::from_bits(scale[(size_t)b * T + tok]), zero[(size_t)b * T + tok], false);
+        const size_t hidden = (size_t)B * H * kHeadDim;
+        uint8_t *row = codes + (size_t)tok * hidden + ((size_t)b * H + h0) * kHeadDim + l16 * 8;
+#pragma unroll
+        for (int i = 0; i < kQuantHeads; i++) {
+            if (i < nh) {
+                uint32_t a01, a23, b01, b23;
+                quant4<DT, false>(make_uint2(v[i].x, v[i].y), tp, a01, a23);
+                quant4<DT, false>(make_uint2(v[i].z, v[i].w), tp, b01, b23);
+                const uint32_t lo = __builtin_amdgcn_perm(a23, a01, 0x06040200u), hi = __builtin_amdgcn_perm(b23, b01, 0x06040200u);
+                const u16x2 m = __builtin_elementwise_max(__builtin_elementwise_max(as_u16x2(a01 & 0x00FF00FFu), as_u16x2(a23 & 0x00FF00FFu)),
+                                                          __builtin_elementwise_max(as_u16x2(b01 & 0x00FF00FFu), as_u16x2(b23 & 0x00FF00FFu)));
+                cmax = max(cmax, max((uint32_t)m[0], (uint32_t)m[1]));
+                *reinterpret_cast<uint2 *>(row + (size_t)i * kHeadDim) = make_uint2(lo, hi);
+            }
+        }
+    }
+    if (max_code_out) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax = max(cmax, __shfl_xor(cmax, d, 64));
+        // a read first: once the largest code has been seen nobody writes any more (a million atomics on one
+        // address would cost milliseconds)
+        if ((threadIdx.x & 63) == 0 && cmax > __hip_atomic_load(max_code_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax(max_code_out, cmax);
+    }
+}
+
+// ---- uint8 code matrix -> x_hat [B, H, T, 128] -----------------------------------------
+// the same grid and thread roles
+template <int DT>
+__global__ void __launch_bounds__(256) dequantize_kernel(const uint8_t *__restrict__ codes, int H, int T,
+                                                         const uint16_t *__restrict__ scale, const uint16_t *__restrict__ zero,
+                                                         uint16_t *__restrict__ x) {
+    const int b = blockIdx.z, h0 = blockIdx.y * kQuantHeads;
+    const int B = gridDim.z;
+    const int tok = blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int l16 = threadIdx.x & 15;
+    const int nh = min(kQuantHeads, H - h0);               // uniform
+    if (tok >= T) return;
+    const size_t hidden = (size_t)B * H * kHeadDim;
+    const uint8_t *row = codes + (size_t)tok * hidden + ((size_t)b * H + h0) * kHeadDim + l16 * 8;
+    uint2 c[kQuantHeads];
+#pragma unroll
+    for (int i = 0; i < kQuantHeads; i++)
+        if (i < nh) c[i] = *reinterpret_cast<const uint2 *>(row + (size_t)i * kHeadDim);
+    const float sc = T16<DT>::from_bits(scale[(size_t)b * T + tok]);
+    const float z = T16<DT>::from_bits(zero[(size_t)b * T + tok]);
+#pragma unroll
+    for (int i = 0; i < kQuantHeads; i++) {
+        if (i < nh) {
+            uint32_t out[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t w = q < 2 ? c[i].x : c[i].y;
+                const float a0 = (float)((w >> (16 * (q & 1))) & 0xFFu);
+                const float a1 = (float)((w >> (16 * (q & 1) + 8)) & 0xFFu);
+                const uint32_t r0 = T16<DT>::to_bits(round_t<DT>(a0 + z) * sc);
+                const uint32_t r1 = T16<DT>::to_bits(round_t<DT>(a1 + z) * sc);
+                out[q] = r0 | (r1 << 16);
+            }
+            *reinterpret_cast<uint4 *>(x + (((size_t)b * H + h0 + i) * T + tok) * kHeadDim + l16 * 8) =
+                make_uint4(out[0], out[1], out[2], out[3]);
+        }
+    }
+}
+
 // bit_length of both 16-bit halves, clamped to 4 (values above 15 mean the codes overflow the
 // format; the launch reports that through max_code)
 __device__ __forceinline__ uint32_t pk_bitlen4(uint32_t d) {
@@ -339,8 +355,6 @@ __device__ __forceinline__ void minmax8(const uint4 v, float &mn, float &mx) {
     }
 }
 
-struct TokPar;
-template <int DT> __device__ __forceinline__ TokPar token_par(float sc, uint32_t zero_bits, bool general_form = false);
 
 // min and max over the 16 lanes of a row of the wavefront (every lane gets the results): the exchanges are DPP
 // operands of the min / max instructions themselves (quad permutes, then the half-row and row mirrors).
@@ -2027,7 +2041,7 @@ int pkv_quantize(const void *x, int dtype, int B, int H, int T, const void *scal
     PKV_REQUIRE(scale && zero && codes, PKV_ERR_INVALID, "null pointer argument");
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)H, (unsigned)B);
+    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)((H + kQuantHeads - 1) / kQuantHeads), (unsigned)B);
     if (dtype == PKV_F16)
         quantize_kernel<PKV_F16><<<grid, 256, 0, s>>>((const uint16_t *)x, H, T, (const uint16_t *)scale,
                                                       (const uint16_t *)zero, codes, max_code_out);
@@ -2047,7 +2061,7 @@ int pkv_dequantize(const uint8_t *codes, int dtype, int B, int H, int T, const v
     PKV_REQUIRE(scale && zero && codes, PKV_ERR_INVALID, "null pointer argument");
     LaunchTimer tm(s, ms_out != nullptr);
     if ((rc = tm.begin())) return rc;
-    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)H, (unsigned)B);
+    const dim3 grid((unsigned)((T + 15) / 16), (unsigned)((H + kQuantHeads - 1) / kQuantHeads), (unsigned)B);
     if (dtype == PKV_F16)
         dequantize_kernel<PKV_F16><<<grid, 256, 0, s>>>(codes, H, T, (const uint16_t *)scale,
                                                         (const uint16_t *)zero, (uint16_t *)x_out);
