@@ -39,9 +39,11 @@ def test_quantizer_bit_exact(cuda, dtype, rel):
 def test_fused_quant_encode_stream_bit_exact(cuda, oracle_codec, dtype):
     for (B, H, T, rel) in ((1, 2, 128, 0.1), (2, 8, 256, 0.1), (1, 32, 128, 0.1), (2, 4, 256, 0.2), (1, 8, 128, 0.34),
                            (1, 3, 128, 0.1), (2, 5, 256, 0.14), (3, 1, 128, 0.1),
+                           # five to eight heads: the kernels that read x once as cells (unused head slots repeat a head)
+                           (1, 6, 256, 0.1), (3, 7, 128, 0.2), (2, 7, 256, 0.05), (1, 6, 128, 0.03),
                            # few heads: several groups to a workgroup, the last workgroup partly filled
                            (3, 2, 384, 0.1), (5, 1, 256, 0.1), (3, 3, 384, 0.2), (3, 4, 128, 0.1),
-                           # widths 5 and 6 (format extension): round-major kernels up to eight heads, group kernel beyond
+                           # widths 5 and 6 (format extension): cells / round-major kernels up to eight heads, runs of eight beyond
                            (2, 8, 256, 0.05), (1, 4, 384, 0.03), (1, 3, 128, 0.05), (1, 16, 128, 0.05), (2, 12, 256, 0.03)):
         k, v = synth.make_kv(B, H, T, seed=31 + H, dtype=dtype)
         for is_k, x in ((1, k), (0, v)):
