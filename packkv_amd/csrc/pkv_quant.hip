@@ -388,63 +388,10 @@ __device__ __forceinline__ f16x2 pk_max_h(f16x2 a, f16x2 b) {
     return r;
 }
 
-// Token parameters of one round of the round-major encoders.  256 threads per 16 tokens: thread (tt = token, l16)
-// reads 8 channels of every head (slots beyond H - 1 repeat the first row: a repeated row changes no min / max); lane
-// l16 == 0 writes the token's scale and zero and its constants for quant4.  `rows` is x at (sequence, head 0, the
-// round's first token) and uniform, so the eight loads are one 32-bit lane offset on eight scalar bases.
-template <int DT>
-__device__ __forceinline__ void round_token_minmax(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float &mn, float &mx) {
-    const uint32_t lane_off = (uint32_t)(tt * kHeadDim + l16 * 8) * 2u;          // bytes
-    uint4 v[8];
-    v[0] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows) + lane_off);
-#pragma unroll
-    for (int i = 1; i < 8; i++) {                          // (H is uniform: a row that does not exist is not fetched)
-        if (i < H) v[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(rows + (size_t)i * head_stride) + lane_off);
-        else v[i] = v[0];
-    }
-    if (DT == PKV_F16) {               // packed fp16 comparisons all the way down to one word each
-        f16x2 lo[8], hi[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const f16x2 a = __builtin_bit_cast(f16x2, v[i].x), b = __builtin_bit_cast(f16x2, v[i].y),
-                        c = __builtin_bit_cast(f16x2, v[i].z), d = __builtin_bit_cast(f16x2, v[i].w);
-            lo[i] = pk_min_h(pk_min_h(a, b), pk_min_h(c, d));
-            hi[i] = pk_max_h(pk_max_h(a, b), pk_max_h(c, d));
-        }
-#pragma unroll
-        for (int w = 4; w >= 1; w >>= 1)
-#pragma unroll
-            for (int i = 0; i < w; i++) {
-                lo[i] = pk_min_h(lo[i], lo[i + w]);
-                hi[i] = pk_max_h(hi[i], hi[i + w]);
-            }
-        mn = fminf((float)lo[0][0], (float)lo[0][1]);
-        mx = fmaxf((float)hi[0][0], (float)hi[0][1]);
-    } else {
-        mn = INFINITY, mx = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 8; i++) minmax8<DT>(v[i], mn, mx);
-    }
-    row16_minmax(mn, mx);
-}
-
-template <int DT>
-__device__ __forceinline__ void round_token_params(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
-                                                   uint16_t *scale_out, uint16_t *zero_out, TokPar *par_out) {
-    float mn, mx;
-    round_token_minmax<DT>(rows, head_stride, H, tt, l16, mn, mx);
-    if (l16 == 0) {
-        const float range = round_t<DT>(mx - mn);
-        const float sc = round_t<DT>(range * rel);
-        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
-        *scale_out = (uint16_t)T16<DT>::to_bits(sc);
-        *zero_out = (uint16_t)zb;
-        *par_out = token_par<DT>(sc, zb, false);
-    }
-}
-
-
-// The same for groups of up to four heads (several of which share a workgroup): only the rows that exist are
+// Token parameters of one round of the round-major encoders for a group of up to four heads (several of which share
+// a workgroup).  256 threads per 16 tokens: thread (tt = token, l16) reads 8 channels of every head; lane l16 == 0
+// writes the token's scale and zero and its constants for quant4.  `rows` is x at (sequence, head 0, the round's first
+// token) and uniform, so the loads are one 32-bit lane offset on scalar bases; only the rows that exist are
 // fetched and compared.
 template <int DT>
 __device__ __forceinline__ void round_token_params_few(const uint16_t *rows, size_t head_stride, int H, int tt, int l16, float rel,
@@ -721,219 +668,6 @@ constexpr int kSubBlocks = 8;
 #define PKV_EPRIO_EMIT 2
 #endif
 
-// ---- K, all heads in one workgroup: round-major single trip over x --------------------------
-// For H <= 8 the eight blocks of a (context block, sequence) group are the eight heads, so one
-// workgroup of 256 threads (head j = tid / 32, lane t = tid % 32) can go through the group ROUND BY
-// ROUND (16 tokens): read the round's rows of all heads for the token parameters (32 KiB per
-// workgroup), then at once re-read them as cells -- the lines are still in L2 -- quantize, and emit
-// unit `round` of every block behind the units already there.  x therefore crosses HBM once.
-// Blocks sit in worst-case slots in LDS and are compacted by the final copy.
-// PERM: the tokens are encoded in the order of a repacking -- position p of the output holds token
-// (p / perm_block) * perm_block + perm[p] of x (perm_block a multiple of 64) -- so a round's rows are gathered; scale
-// and zero are written in the output order.
-template <int DT, bool WIDE, bool PERM, bool XCH = false>
-__global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
-    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
-    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
-    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger, int gpw, uint32_t ngroups_total,
-    int nsg = 1, uint64_t *xw = nullptr) {
-    extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
-    __shared__ uint32_t s_idx;
-    __shared__ uint64_t s_off;
-    __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the group's bytes
-    __shared__ __attribute__((aligned(16))) TokPar s_par[kSubBlocks * 16];      // [group of the workgroup][token of the round]
-    const int tid = threadIdx.x;
-    stagger_first_generation(stagger);
-    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
-    __syncthreads();
-    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);   // uniform: the rows' addresses become scalar
-    if (gidx >= ngroups) return;
-    // XCH (more than eight heads): a group's heads are cut into nsg runs of eight, one workgroup (one ticket) each,
-    // consecutive in the stream.  A workgroup reads only its own heads: it forms the round's minima and maxima over
-    // them, publishes them per token as one 64-bit word (valid | min | max, a relaxed agent-scope atomic like the
-    // look-back's status words) and takes the other runs' words to form the token parameters, which are therefore
-    // the same bits in every run.  The runs of a group hold consecutive tickets, so all of them are running or next
-    // in line: the oldest unfinished group is always complete on the machine and the waits end.  H_all = all heads.
-    const int H_all = H;
-    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
-    const int hbase = XCH ? 8 * (int)sgi : 0;
-    if (XCH) H = min(8, H_all - hbase);
-    // Fewer than five heads: a workgroup takes gpw = 8 / H (rounded down) consecutive groups -- consecutive in the
-    // stream too -- so that its eight half-wavefronts all have a block; `ngroups` then counts workgroups and
-    // `ngroups_all` groups.  Half-wavefront j serves head j % H of group gidx * gpw + j / H; everything below that is
-    // written for "the group" uses this half-wavefront's group (with gpw == 1 the one group, uniformly).
-    const uint32_t ngroups_all = ngroups_total;
-    const int j = tid >> 5, t = tid & 31;                 // block and lane of the unit
-    const int jg = gpw > 1 ? j / H : 0, jh = gpw > 1 ? j % H : j;
-    const uint32_t grp_first = gidx * (uint32_t)gpw;
-    const int ng = (int)min((uint32_t)gpw, ngroups_all - grp_first);          // groups of this workgroup
-    const int nblk = gpw > 1 ? ng * H : H;                // blocks of this workgroup
-    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : XCH ? gidx / (uint32_t)nsg : gidx;
-    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
-    const size_t tok0 = (size_t)cb * 64;
-    const UnitGeom g = unit_geom(W);
-    const bool active = gpw > 1 ? (jg < ng && j < gpw * H) : j < H;
-    const int jc = gpw > 1 ? jh : min(j, H - 1);
-    const TokPar *my_par = s_par + 16 * (gpw > 1 ? min(jg, ng - 1) : 0);
-    uint8_t *blk = gbuf + (size_t)j * bound;
-    uint32_t my_off = 8u;                                 // bytes of this block so far (uniform per half-wavefront)
-    uint32_t cmax_all = 0;
-    uint32_t src_tok[4] = {0u, 0u, 0u, 0u};               // PERM: the thread's token of every round's parameter pass
-    if (PERM)
-#pragma unroll
-        for (int r = 0; r < 4; r++) src_tok[r] = min(perm[tok0 + 16 * r + (tid >> 4)], (uint32_t)perm_block - 1u);
-#pragma unroll 1
-    for (int r = 0; r < 4; r++) {
-        // token parameters of the round: 16 lanes x 8 channels per token, all heads
-        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
-        {
-            const int tt = tid >> 4, l16 = tid & 15;
-            const size_t tok = (size_t)b * par_stride + tok0 + 16 * r + tt;
-            if (PERM) {
-                const size_t pb = (tok0 / (size_t)perm_block) * (size_t)perm_block;      // first token of the repacking block
-                const uint32_t src = r == 0 ? src_tok[0] : r == 1 ? src_tok[1] : r == 2 ? src_tok[2] : src_tok[3];
-                round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
-                                       (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
-            } else if (XCH) {
-                float mn, mx;
-                round_token_minmax<DT>(x + (((size_t)b * H_all + hbase) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, mn, mx);
-                uint64_t *words = xw + ((size_t)(gidx - sgi) * 4 + r) * 16;       // [run][round][token] of this group
-                if (l16 == 0)
-                    __hip_atomic_store(words + (size_t)sgi * 64 + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(mn) << 16) | (uint64_t)T16<DT>::to_bits(mx),
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                // the first wavefront collects: lane = (run, token) for up to four runs at a time
-                if (tid < 64) {
-                    float amn = INFINITY, amx = -INFINITY;
-                    for (int s0 = 0; s0 < nsg; s0 += 4) {
-                        const int run = s0 + (tid >> 4);
-                        if (run < nsg) {
-                            const uint64_t *wp = words + (size_t)run * 64 + (tid & 15);
-                            uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            int spins = 0;
-                            while ((w >> 63) == 0 && spins < kSpinLimit) {
-                                __builtin_amdgcn_s_sleep(8);
-                                w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                spins++;
-                            }
-                            if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
-                            amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
-                            amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
-                        }
-                    }
-                    amn = fminf(amn, __shfl_xor(amn, 16, 64)); amx = fmaxf(amx, __shfl_xor(amx, 16, 64));
-                    amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
-                    if (tid < 16) {
-                        const float range = round_t<DT>(amx - amn);
-                        const float sc = round_t<DT>(range * rel);
-                        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
-                        if (sgi == 0) {
-                            const size_t tk = (size_t)b * par_stride + tok0 + 16 * r + tid;
-                            scale[tk] = (uint16_t)T16<DT>::to_bits(sc);
-                            zero[tk] = (uint16_t)zb;
-                        }
-                        s_par[tid] = token_par<DT>(sc, zb, false);
-                    }
-                }
-            } else if (gpw == 1) {
-                round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
-                                       scale + tok, zero + tok, s_par + tt);
-            } else {
-                for (int q = 0; q < ng; q++) {              // one group after the other: H rows each
-                    const uint32_t gq = grp_first + (uint32_t)q;
-                    const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
-                    const size_t tq = (size_t)bq * par_stride + (size_t)cq * 64 + 16 * r + tt;
-                    round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 64 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H,
-                                               tt, l16, rel, scale + tq, zero + tq, s_par + 16 * q + tt);
-                }
-            }
-        }
-        // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
-        uint2 xr[16];
-        if (PERM) {
-            const size_t pb = (tok0 / (size_t)perm_block) * (size_t)perm_block;
-            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 16 * r, (uint32_t)perm_block - 1u,
-                           (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
-        } else {
-            cell_load(x + (((size_t)b * H_all + hbase + jc) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
-        }
-        __syncthreads();
-        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
-        typename PacksOf<WIDE>::type u;
-        uint32_t cmax;
-        cell_packs<DT>(xr, my_par, u, cmax);
-        __syncthreads();                                  // s_par is rewritten by the next round
-        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
-        pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
-        const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
-        if (r == 3) {
-            // every block's final size is known before its last unit is written: the group's size is published
-            // now, so that the workgroups behind it in the stream wait that much less for it
-            if (active && t == 0) blk_off[j + 1] = my_off + usz;          // sizes first ...
-            if (tid == 0) blk_off[0] = 0;
-            __syncthreads();
-            if (tid == 0) {                                               // ... then their running sum
-                for (int q = 1; q <= nblk; q++) blk_off[q] += blk_off[q - 1];
-                lookback_publish(st, gidx, blk_off[nblk]);
-            }
-        }
-        if (active) {
-            cmax_all = max(cmax_all, cmax);
-            if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
-            unit_emit_any(blk, my_off, t, g, u);
-            my_off += usz;
-        }
-    }
-    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
-        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
-    }
-    __syncthreads();
-    const uint32_t bytes = blk_off[nblk];
-    if (tid < 64) {
-        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
-        if (tid == 0) {
-            s_off = off;
-            if (gidx == ngroups - 1) st->total = off + bytes;
-            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
-        }
-    }
-    __syncthreads();
-    const uint64_t off = s_off;
-    if (off + bytes > capacity) return;
-    if (tid < nblk) {
-        const uint32_t first = XCH ? grp * (uint32_t)H_all + (uint32_t)hbase : (gpw > 1 ? grp_first : gidx) * (uint32_t)H;      // block index = group * H + head
-        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
-        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
-    }
-    // each half-wavefront copies its own block: head to the first 16-byte boundary of the stream
-    // and tail in 2-byte pieces, the body as aligned 16-byte stores fed by aligned LDS reads and
-    // byte funnel shifts
-    if (active) {
-        uint8_t *dst = stream + off + blk_off[j];
-        const uint32_t nbytes = my_off;
-        const uint32_t head = min(nbytes, (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u));
-        const uint32_t nq = (nbytes - head) >> 4;
-        for (uint32_t i = t; i < (head >> 1); i += 32)
-            reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(blk)[i];
-        const uint32_t *src32 = reinterpret_cast<const uint32_t *>(blk + (head & ~3u));
-        for (uint32_t i = t; i < nq; i += 32) {
-            const uint32_t *q = src32 + 4 * i;
-            const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
-            uint4 v;
-            v.x = __builtin_amdgcn_alignbyte(d1, d0, head);
-            v.y = __builtin_amdgcn_alignbyte(d2, d1, head);
-            v.z = __builtin_amdgcn_alignbyte(d3, d2, head);
-            v.w = __builtin_amdgcn_alignbyte(d4, d3, head);
-            *reinterpret_cast<uint4 *>(dst + head + 16 * (size_t)i) = v;
-        }
-        const uint32_t done = head + 16u * nq;
-        for (uint32_t i = t; i < ((nbytes - done) >> 1); i += 32)
-            reinterpret_cast<uint16_t *>(dst + done)[i] = reinterpret_cast<const uint16_t *>(blk + done)[i];
-    }
-}
-
 // Copy n bytes (even) from LDS (src 4-byte aligned, readable up to 20 bytes past n) to global memory (dst 2-byte
 // aligned) with the 32 lanes of a half-wavefront: head to the first 16-byte boundary and tail in 2-byte pieces, the
 // body as aligned 16-byte stores fed by aligned LDS reads and byte funnel shifts.
@@ -1084,12 +818,12 @@ __device__ __forceinline__ void cell_token_minmax_halves(const uint2 xr[16], flo
 // has one barrier), and the next round's cells are requested as soon as this round's are quantized -- into the same
 // registers -- so that they travel while the packs are formed and emitted.  For 5..8 heads (one group per
 // workgroup); PERM as in the round-major kernel.  Same stream, parameters and block_info as that kernel.
-template <int DT, bool WIDE, bool PERM>
+template <int DT, bool WIDE, bool PERM, bool XCH = false>
 __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride,
-    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger) {
+    const uint32_t *__restrict__ perm, int perm_block, const Stagger stagger, int nsg = 1, uint64_t *xw = nullptr) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // H block slots of `bound` bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1102,22 +836,30 @@ __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
     __syncthreads();
     const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);
     if (gidx >= ngroups) return;
+    // XCH (more than eight heads): runs of eight heads, one workgroup and one ticket each, as in the round-major
+    // kernel: a run forms the minima and maxima over its own heads, publishes them per token and collects the others'.
+    const int H_all = H;
+    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
+    const int hbase = XCH ? 8 * (int)sgi : 0;
+    if (XCH) H = min(8, H_all - hbase);
     const int j = tid >> 5, t = tid & 31, wave = tid >> 6, lane = tid & 63;
-    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const uint32_t grp = XCH ? gidx / (uint32_t)nsg : gidx;
+    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 64;
     const UnitGeom g = unit_geom(W);
     const bool active = j < H;
     const int jc = min(j, H - 1);                          // (a repeated head changes no minimum or maximum)
-    const TokPar *my_par = s_par + 16 * wave;
+    const TokPar *my_par = XCH ? s_par : s_par + 16 * wave;
     uint8_t *blk = gbuf + (size_t)j * bound;
     uint32_t my_off = 8u;
     uint32_t cmax_all = 0;
-    const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0) * kHeadDim + 4 * t;
+    const uint16_t *cells = x + (((size_t)b * H_all + hbase + jc) * T + tok0) * kHeadDim + 4 * t;
     // PERM: the rows of a round are tokens perm[...] of the repacking block that holds this context block
     const uint16_t *pseq = x + (((size_t)b * H) * T + (tok0 / (size_t)(PERM ? perm_block : 1)) * (size_t)(PERM ? perm_block : 1)) * kHeadDim;
     const uint32_t plane = (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2);
-    // (bf16 with the wide packs would need more than 128 registers to keep a round in flight: it asks at the top)
-    constexpr bool AHEAD = !(WIDE && DT != PKV_F16);
+    // (bf16 with the wide packs or with the exchange between runs would need more than 128 registers to keep a round
+    // in flight: it asks at the top)
+    constexpr bool AHEAD = !((WIDE || XCH) && DT != PKV_F16);
     uint2 xr[16];
     if (AHEAD) {
         if (PERM) cell_load_rows(pseq, perm + tok0, (uint32_t)perm_block - 1u, plane, xr);
@@ -1136,7 +878,49 @@ __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
             if ((lane & 3) == 0) s_mm[r & 1][wave][lane >> 2] = make_float2(mn, mx);
         }
         __syncthreads();
-        if (lane < 16) {
+        if (XCH) {
+            if (wave == 0) {
+                const int tk = lane & 15;
+                const float2 p0 = s_mm[r & 1][0][tk], p1 = s_mm[r & 1][1][tk], p2 = s_mm[r & 1][2][tk], p3 = s_mm[r & 1][3][tk];
+                const float rmn = fminf(fminf(p0.x, p1.x), fminf(p2.x, p3.x)), rmx = fmaxf(fmaxf(p0.y, p1.y), fmaxf(p2.y, p3.y));
+                uint64_t *words = xw + ((size_t)(gidx - sgi) * 4 + r) * 16;       // [run][round][token] of this group
+                if (lane < 16)
+                    __hip_atomic_store(words + (size_t)sgi * 64 + lane, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(rmn) << 16) | (uint64_t)T16<DT>::to_bits(rmx),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // lane = (run, token) for up to four runs at a time
+                float amn = INFINITY, amx = -INFINITY;
+                for (int s0 = 0; s0 < nsg; s0 += 4) {
+                    const int run = s0 + (lane >> 4);
+                    if (run < nsg) {
+                        const uint64_t *wp = words + (size_t)run * 64 + tk;
+                        uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        int spins = 0;
+                        while ((w >> 63) == 0 && spins < kSpinLimit) {
+                            __builtin_amdgcn_s_sleep(8);
+                            w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            spins++;
+                        }
+                        if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
+                        amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
+                        amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
+                    }
+                }
+                amn = fminf(amn, __shfl_xor(amn, 16, 64)); amx = fmaxf(amx, __shfl_xor(amx, 16, 64));
+                amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
+                if (lane < 16) {
+                    const float range = round_t<DT>(amx - amn);
+                    const float sc = round_t<DT>(range * rel);
+                    const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
+                    if (sgi == 0) {
+                        const size_t tok = (size_t)b * par_stride + tok0 + 16 * r + lane;
+                        scale[tok] = (uint16_t)T16<DT>::to_bits(sc);
+                        zero[tok] = (uint16_t)zb;
+                    }
+                    s_par[lane] = token_par<DT>(sc, zb, false);
+                }
+            }
+            __syncthreads();
+        } else if (lane < 16) {
             const float2 p0 = s_mm[r & 1][0][lane], p1 = s_mm[r & 1][1][lane], p2 = s_mm[r & 1][2][lane], p3 = s_mm[r & 1][3][lane];
             const float mn = fminf(fminf(p0.x, p1.x), fminf(p2.x, p3.x)), mx = fmaxf(fmaxf(p0.y, p1.y), fmaxf(p2.y, p3.y));
             const float range = round_t<DT>(mx - mn);
@@ -1201,10 +985,122 @@ __global__ void __launch_bounds__(256) k_quant_encode_cells_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < H) {
-        info[2 * (size_t)(gidx * (uint32_t)H + tid)] = (uint32_t)(off + blk_off[tid]);
-        info[2 * (size_t)(gidx * (uint32_t)H + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+        const uint32_t first = XCH ? grp * (uint32_t)H_all + (uint32_t)hbase : gidx * (uint32_t)H;      // block index = group * heads + head
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
     if (active) copy_out32(stream + off + blk_off[j], blk, my_off, t);
+}
+
+// ---- K, up to four heads: round-major, several groups to a workgroup ---------------------------
+// The eight blocks a workgroup of 256 threads owns (block j = tid / 32, lane t = tid % 32) are here the H <= 4 heads
+// of gpw = 8 / H (rounded down) consecutive (context block, sequence) groups -- consecutive in the stream too -- so
+// that all eight half-wavefronts have a block.  The workgroup goes through its groups ROUND BY ROUND (16 tokens):
+// it reads the round's rows row-wise for the token parameters (round_token_params_few, one group after the other),
+// then at once re-reads them as cells -- the lines are still in L2 -- quantizes, and emits unit `round` of every
+// block behind the units already there.  x crosses HBM once.  Blocks sit in worst-case slots in LDS and are
+// compacted by the final copy.  (Five to eight heads, more than eight, and every token order take the cells
+// kernel above, which reads a round once.)  `ngroups` counts workgroups, `ngroups_all` groups.
+template <int DT, bool WIDE>
+__global__ void __launch_bounds__(256) k_quant_encode_rounds_kernel(
+    const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
+    uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
+    ScanState *st, int W, uint32_t ngroups, uint32_t bound, uint64_t base, int par_stride, const Stagger stagger,
+    int gpw, uint32_t ngroups_all) {
+    extern __shared__ __align__(16) uint8_t gbuf[];        // gpw * H block slots of `bound` bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[kSubBlocks + 1];           // byte offset of each block inside the workgroup's bytes
+    __shared__ __attribute__((aligned(16))) TokPar s_par[kSubBlocks * 16];      // [group of the workgroup][token of the round]
+    const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);   // uniform: the rows' addresses become scalar
+    if (gidx >= ngroups) return;
+    // half-wavefront j serves head j % H of group gidx * gpw + j / H
+    const int j = tid >> 5, t = tid & 31;                 // block and lane of the unit
+    const int jg = j / H, jh = j % H;
+    const uint32_t grp_first = gidx * (uint32_t)gpw;
+    const int ng = (int)min((uint32_t)gpw, ngroups_all - grp_first);          // groups of this workgroup
+    const int nblk = ng * H;                              // blocks of this workgroup
+    const uint32_t grp = grp_first + (uint32_t)min(jg, ng - 1);
+    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
+    const size_t tok0 = (size_t)cb * 64;
+    const UnitGeom g = unit_geom(W);
+    const bool active = jg < ng && j < gpw * H;
+    const TokPar *my_par = s_par + 16 * min(jg, ng - 1);
+    uint8_t *blk = gbuf + (size_t)j * bound;
+    uint32_t my_off = 8u;                                 // bytes of this block so far (uniform per half-wavefront)
+    uint32_t cmax_all = 0;
+#pragma unroll 1
+    for (int r = 0; r < 4; r++) {
+        // token parameters of the round: 16 lanes x 8 channels per token, the heads of one group after the other
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
+        {
+            const int tt = tid >> 4, l16 = tid & 15;
+            for (int q = 0; q < ng; q++) {
+                const uint32_t gq = grp_first + (uint32_t)q;
+                const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
+                const size_t tq = (size_t)bq * par_stride + (size_t)cq * 64 + 16 * r + tt;
+                round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 64 + 16 * r) * kHeadDim, (size_t)T * kHeadDim, H,
+                                           tt, l16, rel, scale + tq, zero + tq, s_par + 16 * q + tt);
+            }
+        }
+        // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
+        uint2 xr[16];
+        cell_load(x + (((size_t)b * H + jh) * T + tok0 + 16 * r) * kHeadDim + 4 * t, xr);
+        __syncthreads();
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
+        typename PacksOf<WIDE>::type u;
+        uint32_t cmax;
+        cell_packs<DT>(xr, my_par, u, cmax);
+        __syncthreads();                                  // s_par is rewritten by the next round
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+        pack_offsets(u.len, u.off, u.payload);            // (all lanes: the scan runs on whole wavefronts)
+        const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        if (r == 3) {
+            // every block's final size is known before its last unit is written: the workgroup's size is published
+            // now, so that the workgroups behind it in the stream wait that much less for it
+            if (active && t == 0) blk_off[j + 1] = my_off + usz;          // sizes first ...
+            if (tid == 0) blk_off[0] = 0;
+            __syncthreads();
+            if (tid == 0) {                                               // ... then their running sum
+                for (int q = 1; q <= nblk; q++) blk_off[q] += blk_off[q - 1];
+                lookback_publish(st, gidx, blk_off[nblk]);
+            }
+        }
+        if (active) {
+            cmax_all = max(cmax_all, cmax);
+            if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
+            unit_emit_any(blk, my_off, t, g, u);
+            my_off += usz;
+        }
+    }
+    if (__any(cmax_all >= (1u << W))) {   // codes that do not fit W bits are an error the host reports
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cmax_all = max(cmax_all, __shfl_xor(cmax_all, d, 64));
+        if ((tid & 63) == 0) atomicMax(&st->max_code, cmax_all);
+    }
+    __syncthreads();
+    const uint32_t bytes = blk_off[nblk];
+    if (tid < 64) {
+        const uint64_t off = base + lookback_offset(st, gidx, bytes, true);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < nblk) {
+        const uint32_t first = grp_first * (uint32_t)H;                   // block index = group * H + head
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    if (active) copy_out32(stream + off + blk_off[j], blk, my_off, t);     // each half-wavefront copies its own block
 }
 
 // OR the FB-bit fields f[0..3] of four adjacent lanes 4m..4m+3, slot i, into a unit's LSB-first metadata array
@@ -1248,25 +1144,27 @@ __device__ __forceinline__ uint32_t oct_incl_scan(uint32_t v, int m, uint32_t &t
     return x;
 }
 
-// ---- V, all heads in one workgroup: round-major single trip over x --------------------------
-// For H <= 8 one workgroup of 512 threads owns the 2 H blocks of a (128-token context block, sequence) group and
-// goes through it 32 tokens (two rounds) at a time: read the rows of all heads for the token parameters, then at
-// once re-read them as cells -- still in L2 -- quantize and append.  Thread = (round parity rp, head j, cell lane t):
-// its cell (round 2 it + rp, channels 4t..4t+3 of head j) holds slot (2 it + rp) % 4 of lanes 4m..4m+3, m = t % 8, of
-// unit (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight
-// threads of a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed
-// in with LDS atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.
-template <int DT, bool WIDE, bool PERM, bool XCH = false>
+// ---- V, up to four heads: round-major, several groups to a workgroup ---------------------------
+// One workgroup of 512 threads owns the 2 H blocks of each of gpw = 8 / H (rounded down) consecutive (128-token
+// context block, sequence) groups, H <= 4, and goes through them 32 tokens (two rounds) at a time: read the rows
+// row-wise for the token parameters, then at once re-read them as cells -- still in L2 -- quantize and append.
+// Thread = (round parity rp, head slot j, cell lane t); head slot j serves head j % H of group gidx * gpw + j / H.
+// Its cell (round 2 it + rp, channels 4t..4t+3) holds slot (2 it + rp) % 4 of lanes 4m..4m+3, m = t % 8, of unit
+// (warp (t / 8) % 2, segment it / 2) of block 2 j + t / 16.  A unit's payload is slot-major, so the eight threads of
+// a (unit, slot) append their packs behind the slots already there; the metadata bit-fields are OR-ed in with LDS
+// atomics.  Units sit in worst-case slots in LDS; the final copy compacts them into the stream.  (Five to eight
+// heads, more than eight, and every token order take the cells kernel below.)  `ngroups` counts workgroups,
+// `ngroups_total` groups.
+template <int DT, bool WIDE>
 __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
-    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
-    const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
-    const uint16_t *__restrict__ zero_in, const Stagger stagger, int gpw, uint32_t ngroups_total, int nsg, uint64_t *xw) {
+    ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride, const Stagger stagger,
+    int gpw, uint32_t ngroups_total) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
-    __shared__ uint32_t blk_off[17];                       // byte offset of each block inside the group's bytes
+    __shared__ uint32_t blk_off[17];                       // byte offset of each block inside the workgroup's bytes
     __shared__ uint32_t s_tot[2][8][4];                    // payload bytes the two rounds of an iteration append per unit
     __shared__ uint16_t s_usz[16][4];                      // bytes of every unit (block, unit index 2 w + sg)
     __shared__ __attribute__((aligned(16))) TokPar s_par[kSubBlocks * 32];      // [group of the workgroup][token of the iteration]
@@ -1274,119 +1172,43 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
+    const uint32_t gidx = s_idx;
     if (gidx >= ngroups) return;
-    // XCH (more than eight heads): runs of eight heads, one workgroup each, that exchange the minima and maxima of
-    // their rows per token, as in the K kernel; a run's words are [iteration][token of the iteration]
-    const int H_all = H;
-    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
-    const int hbase = XCH ? 8 * (int)sgi : 0;
-    if (XCH) H = min(8, H_all - hbase);
-    // Fewer than five heads: gpw = 8 / H (rounded down) consecutive groups to a workgroup, as in the K kernel --
-    // `ngroups` counts workgroups, `ngroups_total` groups; head slot j serves head j % H of group gidx * gpw + j / H.
     const int rp = tid >> 8, j = (tid >> 5) & 7, t = tid & 31;
-    const int jg = gpw > 1 ? j / H : 0, jh = gpw > 1 ? j % H : j;
+    const int jg = j / H, jh = j % H;
     const uint32_t grp_first = gidx * (uint32_t)gpw;
     const int ng = (int)min((uint32_t)gpw, ngroups_total - grp_first);        // groups of this workgroup
-    const int nheads = gpw > 1 ? ng * H : H;              // head slots in use
-    const uint32_t grp = gpw > 1 ? grp_first + (uint32_t)min(jg, ng - 1) : XCH ? gidx / (uint32_t)nsg : gidx;
+    const int nheads = ng * H;                            // head slots in use
+    const uint32_t grp = grp_first + (uint32_t)min(jg, ng - 1);
     const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
-    const bool active = gpw > 1 ? jg < ng : j < H;
-    const int jc = gpw > 1 ? jh : min(j, H - 1);
-    const TokPar *my_par = s_par + 32 * (gpw > 1 ? min(jg, ng - 1) : 0) + 16 * rp;
+    const bool active = jg < ng;
+    const TokPar *my_par = s_par + 32 * min(jg, ng - 1) + 16 * rp;
     const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
     // metadata areas start as zeros (fields are OR-ed in)
     for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)
         reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
     uint32_t run_off = 0;                                  // payload bytes of the thread's current unit so far
     uint32_t cmax_all = 0;
-    uint32_t src_tok[4] = {0u, 0u, 0u, 0u};                // PERM: the thread's token of every iteration's parameter pass
-    if (PERM)
-#pragma unroll
-        for (int it = 0; it < 4; it++) src_tok[it] = min(perm[tok0 + 32 * it + (tid >> 4)], (uint32_t)perm_block - 1u);
 #pragma unroll 1
     for (int it = 0; it < 4; it++) {
-        // token parameters of the 32 tokens: 16 lanes x 8 channels per token, all heads
+        // token parameters of the 32 tokens: 16 lanes x 8 channels per token, the heads of one group after the other
         __builtin_amdgcn_s_setprio(PKV_EPRIO_STAT);
         {
             const int tt = tid >> 4, l16 = tid & 15;
-            const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + tt;
-            if (PERM) {     // (the 32 tokens of an iteration lie in one repacking block: perm_block is a multiple of 64)
-                const size_t pb = ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block;
-                const uint32_t src = it == 0 ? src_tok[0] : it == 1 ? src_tok[1] : it == 2 ? src_tok[2] : src_tok[3];
-                if (scale_in) {       // (uniform) the tokens' parameters are known, in the order of x: no pass over the rows
-                    if (l16 == 0) {
-                        const uint32_t sb = scale_in[(size_t)b * T + pb + src], zb = zero_in[(size_t)b * T + pb + src];
-                        scale[tok] = (uint16_t)sb;
-                        zero[tok] = (uint16_t)zb;
-                        s_par[tt] = token_par<DT>(T16<DT>::from_bits(sb), zb, false);
-                    }
-                } else {
-                    round_token_params<DT>(x + (((size_t)b * H) * T + pb) * kHeadDim, (size_t)T * kHeadDim, H,
-                                           (int)src, l16, rel, scale + tok, zero + tok, s_par + tt);
-                }
-            } else if (XCH) {
-                float mn, mx;
-                round_token_minmax<DT>(x + (((size_t)b * H_all + hbase) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, mn, mx);
-                uint64_t *words = xw + (size_t)(gidx - sgi) * 128 + 32 * it;      // [run][iteration][token] of this group
-                if (l16 == 0)
-                    __hip_atomic_store(words + (size_t)sgi * 128 + tt, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(mn) << 16) | (uint64_t)T16<DT>::to_bits(mx),
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                // the first wavefront collects: lane = (parity of the run, token)
-                if (tid < 64) {
-                    float amn = INFINITY, amx = -INFINITY;
-                    for (int run = tid >> 5; run < nsg; run += 2) {
-                        const uint64_t *wp = words + (size_t)run * 128 + (tid & 31);
-                        uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        int spins = 0;
-                        while ((w >> 63) == 0 && spins < kSpinLimit) {
-                            __builtin_amdgcn_s_sleep(8);
-                            w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            spins++;
-                        }
-                        if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
-                        amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
-                        amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
-                    }
-                    amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
-                    if (tid < 32) {
-                        const float range = round_t<DT>(amx - amn);
-                        const float sc = round_t<DT>(range * rel);
-                        const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
-                        if (sgi == 0) {
-                            const size_t tk = (size_t)b * par_stride + tok0 + 32 * it + tid;
-                            scale[tk] = (uint16_t)T16<DT>::to_bits(sc);
-                            zero[tk] = (uint16_t)zb;
-                        }
-                        s_par[tid] = token_par<DT>(sc, zb, false);
-                    }
-                }
-            } else if (gpw == 1) {
-                round_token_params<DT>(x + (((size_t)b * H) * T + tok0 + 32 * it) * kHeadDim, (size_t)T * kHeadDim, H, tt, l16, rel,
-                                       scale + tok, zero + tok, s_par + tt);
-            } else {
-                for (int q = 0; q < ng; q++) {              // one group after the other: H rows each
-                    const uint32_t gq = grp_first + (uint32_t)q;
-                    const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
-                    const size_t tq = (size_t)bq * par_stride + (size_t)cq * 128 + 32 * it + tt;
-                    round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 128 + 32 * it) * kHeadDim, (size_t)T * kHeadDim,
-                                               H, tt, l16, rel, scale + tq, zero + tq, s_par + 32 * q + tt);
-                }
+            for (int q = 0; q < ng; q++) {
+                const uint32_t gq = grp_first + (uint32_t)q;
+                const uint32_t cq = gq / (uint32_t)B, bq = gq % (uint32_t)B;
+                const size_t tq = (size_t)bq * par_stride + (size_t)cq * 128 + 32 * it + tt;
+                round_token_params_few<DT>(x + (((size_t)bq * H) * T + (size_t)cq * 128 + 32 * it) * kHeadDim, (size_t)T * kHeadDim,
+                                           H, tt, l16, rel, scale + tq, zero + tq, s_par + 32 * q + tt);
             }
         }
         // the same rows again, as cells (issued before the barrier; they hit the lines just fetched)
         uint2 xr[16];
-        if (PERM) {
-            const size_t pb = ((tok0 + 32 * it) / (size_t)perm_block) * (size_t)perm_block;
-            const int rps = __builtin_amdgcn_readfirstlane(rp);          // uniform per wavefront
-            cell_load_rows(x + (((size_t)b * H) * T + pb) * kHeadDim, perm + tok0 + 32 * it + 16 * rps, (uint32_t)perm_block - 1u,
-                           (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2), xr);
-        } else {
-            cell_load(x + (((size_t)b * H_all + hbase + jc) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
-        }
+        cell_load(x + (((size_t)b * H + jh) * T + tok0 + 32 * it + 16 * rp) * kHeadDim + 4 * t, xr);
         __syncthreads();
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         typename PacksOf<WIDE>::type u;
@@ -1401,8 +1223,8 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
         __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
         const uint32_t tot_even = s_tot[0][j][t >> 3], tot_odd = s_tot[1][j][t >> 3];
         if (it == 3) {
-            // the last units' sizes are known before their packs are written: the group's size is published now, so
-            // that the workgroups behind it in the stream wait that much less for it
+            // the last units' sizes are known before their packs are written: the workgroup's size is published now,
+            // so that the workgroups behind it in the stream wait that much less for it
             if (active && rp == 0 && m == 0) s_usz[blkid][2 * w + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
             __syncthreads();
             if (tid == 0) {
@@ -1454,7 +1276,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < nblk) {
-        const uint32_t first = XCH ? grp * (uint32_t)(2 * H_all) + (uint32_t)(2 * hbase) : grp_first * (uint32_t)(2 * H);    // block index = group * 2 H + 2 head + half
+        const uint32_t first = grp_first * (uint32_t)(2 * H);             // block index = group * 2 H + 2 head + half
         info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
         info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
@@ -1485,13 +1307,13 @@ __global__ void __launch_bounds__(512) v_quant_encode_rounds_kernel(
 // PERM: the tokens in the order of a repacking, as in the round-major kernel; with scale_in / zero_in (the tokens'
 // parameters in the order of x, known from the pass that made the order) nothing is left to exchange and an
 // iteration has no barrier at all.
-template <int DT, bool WIDE, bool PERM>
+template <int DT, bool WIDE, bool PERM, bool XCH = false>
 __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     const uint16_t *__restrict__ x, int B, int H, int T, float rel, uint16_t *__restrict__ scale,
     uint16_t *__restrict__ zero, uint8_t *__restrict__ stream, uint64_t capacity, uint32_t *__restrict__ info,
     ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, uint64_t base, int par_stride,
     const uint32_t *__restrict__ perm, int perm_block, const uint16_t *__restrict__ scale_in,
-    const uint16_t *__restrict__ zero_in, const Stagger stagger) {
+    const uint16_t *__restrict__ zero_in, const Stagger stagger, int nsg = 1, uint64_t *xw = nullptr) {
     extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
     __shared__ uint32_t s_idx;
     __shared__ uint64_t s_off;
@@ -1505,20 +1327,27 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     __syncthreads();
     const uint32_t gidx = PERM ? (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx) : s_idx;
     if (gidx >= ngroups) return;
+    // XCH (more than eight heads): runs of eight heads that exchange the minima and maxima of their heads per token,
+    // as in the K kernel; a run's words are [iteration][token of the iteration]
+    const int H_all = H;
+    const uint32_t sgi = XCH ? gidx % (uint32_t)nsg : 0u;
+    const int hbase = XCH ? 8 * (int)sgi : 0;
+    if (XCH) H = min(8, H_all - hbase);
     const int j = tid >> 6, rp = (tid >> 5) & 1, t = tid & 31, wave = j, lane = tid & 63;
-    const uint32_t cb = gidx / (uint32_t)B, b = gidx % (uint32_t)B;
+    const uint32_t grp = XCH ? gidx / (uint32_t)nsg : gidx;
+    const uint32_t cb = grp / (uint32_t)B, b = grp % (uint32_t)B;
     const size_t tok0 = (size_t)cb * 128;
     const UnitGeom g = unit_geom(W);
     const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
     const bool active = j < H;
     const int jc = min(j, H - 1);
-    const TokPar *my_par = s_par + 32 * wave + 16 * rp;
+    const TokPar *my_par = (XCH ? s_par : s_par + 32 * wave) + 16 * rp;
     const int blkid = 2 * j + (t >> 4), w = (t >> 3) & 1, m = t & 7;
     for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)                 // metadata areas start as zeros
         reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
     uint32_t run_off = 0;
     uint32_t cmax_all = 0;
-    const uint16_t *cells = x + (((size_t)b * H + jc) * T + tok0 + 16 * rp) * kHeadDim + 4 * t;
+    const uint16_t *cells = x + (((size_t)b * H_all + hbase + jc) * T + tok0 + 16 * rp) * kHeadDim + 4 * t;
     const uint32_t plane = (uint32_t)(((size_t)jc * T * kHeadDim + 4 * t) * 2);
     const bool known = PERM && scale_in != nullptr;              // uniform
     if (known) __syncthreads();                                  // the metadata zeros are in place before the first OR (no barrier below)
@@ -1549,6 +1378,50 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
             if ((lane & 1) == 0) s_mm[it & 1][wave][lane >> 1] = T16<DT>::to_bits(mn) | (T16<DT>::to_bits(mx) << 16);
         }
         __syncthreads();
+        if (XCH) {
+            if (wave == 0) {
+                const int tk = lane & 31;
+                float rmn = INFINITY, rmx = -INFINITY;
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const uint32_t p = s_mm[it & 1][q][tk];
+                    rmn = fminf(rmn, T16<DT>::from_bits(p & 0xFFFFu));
+                    rmx = fmaxf(rmx, T16<DT>::from_bits(p >> 16));
+                }
+                uint64_t *words = xw + (size_t)(gidx - sgi) * 128 + 32 * it;      // [run][iteration][token] of this group
+                if (lane < 32)
+                    __hip_atomic_store(words + (size_t)sgi * 128 + lane, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(rmn) << 16) | (uint64_t)T16<DT>::to_bits(rmx),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // lane = (parity of the run, token)
+                float amn = INFINITY, amx = -INFINITY;
+                for (int run = lane >> 5; run < nsg; run += 2) {
+                    const uint64_t *wp = words + (size_t)run * 128 + tk;
+                    uint64_t w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    int spins = 0;
+                    while ((w >> 63) == 0 && spins < kSpinLimit) {
+                        __builtin_amdgcn_s_sleep(8);
+                        w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        spins++;
+                    }
+                    if ((w >> 63) == 0) atomicExch(&st->error, (uint32_t)PKV_ERR_INTERNAL);     // (bounded wait: the host reports it)
+                    amn = fminf(amn, T16<DT>::from_bits((uint32_t)(w >> 16) & 0xFFFFu));
+                    amx = fmaxf(amx, T16<DT>::from_bits((uint32_t)w & 0xFFFFu));
+                }
+                amn = fminf(amn, __shfl_xor(amn, 32, 64)); amx = fmaxf(amx, __shfl_xor(amx, 32, 64));
+                if (lane < 32) {
+                    const float range = round_t<DT>(amx - amn);
+                    const float sc = round_t<DT>(range * rel);
+                    const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(amn, sc))));
+                    if (sgi == 0) {
+                        const size_t tok = (size_t)b * par_stride + tok0 + 32 * it + lane;
+                        scale[tok] = (uint16_t)T16<DT>::to_bits(sc);
+                        zero[tok] = (uint16_t)zb;
+                    }
+                    s_par[lane] = token_par<DT>(sc, zb, false);
+                }
+            }
+            __syncthreads();
+        } else
         if (lane < 32) {
             float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
@@ -1635,8 +1508,9 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     const uint64_t off = s_off;
     if (off + bytes > capacity) return;
     if (tid < nblk) {
-        info[2 * (size_t)(gidx * (uint32_t)nblk + tid)] = (uint32_t)(off + blk_off[tid]);
-        info[2 * (size_t)(gidx * (uint32_t)nblk + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+        const uint32_t first = XCH ? grp * (uint32_t)(2 * H_all) + (uint32_t)(2 * hbase) : gidx * (uint32_t)nblk;    // block index = group * 2 heads + 2 head + half
+        info[2 * (size_t)(first + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(first + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
     }
     const int q = tid >> 5;
     if (q < nblk) {
@@ -1873,10 +1747,10 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             const int gpw = (H <= 4 && !perm) ? kSubBlocks / H : 1;
             const uint32_t ngroups = (ngroups_all + (uint32_t)gpw - 1u) / (uint32_t)gpw;
             // (a token order always comes with gpw == 1, i.e. the cells kernel)
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true, false>)
-                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false, false>);
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true>)
+                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false>
+                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false>);
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             Stagger sg;
@@ -1894,12 +1768,12 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
                 if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 512, lds, ngroups, &sg))) return rc;
                 cells<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
                                                 stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, perm, perm_block,
-                                                (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg);
+                                                (const uint16_t *)scale_in, (const uint16_t *)zero_in, sg, 1, nullptr);
             } else {
                 if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
                 kern<<<ngroups, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
-                                               stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, nullptr, 0,
-                                               nullptr, nullptr, sg, gpw, ngroups_all, 1, nullptr);
+                                               stream, capacity, info, st, bits, ngroups, unit_slot, base, par_stride, sg, gpw,
+                                               ngroups_all);
             }
         } else if (IS_K && H <= kSubBlocks) {       // nsub == number of groups
             const uint32_t slot = (bound + 15u) & ~15u;
@@ -1909,10 +1783,10 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
             const uint32_t lds = (uint32_t)(gpw * H) * slot + 32u;
             // (a token order always comes with gpw == 1, i.e. the cells kernel: the round-major kernel serves groups of
             // up to four heads in their own order)
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true, false>)
-                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false, false>);
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true>)
+                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false>
+                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false>);
             Stagger sg;
             if (gpw == 1) {                         // five to eight heads: x read once, as cells
                 auto cells = perm ? (bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, true, true>
@@ -1925,39 +1799,39 @@ static int run_quant_encode(const void *x, int dtype, int B, int H, int T, float
                                                                   : k_quant_encode_cells_kernel<PKV_BF16, false, false>));
                 if ((rc = stagger_for(reinterpret_cast<const void *>(cells), 256, lds, nwg, &sg))) return rc;
                 cells<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                            capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg);
+                                            capacity, info, st, bits, nwg, slot, base, par_stride, perm, perm_block, sg, 1, nullptr);
             } else {
                 if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nwg, &sg))) return rc;
                 kern<<<nwg, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                           capacity, info, st, bits, nwg, slot, base, par_stride, nullptr, 0, sg, gpw, nsub, 1, nullptr);
+                                           capacity, info, st, bits, nwg, slot, base, par_stride, sg, gpw, nsub);
             }
         } else if (IS_K) {                           // more than eight heads: runs of eight, one workgroup each, that exchange their minima and maxima
             const uint32_t slot = (bound + 15u) & ~15u;
             const uint32_t lds = (uint32_t)kSubBlocks * slot + 32u;
             const int nsg = (H + kSubBlocks - 1) / kSubBlocks;
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, true, false, true>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, true, false, true>)
-                                 : (dtype == PKV_F16 ? k_quant_encode_rounds_kernel<PKV_F16, false, false, true>
-                                                      : k_quant_encode_rounds_kernel<PKV_BF16, false, false, true>);
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, true, false, true>
+                                                      : k_quant_encode_cells_kernel<PKV_BF16, true, false, true>)
+                                 : (dtype == PKV_F16 ? k_quant_encode_cells_kernel<PKV_F16, false, false, true>
+                                                      : k_quant_encode_cells_kernel<PKV_BF16, false, false, true>);
             Stagger sg;
             if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, nsub, &sg))) return rc;
             kern<<<nsub, 256, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero, stream,
-                                        capacity, info, st, bits, nsub, slot, base, par_stride, nullptr, 0, sg, 1, nsub, nsg,
+                                        capacity, info, st, bits, nsub, slot, base, par_stride, nullptr, 0, sg, nsg,
                                         st->status + nsub);
         } else {                                     // V, more than eight heads: the same runs of eight
             const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
             const uint32_t lds = 64u * unit_slot + 64u;
-            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, true, false, true>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, true, false, true>)
-                                 : (dtype == PKV_F16 ? v_quant_encode_rounds_kernel<PKV_F16, false, false, true>
-                                                      : v_quant_encode_rounds_kernel<PKV_BF16, false, false, true>);
+            auto kern = bits > 4 ? (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, true, false, true>
+                                                      : v_quant_encode_cells_kernel<PKV_BF16, true, false, true>)
+                                 : (dtype == PKV_F16 ? v_quant_encode_cells_kernel<PKV_F16, false, false, true>
+                                                      : v_quant_encode_cells_kernel<PKV_BF16, false, false, true>);
             PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             Stagger sg;
             if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, nruns_all, &sg))) return rc;
             kern<<<nruns_all, 512, lds, s>>>((const uint16_t *)x, B, H, T, rel, (uint16_t *)scale, (uint16_t *)zero,
                                              stream, capacity, info, st, bits, nruns_all, unit_slot, base, par_stride, nullptr, 0,
-                                             nullptr, nullptr, sg, 1, nruns_all, nruns, st->status + nruns_all);
+                                             nullptr, nullptr, sg, nruns, st->status + nruns_all);
         }
         PKV_HIP_CHECK(hipGetLastError());
         if ((rc = tm.end(ms_out))) return rc;
