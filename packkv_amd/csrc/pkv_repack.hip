@@ -703,10 +703,13 @@ typedef unsigned short pk_u16x2 __attribute__((ext_vector_type(2)));
 
 __global__ void __launch_bounds__(256) pack_size_kernel(const uint8_t *__restrict__ codes, int hidden, int pack_len,
                                                         size_t n_items, PackSizeOut *out) {
-    __shared__ uint32_t seen[256];
+    // a presence word per (code value, lane % 32): a lane marks its own column, so the marks of a wavefront never
+    // share a bank however few values the matrix holds (one word per value made every mark a same-address conflict)
+    __shared__ uint32_t seen[256 * 32];
     __shared__ unsigned long long wsum[4];
-    seen[threadIdx.x] = 0u;
+    for (int i = threadIdx.x; i < 256 * 32; i += 256) seen[i] = 0u;
     __syncthreads();
+    uint32_t *col = seen + (threadIdx.x & 31);
     const uint32_t chunks = (uint32_t)hidden / 16u;
     unsigned long long lens = 0;
     for (size_t item = (size_t)blockIdx.x * 256 + threadIdx.x; item < n_items; item += (size_t)gridDim.x * 256) {
@@ -726,10 +729,10 @@ __global__ void __launch_bounds__(256) pack_size_kernel(const uint8_t *__restric
                 mx[2 * i] = __builtin_elementwise_max(mx[2 * i], e);
                 mn[2 * i + 1] = __builtin_elementwise_min(mn[2 * i + 1], o);
                 mx[2 * i + 1] = __builtin_elementwise_max(mx[2 * i + 1], o);
-                seen[e[0]] = 1u;              // every writer stores the same value
-                seen[e[1]] = 1u;
-                seen[o[0]] = 1u;
-                seen[o[1]] = 1u;
+                col[32u * e[0]] = 1u;
+                col[32u * e[1]] = 1u;
+                col[32u * o[0]] = 1u;
+                col[32u * o[1]] = 1u;
             }
         };
         int k = 0;
@@ -756,7 +759,12 @@ __global__ void __launch_bounds__(256) pack_size_kernel(const uint8_t *__restric
     if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = lens;
     __syncthreads();
     if (threadIdx.x == 0) atomicAdd(&out->len_sum, wsum[0] + wsum[1] + wsum[2] + wsum[3]);
-    if (seen[threadIdx.x]) out->present[threadIdx.x] = 1u;
+    {   // value threadIdx.x: any of its 32 columns (read rotated, so that the threads of a wavefront spread over the banks)
+        uint32_t any = 0u;
+#pragma unroll 8
+        for (int c = 0; c < 32; c++) any |= seen[32 * threadIdx.x + ((c + threadIdx.x) & 31)];
+        if (any) out->present[threadIdx.x] = 1u;
+    }
 }
 
 }  // namespace pkv
