@@ -203,7 +203,7 @@ __device__ __forceinline__ void lds_put_meta(uint8_t *arr, int t, int nbits, uin
     } else if (nbits == 2) {
         arr[t] = (uint8_t)w;
     } else if (nbits == 3) {  // 12 bits per lane: an even/odd lane pair shares three bytes
-        const uint32_t hi = __shfl_down(w, 1, 32);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xF5, 0xF, 0xF, false);    // the odd neighbour's word (quad_perm [1,1,3,3])
         if ((t & 1) == 0) {
             const uint32_t v = w | (hi << 12);
             uint8_t *p = arr + (t >> 1) * 3;
@@ -217,7 +217,7 @@ __device__ __forceinline__ void lds_put_meta(uint8_t *arr, int t, int nbits, uin
         p[1] = (uint8_t)(w >> 8);
         p[2] = (uint8_t)(w >> 16);
     } else {                  // nbits == 5: 20 bits per lane, an even/odd lane pair shares five bytes
-        const uint32_t hi = __shfl_down(w, 1, 32);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xF5, 0xF, 0xF, false);    // the odd neighbour's word (quad_perm [1,1,3,3])
         if ((t & 1) == 0) {
             const uint64_t v = (uint64_t)w | ((uint64_t)hi << 20);
             uint8_t *p = arr + (t >> 1) * 5;

@@ -623,20 +623,24 @@ __device__ __forceinline__ void cell_packs(const uint2 xr[16], const TokPar *par
 template <bool WIDE> struct PacksOf { typedef UnitPacks type; };
 template <> struct PacksOf<true> { typedef UnitPacksW type; };
 
-// the 2 * len bytes of pack k at dst (2-byte aligned)
+// the 2 * len bytes of pack k at dst (2-byte aligned): one predicated 16-bit store per piece, written out (a loop
+// over the lane's own length costs a shift, a compare and the loop's control flow per piece)
 __device__ __forceinline__ void put_pack(uint16_t *dst, const UnitPacks &u, int k) {
-    uint64_t wd = u.word[k];
-    for (uint32_t q = 0; q < u.len[k]; q++) {
-        dst[q] = (uint16_t)wd;
-        wd >>= 16;
-    }
+    const uint32_t lo = (uint32_t)u.word[k], hi = (uint32_t)(u.word[k] >> 32), len = u.len[k];
+    if (len > 0u) dst[0] = (uint16_t)lo;
+    if (len > 1u) dst[1] = (uint16_t)(lo >> 16);
+    if (len > 2u) dst[2] = (uint16_t)hi;
+    if (len > 3u) dst[3] = (uint16_t)(hi >> 16);
 }
 __device__ __forceinline__ void put_pack(uint16_t *dst, const UnitPacksW &u, int k) {
-    unsigned __int128 wd = ((unsigned __int128)u.hi[k] << (8u * u.len[k])) | u.lo[k];
-    for (uint32_t q = 0; q < u.len[k]; q++) {
-        dst[q] = (uint16_t)wd;
-        wd >>= 16;
-    }
+    const unsigned __int128 wd = ((unsigned __int128)u.hi[k] << (8u * u.len[k])) | u.lo[k];
+    const uint32_t d0 = (uint32_t)wd, d1 = (uint32_t)(wd >> 32), d2 = (uint32_t)(wd >> 64), len = u.len[k];
+    if (len > 0u) dst[0] = (uint16_t)d0;
+    if (len > 1u) dst[1] = (uint16_t)(d0 >> 16);
+    if (len > 2u) dst[2] = (uint16_t)d1;
+    if (len > 3u) dst[3] = (uint16_t)(d1 >> 16);
+    if (len > 4u) dst[4] = (uint16_t)d2;
+    if (len > 5u) dst[5] = (uint16_t)(d2 >> 16);
 }
 
 // Emit one analysed unit at blk[unit_off] (the K layout: lane t's packs sit where they were computed).
