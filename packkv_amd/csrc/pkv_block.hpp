@@ -241,12 +241,14 @@ __device__ __forceinline__ void unit_emit(uint8_t *blk, uint32_t unit_off, int t
     uint8_t *pay = blk + unit_off + g.mins_bytes + g.lens_bytes;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+        // one predicated 16-bit store per piece, written out (a loop over the lane's own length costs a shift, a
+        // compare and the loop's control flow per piece)
         uint16_t *dst = reinterpret_cast<uint16_t *>(pay + u.off[i]);
-        uint64_t w = u.word[i];
-        for (uint32_t b = 0; b < u.len[i]; b++) {
-            dst[b] = (uint16_t)w;
-            w >>= 16;
-        }
+        const uint32_t lo = (uint32_t)u.word[i], hi = (uint32_t)(u.word[i] >> 32), len = u.len[i];
+        if (len > 0u) dst[0] = (uint16_t)lo;
+        if (len > 1u) dst[1] = (uint16_t)(lo >> 16);
+        if (len > 2u) dst[2] = (uint16_t)hi;
+        if (len > 3u) dst[3] = (uint16_t)(hi >> 16);
     }
 }
 
