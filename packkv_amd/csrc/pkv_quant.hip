@@ -1124,14 +1124,25 @@ __device__ __forceinline__ void meta_or4(uint8_t *arr, int m, int FB, int i, con
         }
         return;
     }
-    uint64_t v = 0;
-#pragma unroll
-    for (int k = 0; k < 4; k++) v |= (uint64_t)f[k] << (4 * FB * k + FB * i);
-    const uint32_t byte = 2u * (uint32_t)FB * (uint32_t)m;
+    if (FB == 4) {                                // fields on 16-bit lanes: two aligned words, 32-bit arithmetic only
+        uint32_t *w = reinterpret_cast<uint32_t *>(arr + 8u * (uint32_t)m);
+        atomicOr(w, (f[0] | (f[1] << 16)) << (4 * i));
+        atomicOr(w + 1, (f[2] | (f[3] << 16)) << (4 * i));
+        return;
+    }
+    if (FB == 2) {                                // fields on byte lanes: one aligned word
+        uint32_t *w = reinterpret_cast<uint32_t *>(arr + 4u * (uint32_t)m);
+        atomicOr(w, (f[0] | (f[1] << 8) | (f[2] << 16) | (f[3] << 24)) << (2 * i));
+        return;
+    }
+    // FB == 3: 48 bits at byte 6 m (odd m: two bytes into the word; 48 + 16 bits still fit two words)
+    const uint32_t lo = (f[0] | (f[1] << 12)) << (3 * i), hi = (f[2] | (f[3] << 12)) << (3 * i);     // 27 bits each
+    uint64_t v = (uint64_t)lo | ((uint64_t)hi << 24);
+    const uint32_t byte = 6u * (uint32_t)m;
     uint32_t *w = reinterpret_cast<uint32_t *>(arr + (byte & ~3u));
-    v <<= 8u * (byte & 3u);                       // FB = 3 puts odd m two bytes into the word; 48 + 16 bits still fit
+    v <<= 8u * (byte & 3u);
     atomicOr(w, (uint32_t)v);
-    if (FB > 2) atomicOr(w + 1, (uint32_t)(v >> 32));
+    atomicOr(w + 1, (uint32_t)(v >> 32));
 }
 
 // Inclusive prefix sum over each run of eight lanes (m = lane % 8) on the DPP data path; `total` receives the run's
