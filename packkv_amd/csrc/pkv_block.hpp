@@ -303,11 +303,11 @@ __device__ __forceinline__ uint32_t unit_encode_wide(const uint8_t *tile, int hi
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         uint16_t *dst = reinterpret_cast<uint16_t *>(pay + off[i]);
-        word128 w = word[i];
-        for (uint32_t b = 0; b < len[i]; b++) {
-            dst[b] = (uint16_t)w;
-            w >>= 16;
-        }
+        const word128 w = word[i];
+        const uint32_t d[4] = {(uint32_t)w, (uint32_t)(w >> 32), (uint32_t)(w >> 64), (uint32_t)(w >> 96)};
+#pragma unroll
+        for (uint32_t b = 0; b < 8; b++)                  // (written out: one predicated 16-bit store per piece)
+            if (b < len[i]) dst[b] = (uint16_t)(d[b >> 1] >> (16u * (b & 1u)));
     }
     return meta + payload;
 }

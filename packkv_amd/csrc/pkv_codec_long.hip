@@ -40,11 +40,13 @@ __device__ __forceinline__ void long_put_sub(uint16_t *dst, const uint32_t c[16]
         hi = (hi << len) | c[k];
         lo = (lo << len) | c[8 + k];
     }
-    unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
-    for (uint32_t q = 0; q < len; q++) {
-        dst[q] = (uint16_t)wd;
-        wd >>= 16;
-    }
+    const unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
+    // one predicated 16-bit store per piece, written out (a loop over the lane's own length costs a 128-bit shift, a
+    // compare and the loop's control flow per piece)
+    const uint32_t d[4] = {(uint32_t)wd, (uint32_t)(wd >> 32), (uint32_t)(wd >> 64), (uint32_t)(wd >> 96)};
+#pragma unroll
+    for (uint32_t q = 0; q < 8; q++)
+        if (q < len) dst[q] = (uint16_t)(d[q >> 1] >> (16u * (q & 1u)));
 }
 
 __device__ __forceinline__ void long_get_sub(const uint16_t *src, uint32_t c[16], uint32_t len) {
@@ -217,11 +219,11 @@ __device__ __forceinline__ void long_put_sub_swz(uint8_t *image, uint32_t off, c
         hi = (hi << len) | c[k];
         lo = (lo << len) | c[8 + k];
     }
-    unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
-    for (uint32_t q = 0; q < len; q++) {
-        *reinterpret_cast<uint16_t *>(image + long_swz(off + 2u * q)) = (uint16_t)wd;
-        wd >>= 16;
-    }
+    const unsigned __int128 wd = ((unsigned __int128)hi << (8u * len)) | lo;       // 8 * len bits are len whole bytes
+    const uint32_t d[4] = {(uint32_t)wd, (uint32_t)(wd >> 32), (uint32_t)(wd >> 64), (uint32_t)(wd >> 96)};
+#pragma unroll
+    for (uint32_t q = 0; q < 8; q++)                      // (written out, as in long_put_sub)
+        if (q < len) *reinterpret_cast<uint16_t *>(image + long_swz(off + 2u * q)) = (uint16_t)(d[q >> 1] >> (16u * (q & 1u)));
 }
 
 // n bytes (even) of the swizzled image -> global memory (dst 2-byte aligned) by the whole workgroup: head to the first
