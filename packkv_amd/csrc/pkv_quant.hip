@@ -726,6 +726,20 @@ __device__ __forceinline__ uint32_t bf16_keys(uint32_t w) {
     const i16x2 m = (v >> (short)15) & (short)0x7FFF;
     return __builtin_bit_cast(uint32_t, (i16x2)(v ^ m));
 }
+// A token's (minimum, maximum) as one word that a packed MINIMUM combines: the minimum in the low half, the negated
+// maximum in the high half (fp16: sign bit flipped; bf16: both as order keys, the maximum's complemented).
+template <int DT>
+__device__ __forceinline__ uint32_t minmax_word(float mn, float mx) {
+    if (DT == PKV_F16) return T16<DT>::to_bits(mn) | ((T16<DT>::to_bits(mx) ^ 0x8000u) << 16);
+    return bf16_keys(T16<DT>::to_bits(mn) | (T16<DT>::to_bits(mx) << 16)) ^ 0xFFFF0000u;
+}
+template <int DT>
+__device__ __forceinline__ void minmax_unword(uint32_t w, float &mn, float &mx) {
+    if (DT != PKV_F16) w = bf16_keys(w ^ 0xFFFF0000u);
+    else w ^= 0x80000000u;
+    mn = T16<DT>::from_bits(w & 0xFFFFu);
+    mx = T16<DT>::from_bits(w >> 16);
+}
 template <bool MAX, bool KEYS>
 __device__ __forceinline__ uint32_t swap32_sel(uint32_t a, uint32_t b) {
     const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
@@ -1335,7 +1349,7 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     __shared__ uint32_t blk_off[17];
     __shared__ uint16_t s_usz[16][4];
     __shared__ __attribute__((aligned(16))) TokPar s_par[8 * 32];       // [wavefront][token of the iteration]
-    __shared__ uint32_t s_mm[2][8][32];                                  // [iteration parity][wavefront][token]: min | max << 16 (16-bit patterns)
+    __shared__ uint32_t s_mm[2][8][32];                                  // [iteration parity][wavefront][token]: minmax_word
     const int tid = threadIdx.x;
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
@@ -1390,19 +1404,17 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
         {
             float mn, mx;
             cell_token_minmax_halves<DT>(xr, mn, mx);
-            if ((lane & 1) == 0) s_mm[it & 1][wave][lane >> 1] = T16<DT>::to_bits(mn) | (T16<DT>::to_bits(mx) << 16);
+            if ((lane & 1) == 0) s_mm[it & 1][wave][lane >> 1] = minmax_word<DT>(mn, mx);
         }
         __syncthreads();
         if (XCH) {
             if (wave == 0) {
                 const int tk = lane & 31;
-                float rmn = INFINITY, rmx = -INFINITY;
+                uint32_t pw = s_mm[it & 1][0][tk];
 #pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    const uint32_t p = s_mm[it & 1][q][tk];
-                    rmn = fminf(rmn, T16<DT>::from_bits(p & 0xFFFFu));
-                    rmx = fmaxf(rmx, T16<DT>::from_bits(p >> 16));
-                }
+                for (int q = 1; q < 8; q++) pw = pk_sel_x<false, DT != PKV_F16>(pw, s_mm[it & 1][q][tk]);
+                float rmn, rmx;
+                minmax_unword<DT>(pw, rmn, rmx);
                 uint64_t *words = xw + (size_t)(gidx - sgi) * 128 + 32 * it;      // [run][iteration][token] of this group
                 if (lane < 32)
                     __hip_atomic_store(words + (size_t)sgi * 128 + lane, (1ull << 63) | ((uint64_t)T16<DT>::to_bits(rmn) << 16) | (uint64_t)T16<DT>::to_bits(rmx),
@@ -1438,13 +1450,11 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
             __syncthreads();
         } else
         if (lane < 32) {
-            float mn = INFINITY, mx = -INFINITY;
+            uint32_t pw = s_mm[it & 1][0][lane];             // the eight heads' words, combined by packed minima
 #pragma unroll
-            for (int q = 0; q < 8; q++) {
-                const uint32_t p = s_mm[it & 1][q][lane];
-                mn = fminf(mn, T16<DT>::from_bits(p & 0xFFFFu));
-                mx = fmaxf(mx, T16<DT>::from_bits(p >> 16));
-            }
+            for (int q = 1; q < 8; q++) pw = pk_sel_x<false, DT != PKV_F16>(pw, s_mm[it & 1][q][lane]);
+            float mn, mx;
+            minmax_unword<DT>(pw, mn, mx);
             const float range = round_t<DT>(mx - mn);
             const float sc = round_t<DT>(range * rel);
             const uint32_t zb = T16<DT>::to_bits(rintf(round_t<DT>(__fdiv_rn(mn, sc))));
