@@ -170,6 +170,35 @@ def test_fused_quant_encode_round_trip_full_size(cuda):
         del r, codes, back
 
 
+@pytest.mark.parametrize("B,H,T,dtype,rel", [(16, 8, 32768, torch.bfloat16, 0.1), (8, 7, 16384, torch.bfloat16, 0.2),
+                                             (2, 40, 8192, torch.float16, 0.05)])
+def test_fused_quant_encode_large_shapes_repeat_and_round_trip(cuda, B, H, T, dtype, rel):
+    """Thousands of workgroups in flight (the in-order stream offsets, the exchange between runs of eight heads, the
+    wavefronts' shared minima and maxima): three launches give the same bytes, the parameters are the stand-alone
+    quantizer's, and the stream unpacks to its codes."""
+    k, v = synth.make_kv(B, H, T, seed=5, device=cuda, dtype=dtype)
+    bits = ops.bits_for_rel(rel)
+    for is_k, x in ((True, k), (False, v)):
+        scale, zero = ops.quant_params(x, rel)
+        codes, _ = ops.quantize(x, scale, zero)
+        first = None
+        for _ in range(3):
+            r = (ops.k_quant_encode if is_k else ops.v_quant_encode)(x, rel, bits)
+            assert torch.equal(scale, r["scale"]) and torch.equal(zero, r["zero"])
+            got = (r["size"], r["stream"][:r["size"]].clone(), r["info"].clone())
+            if first is None:
+                first = got
+            else:
+                assert got[0] == first[0] and torch.equal(got[1], first[1]) and torch.equal(got[2], first[2])
+        back = torch.empty_like(codes)
+        if is_k:
+            ops.k_decode(r["stream"], r["info"], back, 64, 128, bits)
+        else:
+            ops.v_decode(r["stream"], r["info"], back, 128, 64, bits)
+        assert torch.equal(back, codes)
+        del r, codes, back, first, got
+
+
 def test_asynchronous_encode_reports_through_encode_status(cuda):
     """want_size=False keeps the launch asynchronous and reports nothing by itself; ops.encode_status then gives the
     size, or raises what the synchronous form raises: a stream that does not fit, a code wider than bits_len.  A
