@@ -25,12 +25,6 @@ typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
 // ((x | 0x80) - (probe + 1) keeps bit 7 of a byte exactly when the byte is above the probe; no borrow crosses bytes
 // while both are at most 128).  Other rows use a 256-bin histogram in LDS (slow when few values dominate: equal
 // addresses serialise the LDS atomics).
-__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
-    return x;
-}
-
 __global__ void __launch_bounds__(256) token_median_kernel(const uint8_t *__restrict__ codes, int ctx_len, int hidden,
                                                            uint8_t *__restrict__ median) {
     __shared__ uint32_t hist[4][256];
