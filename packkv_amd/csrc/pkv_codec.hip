@@ -378,6 +378,19 @@ static int run_pack(bool is_k, const uint8_t *codes, uint8_t *stream, uint64_t c
     // of LDS leave one workgroup per CU and the per-block kernel is 10 % faster)
     const bool grouped = cs.nunits == 4 && bits <= 7 && hid_blk % 16 == 0 && hidden_dim % 16 == 0 &&
                          (reinterpret_cast<uintptr_t>(codes) & 15u) == 0;
+    // the reference's block shapes over rows that are whole groups of 1024 channels: the cells kernels (no code tile
+    // in LDS, the next round in flight while packs are formed)
+    const bool cells = bits <= 6 && hidden_dim % 1024 == 0 && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
+                       (is_k ? (ctx_blk == 64 && hid_blk == 128) : (ctx_blk == 128 && hid_blk == 64));
+    if (cells) {
+        const uint32_t ngroups = (uint32_t)cs.nblocks / (is_k ? 8u : 16u);
+        if ((rc = prepare_scan_state(ngroups, &st, s))) return rc;
+        LaunchTimer tm(s, ms_out != nullptr);
+        if ((rc = tm.begin())) return rc;
+        if ((rc = launch_code_cells(is_k, codes, ctx_len, hidden_dim, bits, cs.blk_cap, stream, capacity, info, st, ngroups, s))) return rc;
+        if ((rc = tm.end(ms_out))) return rc;
+        return finish_encode(st, size_out, 0, s);
+    }
     if (grouped) {
         const uint32_t ngroups = ((uint32_t)cs.nblocks + kPackGroup - 1) / kPackGroup;
         const uint32_t lds = 2u * (uint32_t)(ctx_blk * hid_blk) + (uint32_t)kPackGroup * cs.blk_cap + 32u;

@@ -1551,6 +1551,225 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
     }
 }
 
+// ---- the block codec from a code matrix, as cells --------------------------------------------------------------
+// The cells encoders with nothing to quantize: the input is the uint8 code matrix [ctx_len, hidden] of pkv_k_encode /
+// pkv_v_encode.  Eight consecutive K blocks (64 x 128) or sixteen consecutive V blocks (128 x 64) of the stream are
+// 1024 adjacent channels of one context block, i.e. exactly the group a cells workgroup owns, with the "heads" being
+// 128-channel slices of the matrix.  A thread reads its cell as sixteen dwords (four codes of one token each; the 32
+// lanes of a half-wavefront one 128-byte line per token), asks for the next round's while it forms and emits this
+// round's packs, and no code tile is staged in LDS.  For hidden a multiple of 1024, the reference's block shapes and
+// widths up to 6; pack_group_kernel takes everything else.
+__device__ __forceinline__ void code_cell_load(const uint8_t *cell, size_t row_bytes, uint32_t w[16]) {
+#pragma unroll
+    for (int k = 0; k < 16; k++) w[k] = *reinterpret_cast<const uint32_t *>(cell + (size_t)k * row_bytes);
+}
+// four codes of a dword as two pairs of 16-bit integers (codes 0, 1 and codes 2, 3)
+__device__ __forceinline__ void code_cell_pairs(const uint32_t w[16], uint32_t c01[16], uint32_t c23[16]) {
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        c01[k] = __builtin_amdgcn_perm(0u, w[k], 0x0C010C00u);
+        c23[k] = __builtin_amdgcn_perm(0u, w[k], 0x0C030C02u);
+    }
+}
+
+template <bool WIDE>
+__global__ void __launch_bounds__(256) k_code_cells_kernel(
+    const uint8_t *__restrict__ codes, int hidden, uint8_t *__restrict__ stream, uint64_t capacity,
+    uint32_t *__restrict__ info, ScanState *st, int W, uint32_t ngroups, uint32_t bound, const Stagger stagger) {
+    extern __shared__ __align__(16) uint8_t gbuf[];        // 8 block slots of `bound` bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[kSubBlocks + 1];
+    const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);
+    if (gidx >= ngroups) return;
+    const int j = tid >> 5, t = tid & 31;                 // block of the group, lane of the unit
+    const uint32_t per_row = (uint32_t)hidden / 1024u;    // groups per context block
+    const uint32_t cb = gidx / per_row, hg = gidx % per_row;
+    const UnitGeom g = unit_geom(W);
+    uint8_t *blk = gbuf + (size_t)j * bound;
+    uint32_t my_off = 8u;
+    const uint8_t *cell = codes + (size_t)cb * 64 * (size_t)hidden + (size_t)hg * 1024 + (size_t)j * 128 + 4 * t;
+    uint32_t w[16];
+    code_cell_load(cell, (size_t)hidden, w);
+#pragma unroll 1
+    for (int r = 0; r < 4; r++) {
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
+        uint32_t c01[16], c23[16];
+        code_cell_pairs(w, c01, c23);
+        if (r < 3) code_cell_load(cell + (size_t)(r + 1) * 16 * (size_t)hidden, (size_t)hidden, w);     // travels while the packs are formed
+        typename PacksOf<WIDE>::type u;
+        uint32_t cmax;
+        cell_build(c01, c23, u, cmax);
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+        pack_offsets(u.len, u.off, u.payload);
+        const uint32_t usz = (uint32_t)(g.mins_bytes + g.lens_bytes) + u.payload;
+        if (r == 3) {                                     // the group's size is known before its last units are written
+            if (t == 0) blk_off[j + 1] = my_off + usz;
+            if (tid == 0) blk_off[0] = 0;
+            __syncthreads();
+            if (tid == 0) {
+                for (int q = 1; q <= kSubBlocks; q++) blk_off[q] += blk_off[q - 1];
+                lookback_publish(st, gidx, blk_off[kSubBlocks]);
+            }
+        }
+        if (t == 0) reinterpret_cast<uint16_t *>(blk)[r] = (uint16_t)(my_off - 8u + usz);
+        unit_emit_any(blk, my_off, t, g, u);
+        my_off += usz;
+    }
+    __syncthreads();
+    const uint32_t bytes = blk_off[kSubBlocks];
+    if (tid < 64) {
+        const uint64_t off = lookback_offset(st, gidx, bytes, true);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < kSubBlocks) {
+        info[2 * (size_t)(gidx * (uint32_t)kSubBlocks + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(gidx * (uint32_t)kSubBlocks + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    copy_out32(stream + off + blk_off[j], blk, my_off, t);
+}
+
+// V: the thread roles of v_quant_encode_cells_kernel (a wavefront = one 128-channel slice with both rounds of an
+// iteration in its halves), no barrier inside an iteration.
+template <bool WIDE>
+__global__ void __launch_bounds__(512) v_code_cells_kernel(
+    const uint8_t *__restrict__ codes, int hidden, uint8_t *__restrict__ stream, uint64_t capacity,
+    uint32_t *__restrict__ info, ScanState *st, int W, uint32_t ngroups, uint32_t unit_slot, const Stagger stagger) {
+    extern __shared__ __align__(16) uint8_t gbuf[];        // 16 blocks x 4 units x unit_slot bytes
+    __shared__ uint32_t s_idx;
+    __shared__ uint64_t s_off;
+    __shared__ uint32_t blk_off[17];
+    __shared__ uint16_t s_usz[16][4];
+    const int tid = threadIdx.x;
+    stagger_first_generation(stagger);
+    if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t gidx = s_idx;
+    if (gidx >= ngroups) return;
+    const int j = tid >> 6, rp = (tid >> 5) & 1, t = tid & 31;
+    const uint32_t per_row = (uint32_t)hidden / 1024u;
+    const uint32_t cb = gidx / per_row, hg = gidx % per_row;
+    const UnitGeom g = unit_geom(W);
+    const uint32_t meta = (uint32_t)(g.mins_bytes + g.lens_bytes);
+    const int blkid = 2 * j + (t >> 4), wq = (t >> 3) & 1, m = t & 7;
+    for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)                 // metadata areas start as zeros
+        reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
+    uint32_t run_off = 0;
+    const uint8_t *cell = codes + ((size_t)cb * 128 + 16 * rp) * (size_t)hidden + (size_t)hg * 1024 + (size_t)j * 128 + 4 * t;
+    __syncthreads();                                       // the metadata zeros are in place before the first OR
+#pragma unroll 1
+    for (int it = 0; it < 4; it++) {
+        // (no request ahead: placing the packs holds too many registers, as in v_quant_encode_cells_kernel)
+        uint32_t w[16];
+        code_cell_load(cell + (size_t)it * 32 * (size_t)hidden, (size_t)hidden, w);
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
+        uint32_t c01[16], c23[16];
+        code_cell_pairs(w, c01, c23);
+        typename PacksOf<WIDE>::type u;
+        uint32_t cmax;
+        cell_build(c01, c23, u, cmax);
+        const uint32_t pb = 2u * (u.len[0] + u.len[1] + u.len[2] + u.len[3]);
+        uint32_t tot;
+        const uint32_t inc = oct_incl_scan(pb, m, tot);
+        __builtin_amdgcn_s_setprio(PKV_EPRIO_EMIT);
+        const auto halves = __builtin_amdgcn_permlane32_swap(tot, tot, false, false);      // the even round's total, the odd round's
+        const uint32_t tot_even = halves[0], tot_odd = halves[1];
+        if (it == 3) {
+            if (rp == 0 && m == 0) s_usz[blkid][2 * wq + 1] = (uint16_t)(meta + run_off + tot_even + tot_odd);
+            __syncthreads();
+            if (tid == 0) {
+                uint32_t run = 0;
+                for (int q = 0; q < 16; q++) {
+                    blk_off[q] = run;
+                    run += 8u + s_usz[q][0] + s_usz[q][1] + s_usz[q][2] + s_usz[q][3];
+                }
+                blk_off[16] = run;
+                lookback_publish(st, gidx, run);
+            }
+        }
+        {
+            const int sg = it >> 1, slot = 2 * (it & 1) + rp;
+            uint8_t *unit = gbuf + (size_t)(blkid * 4 + 2 * wq + sg) * unit_slot;
+            meta_or4(unit, m, g.W, slot, u.mn);
+            meta_or4(unit + g.mins_bytes, m, g.LB, slot, u.len);
+            uint32_t o = meta + run_off + (rp ? tot_even : 0u) + (inc - pb);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                put_pack(reinterpret_cast<uint16_t *>(unit + o), u, k);
+                o += 2u * u.len[k];
+            }
+        }
+        run_off += tot_even + tot_odd;
+        if (it & 1) {
+            if (it == 1 && rp == 0 && m == 0) s_usz[blkid][2 * wq] = (uint16_t)(meta + run_off);
+            run_off = 0;
+        }
+    }
+    __syncthreads();
+    const uint32_t bytes = blk_off[16];
+    if (tid < 64) {
+        const uint64_t off = lookback_offset(st, gidx, bytes, true);
+        if (tid == 0) {
+            s_off = off;
+            if (gidx == ngroups - 1) st->total = off + bytes;
+            if (off + bytes > capacity) atomicExch(&st->error, (uint32_t)PKV_ERR_CAPACITY);
+        }
+    }
+    __syncthreads();
+    const uint64_t off = s_off;
+    if (off + bytes > capacity) return;
+    if (tid < 16) {
+        info[2 * (size_t)(gidx * 16u + tid)] = (uint32_t)(off + blk_off[tid]);
+        info[2 * (size_t)(gidx * 16u + tid) + 1] = blk_off[tid + 1] - blk_off[tid];
+    }
+    const int q = tid >> 5;                                // half-wavefront q copies block q
+    uint8_t *dst = stream + off + blk_off[q];
+    uint32_t cum = 0;
+#pragma unroll
+    for (int un = 0; un < 4; un++) {
+        const uint32_t n = s_usz[q][un];
+        copy_out32(dst + 8 + cum, gbuf + (size_t)(q * 4 + un) * unit_slot, n, t);
+        cum += n;
+        if (t == un) reinterpret_cast<uint16_t *>(dst)[un] = (uint16_t)cum;
+    }
+}
+
+// Launch of the two kernels above (pkv_codec.hip decides when they apply): `st` is a prepared scan state with one
+// status word per group, `bound` the worst-case bytes of a block.
+int launch_code_cells(bool is_k, const uint8_t *codes, int ctx_len, int hidden, int bits, uint32_t bound, uint8_t *stream,
+                      uint64_t capacity, uint32_t *info, ScanState *st, uint32_t ngroups, hipStream_t s) {
+    int rc;
+    Stagger sg;
+    if (is_k) {
+        const uint32_t slot = (bound + 15u) & ~15u;
+        const uint32_t lds = (uint32_t)kSubBlocks * slot + 32u;
+        auto kern = bits > 4 ? k_code_cells_kernel<true> : k_code_cells_kernel<false>;
+        if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 256, lds, ngroups, &sg))) return rc;
+        kern<<<ngroups, 256, lds, s>>>(codes, hidden, stream, capacity, info, st, bits, ngroups, slot, sg);
+    } else {
+        const uint32_t unit_slot = (uint32_t)(((bound - 8u) / 4u + 15u) & ~15u);
+        const uint32_t lds = 64u * unit_slot + 64u;
+        auto kern = bits > 4 ? v_code_cells_kernel<true> : v_code_cells_kernel<false>;
+        PKV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if ((rc = stagger_for(reinterpret_cast<const void *>(kern), 512, lds, ngroups, &sg))) return rc;
+        kern<<<ngroups, 512, lds, s>>>(codes, hidden, stream, capacity, info, st, bits, ngroups, unit_slot, sg);
+    }
+    (void)ctx_len;
+    PKV_HIP_CHECK(hipGetLastError());
+    return PKV_OK;
+}
+
 // ---- per-token median of the V codes, straight from V -----------------------------------------------------------
 // `median_repacking` (utils/compute.py:262-270) orders the tokens of a block by the lower median of each token's
 // V codes over ALL channels of all sequences and heads.  This kernel gets those medians without a code matrix: a

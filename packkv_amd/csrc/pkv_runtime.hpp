@@ -56,5 +56,9 @@ int prepare_scan_state(uint32_t nblocks, ScanState **out, hipStream_t s);
 // Reads back {error, total, max_code}; when `size_out` is NULL returns at once (no sync).
 // `bits` > 0 additionally rejects a launch whose largest code does not fit `bits` bits.
 int finish_encode(ScanState *st, uint64_t *size_out, int bits, hipStream_t s);
+// The block codec from a code matrix through the cells kernels (pkv_quant.hip): eight K / sixteen V blocks per group,
+// for hidden a multiple of 1024, the reference's block shapes, widths up to 6.  `st` holds one status word per group.
+int launch_code_cells(bool is_k, const uint8_t *codes, int ctx_len, int hidden, int bits, uint32_t bound, uint8_t *stream,
+                      uint64_t capacity, uint32_t *info, ScanState *st, uint32_t ngroups, hipStream_t s);
 
 }  // namespace pkv

@@ -197,7 +197,9 @@ def test_wide_codes_stream_matches_restatement(cuda, oracle_codec, W):
     byte, to an exact round trip, and the stream size to the closed form (payload 2 * len bytes per pack, W + LB bits
     of metadata per pack, 8 header bytes per block)."""
     rng = np.random.default_rng(40 + W)
-    for is_k, (cb, hb), (T, H) in ((1, (64, 128), (128, 256)), (0, (128, 64), (256, 192)), (1, (32, 128), (96, 128))):
+    # (rows of 1024 and 2048 channels: the kernels that read the code matrix as cells)
+    for is_k, (cb, hb), (T, H) in ((1, (64, 128), (128, 256)), (0, (128, 64), (256, 192)), (1, (32, 128), (96, 128)),
+                                   (1, (64, 128), (128, 2048)), (0, (128, 64), (256, 1024))):
         codes = rng.integers(0, 2 ** W, size=(T, H), dtype=np.uint8)
         codes[: T // 2, ::2] //= 8                 # mixed widths: some packs narrow, some constant
         codes[:16, :32] = 7
