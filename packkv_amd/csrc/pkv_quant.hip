@@ -1559,9 +1559,11 @@ __global__ void __launch_bounds__(512) v_quant_encode_cells_kernel(
 // lanes of a half-wavefront one 128-byte line per token), asks for the next round's while it forms and emits this
 // round's packs, and no code tile is staged in LDS.  For hidden a multiple of 1024, the reference's block shapes and
 // widths up to 6; pack_group_kernel takes everything else.
-__device__ __forceinline__ void code_cell_load(const uint8_t *cell, size_t row_bytes, uint32_t w[16]) {
+// `rows` (uniform: scalar registers) is the first of the 16 token rows, `lane_off` the lane's byte offset inside a
+// row, so that a load is one 32-bit lane offset on a scalar base
+__device__ __forceinline__ void code_cell_load(const uint8_t *rows, size_t row_bytes, uint32_t lane_off, uint32_t w[16]) {
 #pragma unroll
-    for (int k = 0; k < 16; k++) w[k] = *reinterpret_cast<const uint32_t *>(cell + (size_t)k * row_bytes);
+    for (int k = 0; k < 16; k++) w[k] = *reinterpret_cast<const uint32_t *>(rows + (size_t)k * row_bytes + lane_off);
 }
 // four codes of a dword as two pairs of 16-bit integers (codes 0, 1 and codes 2, 3)
 __device__ __forceinline__ void code_cell_pairs(const uint32_t w[16], uint32_t c01[16], uint32_t c23[16]) {
@@ -1592,15 +1594,16 @@ __global__ void __launch_bounds__(256) k_code_cells_kernel(
     const UnitGeom g = unit_geom(W);
     uint8_t *blk = gbuf + (size_t)j * bound;
     uint32_t my_off = 8u;
-    const uint8_t *cell = codes + (size_t)cb * 64 * (size_t)hidden + (size_t)hg * 1024 + (size_t)j * 128 + 4 * t;
+    const uint8_t *rows = codes + (size_t)cb * 64 * (size_t)hidden + (size_t)hg * 1024;      // uniform
+    const uint32_t lane_off = (uint32_t)(j * 128 + 4 * t);
     uint32_t w[16];
-    code_cell_load(cell, (size_t)hidden, w);
+    code_cell_load(rows, (size_t)hidden, lane_off, w);
 #pragma unroll 1
     for (int r = 0; r < 4; r++) {
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         uint32_t c01[16], c23[16];
         code_cell_pairs(w, c01, c23);
-        if (r < 3) code_cell_load(cell + (size_t)(r + 1) * 16 * (size_t)hidden, (size_t)hidden, w);     // travels while the packs are formed
+        if (r < 3) code_cell_load(rows + (size_t)(r + 1) * 16 * (size_t)hidden, (size_t)hidden, lane_off, w);     // travels while the packs are formed
         typename PacksOf<WIDE>::type u;
         uint32_t cmax;
         cell_build(c01, c23, u, cmax);
@@ -1655,7 +1658,7 @@ __global__ void __launch_bounds__(512) v_code_cells_kernel(
     stagger_first_generation(stagger);
     if (tid == 0) s_idx = atomicAdd(&st->ticket, 1u);
     __syncthreads();
-    const uint32_t gidx = s_idx;
+    const uint32_t gidx = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_idx);      // uniform: the rows' addresses become scalar
     if (gidx >= ngroups) return;
     const int j = tid >> 6, rp = (tid >> 5) & 1, t = tid & 31;
     const uint32_t per_row = (uint32_t)hidden / 1024u;
@@ -1666,13 +1669,15 @@ __global__ void __launch_bounds__(512) v_code_cells_kernel(
     for (uint32_t i = tid; i < 64u * (meta / 4u); i += 512)                 // metadata areas start as zeros
         reinterpret_cast<uint32_t *>(gbuf + (size_t)(i / (meta / 4u)) * unit_slot)[i % (meta / 4u)] = 0u;
     uint32_t run_off = 0;
-    const uint8_t *cell = codes + ((size_t)cb * 128 + 16 * rp) * (size_t)hidden + (size_t)hg * 1024 + (size_t)j * 128 + 4 * t;
+    const uint8_t *rows = codes + (size_t)cb * 128 * (size_t)hidden + (size_t)hg * 1024;      // uniform
+    const uint32_t lane_off = (uint32_t)(16 * rp) * (uint32_t)hidden + (uint32_t)(j * 128 + 4 * t);
     __syncthreads();                                       // the metadata zeros are in place before the first OR
 #pragma unroll 1
     for (int it = 0; it < 4; it++) {
-        // (no request ahead: placing the packs holds too many registers, as in v_quant_encode_cells_kernel)
+        // (no request ahead: with sixteen more registers in flight while the packs are placed the kernel needs 142
+        // and a CU holds one workgroup instead of two)
         uint32_t w[16];
-        code_cell_load(cell + (size_t)it * 32 * (size_t)hidden, (size_t)hidden, w);
+        code_cell_load(rows + (size_t)it * 32 * (size_t)hidden, (size_t)hidden, lane_off, w);
         __builtin_amdgcn_s_setprio(PKV_EPRIO_PACK);
         uint32_t c01[16], c23[16];
         code_cell_pairs(w, c01, c23);
